@@ -1,0 +1,177 @@
+/*
+ * ring_abi.h — C ABI of the MI355X (gfx950) per-rank data path of the ring
+ * allreduce / allgather of tensorflow/contrib/mpi_collectives.
+ *
+ * This is the seam the reference keeps inside its plugin between the ring
+ * algorithm (ring.h) and the device primitives (ring.cc / ring.cu.cc):
+ *
+ *     template <typename Device>
+ *     void CopyTensorData(void* dst, void* src, size_t size);        ring.h:44-45
+ *     template <typename Device, typename T>
+ *     void AccumulateTensorData(T* dst, T* src, size_t size);        ring.h:50-51
+ *     cudaStream_t CudaStreamForMPI();                               ring.h:55-57
+ *
+ * restated as plain C: pointers, sizes, an opaque stream handle, an int
+ * status. Differences from the reference seam, all deliberate:
+ *   - every device entry point is ASYNCHRONOUS on the stream it is given; the
+ *     caller synchronises (the reference blocks the host after every call,
+ *     ring.cu.cc:41-45, :60-66);
+ *   - every entry point returns a status (the reference returns void and
+ *     drops CUDA errors);
+ *   - a whole phase of the ring (all n-1 accumulates, all n-1 allgather
+ *     copies) can be issued as ONE launch from a step table, because the
+ *     steps of one rank write disjoint segments (ring.h:183-205, :211-225);
+ *   - nothing allocates device memory unless its name says "create".
+ *
+ * Conventions: `count` is in elements, `bytes` in bytes; a count of 0 with
+ * null pointers is valid and does nothing (an empty tensor reaches the
+ * reference's primitives the same way); pointers are device pointers unless
+ * the parameter is documented as host; element offsets may be any multiple of
+ * the element size (ragged segments break 16-byte alignment and the kernels
+ * handle it). `stream` is a hipStream_t passed as void* (NULL = the default
+ * stream). One thread per stream.
+ */
+#ifndef RING_ABI_H_
+#define RING_ABI_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RING_ABI_VERSION 1
+
+/* Element types: exactly the three the reference registers and dispatches on
+ * (mpi_ops.cc:1120 `Attr("T: {int32, int64, float32}")`, ring.cu.cc:14-20,
+ * mpi_ops.cc:478-508). */
+enum ring_dtype { RING_F32 = 0, RING_I32 = 1, RING_I64 = 2 };
+
+/* Status codes. RING_ERR_HIP: ring_last_hip_error() has the hipError_t. */
+enum ring_status {
+  RING_OK = 0,
+  RING_ERR_DTYPE = 1,    /* not one of ring_dtype ("Invalid tensor type", mpi_ops.cc:844) */
+  RING_ERR_ARGUMENT = 2, /* null pointer with a non-zero size, n < 1, rank out of range ... */
+  RING_ERR_HIP = 3,      /* a HIP runtime call failed */
+  RING_ERR_NO_DEVICE = 4 /* no usable GPU */
+};
+
+int ring_abi_version(void);
+const char* ring_status_string(int status);
+/* hipError_t of the most recent failing HIP call on this thread (0 if none). */
+int ring_last_hip_error(void);
+/* sizeof(T) for a ring_dtype, 0 if the code is not one. */
+size_t ring_dtype_size(int dtype);
+
+/* Launch-shape knobs for measurement runs (process-wide; not needed for
+ * normal use): "unroll" = 16-byte vectors per lane per tile (2, 4, 8),
+ * "nontemporal" = non-temporal stores (0, 1), "blocks_per_cu" = 0 for one
+ * workgroup per tile, k > 0 for a persistent grid of CUs x k workgroups that
+ * stride over the tiles. No counterpart in the reference, whose launch shape
+ * is the constant <<<32, 256>>> (ring.cu.cc:64). */
+int ring_set_option(const char* name, int value);
+
+/* ---- host-side tables (no GPU involved) ---------------------------------- */
+
+/* Segment split of a `count`-element tensor over n ranks — ring.h:150-166:
+ * count/n each, the first count%n segments one more, starts = exclusive
+ * prefix sum. sizes/starts: host arrays of n. */
+int ring_segment_table(size_t count, int n, size_t* sizes, size_t* starts);
+
+/* Elements of the receive buffer an allreduce needs — mpi_ops.cc:1073-1077:
+ * ceil(count / n). */
+size_t ring_temp_elements(size_t count, int n);
+
+/* Allgather segment starts, in elements — ring.h:255-259. rows[k] is rank k's
+ * first dimension; starts: host array of n. */
+int ring_allgather_table(const size_t* rows, int n, size_t elems_per_row,
+                         size_t* starts);
+
+/* Which segments rank r sends / receives at step i (0 <= i < n-1):
+ *   reduce-scatter  send (r-i),   recv (r-i-1)    ring.h:184-185
+ *   allreduce's allgather  send (r-i+1), recv (r-i)   ring.h:212-213
+ *   standalone allgather   send (r-i),   recv (r-i-1) ring.h:280-281
+ * all modulo n. Neighbours are fixed: receive from r-1, send to r+1
+ * (ring.h:171-174). */
+enum ring_phase { RING_PHASE_REDUCE_SCATTER = 0, RING_PHASE_ALLGATHER = 1, RING_PHASE_GATHER = 2 };
+int ring_schedule(int phase, int n, int r, int step, int* send_seg, int* recv_seg);
+
+/* ---- the dedicated stream — CudaStreamForMPI(), mpi_ops.cc:213-230, 582-583,
+ * 872-876: one non-default stream for all ring copies and accumulates, so a
+ * wait on it never waits for unrelated compute. Default priority. ---------- */
+int ring_stream_create(void** stream);
+int ring_stream_destroy(void* stream);
+int ring_stream_synchronize(void* stream);
+
+/* ---- device primitives ---------------------------------------------------- */
+
+/* CopyTensorData<GPUDevice> — ring.cu.cc:41-45 (call sites ring.h:146-148,
+ * 263-266). Device-to-device byte copy by a hand-written kernel; dst and src
+ * must not overlap. */
+int ring_copy_bytes(void* dst, const void* src, size_t bytes, void* stream);
+
+/* AccumulateTensorData<GPUDevice,T> + elemwise_accum<T> — ring.cu.cc:48-69
+ * (call site ring.h:203-204): dst[i] += src[i], one IEEE binary32 add (or one
+ * wrapping integer add) per element. dst and src must not overlap. */
+int ring_accumulate_f32(float* dst, const float* src, size_t count, void* stream);
+int ring_accumulate_i32(int32_t* dst, const int32_t* src, size_t count, void* stream);
+int ring_accumulate_i64(int64_t* dst, const int64_t* src, size_t count, void* stream);
+int ring_accumulate(int dtype, void* dst, const void* src, size_t count, void* stream);
+
+/* The divide of allreduce(average=True) — __init__.py:160-164
+ * `tf.div(summed, cast(size(), dtype))`: in place data[i] = data[i] / divisor,
+ * true (correctly rounded) division for float32, floor division for the
+ * integer types (math_ops.py:982-985). divisor >= 1. */
+int ring_scale(int dtype, void* data, size_t count, int divisor, void* stream);
+
+/* One row of a step table: the segment received at one ring step. `src` is
+ * where the incoming segment lies in device memory (the reference's `temp`
+ * after MPI_Wait, ring.h:189-200, or the neighbour's send buffer itself when
+ * it is directly addressable); `dst_offset` is segment_starts[recv_seg]. */
+typedef struct ring_step {
+  uint64_t dst_offset; /* elements from the start of `buffer` */
+  const void* src;     /* device pointer, any multiple of the element size */
+  uint64_t count;      /* elements; 0 is allowed */
+} ring_step;
+
+/* All the accumulates of a rank's reduce-scatter (ring.h:183-205) in one
+ * launch: for every row, buffer[dst_offset + i] += src[i]. `steps` is a HOST
+ * array of n_steps rows whose destination ranges are pairwise disjoint and
+ * disjoint from every src (true for the n-1 steps of one rank). Any n_steps
+ * >= 0; tables longer than one launch can carry are split internally. */
+int ring_reduce_scatter_steps(void* buffer, const ring_step* steps, int n_steps,
+                              int dtype, void* stream);
+
+/* All the receives of a rank's allgather phase (ring.h:211-225, and
+ * ring.h:279-298 for the standalone allgather) in one launch: for every row,
+ * buffer[dst_offset + i] = src[i]. Same table rules. */
+int ring_allgather_steps(void* buffer, const ring_step* steps, int n_steps,
+                         int dtype, void* stream);
+
+/* ---- tensor fusion (no counterpart in the reference, which issues one
+ * MPIAllreduce per gradient, __init__.py:195-205): k tensors are packed back
+ * to back, in order, without padding, into one buffer that is ring-reduced
+ * as a single tensor and unpacked again. -------------------------------- */
+
+typedef struct ring_fusion_plan ring_fusion_plan;
+
+/* Builds the device-resident offset table for k tensors (`tensors[j]` device
+ * pointer to counts[j] elements; both HOST arrays). Allocates a few KiB of
+ * device memory owned by the plan and copies the table synchronously. Tensor
+ * pointers must stay valid while the plan is used. */
+int ring_fusion_plan_create(const void* const* tensors, const size_t* counts,
+                            int k, int dtype, ring_fusion_plan** plan);
+int ring_fusion_plan_destroy(ring_fusion_plan* plan);
+/* Total elements of the fused buffer (sum of counts). */
+size_t ring_fusion_plan_elements(const ring_fusion_plan* plan);
+/* fused[offset_j + i] = tensors[j][i] for all j. `fused` must be 16-byte
+ * aligned (tensors need only element alignment). */
+int ring_fusion_pack(const ring_fusion_plan* plan, void* fused, void* stream);
+/* tensors[j][i] = fused[offset_j + i] for all j. */
+int ring_fusion_unpack(const ring_fusion_plan* plan, const void* fused, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RING_ABI_H_ */

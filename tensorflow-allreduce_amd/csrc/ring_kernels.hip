@@ -1,0 +1,723 @@
+// Per-rank data path of the ring allreduce / allgather for MI355X (gfx950).
+//
+// Hand-written HIP kernels behind the C ABI of include/ring_abi.h. They take
+// the place of the reference's device primitives
+// (tensorflow/contrib/mpi_collectives/ring.cu.cc:41-69): the D2D copy, and
+// elemwise_accum<<<32,256>>> followed by a host-blocking stream sync at every
+// ring step.
+//
+// Design, in the order it matters for an HBM-bound stream:
+//   * every lane moves 16 bytes per access (global_load/store_dwordx4), a
+//     wave64 touches 1 KiB of contiguous memory per instruction;
+//   * a workgroup is 4 waves; one tile is kUnroll x 256 x 16 B per operand, all
+//     loads of a tile are issued before the first add/store, so each wave
+//     keeps 2*kUnroll KiB in flight;
+//   * workgroups walk the tiles of ALL rows of a step table in one grid-stride
+//     loop, so the n-1 accumulates (or copies) of a rank are one launch, not
+//     n-1 launches and n-1 host syncs;
+//   * stores are 16-byte aligned: up to 3 head elements are peeled per row so
+//     the destination is aligned, the source is read with element-aligned
+//     (possibly 16-byte-unaligned) dwordx4 loads. Ragged segment starts only
+//     cost those few scalar elements;
+//   * streams that are written once and not re-read by this launch use
+//     non-temporal stores;
+//   * LDS is used only by the fusion kernels, for the offset table of a tile
+//     that spans several small tensors.
+// No MFMA: the path is one add per 12 bytes.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <new>
+#include <vector>
+
+#include "ring_abi.h"
+
+namespace {
+
+constexpr int kBlock = 256;   // threads per workgroup: 4 wave64
+constexpr int kMaxRows = 64;  // rows one launch carries in its kernel arguments
+
+thread_local int g_last_hip_error = 0;
+
+inline int hip_fail(hipError_t e) {
+  g_last_hip_error = static_cast<int>(e);
+  return RING_ERR_HIP;
+}
+#define RING_HIP(call)                                   \
+  do {                                                   \
+    hipError_t e_ = (call);                              \
+    if (e_ != hipSuccess) return hip_fail(e_);           \
+  } while (0)
+
+// ---- element / vector types -------------------------------------------------
+
+template <typename T> struct VecOf;
+template <> struct VecOf<float> { typedef float type __attribute__((ext_vector_type(4))); };
+// integers are added as unsigned so overflow wraps (what the reference's
+// hardware add does) instead of being undefined
+template <> struct VecOf<uint32_t> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
+template <> struct VecOf<uint64_t> { typedef uint64_t type __attribute__((ext_vector_type(2))); };
+
+enum Mode { kCopy = 0, kAccumulate = 1 };
+
+// Rows of one launch, passed by value in the kernel arguments (read with
+// scalar loads; uniform per workgroup).
+struct RowTable {
+  int n_rows;
+  uint32_t tile_begin[kMaxRows + 1];  // prefix sum of tiles per row
+  void* dst[kMaxRows];
+  const void* src[kMaxRows];
+  uint64_t count[kMaxRows];  // elements
+};
+
+template <typename T, bool NT>
+__device__ __forceinline__ void store_vec(typename VecOf<T>::type* p, typename VecOf<T>::type v) {
+  if (NT) __builtin_nontemporal_store(v, p); else *p = v;
+}
+
+// One workgroup-tile of a row: vectors [v0, v0 + 256*UNROLL) of the aligned
+// body, plus the row's scalar head (tile 0) and tail (last tile).
+template <typename T, int MODE, int UNROLL, bool NT>
+__device__ __forceinline__ void row_tile(T* __restrict__ dst, const T* __restrict__ src,
+                                         uint64_t count, uint32_t tile, uint32_t tiles_in_row) {
+  typedef typename VecOf<T>::type V;
+  typedef V VU __attribute__((aligned(sizeof(T))));  // element-aligned 16-byte load
+  constexpr uint32_t VEC = 16 / sizeof(T);
+  constexpr uint32_t kTileVecs = kBlock * UNROLL;
+
+  uint64_t head = ((16u - (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(dst)) & 15u)) & 15u) / sizeof(T);
+  if (head > count) head = count;
+  const uint64_t nvec = (count - head) / VEC;
+  const uint32_t tid = threadIdx.x;
+
+  if (tile == 0 && tid < head) {
+    if (MODE == kAccumulate) dst[tid] = dst[tid] + src[tid]; else dst[tid] = src[tid];
+  }
+  if (tile + 1 == tiles_in_row) {
+    const uint64_t tail_start = head + nvec * VEC;
+    const uint64_t e = tail_start + tid;
+    if (e < count) {
+      if (MODE == kAccumulate) dst[e] = dst[e] + src[e]; else dst[e] = src[e];
+    }
+  }
+
+  V* __restrict__ dv = reinterpret_cast<V*>(dst + head);
+  const VU* __restrict__ sv = reinterpret_cast<const VU*>(src + head);
+  const uint64_t v0 = static_cast<uint64_t>(tile) * kTileVecs + tid;
+
+  if (static_cast<uint64_t>(tile + 1) * kTileVecs <= nvec) {
+    V s[UNROLL], d[UNROLL];
+#pragma unroll
+    for (int j = 0; j < UNROLL; j++) s[j] = __builtin_nontemporal_load(&sv[v0 + j * kBlock]);
+    if (MODE == kAccumulate) {
+#pragma unroll
+      for (int j = 0; j < UNROLL; j++) d[j] = __builtin_nontemporal_load(&dv[v0 + j * kBlock]);
+#pragma unroll
+      for (int j = 0; j < UNROLL; j++) s[j] = d[j] + s[j];
+    }
+#pragma unroll
+    for (int j = 0; j < UNROLL; j++) store_vec<T, NT>(&dv[v0 + j * kBlock], s[j]);
+  } else {
+#pragma unroll
+    for (int j = 0; j < UNROLL; j++) {
+      const uint64_t v = v0 + j * kBlock;
+      if (v < nvec) {
+        V s = __builtin_nontemporal_load(&sv[v]);
+        if (MODE == kAccumulate) s = __builtin_nontemporal_load(&dv[v]) + s;
+        store_vec<T, NT>(&dv[v], s);
+      }
+    }
+  }
+}
+
+template <typename T, int MODE, int UNROLL, bool NT>
+__global__ void __launch_bounds__(kBlock) rows_kernel(const RowTable tab) {
+  const uint32_t total = tab.tile_begin[tab.n_rows];
+  for (uint32_t t = blockIdx.x; t < total; t += gridDim.x) {
+    // largest row with tile_begin[row] <= t (uniform: scalar code)
+    int lo = 0, hi = tab.n_rows;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (tab.tile_begin[mid] <= t) lo = mid; else hi = mid;
+    }
+    const uint32_t first = tab.tile_begin[lo];
+    row_tile<T, MODE, UNROLL, NT>(static_cast<T*>(tab.dst[lo]), static_cast<const T*>(tab.src[lo]),
+                                  tab.count[lo], t - first, tab.tile_begin[lo + 1] - first);
+  }
+}
+
+// Byte copy for operands that are not 4-byte compatible (never produced by the
+// three element types; kept so ring_copy_bytes is total).
+__global__ void __launch_bounds__(kBlock) bytes_kernel(uint8_t* __restrict__ dst,
+                                                       const uint8_t* __restrict__ src, uint64_t n) {
+  for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x; i < n;
+       i += static_cast<uint64_t>(gridDim.x) * kBlock)
+    dst[i] = src[i];
+}
+
+// ---- average: sum / n ---------------------------------------------------------
+// tf.div semantics of the reference's allreduce(average=True)
+// (__init__.py:160-164): true division for float32 (a correctly rounded
+// divide, NOT a multiply by 1/n), floor division for the integer types.
+
+template <typename T> struct ScaleOp;
+template <> struct ScaleOp<float> {
+  typedef float V __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ float one(float x, int n) { return x / static_cast<float>(n); }
+};
+template <> struct ScaleOp<int32_t> {
+  typedef int32_t V __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ int32_t one(int32_t x, int n) {
+    int32_t q = x / n;
+    return q - ((x % n != 0) && (x < 0));  // n > 0: floor differs from trunc only for x < 0
+  }
+};
+template <> struct ScaleOp<int64_t> {
+  typedef int64_t V __attribute__((ext_vector_type(2)));
+  static __device__ __forceinline__ int64_t one(int64_t x, int n) {
+    int64_t q = x / n;
+    return q - ((x % n != 0) && (x < 0));
+  }
+};
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock) scale_kernel(T* __restrict__ data, uint64_t count, int n) {
+  typedef typename ScaleOp<T>::V V;
+  constexpr uint32_t VEC = 16 / sizeof(T);
+  uint64_t head = ((16u - (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(data)) & 15u)) & 15u) / sizeof(T);
+  if (head > count) head = count;
+  const uint64_t nvec = (count - head) / VEC;
+  const uint64_t gtid = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  const uint64_t gsize = static_cast<uint64_t>(gridDim.x) * kBlock;
+  if (gtid < head) data[gtid] = ScaleOp<T>::one(data[gtid], n);
+  const uint64_t tail_at = head + nvec * VEC + gtid;
+  if (tail_at < count) data[tail_at] = ScaleOp<T>::one(data[tail_at], n);
+  V* __restrict__ dv = reinterpret_cast<V*>(data + head);
+  for (uint64_t v = gtid; v < nvec; v += gsize) {
+    V x = dv[v];
+#pragma unroll
+    for (uint32_t c = 0; c < VEC; c++) x[c] = ScaleOp<T>::one(x[c], n);
+    dv[v] = x;
+  }
+}
+
+// ---- tensor fusion: pack / unpack -----------------------------------------------
+// The fused buffer is cut into tiles of 1024 16-byte groups. A tile that lies
+// inside one tensor (all of the bytes of a ResNet-sized gradient set, bar a few
+// hundred KiB) is a plain aligned-store span copy. A tile that spans several
+// tensors stages the offsets and base pointers of just those tensors in LDS
+// and every lane finds the tensor of its 16-byte group by binary search there.
+
+constexpr uint32_t kFusionTileVecs = 1024;
+constexpr uint32_t kFusionLdsCap = 512;  // tensors of one tile staged in LDS
+
+template <typename T, bool PACK, bool NT>
+__global__ void __launch_bounds__(kBlock)
+fusion_kernel(T* __restrict__ fused, const uint64_t* __restrict__ offsets, T* const* __restrict__ ptrs,
+              const uint32_t* __restrict__ tile_first, const uint32_t* __restrict__ tile_last,
+              uint32_t ntiles, uint64_t total) {
+  typedef typename VecOf<T>::type V;
+  typedef V VU __attribute__((aligned(sizeof(T))));
+  constexpr uint32_t VEC = 16 / sizeof(T);
+  constexpr uint64_t kTileElems = static_cast<uint64_t>(kFusionTileVecs) * VEC;
+  __shared__ uint64_t s_off[kFusionLdsCap + 1];
+  __shared__ T* s_ptr[kFusionLdsCap];
+
+  for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+    const uint64_t e0 = static_cast<uint64_t>(tile) * kTileElems;
+    const uint64_t e1 = (e0 + kTileElems < total) ? e0 + kTileElems : total;
+    const uint32_t t0 = tile_first[tile];
+    const uint32_t t1 = tile_last[tile];
+    if (t0 == t1) {
+      T* tensor = ptrs[t0] + (e0 - offsets[t0]);
+      if (PACK) row_tile<T, kCopy, 4, NT>(fused + e0, tensor, e1 - e0, 0, 1);
+      else row_tile<T, kCopy, 4, NT>(tensor, fused + e0, e1 - e0, 0, 1);
+      continue;
+    }
+    const uint32_t span = t1 - t0 + 1;
+    const uint64_t* off_tab = offsets + t0;
+    T* const* ptr_tab = ptrs + t0;
+    const bool staged = span <= kFusionLdsCap;  // uniform per workgroup
+    if (staged) {
+      for (uint32_t i = threadIdx.x; i <= span; i += kBlock) s_off[i] = offsets[t0 + i];
+      for (uint32_t i = threadIdx.x; i < span; i += kBlock) s_ptr[i] = ptrs[t0 + i];
+      __syncthreads();
+      off_tab = s_off;
+      ptr_tab = s_ptr;
+    }
+    const uint32_t ngroups = static_cast<uint32_t>((e1 - e0 + VEC - 1) / VEC);
+    for (uint32_t g = threadIdx.x; g < ngroups; g += kBlock) {
+      uint64_t e = e0 + static_cast<uint64_t>(g) * VEC;
+      uint32_t lo = 0, hi = span;  // off_tab[lo] <= e < off_tab[hi]
+      while (hi - lo > 1) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (off_tab[mid] <= e) lo = mid; else hi = mid;
+      }
+      if (e + VEC <= off_tab[lo + 1] && e + VEC <= e1) {
+        T* tensor = ptr_tab[lo] + (e - off_tab[lo]);
+        if (PACK) store_vec<T, NT>(reinterpret_cast<V*>(fused + e), *reinterpret_cast<const VU*>(tensor));
+        else *reinterpret_cast<VU*>(tensor) = *reinterpret_cast<const V*>(fused + e);
+      } else {
+        const uint64_t end = (e + VEC < e1) ? e + VEC : e1;
+        for (; e < end; e++) {
+          while (e >= off_tab[lo + 1]) lo++;
+          T* tensor = ptr_tab[lo] + (e - off_tab[lo]);
+          if (PACK) fused[e] = *tensor; else *tensor = fused[e];
+        }
+      }
+    }
+    if (staged) __syncthreads();  // before the next tile overwrites the table
+  }
+}
+
+// ---- launch configuration -----------------------------------------------------
+
+struct Tuning {
+  int unroll = 4;          // 16-byte vectors per lane per tile: 2, 4 or 8
+  int nontemporal = 1;     // non-temporal stores
+  int blocks_per_cu = 0;   // 0: one workgroup per tile; >0: persistent grid of CUs x this
+};
+Tuning g_tuning;
+
+struct DeviceInfo {
+  bool ok = false;
+  int cus = 0;
+};
+
+int device_info(DeviceInfo* out) {
+  static thread_local DeviceInfo cached[64];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) { hip_fail(e); return RING_ERR_NO_DEVICE; }
+  if (dev < 0 || dev >= 64) return RING_ERR_NO_DEVICE;
+  if (!cached[dev].ok) {
+    int cus = 0;
+    RING_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    cached[dev].cus = cus > 0 ? cus : 256;
+    cached[dev].ok = true;
+  }
+  *out = cached[dev];
+  return RING_OK;
+}
+
+template <typename T, int MODE>
+int launch_rows_typed(const RowTable& tab, uint32_t grid, hipStream_t stream) {
+  const bool nt = g_tuning.nontemporal != 0;
+#define RING_LAUNCH(U, N) \
+  hipLaunchKernelGGL((rows_kernel<T, MODE, U, N>), dim3(grid), dim3(kBlock), 0, stream, tab)
+  switch (g_tuning.unroll) {
+    case 2: if (nt) RING_LAUNCH(2, true); else RING_LAUNCH(2, false); break;
+    case 8: if (nt) RING_LAUNCH(8, true); else RING_LAUNCH(8, false); break;
+    default: if (nt) RING_LAUNCH(4, true); else RING_LAUNCH(4, false); break;
+  }
+#undef RING_LAUNCH
+  RING_HIP(hipGetLastError());
+  return RING_OK;
+}
+
+struct HostRow {
+  void* dst;
+  const void* src;
+  uint64_t count;  // elements of `esz` bytes
+};
+
+// Launches rows (any number) in groups of kMaxRows. esz: 4 or 8.
+template <int MODE>
+int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, hipStream_t stream) {
+  const int unroll = (g_tuning.unroll == 2 || g_tuning.unroll == 8) ? g_tuning.unroll : 4;
+  const uint64_t tile_vecs = static_cast<uint64_t>(kBlock) * unroll;
+  const uint64_t vec = 16 / esz;
+  DeviceInfo info;
+  size_t i = 0;
+  while (i < n_rows) {
+    RowTable tab;
+    tab.n_rows = 0;
+    tab.tile_begin[0] = 0;
+    uint64_t tiles = 0;
+    while (i < n_rows && tab.n_rows < kMaxRows) {
+      const HostRow& r = rows[i];
+      if (r.count == 0) { i++; continue; }
+      const uintptr_t d = reinterpret_cast<uintptr_t>(r.dst);
+      uint64_t head = ((16u - (d & 15u)) & 15u) / esz;
+      if (head > r.count) head = r.count;
+      const uint64_t nvec = (r.count - head) / vec;
+      uint64_t t = (nvec + tile_vecs - 1) / tile_vecs;
+      if (t == 0) t = 1;
+      if (tiles + t > 0x7fffffffull) {
+        if (tab.n_rows == 0) return RING_ERR_ARGUMENT;  // a single row beyond 2^31 tiles
+        break;
+      }
+      const int k = tab.n_rows++;
+      tab.dst[k] = r.dst;
+      tab.src[k] = r.src;
+      tab.count[k] = r.count;
+      tiles += t;
+      tab.tile_begin[k + 1] = static_cast<uint32_t>(tiles);
+      i++;
+    }
+    if (tab.n_rows == 0) continue;
+    uint32_t grid = static_cast<uint32_t>(tiles);
+    if (g_tuning.blocks_per_cu > 0) {
+      int rc = device_info(&info);
+      if (rc != RING_OK) return rc;
+      const uint64_t cap = static_cast<uint64_t>(info.cus) * g_tuning.blocks_per_cu;
+      if (grid > cap) grid = static_cast<uint32_t>(cap);
+    }
+    int rc;
+    if (esz == 8) rc = launch_rows_typed<uint64_t, MODE>(tab, grid, stream);
+    else if (is_float && MODE == kAccumulate) rc = launch_rows_typed<float, MODE>(tab, grid, stream);
+    else rc = launch_rows_typed<uint32_t, MODE>(tab, grid, stream);
+    if (rc != RING_OK) return rc;
+  }
+  return RING_OK;
+}
+
+inline bool dtype_ok(int dtype) { return dtype == RING_F32 || dtype == RING_I32 || dtype == RING_I64; }
+inline size_t dtype_size(int dtype) { return dtype == RING_I64 ? 8 : (dtype_ok(dtype) ? 4 : 0); }
+
+int steps_common(void* buffer, const ring_step* steps, int n_steps, int dtype, void* stream, bool accumulate) {
+  if (!dtype_ok(dtype)) return RING_ERR_DTYPE;
+  if (n_steps < 0) return RING_ERR_ARGUMENT;
+  if (n_steps == 0) return RING_OK;
+  if (!steps) return RING_ERR_ARGUMENT;
+  const size_t esz = dtype_size(dtype);
+  std::vector<HostRow> rows;
+  rows.reserve(static_cast<size_t>(n_steps));
+  for (int i = 0; i < n_steps; i++) {
+    if (steps[i].count == 0) continue;
+    if (!buffer || !steps[i].src) return RING_ERR_ARGUMENT;
+    char* d = static_cast<char*>(buffer) + steps[i].dst_offset * esz;
+    if ((reinterpret_cast<uintptr_t>(d) | reinterpret_cast<uintptr_t>(steps[i].src)) & (esz - 1))
+      return RING_ERR_ARGUMENT;
+    rows.push_back(HostRow{d, steps[i].src, steps[i].count});
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (accumulate) return launch_rows<kAccumulate>(rows.data(), rows.size(), esz, dtype == RING_F32, s);
+  return launch_rows<kCopy>(rows.data(), rows.size(), esz, false, s);
+}
+
+}  // namespace
+
+// Host side of a fusion plan. The device table is one allocation:
+// offsets[m+1] | ptrs[m] | tile_first[ntiles] | tile_last[ntiles].
+struct ring_fusion_plan {
+  int dtype = 0;
+  size_t esz = 0;
+  int device = 0;
+  uint32_t m = 0;        // non-empty tensors
+  uint32_t ntiles = 0;
+  uint64_t total = 0;    // elements
+  void* d_table = nullptr;
+  uint64_t* d_offsets = nullptr;
+  void** d_ptrs = nullptr;
+  uint32_t* d_tile_first = nullptr;
+  uint32_t* d_tile_last = nullptr;
+};
+
+namespace {
+
+template <typename T, bool PACK>
+int launch_fusion(const ring_fusion_plan* p, void* fused, hipStream_t stream) {
+  uint32_t grid = p->ntiles;
+  if (g_tuning.blocks_per_cu > 0) {
+    DeviceInfo info;
+    int rc = device_info(&info);
+    if (rc != RING_OK) return rc;
+    const uint64_t cap = static_cast<uint64_t>(info.cus) * g_tuning.blocks_per_cu;
+    if (grid > cap) grid = static_cast<uint32_t>(cap);
+  }
+  if (g_tuning.nontemporal)
+    hipLaunchKernelGGL((fusion_kernel<T, PACK, true>), dim3(grid), dim3(kBlock), 0, stream,
+                       static_cast<T*>(fused), p->d_offsets, reinterpret_cast<T* const*>(p->d_ptrs),
+                       p->d_tile_first, p->d_tile_last, p->ntiles, p->total);
+  else
+    hipLaunchKernelGGL((fusion_kernel<T, PACK, false>), dim3(grid), dim3(kBlock), 0, stream,
+                       static_cast<T*>(fused), p->d_offsets, reinterpret_cast<T* const*>(p->d_ptrs),
+                       p->d_tile_first, p->d_tile_last, p->ntiles, p->total);
+  RING_HIP(hipGetLastError());
+  return RING_OK;
+}
+
+int fusion_run(const ring_fusion_plan* p, void* fused, void* stream, bool pack) {
+  if (!p) return RING_ERR_ARGUMENT;
+  if (p->total == 0) return RING_OK;
+  if (!fused || (reinterpret_cast<uintptr_t>(fused) & 15u)) return RING_ERR_ARGUMENT;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (p->esz == 8) return pack ? launch_fusion<uint64_t, true>(p, fused, s) : launch_fusion<uint64_t, false>(p, fused, s);
+  return pack ? launch_fusion<uint32_t, true>(p, fused, s) : launch_fusion<uint32_t, false>(p, fused, s);
+}
+
+}  // namespace
+
+// =============================================================================
+// C ABI
+// =============================================================================
+extern "C" {
+
+int ring_abi_version(void) { return RING_ABI_VERSION; }
+
+const char* ring_status_string(int status) {
+  switch (status) {
+    case RING_OK: return "ok";
+    case RING_ERR_DTYPE: return "Invalid tensor type passed.";
+    case RING_ERR_ARGUMENT: return "invalid argument";
+    case RING_ERR_HIP: return "HIP runtime call failed";
+    case RING_ERR_NO_DEVICE: return "no usable GPU";
+    default: return "unknown status";
+  }
+}
+
+int ring_last_hip_error(void) { return g_last_hip_error; }
+
+size_t ring_dtype_size(int dtype) { return dtype_size(dtype); }
+
+// Tuning knobs for measurement runs; not part of the drop-in surface.
+// name: "unroll" (2|4|8), "nontemporal" (0|1), "blocks_per_cu" (0 = one
+// workgroup per tile).
+int ring_set_option(const char* name, int value) {
+  if (!name) return RING_ERR_ARGUMENT;
+  if (!strcmp(name, "unroll")) {
+    if (value != 2 && value != 4 && value != 8) return RING_ERR_ARGUMENT;
+    g_tuning.unroll = value;
+  } else if (!strcmp(name, "nontemporal")) {
+    g_tuning.nontemporal = value ? 1 : 0;
+  } else if (!strcmp(name, "blocks_per_cu")) {
+    if (value < 0 || value > 64) return RING_ERR_ARGUMENT;
+    g_tuning.blocks_per_cu = value;
+  } else {
+    return RING_ERR_ARGUMENT;
+  }
+  return RING_OK;
+}
+
+// ---- host tables ------------------------------------------------------------
+
+int ring_segment_table(size_t count, int n, size_t* sizes, size_t* starts) {
+  if (n < 1 || !sizes || !starts) return RING_ERR_ARGUMENT;
+  const size_t un = static_cast<size_t>(n);
+  const size_t q = count / un, rem = count % un;
+  size_t at = 0;
+  for (size_t i = 0; i < un; i++) {
+    sizes[i] = q + (i < rem ? 1 : 0);
+    starts[i] = at;
+    at += sizes[i];
+  }
+  return RING_OK;
+}
+
+size_t ring_temp_elements(size_t count, int n) {
+  if (n < 1) return 0;
+  const size_t un = static_cast<size_t>(n);
+  return count / un + (count % un ? 1 : 0);
+}
+
+int ring_allgather_table(const size_t* rows, int n, size_t elems_per_row, size_t* starts) {
+  if (n < 1 || !rows || !starts) return RING_ERR_ARGUMENT;
+  size_t at = 0;
+  for (int i = 0; i < n; i++) {
+    starts[i] = at;
+    at += elems_per_row * rows[i];
+  }
+  return RING_OK;
+}
+
+int ring_schedule(int phase, int n, int r, int step, int* send_seg, int* recv_seg) {
+  if (n < 1 || r < 0 || r >= n || step < 0 || step >= n - 1 || !send_seg || !recv_seg)
+    return RING_ERR_ARGUMENT;
+  int send, recv;
+  switch (phase) {
+    case RING_PHASE_REDUCE_SCATTER:
+    case RING_PHASE_GATHER:
+      send = r - step; recv = r - step - 1; break;
+    case RING_PHASE_ALLGATHER:
+      send = r - step + 1; recv = r - step; break;
+    default: return RING_ERR_ARGUMENT;
+  }
+  *send_seg = ((send % n) + n) % n;
+  *recv_seg = ((recv % n) + n) % n;
+  return RING_OK;
+}
+
+// ---- stream -------------------------------------------------------------------
+
+int ring_stream_create(void** stream) {
+  if (!stream) return RING_ERR_ARGUMENT;
+  hipStream_t s = nullptr;
+  RING_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+  *stream = s;
+  return RING_OK;
+}
+
+int ring_stream_destroy(void* stream) {
+  if (!stream) return RING_OK;
+  RING_HIP(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+  return RING_OK;
+}
+
+int ring_stream_synchronize(void* stream) {
+  RING_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  return RING_OK;
+}
+
+// ---- primitives -----------------------------------------------------------------
+
+int ring_copy_bytes(void* dst, const void* src, size_t bytes, void* stream) {
+  if (bytes == 0) return RING_OK;
+  if (!dst || !src) return RING_ERR_ARGUMENT;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const uintptr_t all = reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src) | bytes;
+  if ((all & 3u) == 0) {
+    HostRow row{dst, src, bytes / 4};
+    return launch_rows<kCopy>(&row, 1, 4, false, s);
+  }
+  uint64_t blocks = (bytes + kBlock - 1) / kBlock;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(bytes_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, s,
+                     static_cast<uint8_t*>(dst), static_cast<const uint8_t*>(src),
+                     static_cast<uint64_t>(bytes));
+  RING_HIP(hipGetLastError());
+  return RING_OK;
+}
+
+int ring_accumulate(int dtype, void* dst, const void* src, size_t count, void* stream) {
+  if (!dtype_ok(dtype)) return RING_ERR_DTYPE;
+  if (count == 0) return RING_OK;
+  if (!dst || !src) return RING_ERR_ARGUMENT;
+  const size_t esz = dtype_size(dtype);
+  if ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & (esz - 1))
+    return RING_ERR_ARGUMENT;
+  HostRow row{dst, src, count};
+  return launch_rows<kAccumulate>(&row, 1, esz, dtype == RING_F32, static_cast<hipStream_t>(stream));
+}
+
+int ring_accumulate_f32(float* dst, const float* src, size_t count, void* stream) {
+  return ring_accumulate(RING_F32, dst, src, count, stream);
+}
+int ring_accumulate_i32(int32_t* dst, const int32_t* src, size_t count, void* stream) {
+  return ring_accumulate(RING_I32, dst, src, count, stream);
+}
+int ring_accumulate_i64(int64_t* dst, const int64_t* src, size_t count, void* stream) {
+  return ring_accumulate(RING_I64, dst, src, count, stream);
+}
+
+int ring_reduce_scatter_steps(void* buffer, const ring_step* steps, int n_steps, int dtype, void* stream) {
+  return steps_common(buffer, steps, n_steps, dtype, stream, true);
+}
+
+int ring_allgather_steps(void* buffer, const ring_step* steps, int n_steps, int dtype, void* stream) {
+  return steps_common(buffer, steps, n_steps, dtype, stream, false);
+}
+
+int ring_scale(int dtype, void* data, size_t count, int divisor, void* stream) {
+  if (!dtype_ok(dtype)) return RING_ERR_DTYPE;
+  if (divisor < 1) return RING_ERR_ARGUMENT;
+  if (count == 0) return RING_OK;
+  if (!data || (reinterpret_cast<uintptr_t>(data) & (dtype_size(dtype) - 1))) return RING_ERR_ARGUMENT;
+  const uint64_t vecs = count / (16 / dtype_size(dtype)) + 1;
+  uint64_t blocks = (vecs + kBlock - 1) / kBlock;
+  if (blocks > 16384) blocks = 16384;
+  const dim3 grid(static_cast<uint32_t>(blocks)), block(kBlock);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (dtype) {
+    case RING_F32: hipLaunchKernelGGL(scale_kernel<float>, grid, block, 0, s, static_cast<float*>(data), static_cast<uint64_t>(count), divisor); break;
+    case RING_I32: hipLaunchKernelGGL(scale_kernel<int32_t>, grid, block, 0, s, static_cast<int32_t*>(data), static_cast<uint64_t>(count), divisor); break;
+    default: hipLaunchKernelGGL(scale_kernel<int64_t>, grid, block, 0, s, static_cast<int64_t*>(data), static_cast<uint64_t>(count), divisor); break;
+  }
+  RING_HIP(hipGetLastError());
+  return RING_OK;
+}
+
+// ---- fusion ------------------------------------------------------------------------
+
+int ring_fusion_plan_create(const void* const* tensors, const size_t* counts, int k, int dtype,
+                            ring_fusion_plan** plan) {
+  if (!plan) return RING_ERR_ARGUMENT;
+  *plan = nullptr;
+  if (!dtype_ok(dtype)) return RING_ERR_DTYPE;
+  if (k < 0 || (k > 0 && (!tensors || !counts))) return RING_ERR_ARGUMENT;
+  const size_t esz = dtype_size(dtype);
+  const uint64_t tile_elems = static_cast<uint64_t>(kFusionTileVecs) * (16 / esz);
+
+  std::vector<uint64_t> offsets;
+  std::vector<void*> ptrs;
+  uint64_t total = 0;
+  for (int j = 0; j < k; j++) {
+    if (counts[j] == 0) continue;  // empty tensors occupy nothing in the fused buffer
+    if (!tensors[j] || (reinterpret_cast<uintptr_t>(tensors[j]) & (esz - 1))) return RING_ERR_ARGUMENT;
+    offsets.push_back(total);
+    ptrs.push_back(const_cast<void*>(tensors[j]));
+    total += counts[j];
+  }
+  offsets.push_back(total);
+  const uint64_t ntiles64 = (total + tile_elems - 1) / tile_elems;
+  if (ntiles64 > 0x7fffffffull || ptrs.size() > 0x7fffffffull) return RING_ERR_ARGUMENT;
+
+  ring_fusion_plan* p = new (std::nothrow) ring_fusion_plan();
+  if (!p) return RING_ERR_ARGUMENT;
+  p->dtype = dtype;
+  p->esz = esz;
+  p->m = static_cast<uint32_t>(ptrs.size());
+  p->ntiles = static_cast<uint32_t>(ntiles64);
+  p->total = total;
+  if (total == 0) { *plan = p; return RING_OK; }
+
+  std::vector<uint32_t> first(p->ntiles), last(p->ntiles);
+  uint32_t t = 0;
+  for (uint32_t tile = 0; tile < p->ntiles; tile++) {
+    const uint64_t e0 = static_cast<uint64_t>(tile) * tile_elems;
+    const uint64_t e1 = (e0 + tile_elems < total) ? e0 + tile_elems : total;
+    while (offsets[t + 1] <= e0) t++;
+    first[tile] = t;
+    uint32_t u = t;
+    while (offsets[u + 1] < e1) u++;
+    last[tile] = u;
+  }
+
+  const size_t b_off = offsets.size() * sizeof(uint64_t);
+  const size_t b_ptr = ptrs.size() * sizeof(void*);
+  const size_t b_tile = static_cast<size_t>(p->ntiles) * sizeof(uint32_t);
+  std::vector<char> host(b_off + b_ptr + 2 * b_tile);
+  memcpy(host.data(), offsets.data(), b_off);
+  memcpy(host.data() + b_off, ptrs.data(), b_ptr);
+  memcpy(host.data() + b_off + b_ptr, first.data(), b_tile);
+  memcpy(host.data() + b_off + b_ptr + b_tile, last.data(), b_tile);
+
+  hipError_t e = hipGetDevice(&p->device);
+  if (e == hipSuccess) e = hipMalloc(&p->d_table, host.size());
+  if (e == hipSuccess) e = hipMemcpy(p->d_table, host.data(), host.size(), hipMemcpyHostToDevice);
+  if (e != hipSuccess) {
+    if (p->d_table) (void)hipFree(p->d_table);
+    delete p;
+    return hip_fail(e);
+  }
+  char* base = static_cast<char*>(p->d_table);
+  p->d_offsets = reinterpret_cast<uint64_t*>(base);
+  p->d_ptrs = reinterpret_cast<void**>(base + b_off);
+  p->d_tile_first = reinterpret_cast<uint32_t*>(base + b_off + b_ptr);
+  p->d_tile_last = reinterpret_cast<uint32_t*>(base + b_off + b_ptr + b_tile);
+  *plan = p;
+  return RING_OK;
+}
+
+int ring_fusion_plan_destroy(ring_fusion_plan* plan) {
+  if (!plan) return RING_OK;
+  hipError_t e = plan->d_table ? hipFree(plan->d_table) : hipSuccess;
+  delete plan;
+  if (e != hipSuccess) return hip_fail(e);
+  return RING_OK;
+}
+
+size_t ring_fusion_plan_elements(const ring_fusion_plan* plan) { return plan ? plan->total : 0; }
+
+int ring_fusion_pack(const ring_fusion_plan* plan, void* fused, void* stream) {
+  return fusion_run(plan, fused, stream, true);
+}
+
+int ring_fusion_unpack(const ring_fusion_plan* plan, const void* fused, void* stream) {
+  return fusion_run(plan, const_cast<void*>(fused), stream, false);
+}
+
+}  // extern "C"

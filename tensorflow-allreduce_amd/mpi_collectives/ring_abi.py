@@ -1,0 +1,214 @@
+"""ctypes binding of the C ABI in include/ring_abi.h (lib/libring_hip.so).
+
+The library holds the hand-written gfx950 kernels of the ring's per-rank data
+path. There is no CPU fallback: if the library is missing, or an entry point
+fails, a RingError is raised.
+"""
+import ctypes
+import os
+
+F32, I32, I64 = 0, 1, 2
+DTYPE_SIZE = {F32: 4, I32: 4, I64: 8}
+PHASE_REDUCE_SCATTER, PHASE_ALLGATHER, PHASE_GATHER = 0, 1, 2
+
+_PKG_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(_PKG_ROOT, "lib", "libring_hip.so")
+
+# Every symbol include/ring_abi.h declares.
+EXPORTS = (
+    "ring_abi_version", "ring_status_string", "ring_last_hip_error", "ring_dtype_size",
+    "ring_set_option", "ring_segment_table", "ring_temp_elements", "ring_allgather_table",
+    "ring_schedule", "ring_stream_create", "ring_stream_destroy", "ring_stream_synchronize",
+    "ring_copy_bytes", "ring_accumulate_f32", "ring_accumulate_i32", "ring_accumulate_i64",
+    "ring_accumulate", "ring_reduce_scatter_steps", "ring_allgather_steps",
+    "ring_fusion_plan_create", "ring_fusion_plan_destroy", "ring_fusion_plan_elements",
+    "ring_fusion_pack", "ring_fusion_unpack", "ring_scale",
+)
+
+
+class RingError(RuntimeError):
+    def __init__(self, status, where):
+        self.status = status
+        msg = "%s: %s (status %d" % (where, status_string(status), status)
+        if status == 3:
+            msg += ", hipError %d" % lib().ring_last_hip_error()
+        super().__init__(msg + ")")
+
+
+class Step(ctypes.Structure):
+    """ring_step: one received segment of a step table."""
+    _fields_ = [("dst_offset", ctypes.c_uint64), ("src", ctypes.c_void_p),
+                ("count", ctypes.c_uint64)]
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "%s is missing: build it with `python tensorflow-allreduce_amd/build.py` "
+                "(the ring data path has no CPU fallback)" % LIB_PATH)
+        L = ctypes.CDLL(LIB_PATH)
+        ci, sz, vp = ctypes.c_int, ctypes.c_size_t, ctypes.c_void_p
+        psz = ctypes.POINTER(ctypes.c_size_t)
+        pint = ctypes.POINTER(ctypes.c_int)
+        sig = {
+            "ring_abi_version": (ci, []),
+            "ring_status_string": (ctypes.c_char_p, [ci]),
+            "ring_last_hip_error": (ci, []),
+            "ring_dtype_size": (sz, [ci]),
+            "ring_set_option": (ci, [ctypes.c_char_p, ci]),
+            "ring_segment_table": (ci, [sz, ci, psz, psz]),
+            "ring_temp_elements": (sz, [sz, ci]),
+            "ring_allgather_table": (ci, [psz, ci, sz, psz]),
+            "ring_schedule": (ci, [ci, ci, ci, ci, pint, pint]),
+            "ring_stream_create": (ci, [ctypes.POINTER(vp)]),
+            "ring_stream_destroy": (ci, [vp]),
+            "ring_stream_synchronize": (ci, [vp]),
+            "ring_copy_bytes": (ci, [vp, vp, sz, vp]),
+            "ring_accumulate_f32": (ci, [vp, vp, sz, vp]),
+            "ring_accumulate_i32": (ci, [vp, vp, sz, vp]),
+            "ring_accumulate_i64": (ci, [vp, vp, sz, vp]),
+            "ring_accumulate": (ci, [ci, vp, vp, sz, vp]),
+            "ring_reduce_scatter_steps": (ci, [vp, ctypes.POINTER(Step), ci, ci, vp]),
+            "ring_allgather_steps": (ci, [vp, ctypes.POINTER(Step), ci, ci, vp]),
+            "ring_fusion_plan_create": (ci, [ctypes.POINTER(vp), psz, ci, ci, ctypes.POINTER(vp)]),
+            "ring_fusion_plan_destroy": (ci, [vp]),
+            "ring_fusion_plan_elements": (sz, [vp]),
+            "ring_fusion_pack": (ci, [vp, vp, vp]),
+            "ring_fusion_unpack": (ci, [vp, vp, vp]),
+            "ring_scale": (ci, [ci, vp, sz, ci, vp]),
+        }
+        for name in EXPORTS:
+            fn = getattr(L, name)          # AttributeError if the symbol is missing
+            fn.restype, fn.argtypes = sig[name]
+        if L.ring_abi_version() != 1:
+            raise RuntimeError("libring_hip.so has ABI version %d, expected 1" % L.ring_abi_version())
+        _lib = L
+    return _lib
+
+
+def status_string(status):
+    return lib().ring_status_string(status).decode()
+
+
+def check(status, where):
+    if status != 0:
+        raise RingError(status, where)
+
+
+def set_option(name, value):
+    check(lib().ring_set_option(name.encode(), int(value)), "ring_set_option(%s)" % name)
+
+
+# ---- host tables ----------------------------------------------------------------
+
+def segment_table(count, n):
+    sizes = (ctypes.c_size_t * max(n, 1))()
+    starts = (ctypes.c_size_t * max(n, 1))()
+    check(lib().ring_segment_table(count, n, sizes, starts), "ring_segment_table")
+    return list(sizes), list(starts)
+
+
+def temp_elements(count, n):
+    return int(lib().ring_temp_elements(count, n))
+
+
+def allgather_table(rows, elems_per_row):
+    n = len(rows)
+    r = (ctypes.c_size_t * max(n, 1))(*rows)
+    starts = (ctypes.c_size_t * max(n, 1))()
+    check(lib().ring_allgather_table(r, n, elems_per_row, starts), "ring_allgather_table")
+    return list(starts)[:n]
+
+
+def schedule(phase, n, r, step):
+    send, recv = ctypes.c_int(), ctypes.c_int()
+    check(lib().ring_schedule(phase, n, r, step, ctypes.byref(send), ctypes.byref(recv)),
+          "ring_schedule")
+    return send.value, recv.value
+
+
+# ---- stream ---------------------------------------------------------------------
+
+def stream_create():
+    s = ctypes.c_void_p()
+    check(lib().ring_stream_create(ctypes.byref(s)), "ring_stream_create")
+    return s.value
+
+
+def stream_destroy(stream):
+    check(lib().ring_stream_destroy(stream), "ring_stream_destroy")
+
+
+def stream_synchronize(stream):
+    check(lib().ring_stream_synchronize(stream), "ring_stream_synchronize")
+
+
+# ---- device primitives (raw pointers) ---------------------------------------------
+
+def copy_bytes(dst, src, nbytes, stream):
+    check(lib().ring_copy_bytes(dst, src, nbytes, stream), "ring_copy_bytes")
+
+
+def accumulate(dtype, dst, src, count, stream):
+    check(lib().ring_accumulate(dtype, dst, src, count, stream), "ring_accumulate")
+
+
+def make_steps(rows):
+    """rows: iterable of (dst_offset_elems, src_ptr, count) -> ctypes array."""
+    rows = list(rows)
+    arr = (Step * max(len(rows), 1))()
+    for i, (off, src, cnt) in enumerate(rows):
+        arr[i].dst_offset, arr[i].src, arr[i].count = off, src, cnt
+    return arr, len(rows)
+
+
+def reduce_scatter_steps(buffer, steps, n_steps, dtype, stream):
+    check(lib().ring_reduce_scatter_steps(buffer, steps, n_steps, dtype, stream),
+          "ring_reduce_scatter_steps")
+
+
+def allgather_steps(buffer, steps, n_steps, dtype, stream):
+    check(lib().ring_allgather_steps(buffer, steps, n_steps, dtype, stream),
+          "ring_allgather_steps")
+
+
+def scale(dtype, data, count, divisor, stream):
+    check(lib().ring_scale(dtype, data, count, divisor, stream), "ring_scale")
+
+
+class FusionPlan:
+    """Offset table of k tensors packed back to back (ring_fusion_plan)."""
+
+    def __init__(self, ptrs, counts, dtype):
+        k = len(ptrs)
+        p = (ctypes.c_void_p * max(k, 1))(*ptrs)
+        c = (ctypes.c_size_t * max(k, 1))(*counts)
+        h = ctypes.c_void_p()
+        check(lib().ring_fusion_plan_create(p, c, k, dtype, ctypes.byref(h)),
+              "ring_fusion_plan_create")
+        self._h = h.value
+        self.dtype = dtype
+        self.elements = int(lib().ring_fusion_plan_elements(self._h))
+
+    def pack(self, fused, stream):
+        check(lib().ring_fusion_pack(self._h, fused, stream), "ring_fusion_pack")
+
+    def unpack(self, fused, stream):
+        check(lib().ring_fusion_unpack(self._h, fused, stream), "ring_fusion_unpack")
+
+    def close(self):
+        if self._h:
+            check(lib().ring_fusion_plan_destroy(self._h), "ring_fusion_plan_destroy")
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

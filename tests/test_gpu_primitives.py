@@ -1,0 +1,259 @@
+"""GPU parity of the device primitives behind the C ABI against the CPU oracle:
+accumulate (ring.cu.cc:48-69), copy (ring.cu.cc:41-45), the batched step
+tables, the average divide and fusion pack/unpack. Integer and float32 results
+must match bit for bit."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import gpu_util as G
+from gpu_util import ring_abi
+
+pytestmark = pytest.mark.gpu
+
+COUNTS = [0, 1, 2, 3, 4, 5, 7, 8, 1023, 1024, 1025, 4096, 4097, 3 * 4096 + 7, 262_144, 1_000_003]
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _gpu():
+    G.require_gpu()
+    yield
+    for k, v in (("unroll", 4), ("nontemporal", 1), ("blocks_per_cu", 0)):
+        ring_abi.set_option(k, v)
+
+
+def special_f32():
+    return np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 1.1754942e-38,
+                     1.17549435e-38, 3.4028235e38, -3.4028235e38, 1.0, 16777216.0, 1e-30],
+                    dtype=np.float32)
+
+
+@pytest.mark.parametrize("dtype", G.DTYPES)
+def test_accumulate_matches_oracle(oracle, dtype):
+    rng = np.random.default_rng(11)
+    for count in COUNTS:
+        for doff, soff in ((0, 0), (1, 0), (0, 1), (3, 2), (2, 3), (1, 1)):
+            a = G.random_array(rng, count, dtype, wide=True)
+            b = G.random_array(rng, count, dtype, wide=True)
+            if dtype == np.float32 and count >= 1024:
+                sp = special_f32()
+                k = sp.size
+                for i in range(k):                      # every special against every special
+                    a[i * k:(i + 1) * k] = sp[i]
+                    b[i * k:(i + 1) * k] = sp
+            da, keep_a = G.dev(a, doff)
+            db, keep_b = G.dev(b, soff)
+            ring_abi.accumulate(G.NP2ABI[np.dtype(dtype)], da.data_ptr(), db.data_ptr(), count, None)
+            G.sync()
+            want = oracle.accumulate(a.copy(), b)
+            G.assert_same_bits(G.host(da), want, "accumulate %s n=%d off=%d/%d" % (dtype.__name__, count, doff, soff))
+            # nothing outside the destination range moved, the source is untouched
+            assert np.all(G.host(keep_a[:doff]) == 0) and np.all(G.host(keep_a[doff + count:]) == 0)
+            G.assert_same_bits(G.host(db), b)
+
+
+def test_typed_entry_points_and_errors():
+    L = ring_abi.lib()
+    a, _ = G.dev(np.arange(10, dtype=np.float32))
+    b, _ = G.dev(np.ones(10, dtype=np.float32))
+    assert L.ring_accumulate_f32(a.data_ptr(), b.data_ptr(), 10, None) == 0
+    ai, _ = G.dev(np.arange(10, dtype=np.int32))
+    bi, _ = G.dev(np.full(10, 2**31 - 1, dtype=np.int32))
+    assert L.ring_accumulate_i32(ai.data_ptr(), bi.data_ptr(), 10, None) == 0
+    al, _ = G.dev(np.arange(10, dtype=np.int64))
+    bl, _ = G.dev(np.full(10, -2**63, dtype=np.int64))
+    assert L.ring_accumulate_i64(al.data_ptr(), bl.data_ptr(), 10, None) == 0
+    G.sync()
+    assert np.array_equal(G.host(a), np.arange(10, dtype=np.float32) + 1)
+    with np.errstate(over="ignore"):
+        assert np.array_equal(G.host(ai), np.arange(10, dtype=np.int32) + np.int32(2**31 - 1))
+        assert np.array_equal(G.host(al), np.arange(10, dtype=np.int64) + np.int64(-2**63))
+    # error behaviour: bad dtype, null with a size, misaligned element pointer
+    assert L.ring_accumulate(7, a.data_ptr(), b.data_ptr(), 10, None) == 1
+    assert ring_abi.status_string(1) == "Invalid tensor type passed."       # mpi_ops.cc:844
+    assert L.ring_accumulate(0, None, b.data_ptr(), 10, None) == 2
+    assert L.ring_accumulate(0, a.data_ptr() + 2, b.data_ptr(), 4, None) == 2
+    assert L.ring_accumulate(0, None, None, 0, None) == 0                   # empty tensor: null, 0
+    assert L.ring_copy_bytes(None, None, 0, None) == 0
+    assert L.ring_copy_bytes(None, b.data_ptr(), 4, None) == 2
+
+
+def test_copy_bytes():
+    rng = np.random.default_rng(3)
+    for nbytes in (0, 1, 3, 4, 5, 15, 16, 17, 4096, 65_536 + 4, 1_000_003, 4_000_012):
+        for doff, soff in ((0, 0), (4, 0), (0, 8), (12, 4), (1, 0), (0, 3), (2, 2)):
+            src = rng.integers(0, 256, nbytes + 32, dtype=np.uint8)
+            import torch
+            dsrc = torch.from_numpy(src).cuda()
+            ddst = torch.zeros(nbytes + 64, dtype=torch.uint8, device="cuda")
+            ring_abi.copy_bytes(ddst.data_ptr() + doff, dsrc.data_ptr() + soff, nbytes, None)
+            G.sync()
+            out = G.host(ddst)
+            assert np.array_equal(out[doff:doff + nbytes], src[soff:soff + nbytes]), (nbytes, doff, soff)
+            assert not out[:doff].any() and not out[doff + nbytes:].any()
+
+
+def _random_table(rng, n_rows, dtype, max_count):
+    """Disjoint destination ranges inside one buffer, at ragged offsets."""
+    counts = [int(c) for c in rng.integers(0, max_count, n_rows)]
+    counts[rng.integers(0, n_rows)] = 0
+    gaps = [int(g) for g in rng.integers(0, 4, n_rows)]
+    offs, at = [], int(rng.integers(0, 4))
+    for c, g in zip(counts, gaps):
+        offs.append(at)
+        at += c + g
+    order = rng.permutation(n_rows)            # rows need not be sorted by offset
+    return [(offs[i], counts[i]) for i in order], at
+
+
+@pytest.mark.parametrize("dtype", G.DTYPES)
+@pytest.mark.parametrize("n_rows", [1, 7, 63, 64, 65, 150])
+def test_step_tables_match_oracle(oracle, dtype, n_rows):
+    rng = np.random.default_rng(100 + n_rows)
+    code = G.NP2ABI[np.dtype(dtype)]
+    table, total = _random_table(rng, n_rows, dtype, 20_000 if n_rows < 100 else 3_000)
+    for accumulate in (True, False):
+        buf = G.random_array(rng, total + 5, dtype)
+        dbuf, _ = G.dev(buf, int(rng.integers(0, 4)))
+        srcs, rows, keep = [], [], []
+        for off, cnt in table:
+            s = G.random_array(rng, cnt, dtype)
+            ds, base = G.dev(s, int(rng.integers(0, 4)))
+            srcs.append(s)
+            keep.append(base)
+            rows.append((off, ds.data_ptr() if cnt else None, cnt))
+        steps, n = ring_abi.make_steps(rows)
+        want = buf.copy()
+        for (off, cnt), s in zip(table, srcs):
+            if accumulate:
+                oracle.accumulate(want[off:off + cnt], s)
+            else:
+                want[off:off + cnt] = s
+        fn = ring_abi.reduce_scatter_steps if accumulate else ring_abi.allgather_steps
+        fn(dbuf.data_ptr(), steps, n, code, None)
+        G.sync()
+        G.assert_same_bits(G.host(dbuf), want, "table rows=%d acc=%s" % (n_rows, accumulate))
+
+
+@pytest.mark.parametrize("opt", [("unroll", 2), ("unroll", 8), ("nontemporal", 0),
+                                 ("blocks_per_cu", 1), ("blocks_per_cu", 8)])
+def test_launch_options_do_not_change_results(oracle, opt):
+    ring_abi.set_option(*opt)
+    try:
+        rng = np.random.default_rng(5)
+        for dtype in G.DTYPES:
+            for count in (5, 4097, 2_000_003):
+                a = G.random_array(rng, count, dtype)
+                b = G.random_array(rng, count, dtype)
+                da, _ = G.dev(a, 1)
+                db, _ = G.dev(b, 2)
+                ring_abi.accumulate(G.NP2ABI[np.dtype(dtype)], da.data_ptr(), db.data_ptr(), count, None)
+                dc, _ = G.dev(np.zeros(count, dtype=dtype), 3)
+                ring_abi.copy_bytes(dc.data_ptr(), db.data_ptr(), count * a.itemsize, None)
+                G.sync()
+                G.assert_same_bits(G.host(da), oracle.accumulate(a.copy(), b), str(opt))
+                G.assert_same_bits(G.host(dc), b, str(opt))
+    finally:
+        for k, v in (("unroll", 4), ("nontemporal", 1), ("blocks_per_cu", 0)):
+            ring_abi.set_option(k, v)
+
+
+@pytest.mark.parametrize("dtype", G.DTYPES)
+def test_scale_is_tf_div(dtype):
+    """allreduce(average=True) divides with tf.div (__init__.py:160-164): true
+    division for float32, floor division for integers."""
+    rng = np.random.default_rng(9)
+    for n in (1, 2, 3, 6, 7, 8, 13, 64):
+        for count, off in ((0, 0), (1, 0), (5, 1), (4099, 3), (300_001, 2)):
+            x = G.random_array(rng, count, dtype, wide=True)
+            if dtype == np.float32 and count > 100:
+                x[:14] = special_f32()
+            dx, keep = G.dev(x, off)
+            ring_abi.scale(G.NP2ABI[np.dtype(dtype)], dx.data_ptr(), count, n, None)
+            G.sync()
+            with np.errstate(all="ignore"):
+                want = x / np.float32(n) if dtype == np.float32 else x // dtype(n)
+            G.assert_same_bits(G.host(dx), want.astype(dtype), "scale %s /%d n=%d" % (dtype.__name__, n, count))
+            assert np.all(G.host(keep[:off]) == 0) and np.all(G.host(keep[off + count:]) == 0)
+
+
+def resnet50_shapes():
+    """The 161 trainable tensors of ResNet-50 v1, in layer order."""
+    shapes = [(7, 7, 3, 64), (64,), (64,)]
+    cin = 64
+    for width, blocks in ((64, 3), (128, 4), (256, 6), (512, 3)):
+        for b in range(blocks):
+            shapes += [(1, 1, cin, width), (width,), (width,),
+                       (3, 3, width, width), (width,), (width,),
+                       (1, 1, width, 4 * width), (4 * width,), (4 * width,)]
+            if b == 0:
+                shapes += [(1, 1, cin, 4 * width), (4 * width,), (4 * width,)]
+            cin = 4 * width
+    shapes += [(2048, 1000), (1000,)]
+    return shapes
+
+
+def test_resnet50_shape_set():
+    shapes = resnet50_shapes()
+    sizes = [int(np.prod(s)) for s in shapes]
+    assert len(shapes) == 161 and sum(sizes) == 25_557_032
+    assert min(sizes) == 64 and max(sizes) == 2_359_296
+    assert sum(1 for s in sizes if s <= 2048) == 107
+
+
+def _fusion_roundtrip(counts, dtype, rng, offsets=None):
+    code = G.NP2ABI[np.dtype(dtype)]
+    hosts, devs, keep = [], [], []
+    for j, c in enumerate(counts):
+        h = G.random_array(rng, c, dtype)
+        d, base = G.dev(h, (offsets[j] if offsets else int(rng.integers(0, 4))))
+        hosts.append(h)
+        devs.append(d)
+        keep.append(base)
+    plan = ring_abi.FusionPlan([d.data_ptr() if c else None for d, c in zip(devs, counts)], counts, code)
+    total = sum(counts)
+    assert plan.elements == total
+    import torch
+    fused = torch.zeros(total + 8, dtype=G.NP2TORCH[np.dtype(dtype)], device="cuda")
+    plan.pack(fused.data_ptr(), None)
+    G.sync()
+    want = np.concatenate(hosts) if hosts else np.empty(0, dtype=dtype)
+    G.assert_same_bits(G.host(fused)[:total], want, "pack")
+    assert not G.host(fused)[total:].any()
+    # unpack different data into zeroed tensors
+    new = G.random_array(rng, total, dtype)
+    fused[:total].copy_(torch.from_numpy(new))
+    for base in keep:
+        base.zero_()
+    plan.unpack(fused.data_ptr(), None)
+    G.sync()
+    at = 0
+    for j, (d, base, c) in enumerate(zip(devs, keep, counts)):
+        G.assert_same_bits(G.host(d), new[at:at + c], "unpack tensor %d" % j)
+        assert int(torch.count_nonzero(base)) == int(np.count_nonzero(new[at:at + c]))  # nothing outside
+        at += c
+    plan.close()
+
+
+@pytest.mark.parametrize("dtype", G.DTYPES)
+def test_fusion_pack_unpack(dtype):
+    rng = np.random.default_rng(21)
+    _fusion_roundtrip([int(np.prod(s)) for s in resnet50_shapes()], dtype, rng)
+    _fusion_roundtrip([], dtype, rng)
+    _fusion_roundtrip([0, 0], dtype, rng)
+    _fusion_roundtrip([1], dtype, rng)
+    _fusion_roundtrip([5, 0, 4096, 1, 0, 3, 8191, 2], dtype, rng)
+    # thousands of tiny tensors inside one tile: more than the LDS table holds
+    _fusion_roundtrip([int(c) for c in rng.integers(0, 4, 3000)], dtype, rng)
+    _fusion_roundtrip([int(c) for c in rng.integers(1, 200, 700)], dtype, rng)
+
+
+def test_fusion_errors():
+    L = ring_abi.lib()
+    h = ctypes.c_void_p()
+    p = (ctypes.c_void_p * 1)(None)
+    c = (ctypes.c_size_t * 1)(4)
+    assert L.ring_fusion_plan_create(p, c, 1, 0, ctypes.byref(h)) == 2      # null tensor with a size
+    assert L.ring_fusion_plan_create(p, c, 1, 9, ctypes.byref(h)) == 1      # bad dtype
+    assert L.ring_fusion_plan_destroy(None) == 0
