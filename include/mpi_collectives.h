@@ -1,0 +1,137 @@
+/*
+ * mpi_collectives.h — C interface of the plugin library (libmpi_collectives.so),
+ * the counterpart of the reference's mpi_collectives.so
+ * (tensorflow/contrib/mpi_collectives/mpi_ops.cc, ring.h): the op registry
+ * with the six MPI ops, their OpKernels, the readiness table / background
+ * thread, and the host-side ring driver. It contains no GPU code; every
+ * device operation goes through the C ABI of ring_abi.h.
+ *
+ * The reference is loaded into TensorFlow with tf.load_op_library() and driven
+ * by the TF executor (mpi_ops.py:30-59). Without TensorFlow the same ops are
+ * driven through the `mpic_context_*` calls below, which play the part of
+ * OpKernelContext / AsyncOpKernel::ComputeAsync(ctx, done)
+ * (tensorflow/core/framework/op_kernel.h:181-198).
+ *
+ * Ranks are VIRTUAL: one process, one GPU. A world either holds all `size`
+ * ranks (each submits its own tensor under the same node name, as separate
+ * MPI processes would) or a single real rank whose peers' incoming segments
+ * were staged in device memory beforehand.
+ *
+ * Status codes are TensorFlow's (tensorflow/core/lib/core/error_codes.proto):
+ * 0 OK, 2 UNKNOWN, 3 INVALID_ARGUMENT, 5 NOT_FOUND, 9 FAILED_PRECONDITION,
+ * 13 INTERNAL. Data types use TensorFlow's DataType numbering
+ * (tensorflow/core/framework/types.proto): 1 float32, 3 int32, 9 int64; any
+ * other value is rejected with "Invalid tensor type passed." (mpi_ops.cc:844).
+ */
+#ifndef MPI_COLLECTIVES_H_
+#define MPI_COLLECTIVES_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum mpic_code {
+  MPIC_OK = 0, MPIC_UNKNOWN = 2, MPIC_INVALID_ARGUMENT = 3, MPIC_NOT_FOUND = 5,
+  MPIC_FAILED_PRECONDITION = 9, MPIC_INTERNAL = 13
+};
+enum mpic_dtype { MPIC_DT_INVALID = 0, MPIC_DT_FLOAT = 1, MPIC_DT_DOUBLE = 2, MPIC_DT_INT32 = 3, MPIC_DT_INT64 = 9 };
+
+typedef struct mpic_world mpic_world;
+typedef struct mpic_context mpic_context;
+
+/* ---- op registry: what REGISTER_OP / REGISTER_KERNEL_BUILDER recorded at load
+ * time (mpi_ops.cc:900-907, 937-950, 979-992, 1024-1037, 1119-1139, 1233-1259).
+ * The Python loader checks the op list as mpi_ops.py:57-59 does. ------------ */
+int mpic_op_count(void);
+const char* mpic_op_name(int index);
+/* One-line signature, e.g. "MPIAllreduce(tensor: T) -> (sum: T); T: {int32, int64, float32}";
+ * NULL if the op is not registered. */
+const char* mpic_op_signature(const char* op);
+const char* mpic_op_doc(const char* op);
+/* 1 if a kernel is registered for (op, device), device = "CPU" or "GPU". */
+int mpic_op_has_kernel(const char* op, const char* device);
+/* Shape function of the op (mpi_ops.cc:1123-1126, 1239-1245): writes the
+ * output shape for input 0's shape; unknown dimensions are -1. Returns the
+ * output rank, or -1 if the op has no outputs / is unknown. */
+int mpic_op_infer_shape(const char* op, int ndims, const int64_t* dims, int64_t* out_dims);
+
+/* ---- worlds (MPIGlobalState, mpi_ops.cc:165-240) ------------------------- */
+
+/* All `size` ranks live in this process and share the current GPU. A
+ * collective starts when every rank has submitted it (mpi_ops.cc:255-269). */
+int mpic_world_create(int size, mpic_world** world);
+/* Only `rank` is real; what its neighbour would send is staged with
+ * mpic_stage_* before the op runs. */
+int mpic_world_create_prestaged(int size, int rank, mpic_world** world);
+/* Stops the background thread (SHUTDOWN, mpi_ops.cc:744-753) and frees the
+ * world. Pending ops fail with UNKNOWN. */
+int mpic_world_destroy(mpic_world* world);
+int mpic_world_size(const mpic_world* world);
+/* The dedicated stream of the world (CudaStreamForMPI, mpi_ops.cc:872-876), as
+ * a hipStream_t. Valid after MPIInit has run. */
+void* mpic_world_stream(const mpic_world* world);
+/* Options: "batched" (1: one launch per ring phase, 0: one launch per ring
+ * step as in ring.h:183-225), "fuse_copy" (1: fold the in->out copy of
+ * ring.h:146-148 into the reduce-scatter), "sync" (1: done() is called after
+ * the stream has drained, 0: as soon as the work is enqueued). */
+int mpic_world_set_option(mpic_world* world, const char* name, int value);
+
+/* Pre-staged peers for the op with node name `name`, consumed by the next
+ * collective of that name: rs_segments[i] / ag_segments[i] are device pointers
+ * to what the left neighbour sends at reduce-scatter / allgather step i
+ * (n-1 each; sizes follow ring_segment_table). For an allgather pass
+ * rs_segments = NULL and ag_segments[i] = the segment received at step i. */
+int mpic_stage_peers(mpic_world* world, const char* name,
+                     const void* const* rs_segments, const void* const* ag_segments);
+
+/* ---- running one op instance (OpKernelContext + ComputeAsync) -------------- */
+
+/* Output allocator supplied by the embedding framework (allocate_output,
+ * op_kernel.h:803-832): returns memory for a tensor of the given type and
+ * shape, on the host if `host_memory`, else on the GPU; NULL on failure. */
+typedef void* (*mpic_alloc_fn)(void* user, int dtype, int ndims, const int64_t* dims, int host_memory);
+
+/* `op`: registered op name; `node_name`: the graph node name collectives are
+ * matched by across ranks (mpi_ops.cc:1062, 1127-1131); `device`: "CPU"/"GPU". */
+int mpic_context_create(mpic_world* world, int rank, const char* op, const char* node_name,
+                        const char* device, mpic_alloc_fn alloc, void* user, mpic_context** ctx);
+int mpic_context_add_input(mpic_context* ctx, int dtype, int ndims, const int64_t* dims,
+                           const void* data, int host_memory);
+/* Runs Compute / ComputeAsync on the calling thread and returns. */
+int mpic_context_compute(mpic_context* ctx);
+/* Blocks until the op's done() ran; returns its status code. */
+int mpic_context_wait(mpic_context* ctx);
+const char* mpic_context_message(const mpic_context* ctx);
+int mpic_context_num_outputs(const mpic_context* ctx);
+int mpic_context_output(const mpic_context* ctx, int index, int* dtype, int* ndims,
+                        int64_t* dims /* room for 8 */, void** data);
+int mpic_context_destroy(mpic_context* ctx);
+
+/* ---- the ring driver, callable without the op layer ------------------------
+ * RingAllreduce (ring.h:136-228) for rank r of n whose incoming segments are
+ * already in device memory. `flags`: bit 0 = batched, bit 1 = fuse the
+ * in->out copy. Asynchronous on `stream`. `dtype` is an mpic_dtype. */
+int mpic_ring_allreduce_prestaged(int n, int r, int dtype, const void* input, void* output,
+                                  size_t count, const void* const* rs_segments,
+                                  const void* const* ag_segments, void* stream, int flags);
+/* RingAllgather (ring.h:236-301) for rank r: rows[k] = rank k's first
+ * dimension, segments[i] = what arrives at step i. */
+int mpic_ring_allgather_prestaged(int n, int r, int dtype, const void* input, const size_t* rows,
+                                  size_t elems_per_row, void* output,
+                                  const void* const* segments, void* stream, int flags);
+/* All n ranks resident on this GPU: inputs[k] / outputs[k] are rank k's
+ * tensors; a neighbour's buffer is read in place of a transfer. */
+int mpic_ring_allreduce_all_ranks(int n, int dtype, const void* const* inputs,
+                                  void* const* outputs, size_t count, void* stream, int flags);
+int mpic_ring_allgather_all_ranks(int n, int dtype, const void* const* inputs, const size_t* rows,
+                                  size_t elems_per_row, void* const* outputs, void* stream, int flags);
+/* Message of the last failing mpic_ring_* call on this thread. */
+const char* mpic_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MPI_COLLECTIVES_H_ */

@@ -143,11 +143,37 @@ typedef struct ring_step {
 int ring_reduce_scatter_steps(void* buffer, const ring_step* steps, int n_steps,
                               int dtype, void* stream);
 
+/* The same reduce-scatter with the in->out copy of ring.h:146-148 folded in:
+ * for every row, buffer[dst_offset + i] = input[dst_offset + i] + src[i].
+ * `input` is the rank's unmodified tensor, `buffer` its output; the sum is the
+ * same single add, so results are bit-identical to copy-then-accumulate while
+ * the accumulated segments are never copied (12 instead of 20 bytes moved
+ * per element). The one segment no step touches (segment r) is not written;
+ * the caller copies it if it needs it before the allgather phase fills it.
+ * input == buffer degenerates to ring_reduce_scatter_steps. */
+int ring_reduce_scatter_steps_from(const void* input, void* buffer,
+                                   const ring_step* steps, int n_steps,
+                                   int dtype, void* stream);
+
 /* All the receives of a rank's allgather phase (ring.h:211-225, and
  * ring.h:279-298 for the standalone allgather) in one launch: for every row,
  * buffer[dst_offset + i] = src[i]. Same table rules. */
 int ring_allgather_steps(void* buffer, const ring_step* steps, int n_steps,
                          int dtype, void* stream);
+
+/* The general form the step tables reduce to, for callers whose rows live in
+ * different buffers (all ranks of a virtual ring advancing one step in a
+ * single launch): for every row, dst[i] = a[i] when b is NULL, else
+ * dst[i] = b[i] + a[i]. b may be dst itself (in-place accumulate); otherwise
+ * no operand of a row may overlap a destination of the same call. `rows` is a
+ * HOST array. */
+typedef struct ring_row {
+  void* dst;
+  const void* a;
+  const void* b;
+  uint64_t count; /* elements */
+} ring_row;
+int ring_apply_rows(const ring_row* rows, int n_rows, int dtype, void* stream);
 
 /* ---- tensor fusion (no counterpart in the reference, which issues one
  * MPIAllreduce per gradient, __init__.py:195-205): k tensors are packed back

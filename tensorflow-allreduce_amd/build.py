@@ -5,6 +5,12 @@
   lib/libring_hip.so      HIP kernels + the C ABI of include/ring_abi.h
                           (csrc/ring_kernels.hip), linked against the HIP
                           runtime only.
+  lib/libmpi_collectives.so
+                          the plugin library (csrc/host/*.cc): op registry, the
+                          six MPI ops and their kernels, readiness table,
+                          background thread and host-side ring driver. Plain
+                          C++ (g++), no GPU code; calls libring_hip.so through
+                          the C ABI.
 
 hipcc cross-compiles for gfx950 without a GPU. Packed FP32 instructions are
 disabled for all device code.
@@ -18,6 +24,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 LIB_DIR = os.path.join(HERE, "lib")
 RING_HIP_SO = os.path.join(LIB_DIR, "libring_hip.so")
+PLUGIN_SO = os.path.join(LIB_DIR, "libmpi_collectives.so")
+HOST_SOURCES = ["framework.cc", "ring_driver.cc", "collective_ops.cc"]
+CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-pthread", "-Wall", "-Wextra"]
 
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
@@ -53,8 +62,29 @@ def build_ring_hip(verbose=True):
     return RING_HIP_SO
 
 
+def build_plugin(verbose=True):
+    """libmpi_collectives.so; needs libring_hip.so to link against."""
+    cxx = shutil.which("g++") or shutil.which("c++")
+    if not cxx:
+        raise RuntimeError("g++ not found")
+    cmd = [cxx] + CXX_FLAGS + [
+        "-I", os.path.join(ROOT, "include"), "-I", os.path.join(HERE, "csrc", "host"),
+        "-o", PLUGIN_SO,
+    ] + [os.path.join(HERE, "csrc", "host", f) for f in HOST_SOURCES] + [
+        "-L", LIB_DIR, "-lring_hip", "-Wl,-rpath,$ORIGIN",
+    ]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("g++ failed:\n" + res.stdout)
+    if verbose and res.stdout.strip():
+        print(res.stdout)
+    return PLUGIN_SO
+
+
 def build_all(verbose=True):
-    return [build_ring_hip(verbose)]
+    return [build_ring_hip(verbose), build_plugin(verbose)]
 
 
 if __name__ == "__main__":

@@ -1,0 +1,889 @@
+// The MPI ops of tensorflow/contrib/mpi_collectives (mpi_ops.cc) for virtual
+// ranks on one MI355X: op registrations, OpKernels, the per-op record, the
+// readiness table with its validation messages, the background thread that
+// performs every collective, and the C interface of include/mpi_collectives.h.
+//
+// What differs from the reference, on purpose:
+//   * ranks are virtual (one process, one GPU), so the coordinator's MPI
+//     messages (mpi_ops.cc:666-790) become in-process queue entries; the
+//     request/response records and the validation rules are kept;
+//   * the background thread sleeps on a condition variable instead of polling
+//     every millisecond (mpi_ops.cc:635), and initialisation waits on a
+//     predicate (the reference's cv.wait at :816-818 can miss its wake-up);
+//   * there is no temp tensor: where MPI_Irecv would fill one (ring.h:189-200)
+//     the incoming segment is read in place, from the neighbour's buffer or
+//     from a pre-staged one;
+//   * collectives only have GPU kernels. A CPU tensor is an error, not a
+//     silent host path.
+#include <atomic>
+#include <condition_variable>
+#include <cstring>
+#include <mutex>
+#include <queue>
+#include <sstream>
+#include <thread>
+#include <unordered_map>
+
+#include "framework.h"
+#include "mpi_collectives.h"
+#include "ring_abi.h"
+#include "ring_driver.h"
+
+namespace mpic {
+namespace {
+
+using CPUDevice = struct CPUDeviceTag {};
+using GPUDevice = struct GPUDeviceTag {};
+template <typename T> bool IsGPUDevice();
+template <> bool IsGPUDevice<GPUDevice>() { return true; }
+template <> bool IsGPUDevice<CPUDevice>() { return false; }
+
+// mpi_message.proto:12-17
+enum MPIDataType { TF_MPI_INVALID_TYPE = 0, TF_MPI_FLOAT32 = 1, TF_MPI_INT32 = 2, TF_MPI_INT64 = 3 };
+const char* MPIDataType_Name(MPIDataType t) {
+  switch (t) {
+    case TF_MPI_FLOAT32: return "TF_MPI_FLOAT32";
+    case TF_MPI_INT32: return "TF_MPI_INT32";
+    case TF_MPI_INT64: return "TF_MPI_INT64";
+    default: return "TF_MPI_INVALID_TYPE";
+  }
+}
+
+// mpi_message.proto:22-40
+struct MPIRequest {
+  enum RequestType { ALLREDUCE = 0, ALLGATHER = 1 };
+  int request_rank = 0;
+  RequestType request_type = ALLREDUCE;
+  MPIDataType tensor_type = TF_MPI_INVALID_TYPE;
+  std::string tensor_name;
+  std::vector<int64_t> tensor_shape;
+};
+
+// mpi_message.proto:49-63
+struct MPIResponse {
+  enum ResponseType { ALLREDUCE = 0, ALLGATHER = 1, ERROR = 2, DONE = 3, SHUTDOWN = 4 };
+  ResponseType response_type = DONE;
+  std::string tensor_name;
+  std::string error_message;
+};
+
+typedef std::function<void(const Status&)> CommunicationDoneCallback;
+
+// mpi_ops.cc:123-153
+struct CollectiveOpRecord {
+  int rank = 0;                   // the (virtual) rank performing this piece of the op
+  std::string name;               // node name: the key collectives are matched by
+  OpKernelContext* context = nullptr;
+  MPIDataType dtype = TF_MPI_INVALID_TYPE;
+  const Tensor* in_t = nullptr;
+  std::vector<size_t> sizes_vec;  // allgather: per-rank first-dimension sizes
+  size_t temp_elements = 0;       // what the reference's temp tensor would hold (mpi_ops.cc:1073-1077)
+  Tensor* out_t = nullptr;
+  bool on_gpu = false;
+  CommunicationDoneCallback callback;
+};
+
+struct StagedPeers {
+  std::vector<const void*> rs, ag;
+};
+
+typedef std::unordered_map<std::string, std::map<int, CollectiveOpRecord>> TensorTable;
+typedef std::unordered_map<std::string, std::vector<MPIRequest>> MessageTable;
+
+}  // namespace
+}  // namespace mpic
+
+// mpi_ops.cc:165-240 (MPIGlobalState), one per world instead of one per process.
+struct mpic_world {
+  std::atomic_flag initialized_flag = ATOMIC_FLAG_INIT;
+  std::condition_variable cv;       // initialisation
+  std::condition_variable work_cv;  // requests for the background thread
+  bool initialization_done = false;
+  mpic::Status init_status;
+  std::mutex mu;
+  mpic::TensorTable tensor_table;
+  std::queue<mpic::MPIRequest> message_queue;
+  std::thread background_thread;
+  bool shut_down = false;
+  mpic::MessageTable message_table;  // coordinator side
+  std::unordered_map<std::string, mpic::StagedPeers> staged;
+  int size = 1;
+  int real_rank = -1;  // -1: every rank lives in this process
+  int device = -1;     // -1 for no GPU
+  void* stream = nullptr;
+  mpic::RingOptions ring_options;
+  bool sync_on_done = true;
+
+  int expected_requests() const { return real_rank >= 0 ? 1 : size; }
+};
+
+namespace mpic {
+namespace {
+
+// mpi_ops.cc:255-269
+bool IncrementTensorCount(MessageTable* table, const MPIRequest& msg, int expected) {
+  std::vector<MPIRequest>& v = (*table)[msg.tensor_name];
+  v.push_back(msg);
+  return static_cast<int>(v.size()) == expected;
+}
+
+TensorShape ShapeOf(const MPIRequest& r) { return TensorShape(r.tensor_shape); }
+
+// mpi_ops.cc:277-432: all the cross-rank checks, with the reference's messages.
+MPIResponse ConstructMPIResponse(MessageTable* table, const std::string& name) {
+  bool error = false;
+  std::vector<MPIRequest> requests = (*table)[name];
+  std::ostringstream err;
+
+  const MPIDataType data_type = requests[0].tensor_type;
+  for (size_t i = 1; i < requests.size(); i++) {
+    if (data_type != requests[i].tensor_type) {
+      error = true;
+      err << "Mismatched data types: One rank had type " << MPIDataType_Name(data_type)
+          << ", but another rank had type " << MPIDataType_Name(requests[i].tensor_type) << ".";
+      break;
+    }
+  }
+
+  const MPIRequest::RequestType message_type = requests[0].request_type;
+  for (size_t i = 1; i < requests.size() && !error; i++) {
+    if (message_type != requests[i].request_type) {
+      error = true;
+      err << "Mismatched MPI operations: One rank did an " << static_cast<int>(message_type)
+          << ", but another rank did an " << static_cast<int>(requests[i].request_type) << ".";
+    }
+  }
+
+  if (message_type == MPIRequest::ALLREDUCE) {
+    const TensorShape tensor_shape = ShapeOf(requests[0]);
+    for (size_t i = 1; i < requests.size() && !error; i++) {
+      const TensorShape request_shape = ShapeOf(requests[i]);
+      if (tensor_shape != request_shape) {
+        error = true;
+        err << "Mismatched allreduce tensor shapes: One rank reduced a tensor of shape "
+            << tensor_shape.DebugString() << ", but another rank sent a tensor of shape "
+            << request_shape.DebugString() << ".";
+      }
+    }
+  }
+
+  if (message_type == MPIRequest::ALLGATHER) {
+    const TensorShape tensor_shape = ShapeOf(requests[0]);
+    if (tensor_shape.dims() == 0 && !error) {
+      error = true;
+      err << "Rank zero tried to gather a rank-zero tensor.";
+    }
+    for (size_t i = 1; i < requests.size() && !error; i++) {
+      const TensorShape request_shape = ShapeOf(requests[i]);
+      if (tensor_shape.dims() != request_shape.dims()) {
+        error = true;
+        err << "Mismatched allgather tensor shapes: One rank gathered a tensor of rank "
+            << tensor_shape.dims() << ", but another rank sent a tensor of rank " << request_shape.dims() << ".";
+        break;
+      }
+      for (int dim = 1; dim < tensor_shape.dims(); dim++) {
+        if (tensor_shape.dim_size(dim) != request_shape.dim_size(dim)) {
+          error = true;
+          err << "Mismatched allgather tensor shapes: One rank gathered a tensor with dimension " << dim
+              << " equal to " << tensor_shape.dim_size(dim)
+              << ", but another rank sent a tensor with dimension " << dim << " equal to "
+              << request_shape.dim_size(dim) << ".";
+          break;
+        }
+      }
+    }
+  }
+
+  MPIResponse response;
+  response.tensor_name = name;
+  if (error) {
+    response.response_type = MPIResponse::ERROR;
+    response.error_message = err.str();
+  } else {
+    response.response_type =
+        message_type == MPIRequest::ALLREDUCE ? MPIResponse::ALLREDUCE : MPIResponse::ALLGATHER;
+  }
+  table->erase(name);
+  return response;
+}
+
+// mpi_ops.cc:435-515: run the collective for every rank that lives here, then
+// resume their ops.
+void PerformCollectiveOp(mpic_world* w, const MPIResponse& response) {
+  std::map<int, CollectiveOpRecord> records;
+  StagedPeers peers;
+  bool have_peers = false;
+  {
+    std::lock_guard<std::mutex> guard(w->mu);
+    auto it = w->tensor_table.find(response.tensor_name);
+    if (it == w->tensor_table.end()) return;
+    records = std::move(it->second);
+    w->tensor_table.erase(it);
+    auto st = w->staged.find(response.tensor_name);
+    if (st != w->staged.end()) {
+      peers = std::move(st->second);
+      w->staged.erase(st);
+      have_peers = true;
+    }
+  }
+  if (records.empty()) return;
+
+  Status status;
+  const CollectiveOpRecord& first = records.begin()->second;
+  const DataType dtype = first.in_t->dtype();
+  const int n = w->size;
+  bool on_gpu = true;
+  for (auto& kv : records) on_gpu = on_gpu && kv.second.on_gpu;
+
+  if (response.response_type == MPIResponse::ERROR) {
+    status = errors::FailedPrecondition(response.error_message);
+  } else if (dtype != DT_FLOAT && dtype != DT_INT32 && dtype != DT_INT64) {
+    status = errors::Unknown(response.response_type == MPIResponse::ALLGATHER
+                                 ? "Invalid tensor type for MPI allgather."
+                                 : "Invalid tensor type for MPI allreduce.");
+  } else if (!on_gpu) {
+    status = errors::FailedPrecondition("MPI collectives have GPU kernels only; the tensor is in host memory.");
+  } else if (w->real_rank >= 0) {
+    const int r = w->real_rank;
+    if (n > 1 && !have_peers) {
+      status = errors::FailedPrecondition("No pre-staged peer segments for " + response.tensor_name + ".");
+    } else if (n > 1 && (peers.ag.size() != static_cast<size_t>(n - 1) ||
+                         (response.response_type == MPIResponse::ALLREDUCE &&
+                          peers.rs.size() != static_cast<size_t>(n - 1)))) {
+      status = errors::FailedPrecondition("Pre-staged peer segments for " + response.tensor_name +
+                                          " do not cover the ring's n-1 steps.");
+    } else if (response.response_type == MPIResponse::ALLREDUCE) {
+      status = RingAllreducePrestaged(n, r, dtype, first.in_t->data(), first.out_t->data(),
+                                      static_cast<size_t>(first.in_t->NumElements()), peers.rs.data(),
+                                      peers.ag.data(), w->stream, w->ring_options);
+    } else {
+      size_t epr = 1;
+      for (int i = 1; i < first.in_t->shape().dims(); i++) epr *= static_cast<size_t>(first.in_t->dim_size(i));
+      status = RingAllgatherPrestaged(n, r, dtype, first.in_t->data(), first.sizes_vec, epr, first.out_t->data(),
+                                      peers.ag.data(), w->stream, w->ring_options);
+    }
+  } else {
+    std::vector<const void*> ins(static_cast<size_t>(n));
+    std::vector<void*> outs(static_cast<size_t>(n));
+    for (auto& kv : records) {
+      ins[static_cast<size_t>(kv.first)] = kv.second.in_t->data();
+      outs[static_cast<size_t>(kv.first)] = kv.second.out_t->data();
+    }
+    if (response.response_type == MPIResponse::ALLREDUCE) {
+      status = RingAllreduceAllRanks(n, dtype, ins.data(), outs.data(),
+                                     static_cast<size_t>(first.in_t->NumElements()), w->stream, w->ring_options);
+    } else {
+      size_t epr = 1;
+      for (int i = 1; i < first.in_t->shape().dims(); i++) epr *= static_cast<size_t>(first.in_t->dim_size(i));
+      // every rank computed the same sizes from the sizing gather; the first
+      // dimension each one actually submitted must agree with them
+      for (auto& kv : records) {
+        if (kv.second.sizes_vec != first.sizes_vec ||
+            static_cast<size_t>(kv.second.in_t->dim_size(0)) != first.sizes_vec[static_cast<size_t>(kv.first)]) {
+          status = errors::FailedPrecondition("Allgather sizes do not match the gathered tensors' first dimensions.");
+          break;
+        }
+      }
+      if (status.ok())
+        status = RingAllgatherAllRanks(n, dtype, ins.data(), first.sizes_vec, epr, outs.data(), w->stream,
+                                       w->ring_options);
+    }
+  }
+
+  if (status.ok() && w->sync_on_done && response.response_type != MPIResponse::ERROR) {
+    const int rc = ring_stream_synchronize(w->stream);
+    if (rc != RING_OK) status = errors::Unknown("MPI operation failed unexpectedly.");  // ring.h:36-39
+  }
+  for (auto& kv : records) kv.second.callback(status);
+}
+
+// mpi_ops.cc:572-795. Ticks are driven by arrivals, not by a 1 ms sleep.
+void BackgroundThreadLoop(mpic_world* w) {
+  Status init;
+  if (w->device >= 0) {
+    // the dedicated stream (mpi_ops.cc:582-583)
+    const int rc = ring_stream_create(&w->stream);
+    if (rc != RING_OK)
+      init = errors::Unknown(std::string("Could not create the MPI stream: ") + ring_status_string(rc));
+  }
+  {
+    std::lock_guard<std::mutex> guard(w->mu);
+    w->init_status = init;
+    w->initialization_done = true;
+  }
+  w->cv.notify_all();
+  if (!init.ok()) return;
+
+  bool should_shut_down = false;
+  do {
+    std::queue<MPIRequest> message_queue;
+    {
+      std::unique_lock<std::mutex> lock(w->mu);
+      w->work_cv.wait(lock, [w] { return w->shut_down || !w->message_queue.empty(); });
+      std::swap(message_queue, w->message_queue);
+      should_shut_down = w->shut_down;
+    }
+    std::vector<std::string> ready_to_reduce;
+    while (!message_queue.empty()) {
+      const MPIRequest& message = message_queue.front();
+      if (IncrementTensorCount(&w->message_table, message, w->expected_requests()))
+        ready_to_reduce.push_back(message.tensor_name);
+      message_queue.pop();
+    }
+    for (const std::string& name : ready_to_reduce) {
+      MPIResponse response = ConstructMPIResponse(&w->message_table, name);
+      PerformCollectiveOp(w, response);
+    }
+  } while (!should_shut_down);
+
+  // ops still waiting for absent ranks can never run: fail them
+  TensorTable leftover;
+  {
+    std::lock_guard<std::mutex> guard(w->mu);
+    leftover.swap(w->tensor_table);
+  }
+  for (auto& named : leftover)
+    for (auto& kv : named.second) kv.second.callback(errors::Unknown("MPI was shut down before the collective ran."));
+  if (w->stream) {
+    ring_stream_synchronize(w->stream);
+    ring_stream_destroy(w->stream);
+    w->stream = nullptr;
+  }
+}
+
+// mpi_ops.cc:799-824
+Status InitializeMPIOnce(mpic_world* w, bool gpu) {
+  if (w->initialized_flag.test_and_set()) {
+    std::unique_lock<std::mutex> lock(w->mu);
+    w->cv.wait(lock, [w] { return w->initialization_done; });
+    return w->init_status;
+  }
+  w->device = gpu ? 0 : -1;
+  w->background_thread = std::thread(BackgroundThreadLoop, w);
+  std::unique_lock<std::mutex> lock(w->mu);
+  w->cv.wait(lock, [w] { return w->initialization_done; });
+  return w->init_status;
+}
+
+// mpi_ops.cc:827-833
+Status IsMPIInitialized(mpic_world* w) {
+  std::lock_guard<std::mutex> guard(w->mu);
+  if (!w->initialization_done)
+    return errors::FailedPrecondition("MPI has not been initialized; use tf.contrib.mpi.Session.");
+  return w->init_status;
+}
+
+// mpi_ops.cc:836-847
+Status DataTypeToMPIType(DataType tf_dtype, MPIDataType* mpi_dtype) {
+  if (tf_dtype == DT_FLOAT) *mpi_dtype = TF_MPI_FLOAT32;
+  else if (tf_dtype == DT_INT32) *mpi_dtype = TF_MPI_INT32;
+  else if (tf_dtype == DT_INT64) *mpi_dtype = TF_MPI_INT64;
+  else return errors::FailedPrecondition("Invalid tensor type passed.");
+  return Status::OK();
+}
+
+// mpi_ops.cc:853-868
+void EnqueueTensorCollective(mpic_world* w, const CollectiveOpRecord& record, MPIRequest::RequestType rtype) {
+  MPIRequest message;
+  message.request_rank = record.rank;
+  message.tensor_name = record.name;
+  message.tensor_type = record.dtype;
+  message.request_type = rtype;
+  message.tensor_shape = record.in_t->shape().dim_sizes();
+  {
+    std::lock_guard<std::mutex> guard(w->mu);
+    w->tensor_table[record.name][record.rank] = record;
+    w->message_queue.push(message);
+  }
+  w->work_cv.notify_one();
+}
+
+mpic_world* WorldOf(OpKernelContext* context) { return static_cast<mpic_world*>(context->world()); }
+
+// ---- ops -------------------------------------------------------------------------
+
+// mpi_ops.cc:880-907
+template <typename Device>
+class MPIInitOp : public OpKernel {
+ public:
+  explicit MPIInitOp(OpKernelConstruction* context) : OpKernel(context) {}
+  void Compute(OpKernelContext* context) override {
+    OP_REQUIRES_OK(context, InitializeMPIOnce(WorldOf(context), IsGPUDevice<Device>()));
+  }
+};
+REGISTER_KERNEL_BUILDER(Name("MPIInit").Device(DEVICE_CPU), MPIInitOp<CPUDevice>);
+REGISTER_KERNEL_BUILDER(Name("MPIInit").Device(DEVICE_GPU), MPIInitOp<GPUDevice>);
+REGISTER_OP("MPIInit").Doc(R"doc(
+Initialize MPI for the current process.
+
+If this is run on a GPU, then that GPU must be used for all future MPI
+operations. If it is run on CPU, then all future MPI operations must also
+run on CPU.
+)doc");
+
+// A scalar int32 in host memory (the GPU kernels of these three ops pin their
+// output to the host, mpi_ops.cc:933, 975, 1018-1020).
+void ScalarOutput(OpKernelContext* context, int value) {
+  OP_REQUIRES_OK(context, IsMPIInitialized(WorldOf(context)));
+  Tensor* output = nullptr;
+  OP_REQUIRES_OK(context, context->allocate_output(0, TensorShape(), DT_INT32, true, &output));
+  *static_cast<int32_t*>(output->data()) = value;
+}
+
+// mpi_ops.cc:910-950
+template <typename Device>
+class MPISizeOp : public OpKernel {
+ public:
+  explicit MPISizeOp(OpKernelConstruction* context) : OpKernel(context) {}
+  void Compute(OpKernelContext* context) override { ScalarOutput(context, WorldOf(context)->size); }
+};
+REGISTER_KERNEL_BUILDER(Name("MPISize").Device(DEVICE_CPU), MPISizeOp<CPUDevice>);
+REGISTER_KERNEL_BUILDER(Name("MPISize").Device(DEVICE_GPU).HostMemory("size"), MPISizeOp<GPUDevice>);
+REGISTER_OP("MPISize")
+    .Output("size: int32")
+    .SetShapeFn([](const std::vector<int64_t>&, std::vector<int64_t>* out) { out->clear(); return Status::OK(); })
+    .Doc(R"doc(
+Returns the number of running MPI processes.
+
+More precisely, returns the number of MPI processes in the group associated
+with the MPI_COMM_WORLD communicator.
+
+size:   Size of the MPI group.
+)doc");
+
+// mpi_ops.cc:953-992
+template <typename Device>
+class MPIRankOp : public OpKernel {
+ public:
+  explicit MPIRankOp(OpKernelConstruction* context) : OpKernel(context) {}
+  void Compute(OpKernelContext* context) override { ScalarOutput(context, context->rank()); }
+};
+REGISTER_KERNEL_BUILDER(Name("MPIRank").Device(DEVICE_CPU), MPIRankOp<CPUDevice>);
+REGISTER_KERNEL_BUILDER(Name("MPIRank").Device(DEVICE_GPU).HostMemory("rank"), MPIRankOp<GPUDevice>);
+REGISTER_OP("MPIRank")
+    .Output("rank: int32")
+    .SetShapeFn([](const std::vector<int64_t>&, std::vector<int64_t>* out) { out->clear(); return Status::OK(); })
+    .Doc(R"doc(
+Returns the index of the current process in the MPI group.
+
+More precisely, returns the rank of the calling process in the MPI_COMM_WORLD
+communicator.
+
+rank:   Rank of the calling process.
+)doc");
+
+// mpi_ops.cc:996-1037. All virtual ranks share one node, so the local rank is
+// the rank.
+template <typename Device>
+class MPILocalRankOp : public OpKernel {
+ public:
+  explicit MPILocalRankOp(OpKernelConstruction* context) : OpKernel(context) {}
+  void Compute(OpKernelContext* context) override { ScalarOutput(context, context->rank()); }
+};
+REGISTER_KERNEL_BUILDER(Name("MPILocalRank").Device(DEVICE_CPU), MPILocalRankOp<CPUDevice>);
+REGISTER_KERNEL_BUILDER(Name("MPILocalRank").Device(DEVICE_GPU).HostMemory("rank"), MPILocalRankOp<GPUDevice>);
+REGISTER_OP("MPILocalRank")
+    .Output("rank: int32")
+    .SetShapeFn([](const std::vector<int64_t>&, std::vector<int64_t>* out) { out->clear(); return Status::OK(); })
+    .Doc(R"doc(
+Returns the index of the current process in the node it is on.
+
+More precisely, returns the rank of the calling process in communicator that
+only spans the MPI processes running on that node.
+
+rank:   Rank of the calling process on the node it is on.
+)doc");
+
+// mpi_ops.cc:1039-1139
+template <typename Device>
+class MPIAllreduceOp : public AsyncOpKernel {
+ public:
+  explicit MPIAllreduceOp(OpKernelConstruction* context) : AsyncOpKernel(context) {}
+  // ComputeAsync only files a record for the background thread.
+  bool IsExpensive() override { return false; }
+
+  void ComputeAsync(OpKernelContext* context, DoneCallback done) override {
+    mpic_world* world = WorldOf(context);
+    OP_REQUIRES_OK_ASYNC(context, IsMPIInitialized(world), done);
+    OP_REQUIRES_OK_ASYNC(context,
+                         context->num_inputs() == 1 ? Status::OK()
+                                                    : errors::InvalidArgument("MPIAllreduce takes one input."),
+                         done);
+    const Tensor* input_tensor = &context->input(0);
+
+    CollectiveOpRecord record;
+    record.dtype = TF_MPI_INVALID_TYPE;
+    OP_REQUIRES_OK_ASYNC(context, DataTypeToMPIType(input_tensor->dtype(), &record.dtype), done);
+
+    Tensor* output_tensor = nullptr;
+    OP_REQUIRES_OK_ASYNC(
+        context, context->allocate_output(0, input_tensor->shape(), input_tensor->dtype(), false, &output_tensor),
+        done);
+
+    record.rank = context->rank();
+    record.name = name();
+    record.context = context;
+    record.in_t = input_tensor;
+    record.out_t = output_tensor;
+    record.on_gpu = IsGPUDevice<Device>() && !input_tensor->host_memory();
+    record.temp_elements = ring_temp_elements(static_cast<size_t>(input_tensor->NumElements()), world->size);
+    record.callback = [done, context](const Status& status) {
+      context->SetStatus(status);
+      done();
+    };
+    // The caller's producer work is ordered before the collective by the
+    // embedding framework (the reference defers this call with a stream host
+    // callback, mpi_ops.cc:1099-1105).
+    EnqueueTensorCollective(world, record, MPIRequest::ALLREDUCE);
+  }
+};
+REGISTER_KERNEL_BUILDER(Name("MPIAllreduce").Device(DEVICE_GPU), MPIAllreduceOp<GPUDevice>);
+REGISTER_OP("MPIAllreduce")
+    .Attr("T: {int32, int64, float32}")
+    .Input("tensor: T")
+    .Output("sum: T")
+    .SetShapeFn([](const std::vector<int64_t>& in, std::vector<int64_t>* out) { *out = in; return Status::OK(); })
+    .Doc(R"doc(
+Perform an MPI Allreduce on a tensor. All other processes that do a reduction
+on a tensor with the same name must have the same dimension for that tensor.
+Tensors are reduced with other tensors that have the same node name for the
+allreduce.
+
+Arguments
+    tensor:     A tensor to reduce.
+
+Output
+    sum:        A tensor with the same shape as `tensor`, summed across all
+                MPI processes.
+)doc");
+
+// mpi_ops.cc:1141-1270
+template <typename Device>
+class MPIAllgatherOp : public AsyncOpKernel {
+ public:
+  explicit MPIAllgatherOp(OpKernelConstruction* context) : AsyncOpKernel(context) {}
+  bool IsExpensive() override { return false; }
+
+  void ComputeAsync(OpKernelContext* context, DoneCallback done) override {
+    mpic_world* world = WorldOf(context);
+    OP_REQUIRES_OK_ASYNC(context, IsMPIInitialized(world), done);
+    OP_REQUIRES_OK_ASYNC(context,
+                         context->num_inputs() == 2 ? Status::OK()
+                                                    : errors::InvalidArgument("MPIAllgather takes two inputs."),
+                         done);
+    const Tensor* input_tensor = &context->input(0);
+    const Tensor* sizing_tensor = &context->input(1);
+
+    CollectiveOpRecord record;
+    record.rank = context->rank();
+    record.name = name();
+    record.context = context;
+    record.in_t = input_tensor;
+    record.on_gpu = IsGPUDevice<Device>() && !input_tensor->host_memory();
+
+    // A scalar sizing tensor means one element per rank (the sizing pre-pass,
+    // mpi_ops.cc:1167-1173); otherwise it lists every rank's first dimension
+    // and lives in host memory (:1176-1183).
+    size_t output_first_dim = 0;
+    if (sizing_tensor->shape().dims() == 0) {
+      output_first_dim = static_cast<size_t>(world->size);
+      record.sizes_vec.assign(static_cast<size_t>(world->size), 1);
+    } else {
+      OP_REQUIRES_OK_ASYNC(
+          context,
+          (sizing_tensor->host_memory() && sizing_tensor->dtype() == DT_INT64 &&
+           sizing_tensor->NumElements() >= world->size)
+              ? Status::OK()
+              : errors::InvalidArgument("sizes must be an int64 host tensor with one entry per rank."),
+          done);
+      const int64_t* sizing_array = static_cast<const int64_t*>(sizing_tensor->data());
+      for (int i = 0; i < world->size; i++) {
+        record.sizes_vec.push_back(static_cast<size_t>(sizing_array[i]));
+        output_first_dim += static_cast<size_t>(sizing_array[i]);
+      }
+    }
+
+    record.dtype = TF_MPI_INVALID_TYPE;
+    OP_REQUIRES_OK_ASYNC(context, DataTypeToMPIType(input_tensor->dtype(), &record.dtype), done);
+
+    TensorShape output_shape;
+    output_shape.AddDim(static_cast<int64_t>(output_first_dim));
+    for (int i = 1; i < input_tensor->shape().dims(); i++) output_shape.AddDim(input_tensor->dim_size(i));
+    Tensor* output_tensor = nullptr;
+    OP_REQUIRES_OK_ASYNC(context,
+                         context->allocate_output(0, output_shape, input_tensor->dtype(), false, &output_tensor), done);
+    record.out_t = output_tensor;
+    record.callback = [done, context](const Status& status) {
+      context->SetStatus(status);
+      done();
+    };
+    EnqueueTensorCollective(world, record, MPIRequest::ALLGATHER);
+  }
+};
+REGISTER_OP("MPIAllgather")
+    .Attr("T: {int32, int64, float32}")
+    .Attr("S: {int64}")
+    .Input("tensor: T")
+    .Input("sizes: S")
+    .Output("gathered: T")
+    .SetShapeFn([](const std::vector<int64_t>& in, std::vector<int64_t>* out) {
+      if (in.empty()) return errors::InvalidArgument("Shape must be at least rank 1 but is rank 0");
+      *out = in;
+      (*out)[0] = -1;  // ReplaceDim(input, 0, UnknownDim)
+      return Status::OK();
+    })
+    .Doc(R"doc(
+Perform an MPI Allgather on a tensor. All other processes that do a gather on a
+tensor with the same name must have the same rank for that tensor, and have the
+same dimension on all but the first dimension.
+
+Arguments
+    tensor:     A tensor to gather.
+    sizes:      A tensor containing the first-dimension sizes of tensors to be
+                gathered from other ranks
+
+Output
+    gathered:   A tensor with the same shape as `tensor` except for the first
+                dimension, which is the sum of dimensions in `sizes`.
+)doc");
+REGISTER_KERNEL_BUILDER(Name("MPIAllgather").Device(DEVICE_GPU).HostMemory("sizes"), MPIAllgatherOp<GPUDevice>);
+
+thread_local std::string g_last_error;
+int Fail(const Status& s) {
+  g_last_error = s.error_message();
+  return static_cast<int>(s.code());
+}
+
+}  // namespace
+}  // namespace mpic
+
+// =============================================================================
+// C interface
+// =============================================================================
+struct mpic_context {
+  std::unique_ptr<mpic::OpKernelContext> ctx;
+  std::unique_ptr<mpic::OpKernel> kernel;
+  std::mutex mu;
+  std::condition_variable cv;
+  bool started = false;
+  bool done = false;
+};
+
+using mpic::OpRegistry;
+
+extern "C" {
+
+int mpic_op_count(void) { return static_cast<int>(OpRegistry::Global()->op_names().size()); }
+
+const char* mpic_op_name(int index) {
+  const auto& names = OpRegistry::Global()->op_names();
+  if (index < 0 || static_cast<size_t>(index) >= names.size()) return nullptr;
+  return names[static_cast<size_t>(index)].c_str();
+}
+
+const char* mpic_op_signature(const char* op) {
+  static thread_local std::string text;
+  const mpic::OpDef* def = op ? OpRegistry::Global()->LookUp(op) : nullptr;
+  if (!def) return nullptr;
+  text = def->Signature();
+  return text.c_str();
+}
+
+const char* mpic_op_doc(const char* op) {
+  const mpic::OpDef* def = op ? OpRegistry::Global()->LookUp(op) : nullptr;
+  return def ? def->doc.c_str() : nullptr;
+}
+
+int mpic_op_has_kernel(const char* op, const char* device) {
+  return op && device && OpRegistry::Global()->FindKernel(op, device) ? 1 : 0;
+}
+
+int mpic_op_infer_shape(const char* op, int ndims, const int64_t* dims, int64_t* out_dims) {
+  const mpic::OpDef* def = op ? OpRegistry::Global()->LookUp(op) : nullptr;
+  if (!def || !def->shape_fn || def->outputs.empty() || ndims < 0) return -1;
+  std::vector<int64_t> in(dims, dims + ndims), out;
+  if (!def->shape_fn(in, &out).ok()) return -1;
+  for (size_t i = 0; i < out.size(); i++) out_dims[i] = out[i];
+  return static_cast<int>(out.size());
+}
+
+static int world_create(int size, int rank, mpic_world** world) {
+  if (!world || size < 1 || rank >= size) return MPIC_INVALID_ARGUMENT;
+  mpic_world* w = new mpic_world();
+  w->size = size;
+  w->real_rank = rank;
+  *world = w;
+  return MPIC_OK;
+}
+
+int mpic_world_create(int size, mpic_world** world) { return world_create(size, -1, world); }
+
+int mpic_world_create_prestaged(int size, int rank, mpic_world** world) {
+  if (rank < 0) return MPIC_INVALID_ARGUMENT;
+  return world_create(size, rank, world);
+}
+
+int mpic_world_destroy(mpic_world* w) {
+  if (!w) return MPIC_OK;
+  if (w->background_thread.joinable()) {
+    {
+      std::lock_guard<std::mutex> guard(w->mu);
+      w->shut_down = true;
+    }
+    w->work_cv.notify_all();
+    w->background_thread.join();
+  }
+  delete w;
+  return MPIC_OK;
+}
+
+int mpic_world_size(const mpic_world* w) { return w ? w->size : 0; }
+void* mpic_world_stream(const mpic_world* w) { return w ? w->stream : nullptr; }
+
+int mpic_world_set_option(mpic_world* w, const char* name, int value) {
+  if (!w || !name) return MPIC_INVALID_ARGUMENT;
+  std::lock_guard<std::mutex> guard(w->mu);
+  if (!strcmp(name, "batched")) w->ring_options.batched = value != 0;
+  else if (!strcmp(name, "fuse_copy")) w->ring_options.fuse_copy = value != 0;
+  else if (!strcmp(name, "sync")) w->sync_on_done = value != 0;
+  else return MPIC_INVALID_ARGUMENT;
+  return MPIC_OK;
+}
+
+int mpic_stage_peers(mpic_world* w, const char* name, const void* const* rs_segments,
+                     const void* const* ag_segments) {
+  if (!w || !name || w->real_rank < 0 || (w->size > 1 && !ag_segments)) return MPIC_INVALID_ARGUMENT;
+  mpic::StagedPeers peers;
+  for (int i = 0; i < w->size - 1; i++) {
+    if (rs_segments) peers.rs.push_back(rs_segments[i]);
+    peers.ag.push_back(ag_segments[i]);
+  }
+  std::lock_guard<std::mutex> guard(w->mu);
+  w->staged[name] = std::move(peers);
+  return MPIC_OK;
+}
+
+int mpic_context_create(mpic_world* world, int rank, const char* op, const char* node_name, const char* device,
+                        mpic_alloc_fn alloc, void* user, mpic_context** out) {
+  if (!world || !op || !device || !out) return MPIC_INVALID_ARGUMENT;
+  if (rank < 0 || rank >= world->size || (world->real_rank >= 0 && rank != world->real_rank))
+    return MPIC_INVALID_ARGUMENT;
+  if (!OpRegistry::Global()->LookUp(op)) return MPIC_NOT_FOUND;
+  const mpic::KernelDef* kdef = OpRegistry::Global()->FindKernel(op, device);
+  if (!kdef) return MPIC_NOT_FOUND;  // "No OpKernel was registered to support Op ... on this device"
+  mpic_context* c = new mpic_context();
+  mpic::OpKernelConstruction construction(node_name && *node_name ? node_name : op);
+  c->kernel.reset(kdef->factory(&construction));
+  mpic::OutputAllocator allocator;
+  if (alloc) {
+    allocator = [alloc, user](mpic::DataType dt, const mpic::TensorShape& shape, bool host) -> void* {
+      return alloc(user, static_cast<int>(dt), shape.dims(), shape.dim_sizes().data(), host ? 1 : 0);
+    };
+  }
+  c->ctx.reset(new mpic::OpKernelContext(world, rank, !strcmp(device, "GPU"), allocator));
+  *out = c;
+  return MPIC_OK;
+}
+
+int mpic_context_add_input(mpic_context* c, int dtype, int ndims, const int64_t* dims, const void* data,
+                           int host_memory) {
+  if (!c || c->started || ndims < 0 || ndims > 8 || (ndims > 0 && !dims)) return MPIC_INVALID_ARGUMENT;
+  std::vector<int64_t> d(dims, dims + ndims);
+  c->ctx->AddInput(mpic::Tensor(static_cast<mpic::DataType>(dtype), mpic::TensorShape(d), const_cast<void*>(data),
+                                host_memory != 0));
+  return MPIC_OK;
+}
+
+int mpic_context_compute(mpic_context* c) {
+  if (!c || c->started) return MPIC_INVALID_ARGUMENT;
+  c->started = true;
+  auto done = [c] {
+    {
+      std::lock_guard<std::mutex> guard(c->mu);
+      c->done = true;
+    }
+    c->cv.notify_all();
+  };
+  if (c->kernel->IsAsync()) {
+    static_cast<mpic::AsyncOpKernel*>(c->kernel.get())->ComputeAsync(c->ctx.get(), done);
+  } else {
+    c->kernel->Compute(c->ctx.get());
+    done();
+  }
+  return MPIC_OK;
+}
+
+int mpic_context_wait(mpic_context* c) {
+  if (!c || !c->started) return MPIC_INVALID_ARGUMENT;
+  std::unique_lock<std::mutex> lock(c->mu);
+  c->cv.wait(lock, [c] { return c->done; });
+  return static_cast<int>(c->ctx->status().code());
+}
+
+const char* mpic_context_message(const mpic_context* c) {
+  return c ? c->ctx->status().error_message().c_str() : "";
+}
+
+int mpic_context_num_outputs(const mpic_context* c) { return c ? c->ctx->num_outputs() : 0; }
+
+int mpic_context_output(const mpic_context* c, int index, int* dtype, int* ndims, int64_t* dims, void** data) {
+  if (!c || index < 0 || index >= c->ctx->num_outputs()) return MPIC_INVALID_ARGUMENT;
+  const mpic::Tensor* t = c->ctx->output(index);
+  if (!t) return MPIC_INVALID_ARGUMENT;
+  if (dtype) *dtype = static_cast<int>(t->dtype());
+  if (ndims) *ndims = t->shape().dims();
+  if (dims) for (int i = 0; i < t->shape().dims() && i < 8; i++) dims[i] = t->dim_size(i);
+  if (data) *data = t->data();
+  return MPIC_OK;
+}
+
+int mpic_context_destroy(mpic_context* c) {
+  if (!c) return MPIC_OK;
+  if (c->started) {  // never free a context the background thread may still call back into
+    std::unique_lock<std::mutex> lock(c->mu);
+    c->cv.wait(lock, [c] { return c->done; });
+  }
+  delete c;
+  return MPIC_OK;
+}
+
+// ---- the ring driver without the op layer --------------------------------------------
+
+int mpic_ring_allreduce_prestaged(int n, int r, int dtype, const void* input, void* output, size_t count,
+                                  const void* const* rs_segments, const void* const* ag_segments, void* stream,
+                                  int flags) {
+  mpic::Status s = mpic::RingAllreducePrestaged(n, r, static_cast<mpic::DataType>(dtype), input, output, count,
+                                                rs_segments, ag_segments, stream, mpic::RingOptions::FromFlags(flags));
+  return s.ok() ? MPIC_OK : mpic::Fail(s);
+}
+
+int mpic_ring_allgather_prestaged(int n, int r, int dtype, const void* input, const size_t* rows,
+                                  size_t elems_per_row, void* output, const void* const* segments, void* stream,
+                                  int flags) {
+  if (n < 1 || !rows) return MPIC_INVALID_ARGUMENT;
+  std::vector<size_t> rv(rows, rows + n);
+  mpic::Status s = mpic::RingAllgatherPrestaged(n, r, static_cast<mpic::DataType>(dtype), input, rv, elems_per_row,
+                                                output, segments, stream, mpic::RingOptions::FromFlags(flags));
+  return s.ok() ? MPIC_OK : mpic::Fail(s);
+}
+
+int mpic_ring_allreduce_all_ranks(int n, int dtype, const void* const* inputs, void* const* outputs, size_t count,
+                                  void* stream, int flags) {
+  if (n < 1 || !inputs || !outputs) return MPIC_INVALID_ARGUMENT;
+  mpic::Status s = mpic::RingAllreduceAllRanks(n, static_cast<mpic::DataType>(dtype), inputs, outputs, count, stream,
+                                               mpic::RingOptions::FromFlags(flags));
+  return s.ok() ? MPIC_OK : mpic::Fail(s);
+}
+
+int mpic_ring_allgather_all_ranks(int n, int dtype, const void* const* inputs, const size_t* rows,
+                                  size_t elems_per_row, void* const* outputs, void* stream, int flags) {
+  if (n < 1 || !inputs || !outputs || !rows) return MPIC_INVALID_ARGUMENT;
+  std::vector<size_t> rv(rows, rows + n);
+  mpic::Status s = mpic::RingAllgatherAllRanks(n, static_cast<mpic::DataType>(dtype), inputs, rv, elems_per_row,
+                                               outputs, stream, mpic::RingOptions::FromFlags(flags));
+  return s.ok() ? MPIC_OK : mpic::Fail(s);
+}
+
+const char* mpic_last_error(void) { return mpic::g_last_error.c_str(); }
+
+}  // extern "C"

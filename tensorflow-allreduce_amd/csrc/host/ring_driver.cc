@@ -1,0 +1,226 @@
+#include "ring_driver.h"
+
+#include <string>
+
+#include "ring_abi.h"
+
+namespace mpic {
+namespace {
+
+// The reference's MPI_REQUIRES_OK (ring.h:36-39) for the device layer.
+Status FromRing(int rc, const char* what) {
+  if (rc == RING_OK) return Status::OK();
+  std::string msg = std::string(what) + ": " + ring_status_string(rc);
+  if (rc == RING_ERR_HIP) msg += " (hipError " + std::to_string(ring_last_hip_error()) + ")";
+  if (rc == RING_ERR_DTYPE) return errors::FailedPrecondition(ring_status_string(rc));
+  return errors::Unknown(msg);
+}
+#define RING_RETURN_IF_ERROR(call, what)      \
+  do {                                        \
+    Status s_ = FromRing((call), (what));     \
+    if (!s_.ok()) return s_;                  \
+  } while (0)
+
+inline const char* at(const void* base, size_t elems, size_t esz) {
+  return static_cast<const char*>(base) + elems * esz;
+}
+inline char* at(void* base, size_t elems, size_t esz) { return static_cast<char*>(base) + elems * esz; }
+
+int Seg(int phase, int n, int r, int step, bool recv) {
+  int s = 0, v = 0;
+  ring_schedule(phase, n, r, step, &s, &v);
+  return recv ? v : s;
+}
+
+}  // namespace
+
+Status RingDataType(DataType dt, int* ring_dtype) {
+  switch (dt) {
+    case DT_FLOAT: *ring_dtype = RING_F32; return Status::OK();
+    case DT_INT32: *ring_dtype = RING_I32; return Status::OK();
+    case DT_INT64: *ring_dtype = RING_I64; return Status::OK();
+    default: return errors::FailedPrecondition("Invalid tensor type passed.");
+  }
+}
+
+Status RingAllreducePrestaged(int n, int r, DataType dt, const void* input, void* output, size_t count,
+                              const void* const* rs_recv, const void* const* ag_recv, void* stream,
+                              const RingOptions& opts) {
+  int code = 0;
+  Status s = RingDataType(dt, &code);
+  if (!s.ok()) return s;
+  if (n < 1 || r < 0 || r >= n) return errors::InvalidArgument("rank out of range for the ring");
+  const size_t esz = ring_dtype_size(code);
+  if (count == 0) return Status::OK();
+  if (!input || !output) return errors::InvalidArgument("null tensor with a non-zero element count");
+  if (n > 1 && (!rs_recv || !ag_recv)) return errors::InvalidArgument("no staged peer segments");
+
+  std::vector<size_t> sizes(static_cast<size_t>(n)), starts(static_cast<size_t>(n));
+  RING_RETURN_IF_ERROR(ring_segment_table(count, n, sizes.data(), starts.data()), "ring_segment_table");
+
+  const bool fuse = opts.fuse_copy && opts.batched && input != output && n > 1;
+  if (!fuse && input != output)  // ring.h:146-148
+    RING_RETURN_IF_ERROR(ring_copy_bytes(output, input, count * esz, stream), "ring_copy_bytes");
+  if (n == 1) return Status::OK();
+
+  // ring.h:183-205: step i receives segment (r-i-1) and adds it into the buffer
+  if (fuse) {
+    std::vector<ring_row> rows;
+    for (int i = 0; i < n - 1; i++) {
+      const size_t seg = static_cast<size_t>(Seg(RING_PHASE_REDUCE_SCATTER, n, r, i, true));
+      rows.push_back(ring_row{at(output, starts[seg], esz), rs_recv[i], at(input, starts[seg], esz), sizes[seg]});
+    }
+    // segment r is only ever sent, never accumulated: plain copy
+    const size_t own = static_cast<size_t>(r);
+    rows.push_back(ring_row{at(output, starts[own], esz), at(input, starts[own], esz), nullptr, sizes[own]});
+    RING_RETURN_IF_ERROR(ring_apply_rows(rows.data(), static_cast<int>(rows.size()), code, stream),
+                         "ring_apply_rows");
+  } else if (opts.batched) {
+    std::vector<ring_step> steps;
+    for (int i = 0; i < n - 1; i++) {
+      const size_t seg = static_cast<size_t>(Seg(RING_PHASE_REDUCE_SCATTER, n, r, i, true));
+      steps.push_back(ring_step{starts[seg], rs_recv[i], sizes[seg]});
+    }
+    RING_RETURN_IF_ERROR(ring_reduce_scatter_steps(output, steps.data(), n - 1, code, stream),
+                         "ring_reduce_scatter_steps");
+  } else {
+    for (int i = 0; i < n - 1; i++) {
+      const size_t seg = static_cast<size_t>(Seg(RING_PHASE_REDUCE_SCATTER, n, r, i, true));
+      RING_RETURN_IF_ERROR(ring_accumulate(code, at(output, starts[seg], esz), rs_recv[i], sizes[seg], stream),
+                           "ring_accumulate");
+    }
+  }
+
+  // ring.h:211-225: step i receives segment (r-i) straight into the buffer
+  if (opts.batched) {
+    std::vector<ring_step> steps;
+    for (int i = 0; i < n - 1; i++) {
+      const size_t seg = static_cast<size_t>(Seg(RING_PHASE_ALLGATHER, n, r, i, true));
+      steps.push_back(ring_step{starts[seg], ag_recv[i], sizes[seg]});
+    }
+    RING_RETURN_IF_ERROR(ring_allgather_steps(output, steps.data(), n - 1, code, stream), "ring_allgather_steps");
+  } else {
+    for (int i = 0; i < n - 1; i++) {
+      const size_t seg = static_cast<size_t>(Seg(RING_PHASE_ALLGATHER, n, r, i, true));
+      RING_RETURN_IF_ERROR(ring_copy_bytes(at(output, starts[seg], esz), ag_recv[i], sizes[seg] * esz, stream),
+                           "ring_copy_bytes");
+    }
+  }
+  return Status::OK();
+}
+
+Status RingAllgatherPrestaged(int n, int r, DataType dt, const void* input, const std::vector<size_t>& rows,
+                              size_t elems_per_row, void* output, const void* const* recv, void* stream,
+                              const RingOptions& opts) {
+  int code = 0;
+  Status s = RingDataType(dt, &code);
+  if (!s.ok()) return s;
+  if (n < 1 || r < 0 || r >= n || rows.size() != static_cast<size_t>(n))
+    return errors::InvalidArgument("rank or sizes do not match the ring");
+  const size_t esz = ring_dtype_size(code);
+  std::vector<size_t> starts(static_cast<size_t>(n));
+  RING_RETURN_IF_ERROR(ring_allgather_table(rows.data(), n, elems_per_row, starts.data()), "ring_allgather_table");
+
+  // ring.h:263-266: own slice to its offset
+  const size_t own = elems_per_row * rows[static_cast<size_t>(r)];
+  if (own && (!input || !output)) return errors::InvalidArgument("null tensor with a non-zero element count");
+  if (n > 1 && !recv) return errors::InvalidArgument("no staged peer segments");
+
+  // ring.h:279-298: step i receives segment (r-i-1) in place. With a step table
+  // the own-slice copy is one more row of the same launch.
+  if (opts.batched) {
+    std::vector<ring_step> steps;
+    steps.push_back(ring_step{starts[static_cast<size_t>(r)], input, own});
+    for (int i = 0; i < n - 1; i++) {
+      const size_t seg = static_cast<size_t>(Seg(RING_PHASE_GATHER, n, r, i, true));
+      steps.push_back(ring_step{starts[seg], recv[i], elems_per_row * rows[seg]});
+    }
+    RING_RETURN_IF_ERROR(ring_allgather_steps(output, steps.data(), n, code, stream), "ring_allgather_steps");
+  } else {
+    RING_RETURN_IF_ERROR(ring_copy_bytes(at(output, starts[static_cast<size_t>(r)], esz), input, own * esz, stream),
+                         "ring_copy_bytes");
+    for (int i = 0; i < n - 1; i++) {
+      const size_t seg = static_cast<size_t>(Seg(RING_PHASE_GATHER, n, r, i, true));
+      RING_RETURN_IF_ERROR(
+          ring_copy_bytes(at(output, starts[seg], esz), recv[i], elems_per_row * rows[seg] * esz, stream),
+          "ring_copy_bytes");
+    }
+  }
+  return Status::OK();
+}
+
+Status RingAllreduceAllRanks(int n, DataType dt, const void* const* inputs, void* const* outputs, size_t count,
+                             void* stream, const RingOptions& opts) {
+  (void)opts;
+  int code = 0;
+  Status s = RingDataType(dt, &code);
+  if (!s.ok()) return s;
+  if (n < 1) return errors::InvalidArgument("empty ring");
+  if (count == 0) return Status::OK();
+  const size_t esz = ring_dtype_size(code);
+  std::vector<size_t> sizes(static_cast<size_t>(n)), starts(static_cast<size_t>(n));
+  RING_RETURN_IF_ERROR(ring_segment_table(count, n, sizes.data(), starts.data()), "ring_segment_table");
+
+  std::vector<ring_row> rows(static_cast<size_t>(n));
+  // ring.h:146-148 on every rank
+  for (int r = 0; r < n; r++) {
+    if (!inputs[r] || !outputs[r]) return errors::InvalidArgument("null tensor with a non-zero element count");
+    rows[static_cast<size_t>(r)] = ring_row{outputs[r], inputs[r], nullptr, count};
+  }
+  RING_RETURN_IF_ERROR(ring_apply_rows(rows.data(), n, code, stream), "ring_apply_rows");
+
+  // ring.h:183-205: at step i rank r adds its left neighbour's segment (r-i-1)
+  for (int i = 0; i < n - 1; i++) {
+    for (int r = 0; r < n; r++) {
+      const int left = (r - 1 + n) % n;
+      const size_t seg = static_cast<size_t>(Seg(RING_PHASE_REDUCE_SCATTER, n, r, i, true));
+      char* dst = at(outputs[r], starts[seg], esz);
+      rows[static_cast<size_t>(r)] = ring_row{dst, at(static_cast<const void*>(outputs[left]), starts[seg], esz), dst, sizes[seg]};
+    }
+    RING_RETURN_IF_ERROR(ring_apply_rows(rows.data(), n, code, stream), "ring_apply_rows");
+  }
+  // ring.h:211-225: at step i rank r receives segment (r-i) from the left
+  for (int i = 0; i < n - 1; i++) {
+    for (int r = 0; r < n; r++) {
+      const int left = (r - 1 + n) % n;
+      const size_t seg = static_cast<size_t>(Seg(RING_PHASE_ALLGATHER, n, r, i, true));
+      rows[static_cast<size_t>(r)] = ring_row{at(outputs[r], starts[seg], esz),
+                                              at(static_cast<const void*>(outputs[left]), starts[seg], esz), nullptr, sizes[seg]};
+    }
+    RING_RETURN_IF_ERROR(ring_apply_rows(rows.data(), n, code, stream), "ring_apply_rows");
+  }
+  return Status::OK();
+}
+
+Status RingAllgatherAllRanks(int n, DataType dt, const void* const* inputs, const std::vector<size_t>& rows_per_rank,
+                             size_t elems_per_row, void* const* outputs, void* stream, const RingOptions& opts) {
+  (void)opts;
+  int code = 0;
+  Status s = RingDataType(dt, &code);
+  if (!s.ok()) return s;
+  if (n < 1 || rows_per_rank.size() != static_cast<size_t>(n)) return errors::InvalidArgument("sizes do not match the ring");
+  const size_t esz = ring_dtype_size(code);
+  std::vector<size_t> starts(static_cast<size_t>(n));
+  RING_RETURN_IF_ERROR(ring_allgather_table(rows_per_rank.data(), n, elems_per_row, starts.data()), "ring_allgather_table");
+
+  std::vector<ring_row> rows(static_cast<size_t>(n));
+  for (int r = 0; r < n; r++) {  // ring.h:263-266
+    const size_t own = elems_per_row * rows_per_rank[static_cast<size_t>(r)];
+    if (own && (!inputs[r] || !outputs[r])) return errors::InvalidArgument("null tensor with a non-zero element count");
+    rows[static_cast<size_t>(r)] = ring_row{own ? at(outputs[r], starts[static_cast<size_t>(r)], esz) : nullptr, inputs[r], nullptr, own};
+  }
+  RING_RETURN_IF_ERROR(ring_apply_rows(rows.data(), n, code, stream), "ring_apply_rows");
+  for (int i = 0; i < n - 1; i++) {  // ring.h:279-298
+    for (int r = 0; r < n; r++) {
+      const int left = (r - 1 + n) % n;
+      const size_t seg = static_cast<size_t>(Seg(RING_PHASE_GATHER, n, r, i, true));
+      const size_t cnt = elems_per_row * rows_per_rank[seg];
+      rows[static_cast<size_t>(r)] = ring_row{cnt ? at(outputs[r], starts[seg], esz) : nullptr,
+                                              cnt ? at(static_cast<const void*>(outputs[left]), starts[seg], esz) : nullptr, nullptr, cnt};
+    }
+    RING_RETURN_IF_ERROR(ring_apply_rows(rows.data(), n, code, stream), "ring_apply_rows");
+  }
+  return Status::OK();
+}
+
+}  // namespace mpic

@@ -1,0 +1,59 @@
+// Host side of the ring: segmenting, step schedule and step tables for one
+// rank (or for all virtual ranks at once), issued through the C ABI of
+// ring_abi.h. The counterpart of RingAllreduce / RingAllgather in
+// tensorflow/contrib/mpi_collectives/ring.h:136-301 with the MPI
+// point-to-point calls replaced by segments that are already addressable in
+// device memory.
+#ifndef MPIC_RING_DRIVER_H_
+#define MPIC_RING_DRIVER_H_
+
+#include <cstddef>
+#include <vector>
+
+#include "framework.h"
+
+namespace mpic {
+
+struct RingOptions {
+  // One launch per ring phase (all n-1 steps of a rank) instead of one per
+  // step. Steps of one rank write disjoint segments, so the order inside a
+  // phase does not matter and the result is bit-identical.
+  bool batched = true;
+  // Fold the in->out copy (ring.h:146-148) into the reduce-scatter:
+  // out[seg] = in[seg] + received, the same single add per element.
+  bool fuse_copy = false;
+  static RingOptions FromFlags(int flags) {
+    RingOptions o;
+    o.batched = (flags & 1) != 0;
+    o.fuse_copy = (flags & 2) != 0;
+    return o;
+  }
+};
+
+// ring.cu.cc:14-20 / mpi_ops.cc:836-847: the three supported element types.
+// Sets *ring_dtype to the ring_abi.h code.
+Status RingDataType(DataType dt, int* ring_dtype);
+
+// ring.h:136-228 for rank r of n. rs_recv[i] / ag_recv[i]: device pointers to
+// the segment the left neighbour sends at reduce-scatter / allgather step i
+// (n-1 each). Asynchronous on `stream`.
+Status RingAllreducePrestaged(int n, int r, DataType dt, const void* input, void* output, size_t count,
+                              const void* const* rs_recv, const void* const* ag_recv, void* stream,
+                              const RingOptions& opts);
+
+// ring.h:236-301 for rank r of n. recv[i]: the segment received at step i
+// (segment (r-i-1) mod n).
+Status RingAllgatherPrestaged(int n, int r, DataType dt, const void* input, const std::vector<size_t>& rows,
+                              size_t elems_per_row, void* output, const void* const* recv, void* stream,
+                              const RingOptions& opts);
+
+// All n ranks on this GPU, advancing in lockstep: at every step each rank
+// reads its left neighbour's buffer where MPI would have delivered a copy
+// (the neighbour does not write that segment during the step).
+Status RingAllreduceAllRanks(int n, DataType dt, const void* const* inputs, void* const* outputs, size_t count,
+                             void* stream, const RingOptions& opts);
+Status RingAllgatherAllRanks(int n, DataType dt, const void* const* inputs, const std::vector<size_t>& rows,
+                             size_t elems_per_row, void* const* outputs, void* stream, const RingOptions& opts);
+
+}  // namespace mpic
+#endif  // MPIC_RING_DRIVER_H_

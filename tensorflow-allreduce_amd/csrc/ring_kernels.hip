@@ -61,7 +61,10 @@ template <> struct VecOf<float> { typedef float type __attribute__((ext_vector_t
 template <> struct VecOf<uint32_t> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
 template <> struct VecOf<uint64_t> { typedef uint64_t type __attribute__((ext_vector_type(2))); };
 
-enum Mode { kCopy = 0, kAccumulate = 1 };
+// kCopy: every row is dst = a. kAdd: a row with a second operand is
+// dst = b + a (b may be dst itself: the in-place accumulate of the reference),
+// a row without one is still a copy, so one launch can mix both.
+enum Mode { kCopy = 0, kAdd = 1 };
 
 // Rows of one launch, passed by value in the kernel arguments (read with
 // scalar loads; uniform per workgroup).
@@ -69,7 +72,8 @@ struct RowTable {
   int n_rows;
   uint32_t tile_begin[kMaxRows + 1];  // prefix sum of tiles per row
   void* dst[kMaxRows];
-  const void* src[kMaxRows];
+  const void* a[kMaxRows];  // incoming segment
+  const void* b[kMaxRows];  // local operand of an add row, null for a copy row
   uint64_t count[kMaxRows];  // elements
 };
 
@@ -79,12 +83,15 @@ __device__ __forceinline__ void store_vec(typename VecOf<T>::type* p, typename V
 }
 
 // One workgroup-tile of a row: vectors [v0, v0 + 256*UNROLL) of the aligned
-// body, plus the row's scalar head (tile 0) and tail (last tile).
-template <typename T, int MODE, int UNROLL, bool NT>
-__device__ __forceinline__ void row_tile(T* __restrict__ dst, const T* __restrict__ src,
+// body, plus the row's scalar head (tile 0) and tail (last tile). dst is
+// brought to 16-byte alignment by the head; a and b are read with
+// element-aligned 16-byte loads. b == dst is allowed (every element is read
+// before it is written, by the same lane).
+template <typename T, bool ADD, int UNROLL, bool NT>
+__device__ __forceinline__ void row_tile(T* dst, const T* __restrict__ a, const T* b,
                                          uint64_t count, uint32_t tile, uint32_t tiles_in_row) {
   typedef typename VecOf<T>::type V;
-  typedef V VU __attribute__((aligned(sizeof(T))));  // element-aligned 16-byte load
+  typedef V VU __attribute__((aligned(sizeof(T))));  // element-aligned 16-byte access
   constexpr uint32_t VEC = 16 / sizeof(T);
   constexpr uint32_t kTileVecs = kBlock * UNROLL;
 
@@ -94,40 +101,40 @@ __device__ __forceinline__ void row_tile(T* __restrict__ dst, const T* __restric
   const uint32_t tid = threadIdx.x;
 
   if (tile == 0 && tid < head) {
-    if (MODE == kAccumulate) dst[tid] = dst[tid] + src[tid]; else dst[tid] = src[tid];
+    if (ADD) dst[tid] = b[tid] + a[tid]; else dst[tid] = a[tid];
   }
   if (tile + 1 == tiles_in_row) {
-    const uint64_t tail_start = head + nvec * VEC;
-    const uint64_t e = tail_start + tid;
+    const uint64_t e = head + nvec * VEC + tid;
     if (e < count) {
-      if (MODE == kAccumulate) dst[e] = dst[e] + src[e]; else dst[e] = src[e];
+      if (ADD) dst[e] = b[e] + a[e]; else dst[e] = a[e];
     }
   }
 
-  V* __restrict__ dv = reinterpret_cast<V*>(dst + head);
-  const VU* __restrict__ sv = reinterpret_cast<const VU*>(src + head);
+  V* dv = reinterpret_cast<V*>(dst + head);
+  const VU* __restrict__ av = reinterpret_cast<const VU*>(a + head);
+  const VU* bv = reinterpret_cast<const VU*>(b + head);
   const uint64_t v0 = static_cast<uint64_t>(tile) * kTileVecs + tid;
 
   if (static_cast<uint64_t>(tile + 1) * kTileVecs <= nvec) {
-    V s[UNROLL], d[UNROLL];
+    V x[UNROLL], y[UNROLL];
 #pragma unroll
-    for (int j = 0; j < UNROLL; j++) s[j] = __builtin_nontemporal_load(&sv[v0 + j * kBlock]);
-    if (MODE == kAccumulate) {
+    for (int j = 0; j < UNROLL; j++) x[j] = __builtin_nontemporal_load(&av[v0 + j * kBlock]);
+    if (ADD) {
 #pragma unroll
-      for (int j = 0; j < UNROLL; j++) d[j] = __builtin_nontemporal_load(&dv[v0 + j * kBlock]);
+      for (int j = 0; j < UNROLL; j++) y[j] = __builtin_nontemporal_load(&bv[v0 + j * kBlock]);
 #pragma unroll
-      for (int j = 0; j < UNROLL; j++) s[j] = d[j] + s[j];
+      for (int j = 0; j < UNROLL; j++) x[j] = y[j] + x[j];
     }
 #pragma unroll
-    for (int j = 0; j < UNROLL; j++) store_vec<T, NT>(&dv[v0 + j * kBlock], s[j]);
+    for (int j = 0; j < UNROLL; j++) store_vec<T, NT>(&dv[v0 + j * kBlock], x[j]);
   } else {
 #pragma unroll
     for (int j = 0; j < UNROLL; j++) {
       const uint64_t v = v0 + j * kBlock;
       if (v < nvec) {
-        V s = __builtin_nontemporal_load(&sv[v]);
-        if (MODE == kAccumulate) s = __builtin_nontemporal_load(&dv[v]) + s;
-        store_vec<T, NT>(&dv[v], s);
+        V x = __builtin_nontemporal_load(&av[v]);
+        if (ADD) x = __builtin_nontemporal_load(&bv[v]) + x;
+        store_vec<T, NT>(&dv[v], x);
       }
     }
   }
@@ -144,8 +151,12 @@ __global__ void __launch_bounds__(kBlock) rows_kernel(const RowTable tab) {
       if (tab.tile_begin[mid] <= t) lo = mid; else hi = mid;
     }
     const uint32_t first = tab.tile_begin[lo];
-    row_tile<T, MODE, UNROLL, NT>(static_cast<T*>(tab.dst[lo]), static_cast<const T*>(tab.src[lo]),
-                                  tab.count[lo], t - first, tab.tile_begin[lo + 1] - first);
+    const uint32_t tiles = tab.tile_begin[lo + 1] - first;
+    T* dst = static_cast<T*>(tab.dst[lo]);
+    const T* a = static_cast<const T*>(tab.a[lo]);
+    const T* b = static_cast<const T*>(tab.b[lo]);
+    if (MODE == kAdd && b != nullptr) row_tile<T, true, UNROLL, NT>(dst, a, b, tab.count[lo], t - first, tiles);
+    else row_tile<T, false, UNROLL, NT>(dst, a, nullptr, tab.count[lo], t - first, tiles);
   }
 }
 
@@ -233,8 +244,8 @@ fusion_kernel(T* __restrict__ fused, const uint64_t* __restrict__ offsets, T* co
     const uint32_t t1 = tile_last[tile];
     if (t0 == t1) {
       T* tensor = ptrs[t0] + (e0 - offsets[t0]);
-      if (PACK) row_tile<T, kCopy, 4, NT>(fused + e0, tensor, e1 - e0, 0, 1);
-      else row_tile<T, kCopy, 4, NT>(tensor, fused + e0, e1 - e0, 0, 1);
+      if (PACK) row_tile<T, false, 4, NT>(fused + e0, tensor, nullptr, e1 - e0, 0, 1);
+      else row_tile<T, false, 4, NT>(tensor, fused + e0, nullptr, e1 - e0, 0, 1);
       continue;
     }
     const uint32_t span = t1 - t0 + 1;
@@ -320,12 +331,13 @@ int launch_rows_typed(const RowTable& tab, uint32_t grid, hipStream_t stream) {
 
 struct HostRow {
   void* dst;
-  const void* src;
+  const void* a;
+  const void* b;   // null: copy row
   uint64_t count;  // elements of `esz` bytes
 };
 
-// Launches rows (any number) in groups of kMaxRows. esz: 4 or 8.
-template <int MODE>
+// Launches rows (any number) in groups of kMaxRows. esz: 4 or 8. A table with
+// no add row runs the copy-only kernel.
 int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, hipStream_t stream) {
   const int unroll = (g_tuning.unroll == 2 || g_tuning.unroll == 8) ? g_tuning.unroll : 4;
   const uint64_t tile_vecs = static_cast<uint64_t>(kBlock) * unroll;
@@ -337,6 +349,7 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
     tab.n_rows = 0;
     tab.tile_begin[0] = 0;
     uint64_t tiles = 0;
+    bool any_add = false;
     while (i < n_rows && tab.n_rows < kMaxRows) {
       const HostRow& r = rows[i];
       if (r.count == 0) { i++; continue; }
@@ -352,8 +365,10 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
       }
       const int k = tab.n_rows++;
       tab.dst[k] = r.dst;
-      tab.src[k] = r.src;
+      tab.a[k] = r.a;
+      tab.b[k] = r.b;
       tab.count[k] = r.count;
+      any_add = any_add || r.b != nullptr;
       tiles += t;
       tab.tile_begin[k + 1] = static_cast<uint32_t>(tiles);
       i++;
@@ -367,9 +382,16 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
       if (grid > cap) grid = static_cast<uint32_t>(cap);
     }
     int rc;
-    if (esz == 8) rc = launch_rows_typed<uint64_t, MODE>(tab, grid, stream);
-    else if (is_float && MODE == kAccumulate) rc = launch_rows_typed<float, MODE>(tab, grid, stream);
-    else rc = launch_rows_typed<uint32_t, MODE>(tab, grid, stream);
+    if (!any_add) {
+      rc = esz == 8 ? launch_rows_typed<uint64_t, kCopy>(tab, grid, stream)
+                    : launch_rows_typed<uint32_t, kCopy>(tab, grid, stream);
+    } else if (esz == 8) {
+      rc = launch_rows_typed<uint64_t, kAdd>(tab, grid, stream);
+    } else if (is_float) {
+      rc = launch_rows_typed<float, kAdd>(tab, grid, stream);
+    } else {
+      rc = launch_rows_typed<uint32_t, kAdd>(tab, grid, stream);
+    }
     if (rc != RING_OK) return rc;
   }
   return RING_OK;
@@ -378,7 +400,11 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
 inline bool dtype_ok(int dtype) { return dtype == RING_F32 || dtype == RING_I32 || dtype == RING_I64; }
 inline size_t dtype_size(int dtype) { return dtype == RING_I64 ? 8 : (dtype_ok(dtype) ? 4 : 0); }
 
-int steps_common(void* buffer, const ring_step* steps, int n_steps, int dtype, void* stream, bool accumulate) {
+enum StepKind { kStepCopy, kStepAddInPlace, kStepAddFrom };
+
+// input: the local operand of kStepAddFrom rows (same element offsets as buffer).
+int steps_common(const void* input, void* buffer, const ring_step* steps, int n_steps, int dtype,
+                 void* stream, StepKind kind) {
   if (!dtype_ok(dtype)) return RING_ERR_DTYPE;
   if (n_steps < 0) return RING_ERR_ARGUMENT;
   if (n_steps == 0) return RING_OK;
@@ -388,15 +414,15 @@ int steps_common(void* buffer, const ring_step* steps, int n_steps, int dtype, v
   rows.reserve(static_cast<size_t>(n_steps));
   for (int i = 0; i < n_steps; i++) {
     if (steps[i].count == 0) continue;
-    if (!buffer || !steps[i].src) return RING_ERR_ARGUMENT;
+    if (!buffer || !steps[i].src || (kind == kStepAddFrom && !input)) return RING_ERR_ARGUMENT;
     char* d = static_cast<char*>(buffer) + steps[i].dst_offset * esz;
-    if ((reinterpret_cast<uintptr_t>(d) | reinterpret_cast<uintptr_t>(steps[i].src)) & (esz - 1))
+    const char* local = kind == kStepAddFrom ? static_cast<const char*>(input) + steps[i].dst_offset * esz : d;
+    if ((reinterpret_cast<uintptr_t>(d) | reinterpret_cast<uintptr_t>(steps[i].src) |
+         reinterpret_cast<uintptr_t>(local)) & (esz - 1))
       return RING_ERR_ARGUMENT;
-    rows.push_back(HostRow{d, steps[i].src, steps[i].count});
+    rows.push_back(HostRow{d, steps[i].src, kind == kStepCopy ? nullptr : local, steps[i].count});
   }
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  if (accumulate) return launch_rows<kAccumulate>(rows.data(), rows.size(), esz, dtype == RING_F32, s);
-  return launch_rows<kCopy>(rows.data(), rows.size(), esz, false, s);
+  return launch_rows(rows.data(), rows.size(), esz, dtype == RING_F32, static_cast<hipStream_t>(stream));
 }
 
 }  // namespace
@@ -570,8 +596,8 @@ int ring_copy_bytes(void* dst, const void* src, size_t bytes, void* stream) {
   hipStream_t s = static_cast<hipStream_t>(stream);
   const uintptr_t all = reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src) | bytes;
   if ((all & 3u) == 0) {
-    HostRow row{dst, src, bytes / 4};
-    return launch_rows<kCopy>(&row, 1, 4, false, s);
+    HostRow row{dst, src, nullptr, bytes / 4};
+    return launch_rows(&row, 1, 4, false, s);
   }
   uint64_t blocks = (bytes + kBlock - 1) / kBlock;
   if (blocks > 65536) blocks = 65536;
@@ -589,8 +615,8 @@ int ring_accumulate(int dtype, void* dst, const void* src, size_t count, void* s
   const size_t esz = dtype_size(dtype);
   if ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & (esz - 1))
     return RING_ERR_ARGUMENT;
-  HostRow row{dst, src, count};
-  return launch_rows<kAccumulate>(&row, 1, esz, dtype == RING_F32, static_cast<hipStream_t>(stream));
+  HostRow row{dst, src, dst, count};
+  return launch_rows(&row, 1, esz, dtype == RING_F32, static_cast<hipStream_t>(stream));
 }
 
 int ring_accumulate_f32(float* dst, const float* src, size_t count, void* stream) {
@@ -604,11 +630,36 @@ int ring_accumulate_i64(int64_t* dst, const int64_t* src, size_t count, void* st
 }
 
 int ring_reduce_scatter_steps(void* buffer, const ring_step* steps, int n_steps, int dtype, void* stream) {
-  return steps_common(buffer, steps, n_steps, dtype, stream, true);
+  return steps_common(nullptr, buffer, steps, n_steps, dtype, stream, kStepAddInPlace);
+}
+
+int ring_reduce_scatter_steps_from(const void* input, void* buffer, const ring_step* steps, int n_steps,
+                                   int dtype, void* stream) {
+  if (input == buffer) return steps_common(nullptr, buffer, steps, n_steps, dtype, stream, kStepAddInPlace);
+  return steps_common(input, buffer, steps, n_steps, dtype, stream, kStepAddFrom);
+}
+
+int ring_apply_rows(const ring_row* rows, int n_rows, int dtype, void* stream) {
+  if (!dtype_ok(dtype)) return RING_ERR_DTYPE;
+  if (n_rows < 0) return RING_ERR_ARGUMENT;
+  if (n_rows == 0) return RING_OK;
+  if (!rows) return RING_ERR_ARGUMENT;
+  const size_t esz = dtype_size(dtype);
+  std::vector<HostRow> host;
+  host.reserve(static_cast<size_t>(n_rows));
+  for (int i = 0; i < n_rows; i++) {
+    if (rows[i].count == 0) continue;
+    if (!rows[i].dst || !rows[i].a) return RING_ERR_ARGUMENT;
+    if ((reinterpret_cast<uintptr_t>(rows[i].dst) | reinterpret_cast<uintptr_t>(rows[i].a) |
+         reinterpret_cast<uintptr_t>(rows[i].b)) & (esz - 1))
+      return RING_ERR_ARGUMENT;
+    host.push_back(HostRow{rows[i].dst, rows[i].a, rows[i].b, rows[i].count});
+  }
+  return launch_rows(host.data(), host.size(), esz, dtype == RING_F32, static_cast<hipStream_t>(stream));
 }
 
 int ring_allgather_steps(void* buffer, const ring_step* steps, int n_steps, int dtype, void* stream) {
-  return steps_common(buffer, steps, n_steps, dtype, stream, false);
+  return steps_common(nullptr, buffer, steps, n_steps, dtype, stream, kStepCopy);
 }
 
 int ring_scale(int dtype, void* data, size_t count, int divisor, void* stream) {

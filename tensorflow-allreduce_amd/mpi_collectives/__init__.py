@@ -1,1 +1,482 @@
-"""MI355X-native ring collectives with the API of tensorflow.contrib.mpi_collectives."""
+"""MI355X-native ring collectives with the API of tensorflow.contrib.mpi_collectives.
+
+This package mirrors ``tensorflow/contrib/mpi_collectives/__init__.py``:
+``allreduce``, ``allgather``, ``DistributedOptimizer`` and ``Session`` (plus
+``size``, ``rank``, ``local_rank``, ``init``), over torch tensors that live in
+the HBM of one MI355X. The per-rank data path of the ring (segment split,
+reduce-scatter accumulate, allgather copies, fusion pack/unpack) runs in
+hand-written gfx950 kernels behind a C ABI; there is no CPU implementation.
+
+Ranks are *virtual*. Where the reference runs one MPI process per rank, a
+``Session`` here owns all ranks in one process, on one GPU:
+
+    import mpi_collectives as mpi
+
+    with mpi.Session(size=8) as session:            # runs init(), like mpi.Session
+        sums = []
+        for r in range(8):                          # what each process would do
+            with session.as_rank(r):
+                sums.append(mpi.allreduce(x[r], average=False))
+        sums = session.run(sums)                    # list of torch tensors
+
+As in graph-mode TensorFlow the collective calls return handles; a reduction
+"will not start until all processes are ready", so values exist once every
+rank has submitted the op and ``session.run`` has been called. A session can
+instead hold ONE real rank whose peers' incoming segments were staged in HBM
+beforehand (``Session(size=8, rank=3)`` + ``session.stage_peers``); its
+collectives complete at once.
+
+@@Session
+@@DistributedOptimizer
+@@allreduce
+@@allgather
+"""
+import contextlib
+import os
+
+import torch
+
+from . import _plugin, mpi_ops, ring_abi
+from ._plugin import (FailedPreconditionError, InternalError, InvalidArgumentError,  # noqa: F401
+                      NotFoundError, OpError, UnknownError)
+from .mpi_ops import _allreduce, allgather, init, local_rank, rank, size  # noqa: F401
+
+_TORCH2RING = {torch.float32: ring_abi.F32, torch.int32: ring_abi.I32, torch.int64: ring_abi.I64}
+
+
+class PendingTensor:
+    """Handle of a collective's result (the graph tensor of the reference).
+
+    ``session.run(handle)`` or ``handle.result()`` returns the torch tensor once
+    every rank has submitted the op."""
+
+    def __init__(self, session):
+        self._session = session
+        self._value = None
+        self._error = None
+        self._ready = False
+        self._post = []       # fn(tensor) -> tensor applied to the value when it arrives
+
+    def _set(self, value=None, error=None):
+        if error is None:
+            for fn in self._post:
+                value = fn(value)
+        self._value, self._error, self._ready = value, error, True
+
+    def result(self):
+        if not self._ready:
+            self._session.run()
+        if self._error is not None:
+            raise self._error
+        return self._value
+
+
+class IndexedSlices:
+    """A sparse representation of a set of tensor slices at given indices
+    (the tf.IndexedSlices the reference's allreduce accepts)."""
+
+    def __init__(self, values, indices, dense_shape=None):
+        self.values, self.indices, self.dense_shape = values, indices, dense_shape
+
+
+def _env_size():
+    """Ranks from the launcher's environment, the variables the reference's
+    tests read (mpi_ops_test.py:30-62); 1 when not started under mpirun."""
+    for var in ("PMI_SIZE", "OMPI_COMM_WORLD_SIZE"):
+        if os.environ.get(var):
+            return int(os.environ[var])
+    return 1
+
+
+class Session:
+    """Runs MPI ops for a set of virtual ranks; the counterpart of
+    tf.contrib.mpi.Session (``__init__.py:237-273``): it initializes MPI
+    immediately upon starting.
+
+    Args:
+      target, graph, config: accepted for signature compatibility; unused.
+      size: number of ranks in the ring (default: the launcher's environment,
+        else 1).
+      rank: None if all `size` ranks live in this session; otherwise the one
+        real rank, whose peers are pre-staged with `stage_peers`.
+      device: "GPU" (default when a GPU is present) or "CPU": where init() runs.
+        Collectives have GPU kernels only.
+    """
+
+    def __init__(self, target='', graph=None, config=None, size=None, rank=None, device=None):
+        del target, graph, config
+        L = _plugin.load_library('libmpi_collectives.so', mpi_ops._REQUIRED_OPS)
+        self.size = int(size) if size is not None else _env_size()
+        self.real_rank = rank
+        self.device = device or ("GPU" if torch.cuda.is_available() else "CPU")
+        import ctypes
+        h = ctypes.c_void_p()
+        if rank is None:
+            rc = L.mpic_world_create(self.size, ctypes.byref(h))
+        else:
+            rc = L.mpic_world_create_prestaged(self.size, int(rank), ctypes.byref(h))
+        if rc != 0:
+            raise _plugin.error_for(rc, "could not create an MPI world of size %r, rank %r" % (size, rank))
+        self._world = h.value
+        self._pending = []          # ops submitted and not yet waited for
+        self._submitted = {}        # node name -> set of ranks, for the run() guard
+        self._counters = {}         # (rank, op) -> next auto-name index
+        self._keep = []             # staged buffers kept alive until consumed
+        self._prev = None
+        self._enter_scope()
+        try:
+            # Initialize MPI on the relevant device (__init__.py:271-273).
+            self.run(init())
+        except Exception:
+            self.close()
+            raise
+
+    # -- scoping ---------------------------------------------------------------
+    def _enter_scope(self):
+        self._prev = (mpi_ops._scope.session, mpi_ops._scope.rank)
+        mpi_ops._scope.session = self
+        mpi_ops._scope.rank = self.real_rank if self.real_rank is not None else 0
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+        return False
+
+    @contextlib.contextmanager
+    def as_rank(self, r):
+        """Run the enclosed MPI ops as virtual rank `r`."""
+        if not 0 <= r < self.size or (self.real_rank is not None and r != self.real_rank):
+            raise InvalidArgumentError("rank %r is not a rank of this session" % (r,))
+        prev = (mpi_ops._scope.session, mpi_ops._scope.rank)
+        mpi_ops._scope.session, mpi_ops._scope.rank = self, r
+        try:
+            yield self
+        finally:
+            mpi_ops._scope.session, mpi_ops._scope.rank = prev
+
+    def close(self):
+        if self._world is not None:
+            _plugin.lib().mpic_world_destroy(self._world)
+            self._world = None
+            if mpi_ops._scope.session is self and self._prev is not None:
+                mpi_ops._scope.session, mpi_ops._scope.rank = self._prev
+            self._pending, self._keep = [], []
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # -- world ---------------------------------------------------------------------
+    @property
+    def stream(self):
+        """The world's dedicated HIP stream (CudaStreamForMPI), as an integer handle."""
+        return _plugin.lib().mpic_world_stream(self._world)
+
+    def set_option(self, name, value):
+        """"batched", "fuse_copy" or "sync": see mpic_world_set_option."""
+        rc = _plugin.lib().mpic_world_set_option(self._world, name.encode(), int(value))
+        if rc != 0:
+            raise InvalidArgumentError("unknown session option %r" % name)
+
+    def stage_peers(self, name, rs_segments, ag_segments):
+        """Pre-stage what the left neighbour sends for the collective with node
+        name `name`: lists of n-1 CUDA tensors (reduce-scatter steps, allgather
+        steps). For an allgather pass rs_segments=None."""
+        import ctypes
+        n1 = self.size - 1
+        rs = list(rs_segments) if rs_segments is not None else None
+        ag = list(ag_segments)
+        if len(ag) != n1 or (rs is not None and len(rs) != n1):
+            raise InvalidArgumentError("a ring of %d ranks needs %d staged segments per phase" % (self.size, n1))
+        arr_ag = (ctypes.c_void_p * max(n1, 1))(*[t.data_ptr() if t.numel() else None for t in ag])
+        arr_rs = None
+        if rs is not None:
+            arr_rs = (ctypes.c_void_p * max(n1, 1))(*[t.data_ptr() if t.numel() else None for t in rs])
+        rc = _plugin.lib().mpic_stage_peers(self._world, name.encode(), arr_rs, arr_ag)
+        if rc != 0:
+            raise InvalidArgumentError("stage_peers needs a session created with rank=...")
+        self._keep.append((rs, ag))
+
+    # -- op submission (used by mpi_ops) ------------------------------------------------
+    def _node_name(self, r, op, name):
+        """TensorFlow uniquifies node names per graph: op, op_1, op_2, ... Every
+        rank builds the same graph, so the k-th unnamed op matches across ranks."""
+        base = name if name is not None else op
+        k = self._counters.get((r, base), 0)
+        self._counters[(r, base)] = k + 1
+        return base if k == 0 else "%s_%d" % (base, k)
+
+    def _submit(self, r, op, node_name, inputs, device):
+        if any(t.is_cuda for t in inputs):
+            # the inputs' producers must have finished before the ring reads them (the
+            # reference defers the enqueue with a stream host callback, mpi_ops.cc:1099-1105)
+            torch.cuda.current_stream().synchronize()
+        pending = _plugin.PendingOp(self._world, r, op, node_name, inputs, device)
+        pending.rank = r
+        if op in ("MPIAllreduce", "MPIAllgather"):
+            self._submitted.setdefault(node_name, set()).add(r)
+            self._pending.append(pending)
+        return pending
+
+    @property
+    def _immediate(self):
+        return self.real_rank is not None or self.size == 1
+
+    def _result(self, pending):
+        handle = PendingTensor(self)
+        pending.handle = handle
+        pending.on_done = None
+        if self._immediate:
+            self._drain()
+        return handle
+
+    def _chain_allgather(self, r, sizing, tensor, name, dev):
+        handle = PendingTensor(self)
+        sizing.handle = None
+
+        def after_sizing(outputs):
+            sizes = outputs[0].cpu() if outputs[0].is_cuda else outputs[0]   # host-memory `sizes` input
+            node = self._node_name(r, 'MPIAllgather', name)
+            with self.as_rank(r):
+                second = self._submit(r, 'MPIAllgather', node, [tensor, sizes], dev)
+            second.handle = handle
+            second.on_done = None
+
+        sizing.on_done = after_sizing
+        sizing.fail_handle = handle
+        if self._immediate:
+            self._drain()
+        return handle
+
+    def _after(self, handle, fn):
+        """Run fn(tensor) -> tensor on the result of `handle` once it exists."""
+        if not handle._ready:
+            handle._post.append(fn)
+        elif handle._error is None:
+            handle._value = fn(handle._value)
+
+    def _check_all_ranks_submitted(self):
+        if self.real_rank is not None:
+            return
+        for p in self._pending:
+            ranks = self._submitted.get(p.node_name, set())
+            if len(ranks) != self.size:
+                raise FailedPreconditionError(
+                    "collective %r was submitted by ranks %s of %d; every rank must submit it "
+                    "before the session runs" % (p.node_name, sorted(ranks), self.size))
+
+    def _drain(self):
+        first_error = None
+        while self._pending:
+            self._check_all_ranks_submitted()
+            batch, self._pending = self._pending, []
+            for p in batch:
+                self._submitted.pop(p.node_name, None)
+            for p in batch:
+                try:
+                    outputs = p.wait()
+                    if getattr(p, "on_done", None):
+                        p.on_done(outputs)
+                    if getattr(p, "handle", None) is not None:
+                        p.handle._set(value=outputs[0])
+                except OpError as e:
+                    first_error = first_error or e
+                    for h in (getattr(p, "handle", None), getattr(p, "fail_handle", None)):
+                        if h is not None:
+                            h._set(error=e)
+        if self.stream:
+            ring_abi.stream_synchronize(self.stream)
+        if first_error is not None:
+            raise first_error
+
+    def run(self, fetches=None, feed_dict=None):
+        """Completes every submitted collective and returns `fetches` with each
+        handle replaced by its torch tensor."""
+        del feed_dict
+        self._drain()
+        return _resolve(fetches)
+
+
+def _resolve(x):
+    if isinstance(x, PendingTensor):
+        return x.result()
+    if isinstance(x, IndexedSlices):
+        return IndexedSlices(_resolve(x.values), _resolve(x.indices), x.dense_shape)
+    if isinstance(x, (list, tuple)):
+        return type(x)(_resolve(v) for v in x)
+    if isinstance(x, dict):
+        return {k: _resolve(v) for k, v in x.items()}
+    return x
+
+
+def _div(session, handle):
+    """tf.div(x, cast(size(), x.dtype)) applied to a collective's result: true
+    division for float32, floor division for integers (__init__.py:160-164,
+    math_ops.py:982-985), by the ring_scale kernel on the session's stream."""
+    n = session.size
+
+    def fn(t):
+        if t.numel():
+            ring_abi.scale(_TORCH2RING[t.dtype], t.data_ptr(), t.numel(), n, session.stream)
+            ring_abi.stream_synchronize(session.stream)
+        return t
+
+    session._after(handle, fn)
+    return handle
+
+
+def allreduce(tensor, average=True):
+    """Perform an MPI allreduce on a torch.Tensor or an IndexedSlices.
+
+    Arguments:
+        tensor: torch.Tensor (on the GPU) or IndexedSlices to reduce. The
+                shape of the input must be identical across all ranks.
+        average: If True, computes the average over all ranks.
+                 Otherwise, computes the sum over all ranks.
+
+    This function performs a bandwidth-optimal ring allreduce on the input
+    tensor. If the input is an IndexedSlices, the function instead does an
+    allgather on the values and the indices, effectively doing an allreduce on
+    the represented tensor.
+    """
+    session, _ = mpi_ops._current()
+    if isinstance(tensor, IndexedSlices):
+        # For IndexedSlices, do two allgathers instead of an allreduce.
+        values = allgather(tensor.values)
+        indices = allgather(tensor.indices)
+        # To make this operation into an average, divide all gathered values by the MPI size.
+        new_values = _div(session, values) if average else values
+        return IndexedSlices(new_values, indices, dense_shape=tensor.dense_shape)
+    summed_tensor = _allreduce(tensor)
+    return _div(session, summed_tensor) if average else summed_tensor
+
+
+class DistributedOptimizer:
+    """An optimizer that wraps a torch.optim.Optimizer, using an MPI allreduce
+    to average gradient values before applying gradients to model weights
+    (``__init__.py:167-234``).
+
+    Args:
+      optimizer: optimizer to use for applying updates.
+      name: optional name prefix for the collectives this optimizer issues;
+        defaults to "Distributed" followed by the optimizer's type.
+      use_locking: accepted for signature compatibility.
+      fusion: pack all dense float32 gradients into one fusion buffer and
+        reduce them with a single ring allreduce (not in the reference, which
+        issues one allreduce per gradient).
+    """
+
+    def __init__(self, optimizer, name=None, use_locking=False, fusion=False):
+        if name is None:
+            name = "Distributed{}".format(type(optimizer).__name__)
+        self._optimizer = optimizer
+        self._name = name
+        self._use_locking = use_locking
+        self._fusion = fusion
+        self._fused = None      # (FusionPlan, fused buffer, grads) while a fused allreduce is in flight
+
+    @property
+    def param_groups(self):
+        return self._optimizer.param_groups
+
+    def _params(self, var_list=None):
+        if var_list is not None:
+            return list(var_list)
+        return [p for g in self._optimizer.param_groups for p in g["params"]]
+
+    def compute_gradients(self, loss=None, var_list=None):
+        """Gradients of all trainable variables, allreduced (averaged) across
+        ranks. Calls loss.backward() when a loss is given; returns a list of
+        (gradient handle, variable) pairs."""
+        if loss is not None:
+            loss.backward()
+        params = [p for p in self._params(var_list) if p.grad is not None]
+        if self._fusion:
+            return self._compute_fused(params)
+        out = []
+        for p in params:
+            g = p.grad
+            if g.is_sparse:
+                g = g.coalesce()
+                slices = IndexedSlices(g.values().contiguous(), g.indices()[0].contiguous(), dense_shape=g.shape)
+                out.append((allreduce(slices), p))
+            else:
+                out.append((allreduce(g.contiguous()), p))
+        return out
+
+    def _compute_fused(self, params):
+        session, _ = mpi_ops._current()
+        dense = [p for p in params if not p.grad.is_sparse and p.grad.dtype == torch.float32]
+        dense_ids = {id(p) for p in dense}
+        rest = [p for p in params if id(p) not in dense_ids]
+        grads = [p.grad.contiguous() for p in dense]
+        plan = ring_abi.FusionPlan([g.data_ptr() if g.numel() else None for g in grads],
+                                   [g.numel() for g in grads], ring_abi.F32)
+        fused = torch.empty(plan.elements, dtype=torch.float32, device="cuda")
+        torch.cuda.current_stream().synchronize()      # the gradients' producers
+        plan.pack(fused.data_ptr(), session.stream)
+        ring_abi.stream_synchronize(session.stream)
+        handle = allreduce(fused, average=True)
+        unpacked = {"done": False}
+
+        def unpack(t):
+            if not unpacked["done"]:
+                plan.unpack(t.data_ptr(), session.stream)
+                ring_abi.stream_synchronize(session.stream)
+                unpacked["done"] = True
+                plan.close()
+            return t
+
+        session._after(handle, unpack)
+        out = [(_FusedGrad(handle, g), p) for g, p in zip(grads, dense)]
+        for p in rest:
+            out.append((allreduce(p.grad.contiguous()), p))
+        return out
+
+    def apply_gradients(self, grads_and_vars, global_step=None, name=None):
+        """Stores the reduced gradients on their variables and steps the
+        wrapped optimizer."""
+        del global_step, name
+        for g, p in grads_and_vars:
+            g = _resolve(g.resolve() if isinstance(g, _FusedGrad) else g)
+            if isinstance(g, IndexedSlices):
+                idx = g.indices.reshape(1, -1)
+                p.grad = torch.sparse_coo_tensor(idx, g.values, size=tuple(g.dense_shape)).coalesce()
+            else:
+                p.grad = g.reshape(p.shape)
+        return self._optimizer.step()
+
+    def minimize(self, loss, global_step=None, var_list=None):
+        """compute_gradients followed by apply_gradients. In a session that holds
+        several virtual ranks call the two halves yourself, with every rank's
+        compute_gradients before the first apply_gradients."""
+        return self.apply_gradients(self.compute_gradients(loss, var_list), global_step=global_step)
+
+    def step(self, closure=None):
+        if closure is not None:
+            closure()
+        return self.apply_gradients(self.compute_gradients())
+
+    def zero_grad(self, *args, **kwargs):
+        return self._optimizer.zero_grad(*args, **kwargs)
+
+    def state_dict(self):
+        return self._optimizer.state_dict()
+
+    def load_state_dict(self, state):
+        return self._optimizer.load_state_dict(state)
+
+
+class _FusedGrad:
+    """A gradient that comes back through the fusion buffer."""
+
+    def __init__(self, handle, grad):
+        self._handle, self._grad = handle, grad
+
+    def resolve(self):
+        self._handle.result()      # runs the unpack
+        return self._grad

@@ -1,0 +1,245 @@
+"""Loader and op runner for the plugin library (lib/libmpi_collectives.so).
+
+Plays the part of ``tf.load_op_library`` plus the TensorFlow executor for the
+six MPI ops (tensorflow/contrib/mpi_collectives/mpi_ops.py:30-59): the library
+registers its ops at load time, `load_library` verifies the required op list,
+and `run_op` builds an op context, feeds torch tensors as inputs and lets the
+op allocate its outputs through a callback, as an OpKernelContext would.
+"""
+import ctypes
+import os
+
+import torch
+
+from . import ring_abi
+
+_PKG_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(_PKG_ROOT, "lib", "libmpi_collectives.so")
+
+# TensorFlow DataType numbers (types.proto) <-> torch dtypes
+DT_FLOAT, DT_DOUBLE, DT_INT32, DT_INT64 = 1, 2, 3, 9
+TORCH2DT = {torch.float32: DT_FLOAT, torch.float64: DT_DOUBLE, torch.int32: DT_INT32, torch.int64: DT_INT64}
+DT2TORCH = {v: k for k, v in TORCH2DT.items()}
+
+OK, UNKNOWN, INVALID_ARGUMENT, NOT_FOUND, FAILED_PRECONDITION, INTERNAL = 0, 2, 3, 5, 9, 13
+
+EXPORTS = (
+    "mpic_op_count", "mpic_op_name", "mpic_op_signature", "mpic_op_doc", "mpic_op_has_kernel",
+    "mpic_op_infer_shape", "mpic_world_create", "mpic_world_create_prestaged", "mpic_world_destroy",
+    "mpic_world_size", "mpic_world_stream", "mpic_world_set_option", "mpic_stage_peers",
+    "mpic_context_create", "mpic_context_add_input", "mpic_context_compute", "mpic_context_wait",
+    "mpic_context_message", "mpic_context_num_outputs", "mpic_context_output", "mpic_context_destroy",
+    "mpic_ring_allreduce_prestaged", "mpic_ring_allgather_prestaged", "mpic_ring_allreduce_all_ranks",
+    "mpic_ring_allgather_all_ranks", "mpic_last_error",
+)
+
+
+class OpError(RuntimeError):
+    """Base of the op errors; `code` is TensorFlow's error code."""
+    code = UNKNOWN
+
+    def __init__(self, message, code=None):
+        super().__init__(message)
+        self.message = message
+        if code is not None:
+            self.code = code
+
+
+class FailedPreconditionError(OpError):
+    code = FAILED_PRECONDITION
+
+
+class InvalidArgumentError(OpError):
+    code = INVALID_ARGUMENT
+
+
+class NotFoundError(OpError):
+    code = NOT_FOUND
+
+
+class UnknownError(OpError):
+    code = UNKNOWN
+
+
+class InternalError(OpError):
+    code = INTERNAL
+
+
+_ERRORS = {FAILED_PRECONDITION: FailedPreconditionError, INVALID_ARGUMENT: InvalidArgumentError,
+           NOT_FOUND: NotFoundError, UNKNOWN: UnknownError, INTERNAL: InternalError}
+
+
+def error_for(code, message):
+    return _ERRORS.get(code, OpError)(message, code)
+
+
+ALLOC_FN = ctypes.CFUNCTYPE(ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
+                            ctypes.POINTER(ctypes.c_int64), ctypes.c_int)
+
+_lib = None
+
+
+def load_library(name="libmpi_collectives.so", op_list=None):
+    """Loads the plugin and checks it registers every op in `op_list`.
+
+    Raises NameError if one is missing (mpi_ops.py:41-51) and RuntimeError if
+    the library has not been built: there is no fallback implementation.
+    """
+    global _lib
+    if _lib is None:
+        path = os.path.join(_PKG_ROOT, "lib", name)
+        if not os.path.exists(path):
+            raise RuntimeError("%s is missing: build it with `python tensorflow-allreduce_amd/build.py`" % path)
+        ring_abi.lib()   # the kernels library first, so a missing build fails with its own message
+        L = ctypes.CDLL(path)
+        ci, sz, vp, cp = ctypes.c_int, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_char_p
+        p64 = ctypes.POINTER(ctypes.c_int64)
+        pvp = ctypes.POINTER(vp)
+        pint = ctypes.POINTER(ctypes.c_int)
+        psz = ctypes.POINTER(ctypes.c_size_t)
+        sig = {
+            "mpic_op_count": (ci, []),
+            "mpic_op_name": (cp, [ci]),
+            "mpic_op_signature": (cp, [cp]),
+            "mpic_op_doc": (cp, [cp]),
+            "mpic_op_has_kernel": (ci, [cp, cp]),
+            "mpic_op_infer_shape": (ci, [cp, ci, p64, p64]),
+            "mpic_world_create": (ci, [ci, pvp]),
+            "mpic_world_create_prestaged": (ci, [ci, ci, pvp]),
+            "mpic_world_destroy": (ci, [vp]),
+            "mpic_world_size": (ci, [vp]),
+            "mpic_world_stream": (vp, [vp]),
+            "mpic_world_set_option": (ci, [vp, cp, ci]),
+            "mpic_stage_peers": (ci, [vp, cp, pvp, pvp]),
+            "mpic_context_create": (ci, [vp, ci, cp, cp, cp, ALLOC_FN, vp, pvp]),
+            "mpic_context_add_input": (ci, [vp, ci, ci, p64, vp, ci]),
+            "mpic_context_compute": (ci, [vp]),
+            "mpic_context_wait": (ci, [vp]),
+            "mpic_context_message": (cp, [vp]),
+            "mpic_context_num_outputs": (ci, [vp]),
+            "mpic_context_output": (ci, [vp, ci, pint, pint, p64, pvp]),
+            "mpic_context_destroy": (ci, [vp]),
+            "mpic_ring_allreduce_prestaged": (ci, [ci, ci, ci, vp, vp, sz, pvp, pvp, vp, ci]),
+            "mpic_ring_allgather_prestaged": (ci, [ci, ci, ci, vp, psz, sz, vp, pvp, vp, ci]),
+            "mpic_ring_allreduce_all_ranks": (ci, [ci, ci, pvp, pvp, sz, vp, ci]),
+            "mpic_ring_allgather_all_ranks": (ci, [ci, ci, pvp, psz, sz, pvp, vp, ci]),
+            "mpic_last_error": (cp, []),
+        }
+        for sym in EXPORTS:
+            fn = getattr(L, sym)
+            fn.restype, fn.argtypes = sig[sym]
+        _lib = L
+    registered = op_names()
+    for expected_op in (op_list or []):
+        if expected_op not in registered:
+            raise NameError("Could not find operator %s in dynamic library %s" % (expected_op, name))
+    return _lib
+
+
+def lib():
+    return _lib if _lib is not None else load_library()
+
+
+def op_names():
+    L = _lib
+    return [L.mpic_op_name(i).decode() for i in range(L.mpic_op_count())]
+
+
+def op_signature(op):
+    s = lib().mpic_op_signature(op.encode())
+    return s.decode() if s else None
+
+
+def op_doc(op):
+    s = lib().mpic_op_doc(op.encode())
+    return s.decode() if s else None
+
+
+def infer_shape(op, shape):
+    """The op's shape function; unknown dimensions come back as None."""
+    dims = (ctypes.c_int64 * 8)(*shape)
+    out = (ctypes.c_int64 * 8)()
+    n = lib().mpic_op_infer_shape(op.encode(), len(shape), dims, out)
+    if n < 0:
+        raise InvalidArgumentError("shape inference failed for %s on %r" % (op, list(shape)))
+    return [None if out[i] < 0 else int(out[i]) for i in range(n)]
+
+
+class PendingOp:
+    """One op instance in flight: keeps inputs, outputs and the C context alive
+    until the op's done() has run."""
+
+    def __init__(self, world, rank, op, node_name, inputs, device):
+        L = lib()
+        self._outputs = []          # torch tensors the op allocated, in allocation order
+        self._inputs = inputs       # keep-alive
+        self._finalizers = []
+        self._waited = False
+        self.op, self.node_name = op, node_name
+
+        def _alloc(_user, dtype, ndims, dims, host_memory):
+            # Device outputs go to the GPU. On a machine without one the memory is
+            # host memory and no collective can run on it (the ops have GPU kernels
+            # only); the cross-rank checks, which need no device, still can.
+            try:
+                shape = [dims[i] for i in range(ndims)]
+                on_gpu = not host_memory and torch.cuda.is_available()
+                t = torch.empty(shape, dtype=DT2TORCH[dtype], device="cuda" if on_gpu else "cpu")
+                self._outputs.append(t)
+                return t.data_ptr() if t.numel() or host_memory else None
+            except Exception as e:            # never let an exception cross the C boundary
+                self._alloc_error = e
+                return None
+
+        self._alloc_cb = ALLOC_FN(_alloc)
+        h = ctypes.c_void_p()
+        rc = L.mpic_context_create(world, rank, op.encode(), (node_name or "").encode(), device.encode(),
+                                   self._alloc_cb, None, ctypes.byref(h))
+        if rc == NOT_FOUND:
+            raise NotFoundError("No OpKernel was registered to support Op '%s' on device %s" % (op, device))
+        if rc != OK:
+            raise error_for(rc, "could not create a context for %s (rank %d)" % (op, rank))
+        self._h = h.value
+        for t in inputs:
+            host = not t.is_cuda
+            if t.dtype not in TORCH2DT:
+                dt = 0                                  # DT_INVALID: rejected by the op
+            else:
+                dt = TORCH2DT[t.dtype]
+            dims = (ctypes.c_int64 * max(t.dim(), 1))(*t.shape)
+            rc = L.mpic_context_add_input(self._h, dt, t.dim(), dims, t.data_ptr() if t.numel() else None, int(host))
+            if rc != OK:
+                raise error_for(rc, "bad input for %s" % op)
+        rc = L.mpic_context_compute(self._h)
+        if rc != OK:
+            raise error_for(rc, "could not start %s" % op)
+
+    def add_finalizer(self, fn):
+        """fn() runs once after the op completed successfully (e.g. the average divide)."""
+        self._finalizers.append(fn)
+
+    def wait(self):
+        """Blocks until done(); raises the op's error; returns its outputs."""
+        if not self._waited:
+            L = lib()
+            code = L.mpic_context_wait(self._h)
+            msg = L.mpic_context_message(self._h).decode()
+            self._waited = True
+            L.mpic_context_destroy(self._h)
+            self._h = None
+            if code != OK:
+                self._error = error_for(code, msg)
+            else:
+                self._error = None
+                for fn in self._finalizers:
+                    fn()
+        if self._error is not None:
+            raise self._error
+        return self._outputs
+
+    @property
+    def outputs(self):
+        return self._outputs
+
+    # An op that was never waited for keeps its C context: the background
+    # thread may still call back into it, so it is not destroyed from a finalizer.

@@ -20,7 +20,8 @@ EXPORTS = (
     "ring_set_option", "ring_segment_table", "ring_temp_elements", "ring_allgather_table",
     "ring_schedule", "ring_stream_create", "ring_stream_destroy", "ring_stream_synchronize",
     "ring_copy_bytes", "ring_accumulate_f32", "ring_accumulate_i32", "ring_accumulate_i64",
-    "ring_accumulate", "ring_reduce_scatter_steps", "ring_allgather_steps",
+    "ring_accumulate", "ring_reduce_scatter_steps", "ring_reduce_scatter_steps_from",
+    "ring_allgather_steps", "ring_apply_rows",
     "ring_fusion_plan_create", "ring_fusion_plan_destroy", "ring_fusion_plan_elements",
     "ring_fusion_pack", "ring_fusion_unpack", "ring_scale",
 )
@@ -38,6 +39,12 @@ class RingError(RuntimeError):
 class Step(ctypes.Structure):
     """ring_step: one received segment of a step table."""
     _fields_ = [("dst_offset", ctypes.c_uint64), ("src", ctypes.c_void_p),
+                ("count", ctypes.c_uint64)]
+
+
+class Row(ctypes.Structure):
+    """ring_row: dst = a, or dst = b + a when b is not null."""
+    _fields_ = [("dst", ctypes.c_void_p), ("a", ctypes.c_void_p), ("b", ctypes.c_void_p),
                 ("count", ctypes.c_uint64)]
 
 
@@ -75,7 +82,9 @@ def lib():
             "ring_accumulate_i64": (ci, [vp, vp, sz, vp]),
             "ring_accumulate": (ci, [ci, vp, vp, sz, vp]),
             "ring_reduce_scatter_steps": (ci, [vp, ctypes.POINTER(Step), ci, ci, vp]),
+            "ring_reduce_scatter_steps_from": (ci, [vp, vp, ctypes.POINTER(Step), ci, ci, vp]),
             "ring_allgather_steps": (ci, [vp, ctypes.POINTER(Step), ci, ci, vp]),
+            "ring_apply_rows": (ci, [ctypes.POINTER(Row), ci, ci, vp]),
             "ring_fusion_plan_create": (ci, [ctypes.POINTER(vp), psz, ci, ci, ctypes.POINTER(vp)]),
             "ring_fusion_plan_destroy": (ci, [vp]),
             "ring_fusion_plan_elements": (sz, [vp]),
@@ -173,9 +182,23 @@ def reduce_scatter_steps(buffer, steps, n_steps, dtype, stream):
           "ring_reduce_scatter_steps")
 
 
+def reduce_scatter_steps_from(inp, buffer, steps, n_steps, dtype, stream):
+    check(lib().ring_reduce_scatter_steps_from(inp, buffer, steps, n_steps, dtype, stream),
+          "ring_reduce_scatter_steps_from")
+
+
 def allgather_steps(buffer, steps, n_steps, dtype, stream):
     check(lib().ring_allgather_steps(buffer, steps, n_steps, dtype, stream),
           "ring_allgather_steps")
+
+
+def apply_rows(rows, dtype, stream):
+    """rows: iterable of (dst, a, b_or_None, count) raw device pointers."""
+    rows = list(rows)
+    arr = (Row * max(len(rows), 1))()
+    for i, (d, a, b, cnt) in enumerate(rows):
+        arr[i].dst, arr[i].a, arr[i].b, arr[i].count = d, a, b, cnt
+    check(lib().ring_apply_rows(arr, len(rows), dtype, stream), "ring_apply_rows")
 
 
 def scale(dtype, data, count, divisor, stream):

@@ -64,3 +64,19 @@ def assert_same_bits(got, want, what=""):
         bad = np.flatnonzero(got.view(view) != want.view(view))
         raise AssertionError("%s: %d of %d elements differ, first at %d: got %r want %r"
                              % (what, bad.size, got.size, bad[0], got[bad[0]], want[bad[0]]))
+
+
+def resnet50_shapes():
+    """The 161 trainable tensors of ResNet-50 v1, in layer order."""
+    shapes = [(7, 7, 3, 64), (64,), (64,)]
+    cin = 64
+    for width, blocks in ((64, 3), (128, 4), (256, 6), (512, 3)):
+        for b in range(blocks):
+            shapes += [(1, 1, cin, width), (width,), (width,),
+                       (3, 3, width, width), (width,), (width,),
+                       (1, 1, width, 4 * width), (4 * width,), (4 * width,)]
+            if b == 0:
+                shapes += [(1, 1, cin, 4 * width), (4 * width,), (4 * width,)]
+            cin = 4 * width
+    shapes += [(2048, 1000), (1000,)]
+    return shapes

@@ -178,30 +178,6 @@ def test_scale_is_tf_div(dtype):
             assert np.all(G.host(keep[:off]) == 0) and np.all(G.host(keep[off + count:]) == 0)
 
 
-def resnet50_shapes():
-    """The 161 trainable tensors of ResNet-50 v1, in layer order."""
-    shapes = [(7, 7, 3, 64), (64,), (64,)]
-    cin = 64
-    for width, blocks in ((64, 3), (128, 4), (256, 6), (512, 3)):
-        for b in range(blocks):
-            shapes += [(1, 1, cin, width), (width,), (width,),
-                       (3, 3, width, width), (width,), (width,),
-                       (1, 1, width, 4 * width), (4 * width,), (4 * width,)]
-            if b == 0:
-                shapes += [(1, 1, cin, 4 * width), (4 * width,), (4 * width,)]
-            cin = 4 * width
-    shapes += [(2048, 1000), (1000,)]
-    return shapes
-
-
-def test_resnet50_shape_set():
-    shapes = resnet50_shapes()
-    sizes = [int(np.prod(s)) for s in shapes]
-    assert len(shapes) == 161 and sum(sizes) == 25_557_032
-    assert min(sizes) == 64 and max(sizes) == 2_359_296
-    assert sum(1 for s in sizes if s <= 2048) == 107
-
-
 def _fusion_roundtrip(counts, dtype, rng, offsets=None):
     code = G.NP2ABI[np.dtype(dtype)]
     hosts, devs, keep = [], [], []
@@ -239,7 +215,7 @@ def _fusion_roundtrip(counts, dtype, rng, offsets=None):
 @pytest.mark.parametrize("dtype", G.DTYPES)
 def test_fusion_pack_unpack(dtype):
     rng = np.random.default_rng(21)
-    _fusion_roundtrip([int(np.prod(s)) for s in resnet50_shapes()], dtype, rng)
+    _fusion_roundtrip([int(np.prod(s)) for s in G.resnet50_shapes()], dtype, rng)
     _fusion_roundtrip([], dtype, rng)
     _fusion_roundtrip([0, 0], dtype, rng)
     _fusion_roundtrip([1], dtype, rng)

@@ -1,0 +1,401 @@
+"""GPU parity of the whole ring against the CPU oracle, through the op layer
+(mpi_collectives.allreduce / allgather over virtual ranks) and through the
+ring driver's C entry points, on the configurations of the benchmark plan:
+float32 64 MiB at N=8, ragged int32/int64 at N=6, the ResNet-50 fusion set at
+N=8, variable-row allgather at N=16 and 1 GiB float32 at N=64.
+
+Bar: bit-exact for int32, int64 AND float32 (the ring fixes the order of the
+additions per segment); NaNs only have to be NaNs."""
+import ctypes
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+import gpu_util as G
+import mpi_collectives as mpi
+from gpu_util import ring_abi
+from mpi_collectives import _plugin
+
+pytestmark = pytest.mark.gpu
+
+DT = {np.dtype(np.float32): _plugin.DT_FLOAT, np.dtype(np.int32): _plugin.DT_INT32,
+      np.dtype(np.int64): _plugin.DT_INT64}
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _gpu():
+    G.require_gpu()
+
+
+def cuda(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def make_inputs(n, count, dtype, seed=0, wide=True):
+    return [G.random_array(np.random.default_rng(seed + r), count, dtype, wide=wide and dtype == np.float32)
+            for r in range(n)]
+
+
+# ---- all ranks resident: the op layer --------------------------------------------------
+
+@pytest.mark.parametrize("dtype", G.DTYPES)
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 6, 8])
+def test_allreduce_all_ranks_matches_oracle(oracle, dtype, n):
+    for count in sorted({0, 1, max(n - 1, 0), n, n + 1, 17, 4913, 1_000_003}):
+        ins = make_inputs(n, count, dtype, seed=31 * n + count)
+        want = oracle.ring_allreduce(ins)
+        with mpi.Session(size=n) as session:
+            handles = []
+            for r in range(n):
+                with session.as_rank(r):
+                    assert mpi.rank() == r
+                    handles.append(mpi.allreduce(cuda(ins[r]), average=False))
+            outs = session.run(handles)
+        for r in range(n):
+            G.assert_same_bits(G.host(outs[r]), want[r], "allreduce %s n=%d count=%d rank %d" % (dtype.__name__, n, count, r))
+
+
+@pytest.mark.parametrize("size", [1, 2, 3, 4, 7, 9, 12, 14])
+def test_reference_allreduce_gpu_test(oracle, size):
+    """mpi_ops_test.py:114-156 (and :84-112 for int32): every rank reduces the
+    same [17]^dim tensor; the sum equals tensor*size, exactly for size <= 3
+    (the reference's threshold 0). Above that the reference allows 1e-4 / 5e-4;
+    here the result must in addition equal the oracle's bit for bit."""
+    for dtype, dim in itertools.product((np.int32, np.float32), (1, 2, 3)):
+        rng = np.random.default_rng(1234)
+        t = rng.uniform(-100, 100, [17] * dim).astype(np.float32) if dtype == np.float32 \
+            else rng.integers(-100, 100, [17] * dim).astype(np.int32)
+        want = oracle.ring_allreduce([t] * size)[0]
+        with mpi.Session(size=size) as session:
+            hs = []
+            for r in range(size):
+                with session.as_rank(r):
+                    hs.append(mpi.allreduce(cuda(t), average=False))
+            outs = session.run(hs)
+        for o in outs:
+            assert list(o.shape) == [17] * dim
+            G.assert_same_bits(G.host(o), want, "same-input allreduce size=%d dim=%d" % (size, dim))
+            diff = np.max(np.abs(G.host(o) - t * dtype(size)))
+            if size <= 3 or dtype == np.int32:
+                assert diff == 0, "mpi.allreduce on GPU produces incorrect results"
+            else:
+                assert diff <= 1e-3
+
+
+@pytest.mark.parametrize("n", [2, 3, 6])
+def test_allreduce_average_is_tf_div(oracle, n):
+    """allreduce(average=True) = sum then tf.div by the size: true division for
+    float32, floor division for integers (__init__.py:160-164)."""
+    for dtype in G.DTYPES:
+        ins = make_inputs(n, 50_001, dtype, seed=5)
+        summed = oracle.ring_allreduce(ins)[0]
+        with np.errstate(all="ignore"):
+            want = summed / np.float32(n) if dtype == np.float32 else summed // dtype(n)
+        with mpi.Session(size=n) as session:
+            hs = []
+            for r in range(n):
+                with session.as_rank(r):
+                    hs.append(mpi.allreduce(cuda(ins[r])))            # average=True is the default
+            outs = session.run(hs)
+        for o in outs:
+            G.assert_same_bits(G.host(o), want.astype(dtype), "average %s n=%d" % (dtype.__name__, n))
+
+
+@pytest.mark.parametrize("size", [1, 2, 3, 7, 16])
+def test_reference_allgather_tests(size):
+    """mpi_ops_test.py:204-263: rank-stamped tensors, equal and variable first
+    dimension, 1-3 dims, int32 and float32 (int64 added)."""
+    tensor_sizes = ([17, 32, 81, 12, 15, 23, 22] * 5)[:size]
+    for dtype, dim, variable in itertools.product((torch.int32, torch.float32, torch.int64), (1, 2, 3), (False, True)):
+        rows = tensor_sizes if variable else [17] * size
+        with mpi.Session(size=size) as session:
+            hs = []
+            for r in range(size):
+                with session.as_rank(r):
+                    tensor = torch.ones([rows[r]] + [17] * (dim - 1), dtype=dtype, device="cuda") * r
+                    hs.append(mpi.allgather(tensor))
+            outs = session.run(hs)
+        for gathered in outs:
+            assert list(gathered.shape) == [sum(rows)] + [17] * (dim - 1)
+            for i in range(size):
+                part = gathered[sum(rows[:i]):sum(rows[:i + 1])]
+                assert list(part.shape) == [rows[i]] + [17] * (dim - 1)
+                assert bool((part == i).all()), "mpi.allgather produces incorrect gathered tensor"
+
+
+def test_allgather_variable_rows_n16_matches_oracle(oracle):
+    """Rank i contributes [rows_i, 1024] float32 with rows_i uniform in [1, 4096]."""
+    n = 16
+    rows = [int(np.random.default_rng(i).integers(1, 4097)) for i in range(n)]
+    ins = [np.random.default_rng(100 + i).standard_normal((rows[i], 1024)).astype(np.float32) for i in range(n)]
+    want = np.concatenate(ins, axis=0)
+    assert np.array_equal(oracle.ring_allgather([x[:3] for x in ins])[5], np.concatenate([x[:3] for x in ins]))
+    with mpi.Session(size=n) as session:
+        hs = []
+        for r in range(n):
+            with session.as_rank(r):
+                hs.append(mpi.allgather(cuda(ins[r]), name="rows"))
+        outs = session.run(hs)
+    for o in outs:
+        assert list(o.shape) == [sum(rows), 1024]
+    for r in (0, 7, 15):
+        G.assert_same_bits(G.host(outs[r]), want, "allgather n=16 rank %d" % r)
+    for r in range(n):       # all ranks hold the same bytes
+        assert torch.equal(outs[r], outs[0])
+
+
+def test_allgather_with_empty_ranks_and_indexed_slices(oracle):
+    n = 4
+    rows = [3, 0, 5, 1]
+    vals = [np.random.default_rng(r).standard_normal((rows[r], 6)).astype(np.float32) for r in range(n)]
+    idx = [np.arange(rows[r], dtype=np.int64) * 10 + r for r in range(n)]
+    with mpi.Session(size=n) as session:
+        hs = []
+        for r in range(n):
+            with session.as_rank(r):
+                sl = mpi.IndexedSlices(cuda(vals[r]), cuda(idx[r]), dense_shape=(100, 6))
+                hs.append(mpi.allreduce(sl))                        # two allgathers, values / n
+        outs = session.run(hs)
+    want_vals = np.concatenate(vals) / np.float32(n)
+    want_idx = np.concatenate(idx)
+    for o in outs:
+        G.assert_same_bits(G.host(o.values), want_vals, "IndexedSlices values")
+        assert np.array_equal(G.host(o.indices), want_idx)
+        assert o.dense_shape == (100, 6)
+
+
+# ---- ragged integers at N=6 (10,000,019 elements) -------------------------------------------
+
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+def test_ragged_integers_n6(oracle, dtype):
+    n, count = 6, 10_000_019
+    ins = [np.random.default_rng(r).integers(-1000, 1001, count).astype(dtype) for r in range(n)]
+    want = oracle.ring_allreduce_lockstep(ins)[0]
+    assert np.array_equal(want, sum(x.astype(np.int64) for x in ins).astype(dtype))   # integers: any order
+    with mpi.Session(size=n) as session:
+        hs = []
+        for r in range(n):
+            with session.as_rank(r):
+                hs.append(mpi.allreduce(cuda(ins[r]), average=False))
+        outs = session.run(hs)
+    for r in range(n):
+        G.assert_same_bits(G.host(outs[r]), want, "ragged %s rank %d" % (dtype.__name__, r))
+
+
+# ---- one real rank, peers pre-staged: the measured per-rank path ---------------------------
+
+def _prestaged(n, r, ins, rs, ag, flags, dtype):
+    """mpic_ring_allreduce_prestaged for rank r; returns the output tensor."""
+    L = _plugin.load_library()
+    count = ins[r].size
+    sizes, _ = ring_abi.segment_table(count, n)
+    din = cuda(ins[r])
+    dout = torch.zeros(count + 4, dtype=G.NP2TORCH[np.dtype(dtype)], device="cuda")[:count]
+    keep = []
+    rs_ptrs = (ctypes.c_void_p * max(n - 1, 1))()
+    ag_ptrs = (ctypes.c_void_p * max(n - 1, 1))()
+    for i in range(n - 1):
+        rseg = ring_abi.schedule(ring_abi.PHASE_REDUCE_SCATTER, n, r, i)[1]
+        aseg = ring_abi.schedule(ring_abi.PHASE_ALLGATHER, n, r, i)[1]
+        a = cuda(rs[r][i][:sizes[rseg]])
+        b = cuda(ag[r][i][:sizes[aseg]])
+        keep += [a, b]
+        rs_ptrs[i] = a.data_ptr() if a.numel() else None
+        ag_ptrs[i] = b.data_ptr() if b.numel() else None
+    stream = torch.cuda.current_stream().cuda_stream
+    rc = L.mpic_ring_allreduce_prestaged(n, r, DT[np.dtype(dtype)], din.data_ptr() if count else None,
+                                         dout.data_ptr() if count else None, count, rs_ptrs, ag_ptrs, stream, flags)
+    assert rc == 0, L.mpic_last_error()
+    torch.cuda.synchronize()
+    assert torch.equal(din, cuda(ins[r]))            # the input tensor is never written
+    return dout
+
+
+@pytest.mark.parametrize("dtype", G.DTYPES)
+def test_prestaged_rank_matches_oracle_small(oracle, dtype):
+    for n, count in ((1, 9), (2, 7), (3, 3), (4, 2), (6, 4099), (8, 100_003), (5, 0)):
+        ins = make_inputs(n, count, dtype, seed=n)
+        outs, rs, ag = oracle.ring_allreduce(ins, tap=True)
+        for r in sorted({0, n // 2, n - 1}):
+            for flags in (0, 1, 3):                  # per step; batched; batched + fused copy
+                got = _prestaged(n, r, ins, rs, ag, flags, dtype)
+                G.assert_same_bits(G.host(got), outs[r], "prestaged n=%d r=%d flags=%d" % (n, r, flags))
+
+
+def test_prestaged_64mib_float32_n8(oracle):
+    """The headline shape: 16,777,216 float32, N=8, values N(0,1) from seed=rank,
+    peers' segments staged from the oracle's full ring."""
+    n, count = 8, 16_777_216
+    ins = [np.random.default_rng(r).standard_normal(count, dtype=np.float32) for r in range(n)]
+    outs, rs, ag = oracle.ring_allreduce(ins, tap=True)
+    assert np.array_equal(outs[0], outs[5])
+    for r, flags in ((0, 1), (3, 3), (7, 0)):
+        got = _prestaged(n, r, ins, rs, ag, flags, np.float32)
+        G.assert_same_bits(G.host(got), outs[r], "64 MiB rank %d flags %d" % (r, flags))
+
+
+def test_prestaged_through_the_op_layer(oracle):
+    n, r, count = 4, 2, 70_001
+    ins = make_inputs(n, count, np.float32, seed=9)
+    outs, rs, ag = oracle.ring_allreduce(ins, tap=True)
+    sizes, _ = ring_abi.segment_table(count, n)
+    for fuse in (0, 1):
+        with mpi.Session(size=n, rank=r) as session:
+            session.set_option("fuse_copy", fuse)
+            assert mpi.rank() == r and mpi.size() == n
+            rs_t = [cuda(rs[r][i][:sizes[ring_abi.schedule(0, n, r, i)[1]]]) for i in range(n - 1)]
+            ag_t = [cuda(ag[r][i][:sizes[ring_abi.schedule(1, n, r, i)[1]]]) for i in range(n - 1)]
+            session.stage_peers("MPIAllreduce", rs_t, ag_t)
+            out = session.run(mpi.allreduce(cuda(ins[r]), average=False))
+            G.assert_same_bits(G.host(out), outs[r], "op layer, prestaged, fuse=%d" % fuse)
+            # nothing staged for the second call of that name
+            with pytest.raises(mpi.FailedPreconditionError, match="No pre-staged peer segments"):
+                session.run(mpi.allreduce(cuda(ins[r]), average=False))
+
+
+def test_prestaged_1gib_float32_n64():
+    """268,435,456 float32 (1 GiB), N=64: 63 + 63 steps on 16 MiB segments, one
+    launch per phase. Checked against numpy on the host: every reduce-scatter
+    step is input + received on its own segment, every allgather step a copy."""
+    n, r, count = 64, 37, 268_435_456
+    seg = count // n
+    gen = torch.Generator(device="cuda").manual_seed(r)
+    din = torch.randn(count, device="cuda", generator=gen)
+    rs = torch.randn(n - 1, seg, device="cuda", generator=gen)
+    ag = torch.randn(n - 1, seg, device="cuda", generator=gen)
+    dout = torch.empty(count, device="cuda")
+    L = _plugin.load_library()
+    rs_ptrs = (ctypes.c_void_p * (n - 1))(*[rs[i].data_ptr() for i in range(n - 1)])
+    ag_ptrs = (ctypes.c_void_p * (n - 1))(*[ag[i].data_ptr() for i in range(n - 1)])
+    stream = torch.cuda.current_stream().cuda_stream
+    # reduce-scatter only first: n-1 rows through the step-table entry point
+    ring_abi.copy_bytes(dout.data_ptr(), din.data_ptr(), count * 4, stream)
+    rows = [(ring_abi.schedule(0, n, r, i)[1] * seg, rs[i].data_ptr(), seg) for i in range(n - 1)]
+    steps, k = ring_abi.make_steps(rows)
+    ring_abi.reduce_scatter_steps(dout.data_ptr(), steps, k, ring_abi.F32, stream)
+    torch.cuda.synchronize()
+    hin, hrs, hout = G.host(din), G.host(rs), G.host(dout)
+    for i in range(n - 1):
+        s = ring_abi.schedule(0, n, r, i)[1]
+        G.assert_same_bits(hout[s * seg:(s + 1) * seg], hin[s * seg:(s + 1) * seg] + hrs[i], "RS step %d" % i)
+    G.assert_same_bits(hout[r * seg:(r + 1) * seg], hin[r * seg:(r + 1) * seg], "own segment")
+    # then the whole per-rank allreduce, batched and fused
+    dout.zero_()
+    rc = L.mpic_ring_allreduce_prestaged(n, r, _plugin.DT_FLOAT, din.data_ptr(), dout.data_ptr(), count,
+                                         rs_ptrs, ag_ptrs, stream, 3)
+    assert rc == 0, L.mpic_last_error()
+    torch.cuda.synchronize()
+    hout, hag = G.host(dout), G.host(ag)
+    owned = (r + 1) % n
+    for i in range(n - 1):
+        s = ring_abi.schedule(1, n, r, i)[1]
+        G.assert_same_bits(hout[s * seg:(s + 1) * seg], hag[i], "AG step %d" % i)
+    G.assert_same_bits(hout[owned * seg:(owned + 1) * seg],
+                       hin[owned * seg:(owned + 1) * seg] + hrs[n - 2], "owned segment")
+
+
+# ---- tensor fusion: the ResNet-50 gradient set at N=8 ------------------------------------------
+
+def test_fused_resnet50_allreduce_matches_ring_on_the_packed_buffer(oracle):
+    """161 float32 tensors ~N(0, 1e-3) packed into one buffer, ring-reduced at
+    N=8, unpacked. Parity is with the reference ring applied to the packed 1-D
+    buffer (fusion moves an element to another segment, hence another rotation
+    of the sum, than 161 separate allreduces would)."""
+    n = 8
+    shapes = G.resnet50_shapes()
+    counts = [int(np.prod(s)) for s in shapes]
+    grads = [[(np.random.default_rng(1000 * r + j).standard_normal(c) * 1e-3).astype(np.float32)
+              for j, c in enumerate(counts)] for r in range(n)]
+    packed = [np.concatenate(g) for g in grads]
+    want = oracle.ring_allreduce_lockstep(packed)[0]
+    stream = torch.cuda.current_stream().cuda_stream
+    dgrads = [[cuda(t) for t in g] for g in grads]
+    plans = [ring_abi.FusionPlan([t.data_ptr() for t in g], counts, ring_abi.F32) for g in dgrads]
+    fused_in = [torch.empty(sum(counts), device="cuda") for _ in range(n)]
+    fused_out = [torch.empty(sum(counts), device="cuda") for _ in range(n)]
+    for r in range(n):
+        plans[r].pack(fused_in[r].data_ptr(), stream)
+    L = _plugin.load_library()
+    ins = (ctypes.c_void_p * n)(*[t.data_ptr() for t in fused_in])
+    outs = (ctypes.c_void_p * n)(*[t.data_ptr() for t in fused_out])
+    rc = L.mpic_ring_allreduce_all_ranks(n, _plugin.DT_FLOAT, ins, outs, sum(counts), stream, 1)
+    assert rc == 0, L.mpic_last_error()
+    for r in range(n):
+        plans[r].unpack(fused_out[r].data_ptr(), stream)
+    torch.cuda.synchronize()
+    for r in (0, 4, 7):
+        at = 0
+        for j, c in enumerate(counts):
+            G.assert_same_bits(G.host(dgrads[r][j]), want[at:at + c], "fused rank %d tensor %d" % (r, j))
+            at += c
+
+
+def test_distributed_optimizer_fused_and_unfused(oracle):
+    """DistributedOptimizer.compute_gradients averages every gradient across
+    ranks (__init__.py:195-205); with fusion=True through one fused buffer."""
+    n = 3
+    torch.manual_seed(0)
+    base = torch.nn.Sequential(torch.nn.Linear(37, 19), torch.nn.Tanh(), torch.nn.Linear(19, 5)).cuda()
+    for fusion in (False, True):
+        replicas, opts, xs = [], [], []
+        for r in range(n):
+            m = torch.nn.Sequential(torch.nn.Linear(37, 19), torch.nn.Tanh(), torch.nn.Linear(19, 5)).cuda()
+            m.load_state_dict(base.state_dict())
+            replicas.append(m)
+            opts.append(mpi.DistributedOptimizer(torch.optim.SGD(m.parameters(), lr=0.1), fusion=fusion))
+            xs.append(torch.randn(11, 37, generator=torch.Generator().manual_seed(r)).cuda())
+        local = []
+        with mpi.Session(size=n) as session:
+            gvs = []
+            for r in range(n):
+                with session.as_rank(r):
+                    loss = replicas[r](xs[r]).square().mean()
+                    loss.backward()
+                    local.append([G.host(p.grad).reshape(-1).copy() for p in replicas[r].parameters()])
+                    gvs.append(opts[r].compute_gradients())
+            session.run()
+            for r in range(n):
+                with session.as_rank(r):
+                    opts[r].apply_gradients(gvs[r])
+        nparam = len(local[0])
+        if fusion:
+            summed = oracle.ring_allreduce([np.concatenate(local[r]) for r in range(n)])[0] / np.float32(n)
+            want, at = [], 0
+            for j in range(nparam):
+                want.append(summed[at:at + local[0][j].size])
+                at += local[0][j].size
+        else:
+            want = [oracle.ring_allreduce([local[r][j] for r in range(n)])[0] / np.float32(n) for j in range(nparam)]
+        for r in range(n):
+            for j, p in enumerate(replicas[r].parameters()):
+                G.assert_same_bits(G.host(p.grad).reshape(-1), want[j], "fusion=%s rank %d param %d" % (fusion, r, j))
+        # every replica took the same step
+        for p0, p1 in zip(replicas[0].parameters(), replicas[n - 1].parameters()):
+            assert torch.equal(p0, p1)
+        assert not torch.equal(next(replicas[0].parameters()), next(base.parameters()))
+
+
+def test_chained_allreduces_closed_form():
+    """mpi_allreduce_test.py:40-112 at 2 ranks, one iteration: 13 dependent
+    allreduces of a 1331x1331 matrix (odd element count, ragged segments)."""
+    n, stages, side, spread = 2, 13, 1331, 100
+    for average in (False, True):
+        with mpi.Session(size=n) as session:
+            state = [torch.full((side, side), 1.0 + r * spread, device="cuda") for r in range(n)]
+            for i in range(stages):
+                hs = []
+                for r in range(n):
+                    with session.as_rank(r):
+                        hs.append(mpi.allreduce(state[r] + 2.0 ** (i + 1), average=average))
+                state = session.run(hs)
+        ours = 1.0
+        for i in range(stages):
+            cur = ours + 2.0 ** (i + 1)
+            if average:
+                ours = cur + (spread * (n - 1) / 2 if i == 0 else 0)
+            else:
+                ours = cur * n + (spread * n * (n - 1) / 2 if i == 0 else 0)
+        for s in state:
+            assert np.allclose(G.host(s), np.float32(ours))

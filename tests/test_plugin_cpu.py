@@ -1,0 +1,284 @@
+"""CPU-side tests: the two libraries load and export what include/*.h declares,
+the op registry matches the reference's registrations, the host tables agree
+with the oracle, and the error behaviour of the ops follows the reference's
+tests (tensorflow/contrib/mpi_collectives/mpi_ops_test.py:158-202, 265-297)
+and messages (mpi_ops.cc:277-432, 827-847). No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import numpy
+import pytest
+import torch
+
+import gpu_util
+
+import mpi_collectives as mpi
+from mpi_collectives import _plugin, mpi_ops, ring_abi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b((?:ring|mpic)_[a-z0-9_]+)\s*\(", text)) - {"mpic_alloc_fn"})
+
+
+def test_ring_abi_exports_every_declared_symbol():
+    names = declared_functions("ring_abi.h")
+    assert len(names) >= 25
+    L = ctypes.CDLL(ring_abi.LIB_PATH)
+    for n in names:
+        assert hasattr(L, n), n
+    assert sorted(ring_abi.EXPORTS) == names
+    assert ring_abi.lib().ring_abi_version() == 1
+
+
+def test_plugin_exports_every_declared_symbol():
+    names = declared_functions("mpi_collectives.h")
+    L = ctypes.CDLL(_plugin.LIB_PATH)
+    for n in names:
+        assert hasattr(L, n), n
+    assert sorted(_plugin.EXPORTS) == names
+
+
+def test_op_registry_matches_reference_registrations():
+    _plugin.load_library()
+    assert _plugin.op_names() == ['MPIInit', 'MPISize', 'MPIRank', 'MPILocalRank', 'MPIAllreduce', 'MPIAllgather']
+    # mpi_ops.cc:1119-1126, 1233-1245
+    assert _plugin.op_signature('MPIAllreduce') == "MPIAllreduce(tensor: T) -> (sum: T); T: {int32, int64, float32}"
+    assert _plugin.op_signature('MPIAllgather') == \
+        "MPIAllgather(tensor: T, sizes: S) -> (gathered: T); T: {int32, int64, float32}; S: {int64}"
+    assert _plugin.op_signature('MPISize') == "MPISize() -> (size: int32)"
+    assert _plugin.op_signature('NoSuchOp') is None
+    assert "Perform an MPI Allreduce on a tensor" in _plugin.op_doc('MPIAllreduce')
+    L = _plugin.lib()
+    for op in ('MPIInit', 'MPISize', 'MPIRank', 'MPILocalRank'):
+        assert L.mpic_op_has_kernel(op.encode(), b"CPU") and L.mpic_op_has_kernel(op.encode(), b"GPU")
+    for op in ('MPIAllreduce', 'MPIAllgather'):       # collectives: GPU kernels only, no host path
+        assert L.mpic_op_has_kernel(op.encode(), b"GPU") and not L.mpic_op_has_kernel(op.encode(), b"CPU")
+    # shape functions: identity; first dimension unknown
+    assert _plugin.infer_shape('MPIAllreduce', [17, 3]) == [17, 3]
+    assert _plugin.infer_shape('MPIAllgather', [17, 3]) == [None, 3]
+    assert _plugin.infer_shape('MPISize', []) == []
+
+
+def test_load_library_checks_the_op_list():
+    assert mpi_ops._load_library('libmpi_collectives.so', ['MPISize', 'MPIAllreduce']) is not None
+    with pytest.raises(NameError, match="Could not find operator MPIBroadcast in dynamic library"):
+        mpi_ops._load_library('libmpi_collectives.so', ['MPISize', 'MPIBroadcast'])
+
+
+def test_host_tables_agree_with_oracle(oracle):
+    for n in (1, 2, 3, 6, 8, 64):
+        for count in (0, 1, n - 1, n + 1, 4913, 10_000_019):
+            assert ring_abi.segment_table(count, n) == oracle.segment_table(count, n)
+            assert ring_abi.temp_elements(count, n) == oracle.temp_elements(count, n)
+    rows = [17, 32, 81, 12, 15, 23, 22]
+    assert ring_abi.allgather_table(rows, 289) == oracle.allgather_table(rows, 289)
+    L = ring_abi.lib()
+    sizes = (ctypes.c_size_t * 1)()
+    assert L.ring_segment_table(5, 0, sizes, sizes) == 2           # n < 1
+    assert ring_abi.temp_elements(5, 0) == 0
+
+
+def test_schedule_is_the_reference_index_algebra():
+    # ring.h:184-185, 212-213, 280-281
+    for n in (2, 3, 8):
+        for r in range(n):
+            for i in range(n - 1):
+                assert ring_abi.schedule(ring_abi.PHASE_REDUCE_SCATTER, n, r, i) == ((r - i) % n, (r - i - 1) % n)
+                assert ring_abi.schedule(ring_abi.PHASE_ALLGATHER, n, r, i) == ((r - i + 1) % n, (r - i) % n)
+                assert ring_abi.schedule(ring_abi.PHASE_GATHER, n, r, i) == ((r - i) % n, (r - i - 1) % n)
+            # a rank's reduce-scatter touches every segment but its own, once; its
+            # allgather every segment but (r+1)
+            rs = [ring_abi.schedule(0, n, r, i)[1] for i in range(n - 1)]
+            ag = [ring_abi.schedule(1, n, r, i)[1] for i in range(n - 1)]
+            assert sorted(rs) == sorted(set(range(n)) - {r})
+            assert sorted(ag) == sorted(set(range(n)) - {(r + 1) % n})
+    with pytest.raises(ring_abi.RingError):
+        ring_abi.schedule(0, 4, 0, 3)                               # step out of range
+    assert ring_abi.lib().ring_dtype_size(0) == 4 and ring_abi.lib().ring_dtype_size(2) == 8
+    assert ring_abi.lib().ring_dtype_size(5) == 0
+
+
+def test_ops_before_init_fail_like_the_reference():
+    L = _plugin.load_library()
+    w = ctypes.c_void_p()
+    assert L.mpic_world_create(2, ctypes.byref(w)) == 0
+    try:
+        op = _plugin.PendingOp(w.value, 0, 'MPISize', 'MPISize', [], 'CPU')
+        with pytest.raises(mpi.FailedPreconditionError,
+                           match="MPI has not been initialized; use tf.contrib.mpi.Session."):
+            op.wait()
+    finally:
+        L.mpic_world_destroy(w.value)
+    with pytest.raises(mpi.FailedPreconditionError):
+        mpi.size()                                                    # no session at all
+
+
+def test_size_rank_local_rank():
+    with mpi.Session(size=5, device="CPU") as session:
+        assert mpi.size() == 5 and mpi.rank() == 0
+        for r in range(5):
+            with session.as_rank(r):
+                assert (mpi.size(), mpi.rank(), mpi.local_rank()) == (5, r, r)
+        with pytest.raises(mpi.InvalidArgumentError):
+            with session.as_rank(5):
+                pass
+    # outside a launcher the default world has one rank (mpi_ops_test.py:61-62)
+    with mpi.Session(device="CPU") as session:
+        assert mpi.size() == 1 and mpi.rank() == 0
+
+
+def test_size_from_launcher_environment(monkeypatch):
+    monkeypatch.setenv("PMI_SIZE", "3")
+    with mpi.Session(device="CPU"):
+        assert mpi.size() == 3
+
+
+def test_collectives_have_no_cpu_kernel():
+    with mpi.Session(size=2, device="CPU"):
+        with pytest.raises(mpi.NotFoundError, match="No OpKernel was registered to support Op 'MPIAllreduce'"):
+            mpi.allreduce(torch.ones(4))
+        with pytest.raises(mpi.NotFoundError):
+            mpi.allgather(torch.ones(4, 2))
+
+
+def _submit_all(session, op, tensors, name, extra=None):
+    """Submit `op` as every rank through the GPU kernel registration. The
+    tensors are host tensors: the cross-rank checks run before any device work,
+    and a collective that passes them is then refused for being in host memory."""
+    ops = []
+    for r, t in enumerate(tensors):
+        inputs = [t] + ([extra] if extra is not None else [])
+        ops.append(session._submit(r, op, name, inputs, "GPU"))
+    return ops
+
+
+def _errors(ops):
+    out = []
+    for p in ops:
+        with pytest.raises(mpi.OpError) as e:
+            p.wait()
+        out.append(e.value)
+    return out
+
+
+def test_allreduce_error_matrix():
+    """mpi_ops_test.py:158-202: every rank gets FailedPrecondition."""
+    with mpi.Session(size=3, device="CPU") as s:
+        # same rank, different dimension
+        errs = _errors(_submit_all(s, 'MPIAllreduce', [torch.zeros([17 + r] * 3) for r in range(3)], "a"))
+        assert all(isinstance(e, mpi.FailedPreconditionError) for e in errs)
+        assert errs[0].message == ("Mismatched allreduce tensor shapes: One rank reduced a tensor of shape "
+                                   "[17,17,17], but another rank sent a tensor of shape [18,18,18].")
+        assert len({e.message for e in errs}) == 1
+        s._pending.clear()
+        # same number of elements, different rank
+        shapes = [[17, 23 * 57], [17, 23, 57], [17, 23, 57]]
+        errs = _errors(_submit_all(s, 'MPIAllreduce', [torch.zeros(sh) for sh in shapes], "b"))
+        assert all(isinstance(e, mpi.FailedPreconditionError) for e in errs)
+        assert "of shape [17,1311], but another rank sent a tensor of shape [17,23,57]" in errs[0].message
+        s._pending.clear()
+        # different types
+        ts = [torch.ones([17] * 3, dtype=torch.int32 if r % 2 == 0 else torch.float32) for r in range(3)]
+        errs = _errors(_submit_all(s, 'MPIAllreduce', ts, "c"))
+        assert errs[0].message == ("Mismatched data types: One rank had type TF_MPI_INT32, "
+                                   "but another rank had type TF_MPI_FLOAT32.")
+        s._pending.clear()
+        # a consistent request on host tensors is refused, not computed on the CPU
+        errs = _errors(_submit_all(s, 'MPIAllreduce', [torch.zeros(4)] * 3, "d"))
+        assert "GPU kernels only" in errs[0].message
+        s._pending.clear()
+
+
+def test_allgather_error_matrix():
+    """mpi_ops_test.py:265-297 and the remaining branches of mpi_ops.cc:352-411."""
+    sizes = torch.tensor([17, 17, 17], dtype=torch.int64)
+    with mpi.Session(size=3, device="CPU") as s:
+        ts = [torch.ones([17, 10 * (r + 1), 17]) for r in range(3)]
+        errs = _errors(_submit_all(s, 'MPIAllgather', ts, "g1", sizes))
+        assert all(isinstance(e, mpi.FailedPreconditionError) for e in errs)
+        assert errs[0].message == ("Mismatched allgather tensor shapes: One rank gathered a tensor with dimension 1 "
+                                   "equal to 10, but another rank sent a tensor with dimension 1 equal to 20.")
+        s._pending.clear()
+        ts = [torch.ones([17] * 3, dtype=torch.int32 if r % 2 == 0 else torch.float32) for r in range(3)]
+        errs = _errors(_submit_all(s, 'MPIAllgather', ts, "g2", sizes))
+        assert errs[0].message.startswith("Mismatched data types: One rank had type TF_MPI_INT32")
+        s._pending.clear()
+        ts = [torch.ones([17, 17]), torch.ones([17, 17, 1]), torch.ones([17, 17])]
+        errs = _errors(_submit_all(s, 'MPIAllgather', ts, "g3", sizes))
+        assert errs[0].message == ("Mismatched allgather tensor shapes: One rank gathered a tensor of rank 2, "
+                                   "but another rank sent a tensor of rank 3.")
+        s._pending.clear()
+        errs = _errors(_submit_all(s, 'MPIAllgather', [torch.ones([])] * 3, "g4", torch.zeros((), dtype=torch.int64)))
+        assert errs[0].message == "Rank zero tried to gather a rank-zero tensor."
+        s._pending.clear()
+        # one rank reduces while the others gather
+        ops = [s._submit(0, 'MPIAllreduce', "mix", [torch.ones(17, 2)], "GPU")]
+        ops += [s._submit(r, 'MPIAllgather', "mix", [torch.ones(17, 2), sizes], "GPU") for r in (1, 2)]
+        errs = _errors(ops)
+        assert errs[0].message == "Mismatched MPI operations: One rank did an 0, but another rank did an 1."
+        s._pending.clear()
+
+
+def test_unsupported_dtype_is_rejected_before_anything_runs():
+    with mpi.Session(size=2, device="CPU") as s:
+        p = s._submit(0, 'MPIAllreduce', "x", [torch.ones(4, dtype=torch.float64)], "GPU")
+        with pytest.raises(mpi.FailedPreconditionError, match="Invalid tensor type passed."):
+            p.wait()                                                 # mpi_ops.cc:844
+        s._pending.clear()
+        p = s._submit(0, 'MPIAllreduce', "y", [torch.ones(4, dtype=torch.float16)], "GPU")
+        with pytest.raises(mpi.FailedPreconditionError, match="Invalid tensor type passed."):
+            p.wait()
+        s._pending.clear()
+
+
+def test_run_refuses_to_wait_for_ranks_that_never_submitted():
+    with mpi.Session(size=3, device="CPU") as s:
+        s._submit(0, 'MPIAllreduce', "lonely", [torch.zeros(4)], "GPU")
+        with pytest.raises(mpi.FailedPreconditionError, match="submitted by ranks \\[0\\] of 3"):
+            s.run()
+        pending = s._pending[0]
+    # closing the session shuts the background thread down and fails the op
+    with pytest.raises(mpi.UnknownError, match="shut down"):
+        pending.wait()
+
+
+def test_node_names_are_uniquified_like_graph_nodes():
+    with mpi.Session(size=2, device="CPU") as s:
+        assert [s._node_name(0, 'MPIAllreduce', None) for _ in range(3)] == \
+            ['MPIAllreduce', 'MPIAllreduce_1', 'MPIAllreduce_2']
+        assert s._node_name(1, 'MPIAllreduce', None) == 'MPIAllreduce'
+        assert s._node_name(0, 'MPIAllgather', 'allgather') == 'allgather'
+        assert s._node_name(0, 'MPIAllgather', 'allgather') == 'allgather_1'
+
+
+def test_prestaged_world_checks_its_arguments():
+    L = _plugin.load_library()
+    w = ctypes.c_void_p()
+    assert L.mpic_world_create_prestaged(4, 4, ctypes.byref(w)) == 3      # rank out of range
+    assert L.mpic_world_create_prestaged(4, -1, ctypes.byref(w)) == 3
+    assert L.mpic_world_create(0, ctypes.byref(w)) == 3
+    with mpi.Session(size=4, rank=2, device="CPU") as s:
+        assert mpi.rank() == 2 and mpi.size() == 4
+        with pytest.raises(mpi.InvalidArgumentError):
+            with s.as_rank(1):
+                pass
+        with pytest.raises(mpi.InvalidArgumentError):
+            s.stage_peers("x", [torch.zeros(1)], [torch.zeros(1)])        # needs n-1 = 3 segments
+        # nothing staged for this name
+        p = s._submit(2, 'MPIAllreduce', "nostage", [torch.zeros(8)], "GPU")
+        with pytest.raises(mpi.FailedPreconditionError, match="GPU kernels only|No pre-staged"):
+            p.wait()
+        s._pending.clear()
+
+
+def test_resnet50_shape_set():
+    shapes = gpu_util.resnet50_shapes()
+    sizes = [int(numpy.prod(s)) for s in shapes]
+    assert len(shapes) == 161 and sum(sizes) == 25_557_032
+    assert min(sizes) == 64 and max(sizes) == 2_359_296
+    assert sum(1 for s in sizes if s <= 2048) == 107
