@@ -72,6 +72,18 @@ size_t ring_dtype_size(int dtype);
  * is the constant <<<32, 256>>> (ring.cu.cc:64). */
 int ring_set_option(const char* name, int value);
 
+/* Timing of single launches, for benchmarks (no counterpart in the
+ * reference): events created here, and ring_time_next_launch(start, stop)
+ * makes the NEXT step-table / copy / accumulate kernel this thread launches
+ * record its own begin and end into them (the events travel in the dispatch,
+ * so their difference is the kernel's execution time and nothing else). Read
+ * with ring_event_elapsed_us after the stream has been synchronised. A call
+ * that needs several launches times the first one only. */
+int ring_event_create(void** event);
+int ring_event_destroy(void* event);
+int ring_event_elapsed_us(void* start, void* stop, double* us);
+int ring_time_next_launch(void* start_event, void* stop_event);
+
 /* ---- host-side tables (no GPU involved) ---------------------------------- */
 
 /* Segment split of a `count`-element tensor over n ranks — ring.h:150-166:

@@ -26,6 +26,7 @@
 // No MFMA: the path is one add per 12 bytes.
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
@@ -41,6 +42,10 @@ constexpr int kBlock = 256;   // threads per workgroup: 4 wave64
 constexpr int kMaxRows = 64;  // rows one launch carries in its kernel arguments
 
 thread_local int g_last_hip_error = 0;
+// Events the next kernel launch of this thread records its own begin and end
+// into (ring_time_next_launch); cleared by that launch.
+thread_local hipEvent_t g_time_start = nullptr;
+thread_local hipEvent_t g_time_stop = nullptr;
 
 inline int hip_fail(hipError_t e) {
   g_last_hip_error = static_cast<int>(e);
@@ -317,8 +322,18 @@ int device_info(DeviceInfo* out) {
 template <typename T, int MODE>
 int launch_rows_typed(const RowTable& tab, uint32_t grid, hipStream_t stream) {
   const bool nt = g_tuning.nontemporal != 0;
-#define RING_LAUNCH(U, N) \
-  hipLaunchKernelGGL((rows_kernel<T, MODE, U, N>), dim3(grid), dim3(kBlock), 0, stream, tab)
+  // a timed launch carries its events in the dispatch itself, so they bracket
+  // the kernel's execution and nothing else
+  hipEvent_t t0 = g_time_start, t1 = g_time_stop;
+  g_time_start = g_time_stop = nullptr;
+#define RING_LAUNCH(U, N)                                                                            \
+  do {                                                                                               \
+    if (t0 || t1)                                                                                    \
+      hipExtLaunchKernelGGL((rows_kernel<T, MODE, U, N>), dim3(grid), dim3(kBlock), 0, stream, t0,   \
+                            t1, 0, tab);                                                             \
+    else                                                                                             \
+      hipLaunchKernelGGL((rows_kernel<T, MODE, U, N>), dim3(grid), dim3(kBlock), 0, stream, tab);    \
+  } while (0)
   switch (g_tuning.unroll) {
     case 2: if (nt) RING_LAUNCH(2, true); else RING_LAUNCH(2, false); break;
     case 8: if (nt) RING_LAUNCH(8, true); else RING_LAUNCH(8, false); break;
@@ -516,6 +531,36 @@ int ring_set_option(const char* name, int value) {
   } else {
     return RING_ERR_ARGUMENT;
   }
+  return RING_OK;
+}
+
+// ---- measurement hooks --------------------------------------------------------------
+
+int ring_event_create(void** event) {
+  if (!event) return RING_ERR_ARGUMENT;
+  hipEvent_t e = nullptr;
+  RING_HIP(hipEventCreate(&e));
+  *event = e;
+  return RING_OK;
+}
+
+int ring_event_destroy(void* event) {
+  if (!event) return RING_OK;
+  RING_HIP(hipEventDestroy(static_cast<hipEvent_t>(event)));
+  return RING_OK;
+}
+
+int ring_event_elapsed_us(void* start, void* stop, double* us) {
+  if (!start || !stop || !us) return RING_ERR_ARGUMENT;
+  float ms = 0.f;
+  RING_HIP(hipEventElapsedTime(&ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+  *us = static_cast<double>(ms) * 1e3;
+  return RING_OK;
+}
+
+int ring_time_next_launch(void* start_event, void* stop_event) {
+  g_time_start = static_cast<hipEvent_t>(start_event);
+  g_time_stop = static_cast<hipEvent_t>(stop_event);
   return RING_OK;
 }
 

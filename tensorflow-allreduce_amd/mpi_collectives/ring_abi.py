@@ -17,7 +17,8 @@ LIB_PATH = os.path.join(_PKG_ROOT, "lib", "libring_hip.so")
 # Every symbol include/ring_abi.h declares.
 EXPORTS = (
     "ring_abi_version", "ring_status_string", "ring_last_hip_error", "ring_dtype_size",
-    "ring_set_option", "ring_segment_table", "ring_temp_elements", "ring_allgather_table",
+    "ring_set_option", "ring_event_create", "ring_event_destroy", "ring_event_elapsed_us",
+    "ring_time_next_launch", "ring_segment_table", "ring_temp_elements", "ring_allgather_table",
     "ring_schedule", "ring_stream_create", "ring_stream_destroy", "ring_stream_synchronize",
     "ring_copy_bytes", "ring_accumulate_f32", "ring_accumulate_i32", "ring_accumulate_i64",
     "ring_accumulate", "ring_reduce_scatter_steps", "ring_reduce_scatter_steps_from",
@@ -69,6 +70,10 @@ def lib():
             "ring_last_hip_error": (ci, []),
             "ring_dtype_size": (sz, [ci]),
             "ring_set_option": (ci, [ctypes.c_char_p, ci]),
+            "ring_event_create": (ci, [ctypes.POINTER(vp)]),
+            "ring_event_destroy": (ci, [vp]),
+            "ring_event_elapsed_us": (ci, [vp, vp, ctypes.POINTER(ctypes.c_double)]),
+            "ring_time_next_launch": (ci, [vp, vp]),
             "ring_segment_table": (ci, [sz, ci, psz, psz]),
             "ring_temp_elements": (sz, [sz, ci]),
             "ring_allgather_table": (ci, [psz, ci, sz, psz]),
@@ -112,6 +117,28 @@ def check(status, where):
 
 def set_option(name, value):
     check(lib().ring_set_option(name.encode(), int(value)), "ring_set_option(%s)" % name)
+
+
+# ---- timing of single launches -----------------------------------------------------
+
+def event_create():
+    e = ctypes.c_void_p()
+    check(lib().ring_event_create(ctypes.byref(e)), "ring_event_create")
+    return e.value
+
+
+def event_destroy(event):
+    check(lib().ring_event_destroy(event), "ring_event_destroy")
+
+
+def event_elapsed_us(start, stop):
+    us = ctypes.c_double()
+    check(lib().ring_event_elapsed_us(start, stop, ctypes.byref(us)), "ring_event_elapsed_us")
+    return us.value
+
+
+def time_next_launch(start, stop):
+    check(lib().ring_time_next_launch(start, stop), "ring_time_next_launch")
 
 
 # ---- host tables ----------------------------------------------------------------
