@@ -156,7 +156,7 @@ def main():
             return
         # the same three launches through the C ABI, each carrying its own pair of
         # HIP events in the dispatch (on the stream the kernels run on)
-        e = [ring_abi.event_create() for _ in range(6)]
+        e = event_pool.pop()
         ring_abi.time_next_launch(e[0], e[1])
         ring_abi.check(R.ring_copy_bytes(s["out"].data_ptr(), s["inp"].data_ptr(), COUNT * ESZ, stream), "copy")
         ring_abi.time_next_launch(e[2], e[3])
@@ -166,6 +166,10 @@ def main():
         ring_abi.check(R.ring_allgather_steps(s["out"].data_ptr(), s["ag_steps"][0], s["ag_steps"][1],
                                               ring_abi.F32, stream), "allgather")
         sample.append(e)
+
+    # events are created before the timed region: creating them inside it would
+    # let the queue drain and the sampled launches start on an idle GPU
+    event_pool = [[ring_abi.event_create() for _ in range(6)] for _ in range(args.steps // SAMPLE_EVERY + 1)]
 
     def timed(steps, warmup, fused=False, with_samples=False):
         for k in range(warmup):

@@ -208,6 +208,10 @@ size_t ring_fusion_plan_elements(const ring_fusion_plan* plan);
 int ring_fusion_pack(const ring_fusion_plan* plan, void* fused, void* stream);
 /* tensors[j][i] = fused[offset_j + i] for all j. */
 int ring_fusion_unpack(const ring_fusion_plan* plan, const void* fused, void* stream);
+/* tensors[j][i] = fused[offset_j + i] / divisor, with ring_scale's division
+ * (the average of a fused allreduce folded into the unpack). divisor >= 1. */
+int ring_fusion_unpack_scaled(const ring_fusion_plan* plan, const void* fused, int divisor,
+                              void* stream);
 
 #ifdef __cplusplus
 }

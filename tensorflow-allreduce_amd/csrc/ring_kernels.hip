@@ -47,6 +47,17 @@ thread_local int g_last_hip_error = 0;
 thread_local hipEvent_t g_time_start = nullptr;
 thread_local hipEvent_t g_time_stop = nullptr;
 
+// Every kernel launch of the library goes through here. A launch armed by
+// ring_time_next_launch carries its events in the dispatch itself, so they
+// bracket the kernel's execution and nothing else.
+template <typename... Params, typename... Args>
+inline void launch(void (*kernel)(Params...), dim3 grid, dim3 block, hipStream_t stream, Args... args) {
+  hipEvent_t t0 = g_time_start, t1 = g_time_stop;
+  g_time_start = g_time_stop = nullptr;
+  if (t0 || t1) hipExtLaunchKernelGGL(kernel, grid, block, 0, stream, t0, t1, 0, args...);
+  else hipLaunchKernelGGL(kernel, grid, block, 0, stream, args...);
+}
+
 inline int hip_fail(hipError_t e) {
   g_last_hip_error = static_cast<int>(e);
   return RING_ERR_HIP;
@@ -58,28 +69,77 @@ inline int hip_fail(hipError_t e) {
   } while (0)
 
 // ---- element / vector types -------------------------------------------------
+// A lane moves 16 bytes per access. Integers are ADDED as unsigned so overflow
+// wraps (what the reference's hardware add does) instead of being undefined;
+// they are DIVIDED as signed (floor division of the average).
 
 template <typename T> struct VecOf;
 template <> struct VecOf<float> { typedef float type __attribute__((ext_vector_type(4))); };
-// integers are added as unsigned so overflow wraps (what the reference's
-// hardware add does) instead of being undefined
 template <> struct VecOf<uint32_t> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
 template <> struct VecOf<uint64_t> { typedef uint64_t type __attribute__((ext_vector_type(2))); };
+template <> struct VecOf<int32_t> { typedef int32_t type __attribute__((ext_vector_type(4))); };
+template <> struct VecOf<int64_t> { typedef int64_t type __attribute__((ext_vector_type(2))); };
 
-// kCopy: every row is dst = a. kAdd: a row with a second operand is
-// dst = b + a (b may be dst itself: the in-place accumulate of the reference),
-// a row without one is still a copy, so one launch can mix both.
-enum Mode { kCopy = 0, kAdd = 1 };
+// The divide of allreduce(average=True): tf.div semantics (__init__.py:160-164
+// of the reference): true division for float32 (a correctly rounded divide,
+// NOT a multiply by 1/n), floor division for the integer types. n > 0, so
+// floor differs from C's truncation only for negative x with a remainder.
+__device__ __forceinline__ float div_one(float x, int n) { return x / static_cast<float>(n); }
+__device__ __forceinline__ int32_t div_one(int32_t x, int n) {
+  const int32_t q = x / n;
+  return q - ((x % n != 0) && (x < 0));
+}
+__device__ __forceinline__ int64_t div_one(int64_t x, int n) {
+  const int64_t q = x / n;
+  return q - ((x % n != 0) && (x < 0));
+}
+// never instantiated for the unsigned carrier types; present so templates compile
+__device__ __forceinline__ uint32_t div_one(uint32_t x, int) { return x; }
+__device__ __forceinline__ uint64_t div_one(uint64_t x, int) { return x; }
+
+// kOpCopy: dst = a.  kOpAdd: dst = b + a (b may be dst itself: the in-place
+// accumulate of the reference).  kOpDiv: dst = a / n (a may be dst itself).
+enum Op { kOpCopy = 0, kOpAdd = 1, kOpDiv = 2 };
+
+template <typename T, int OP>
+__device__ __forceinline__ T apply_one(T a, T b, int n) {
+  if (OP == kOpAdd) return b + a;
+  if (OP == kOpDiv) return div_one(a, n);
+  return a;
+}
+template <typename T, int OP>
+__device__ __forceinline__ typename VecOf<T>::type apply_vec(typename VecOf<T>::type a, typename VecOf<T>::type b, int n) {
+  if (OP == kOpAdd) return b + a;
+  if (OP == kOpDiv) {
+#pragma unroll
+    for (uint32_t c = 0; c < 16 / sizeof(T); c++) a[c] = div_one(a[c], n);
+  }
+  return a;
+}
+
+// Launch modes of rows_kernel. kCopy: every row is a copy. kAdd: a row with a
+// second operand is an add, a row without one is still a copy, so one launch
+// can mix both. kDiv: every row is divided by the table's divisor.
+enum Mode { kCopy = 0, kAdd = 1, kDiv = 2 };
 
 // Rows of one launch, passed by value in the kernel arguments (read with
 // scalar loads; uniform per workgroup).
+struct Row {
+  void* dst;
+  const void* a;   // incoming segment
+  const void* b;   // local operand of an add row, null for a copy row
+  uint64_t count;  // elements
+};
 struct RowTable {
   int n_rows;
+  // > 0: every row has this many tiles and the grid is (tiles, rows), so a
+  // workgroup reads its row straight from blockIdx.y (the n-1 near-equal
+  // segments of an allreduce). 0: rows differ; the grid is 1-D over all tiles
+  // and a workgroup finds its row by binary search over tile_begin.
+  uint32_t uniform_tiles;
+  int divisor;                        // kDiv only
   uint32_t tile_begin[kMaxRows + 1];  // prefix sum of tiles per row
-  void* dst[kMaxRows];
-  const void* a[kMaxRows];  // incoming segment
-  const void* b[kMaxRows];  // local operand of an add row, null for a copy row
-  uint64_t count[kMaxRows];  // elements
+  Row row[kMaxRows];
 };
 
 template <typename T, bool NT>
@@ -90,11 +150,11 @@ __device__ __forceinline__ void store_vec(typename VecOf<T>::type* p, typename V
 // One workgroup-tile of a row: vectors [v0, v0 + 256*UNROLL) of the aligned
 // body, plus the row's scalar head (tile 0) and tail (last tile). dst is
 // brought to 16-byte alignment by the head; a and b are read with
-// element-aligned 16-byte loads. b == dst is allowed (every element is read
-// before it is written, by the same lane).
-template <typename T, bool ADD, int UNROLL, bool NT>
-__device__ __forceinline__ void row_tile(T* dst, const T* __restrict__ a, const T* b,
-                                         uint64_t count, uint32_t tile, uint32_t tiles_in_row) {
+// element-aligned 16-byte loads. a == dst (divide) and b == dst (add) are
+// allowed: every element is read before it is written, by the same lane.
+template <typename T, int OP, int UNROLL, bool NT>
+__device__ __forceinline__ void row_tile(T* dst, const T* a, const T* b, uint64_t count, uint32_t tile,
+                                         uint32_t tiles_in_row, int n) {
   typedef typename VecOf<T>::type V;
   typedef V VU __attribute__((aligned(sizeof(T))));  // element-aligned 16-byte access
   constexpr uint32_t VEC = 16 / sizeof(T);
@@ -105,18 +165,14 @@ __device__ __forceinline__ void row_tile(T* dst, const T* __restrict__ a, const 
   const uint64_t nvec = (count - head) / VEC;
   const uint32_t tid = threadIdx.x;
 
-  if (tile == 0 && tid < head) {
-    if (ADD) dst[tid] = b[tid] + a[tid]; else dst[tid] = a[tid];
-  }
+  if (tile == 0 && tid < head) dst[tid] = apply_one<T, OP>(a[tid], OP == kOpAdd ? b[tid] : T(), n);
   if (tile + 1 == tiles_in_row) {
     const uint64_t e = head + nvec * VEC + tid;
-    if (e < count) {
-      if (ADD) dst[e] = b[e] + a[e]; else dst[e] = a[e];
-    }
+    if (e < count) dst[e] = apply_one<T, OP>(a[e], OP == kOpAdd ? b[e] : T(), n);
   }
 
   V* dv = reinterpret_cast<V*>(dst + head);
-  const VU* __restrict__ av = reinterpret_cast<const VU*>(a + head);
+  const VU* av = reinterpret_cast<const VU*>(a + head);
   const VU* bv = reinterpret_cast<const VU*>(b + head);
   const uint64_t v0 = static_cast<uint64_t>(tile) * kTileVecs + tid;
 
@@ -124,12 +180,12 @@ __device__ __forceinline__ void row_tile(T* dst, const T* __restrict__ a, const 
     V x[UNROLL], y[UNROLL];
 #pragma unroll
     for (int j = 0; j < UNROLL; j++) x[j] = __builtin_nontemporal_load(&av[v0 + j * kBlock]);
-    if (ADD) {
+    if (OP == kOpAdd) {
 #pragma unroll
       for (int j = 0; j < UNROLL; j++) y[j] = __builtin_nontemporal_load(&bv[v0 + j * kBlock]);
-#pragma unroll
-      for (int j = 0; j < UNROLL; j++) x[j] = y[j] + x[j];
     }
+#pragma unroll
+    for (int j = 0; j < UNROLL; j++) x[j] = apply_vec<T, OP>(x[j], y[j], n);
 #pragma unroll
     for (int j = 0; j < UNROLL; j++) store_vec<T, NT>(&dv[v0 + j * kBlock], x[j]);
   } else {
@@ -138,15 +194,32 @@ __device__ __forceinline__ void row_tile(T* dst, const T* __restrict__ a, const 
       const uint64_t v = v0 + j * kBlock;
       if (v < nvec) {
         V x = __builtin_nontemporal_load(&av[v]);
-        if (ADD) x = __builtin_nontemporal_load(&bv[v]) + x;
-        store_vec<T, NT>(&dv[v], x);
+        V y = x;
+        if (OP == kOpAdd) y = __builtin_nontemporal_load(&bv[v]);
+        store_vec<T, NT>(&dv[v], apply_vec<T, OP>(x, y, n));
       }
     }
   }
 }
 
 template <typename T, int MODE, int UNROLL, bool NT>
+__device__ __forceinline__ void run_row(const Row& r, uint32_t tile, uint32_t tiles, int divisor) {
+  T* dst = static_cast<T*>(r.dst);
+  const T* a = static_cast<const T*>(r.a);
+  const T* b = static_cast<const T*>(r.b);
+  if (MODE == kDiv) row_tile<T, kOpDiv, UNROLL, NT>(dst, a, nullptr, r.count, tile, tiles, divisor);
+  else if (MODE == kAdd && b != nullptr) row_tile<T, kOpAdd, UNROLL, NT>(dst, a, b, r.count, tile, tiles, 0);
+  else row_tile<T, kOpCopy, UNROLL, NT>(dst, a, nullptr, r.count, tile, tiles, 0);
+}
+
+template <typename T, int MODE, int UNROLL, bool NT>
 __global__ void __launch_bounds__(kBlock) rows_kernel(const RowTable tab) {
+  if (tab.uniform_tiles) {
+    const Row r = tab.row[blockIdx.y];  // one scalar load, no search
+    for (uint32_t t = blockIdx.x; t < tab.uniform_tiles; t += gridDim.x)
+      run_row<T, MODE, UNROLL, NT>(r, t, tab.uniform_tiles, tab.divisor);
+    return;
+  }
   const uint32_t total = tab.tile_begin[tab.n_rows];
   for (uint32_t t = blockIdx.x; t < total; t += gridDim.x) {
     // largest row with tile_begin[row] <= t (uniform: scalar code)
@@ -156,12 +229,7 @@ __global__ void __launch_bounds__(kBlock) rows_kernel(const RowTable tab) {
       if (tab.tile_begin[mid] <= t) lo = mid; else hi = mid;
     }
     const uint32_t first = tab.tile_begin[lo];
-    const uint32_t tiles = tab.tile_begin[lo + 1] - first;
-    T* dst = static_cast<T*>(tab.dst[lo]);
-    const T* a = static_cast<const T*>(tab.a[lo]);
-    const T* b = static_cast<const T*>(tab.b[lo]);
-    if (MODE == kAdd && b != nullptr) row_tile<T, true, UNROLL, NT>(dst, a, b, tab.count[lo], t - first, tiles);
-    else row_tile<T, false, UNROLL, NT>(dst, a, nullptr, tab.count[lo], t - first, tiles);
+    run_row<T, MODE, UNROLL, NT>(tab.row[lo], t - first, tab.tile_begin[lo + 1] - first, tab.divisor);
   }
 }
 
@@ -174,71 +242,28 @@ __global__ void __launch_bounds__(kBlock) bytes_kernel(uint8_t* __restrict__ dst
     dst[i] = src[i];
 }
 
-// ---- average: sum / n ---------------------------------------------------------
-// tf.div semantics of the reference's allreduce(average=True)
-// (__init__.py:160-164): true division for float32 (a correctly rounded
-// divide, NOT a multiply by 1/n), floor division for the integer types.
-
-template <typename T> struct ScaleOp;
-template <> struct ScaleOp<float> {
-  typedef float V __attribute__((ext_vector_type(4)));
-  static __device__ __forceinline__ float one(float x, int n) { return x / static_cast<float>(n); }
-};
-template <> struct ScaleOp<int32_t> {
-  typedef int32_t V __attribute__((ext_vector_type(4)));
-  static __device__ __forceinline__ int32_t one(int32_t x, int n) {
-    int32_t q = x / n;
-    return q - ((x % n != 0) && (x < 0));  // n > 0: floor differs from trunc only for x < 0
-  }
-};
-template <> struct ScaleOp<int64_t> {
-  typedef int64_t V __attribute__((ext_vector_type(2)));
-  static __device__ __forceinline__ int64_t one(int64_t x, int n) {
-    int64_t q = x / n;
-    return q - ((x % n != 0) && (x < 0));
-  }
-};
-
-template <typename T>
-__global__ void __launch_bounds__(kBlock) scale_kernel(T* __restrict__ data, uint64_t count, int n) {
-  typedef typename ScaleOp<T>::V V;
-  constexpr uint32_t VEC = 16 / sizeof(T);
-  uint64_t head = ((16u - (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(data)) & 15u)) & 15u) / sizeof(T);
-  if (head > count) head = count;
-  const uint64_t nvec = (count - head) / VEC;
-  const uint64_t gtid = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
-  const uint64_t gsize = static_cast<uint64_t>(gridDim.x) * kBlock;
-  if (gtid < head) data[gtid] = ScaleOp<T>::one(data[gtid], n);
-  const uint64_t tail_at = head + nvec * VEC + gtid;
-  if (tail_at < count) data[tail_at] = ScaleOp<T>::one(data[tail_at], n);
-  V* __restrict__ dv = reinterpret_cast<V*>(data + head);
-  for (uint64_t v = gtid; v < nvec; v += gsize) {
-    V x = dv[v];
-#pragma unroll
-    for (uint32_t c = 0; c < VEC; c++) x[c] = ScaleOp<T>::one(x[c], n);
-    dv[v] = x;
-  }
-}
-
 // ---- tensor fusion: pack / unpack -----------------------------------------------
 // The fused buffer is cut into tiles of 1024 16-byte groups. A tile that lies
 // inside one tensor (all of the bytes of a ResNet-sized gradient set, bar a few
 // hundred KiB) is a plain aligned-store span copy. A tile that spans several
 // tensors stages the offsets and base pointers of just those tensors in LDS
 // and every lane finds the tensor of its 16-byte group by binary search there.
+// With DIV the unpack also divides by n (the average of a fused allreduce), so
+// the sum is not written and read once more just to be scaled.
 
 constexpr uint32_t kFusionTileVecs = 1024;
 constexpr uint32_t kFusionLdsCap = 512;  // tensors of one tile staged in LDS
 
-template <typename T, bool PACK, bool NT>
+template <typename T, bool PACK, bool NT, bool DIV>
 __global__ void __launch_bounds__(kBlock)
 fusion_kernel(T* __restrict__ fused, const uint64_t* __restrict__ offsets, T* const* __restrict__ ptrs,
               const uint32_t* __restrict__ tile_first, const uint32_t* __restrict__ tile_last,
-              uint32_t ntiles, uint64_t total) {
+              uint32_t ntiles, uint64_t total, int divisor) {
   typedef typename VecOf<T>::type V;
   typedef V VU __attribute__((aligned(sizeof(T))));
   constexpr uint32_t VEC = 16 / sizeof(T);
   constexpr uint64_t kTileElems = static_cast<uint64_t>(kFusionTileVecs) * VEC;
+  constexpr int OP = DIV ? kOpDiv : kOpCopy;
   __shared__ uint64_t s_off[kFusionLdsCap + 1];
   __shared__ T* s_ptr[kFusionLdsCap];
 
@@ -249,8 +274,8 @@ fusion_kernel(T* __restrict__ fused, const uint64_t* __restrict__ offsets, T* co
     const uint32_t t1 = tile_last[tile];
     if (t0 == t1) {
       T* tensor = ptrs[t0] + (e0 - offsets[t0]);
-      if (PACK) row_tile<T, false, 4, NT>(fused + e0, tensor, nullptr, e1 - e0, 0, 1);
-      else row_tile<T, false, 4, NT>(tensor, fused + e0, nullptr, e1 - e0, 0, 1);
+      if (PACK) row_tile<T, kOpCopy, 4, NT>(fused + e0, tensor, nullptr, e1 - e0, 0, 1, 0);
+      else row_tile<T, OP, 4, NT>(tensor, fused + e0, nullptr, e1 - e0, 0, 1, divisor);
       continue;
     }
     const uint32_t span = t1 - t0 + 1;
@@ -274,14 +299,18 @@ fusion_kernel(T* __restrict__ fused, const uint64_t* __restrict__ offsets, T* co
       }
       if (e + VEC <= off_tab[lo + 1] && e + VEC <= e1) {
         T* tensor = ptr_tab[lo] + (e - off_tab[lo]);
-        if (PACK) store_vec<T, NT>(reinterpret_cast<V*>(fused + e), *reinterpret_cast<const VU*>(tensor));
-        else *reinterpret_cast<VU*>(tensor) = *reinterpret_cast<const V*>(fused + e);
+        if (PACK) {
+          store_vec<T, NT>(reinterpret_cast<V*>(fused + e), *reinterpret_cast<const VU*>(tensor));
+        } else {
+          const V x = *reinterpret_cast<const V*>(fused + e);
+          *reinterpret_cast<VU*>(tensor) = apply_vec<T, OP>(x, x, divisor);
+        }
       } else {
         const uint64_t end = (e + VEC < e1) ? e + VEC : e1;
         for (; e < end; e++) {
           while (e >= off_tab[lo + 1]) lo++;
           T* tensor = ptr_tab[lo] + (e - off_tab[lo]);
-          if (PACK) fused[e] = *tensor; else *tensor = fused[e];
+          if (PACK) fused[e] = *tensor; else *tensor = apply_one<T, OP>(fused[e], T(), divisor);
         }
       }
     }
@@ -320,20 +349,9 @@ int device_info(DeviceInfo* out) {
 }
 
 template <typename T, int MODE>
-int launch_rows_typed(const RowTable& tab, uint32_t grid, hipStream_t stream) {
+int launch_rows_typed(const RowTable& tab, dim3 grid, hipStream_t stream) {
   const bool nt = g_tuning.nontemporal != 0;
-  // a timed launch carries its events in the dispatch itself, so they bracket
-  // the kernel's execution and nothing else
-  hipEvent_t t0 = g_time_start, t1 = g_time_stop;
-  g_time_start = g_time_stop = nullptr;
-#define RING_LAUNCH(U, N)                                                                            \
-  do {                                                                                               \
-    if (t0 || t1)                                                                                    \
-      hipExtLaunchKernelGGL((rows_kernel<T, MODE, U, N>), dim3(grid), dim3(kBlock), 0, stream, t0,   \
-                            t1, 0, tab);                                                             \
-    else                                                                                             \
-      hipLaunchKernelGGL((rows_kernel<T, MODE, U, N>), dim3(grid), dim3(kBlock), 0, stream, tab);    \
-  } while (0)
+#define RING_LAUNCH(U, N) launch(rows_kernel<T, MODE, U, N>, grid, dim3(kBlock), stream, tab)
   switch (g_tuning.unroll) {
     case 2: if (nt) RING_LAUNCH(2, true); else RING_LAUNCH(2, false); break;
     case 8: if (nt) RING_LAUNCH(8, true); else RING_LAUNCH(8, false); break;
@@ -353,7 +371,10 @@ struct HostRow {
 
 // Launches rows (any number) in groups of kMaxRows. esz: 4 or 8. A table with
 // no add row runs the copy-only kernel.
-int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, hipStream_t stream) {
+// divisor > 0: every row is divided in place / out of place by it (kDiv) and
+// the element type is signed.
+int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, hipStream_t stream,
+                int divisor = 0) {
   const int unroll = (g_tuning.unroll == 2 || g_tuning.unroll == 8) ? g_tuning.unroll : 4;
   const uint64_t tile_vecs = static_cast<uint64_t>(kBlock) * unroll;
   const uint64_t vec = 16 / esz;
@@ -362,9 +383,11 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
   while (i < n_rows) {
     RowTable tab;
     tab.n_rows = 0;
+    tab.divisor = divisor;
     tab.tile_begin[0] = 0;
     uint64_t tiles = 0;
-    bool any_add = false;
+    uint64_t first_tiles = 0;
+    bool any_add = false, uniform = true;
     while (i < n_rows && tab.n_rows < kMaxRows) {
       const HostRow& r = rows[i];
       if (r.count == 0) { i++; continue; }
@@ -379,25 +402,38 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
         break;
       }
       const int k = tab.n_rows++;
-      tab.dst[k] = r.dst;
-      tab.a[k] = r.a;
-      tab.b[k] = r.b;
-      tab.count[k] = r.count;
+      tab.row[k] = Row{r.dst, r.a, r.b, r.count};
       any_add = any_add || r.b != nullptr;
+      if (k == 0) first_tiles = t;
+      uniform = uniform && t == first_tiles;
       tiles += t;
       tab.tile_begin[k + 1] = static_cast<uint32_t>(tiles);
       i++;
     }
     if (tab.n_rows == 0) continue;
-    uint32_t grid = static_cast<uint32_t>(tiles);
+    uint64_t cap = tiles;
     if (g_tuning.blocks_per_cu > 0) {
       int rc = device_info(&info);
       if (rc != RING_OK) return rc;
-      const uint64_t cap = static_cast<uint64_t>(info.cus) * g_tuning.blocks_per_cu;
-      if (grid > cap) grid = static_cast<uint32_t>(cap);
+      cap = static_cast<uint64_t>(info.cus) * g_tuning.blocks_per_cu;
+    }
+    dim3 grid;
+    if (uniform && tab.n_rows <= 65535) {
+      uint64_t per_row = cap / static_cast<uint64_t>(tab.n_rows);
+      if (per_row < 1) per_row = 1;
+      if (per_row > first_tiles) per_row = first_tiles;
+      tab.uniform_tiles = static_cast<uint32_t>(first_tiles);
+      grid = dim3(static_cast<uint32_t>(per_row), static_cast<uint32_t>(tab.n_rows));
+    } else {
+      tab.uniform_tiles = 0;
+      grid = dim3(static_cast<uint32_t>(tiles < cap ? tiles : cap));
     }
     int rc;
-    if (!any_add) {
+    if (divisor > 0) {
+      rc = esz == 8 ? launch_rows_typed<int64_t, kDiv>(tab, grid, stream)
+           : is_float ? launch_rows_typed<float, kDiv>(tab, grid, stream)
+                      : launch_rows_typed<int32_t, kDiv>(tab, grid, stream);
+    } else if (!any_add) {
       rc = esz == 8 ? launch_rows_typed<uint64_t, kCopy>(tab, grid, stream)
                     : launch_rows_typed<uint32_t, kCopy>(tab, grid, stream);
     } else if (esz == 8) {
@@ -460,8 +496,8 @@ struct ring_fusion_plan {
 
 namespace {
 
-template <typename T, bool PACK>
-int launch_fusion(const ring_fusion_plan* p, void* fused, hipStream_t stream) {
+template <typename T, bool PACK, bool DIV>
+int launch_fusion(const ring_fusion_plan* p, void* fused, hipStream_t stream, int divisor) {
   uint32_t grid = p->ntiles;
   if (g_tuning.blocks_per_cu > 0) {
     DeviceInfo info;
@@ -471,24 +507,33 @@ int launch_fusion(const ring_fusion_plan* p, void* fused, hipStream_t stream) {
     if (grid > cap) grid = static_cast<uint32_t>(cap);
   }
   if (g_tuning.nontemporal)
-    hipLaunchKernelGGL((fusion_kernel<T, PACK, true>), dim3(grid), dim3(kBlock), 0, stream,
-                       static_cast<T*>(fused), p->d_offsets, reinterpret_cast<T* const*>(p->d_ptrs),
-                       p->d_tile_first, p->d_tile_last, p->ntiles, p->total);
+    launch(fusion_kernel<T, PACK, true, DIV>, dim3(grid), dim3(kBlock), stream, static_cast<T*>(fused),
+           static_cast<const uint64_t*>(p->d_offsets), reinterpret_cast<T* const*>(p->d_ptrs),
+           static_cast<const uint32_t*>(p->d_tile_first), static_cast<const uint32_t*>(p->d_tile_last), p->ntiles,
+           p->total, divisor);
   else
-    hipLaunchKernelGGL((fusion_kernel<T, PACK, false>), dim3(grid), dim3(kBlock), 0, stream,
-                       static_cast<T*>(fused), p->d_offsets, reinterpret_cast<T* const*>(p->d_ptrs),
-                       p->d_tile_first, p->d_tile_last, p->ntiles, p->total);
+    launch(fusion_kernel<T, PACK, false, DIV>, dim3(grid), dim3(kBlock), stream, static_cast<T*>(fused),
+           static_cast<const uint64_t*>(p->d_offsets), reinterpret_cast<T* const*>(p->d_ptrs),
+           static_cast<const uint32_t*>(p->d_tile_first), static_cast<const uint32_t*>(p->d_tile_last), p->ntiles,
+           p->total, divisor);
   RING_HIP(hipGetLastError());
   return RING_OK;
 }
 
-int fusion_run(const ring_fusion_plan* p, void* fused, void* stream, bool pack) {
+// divisor 0: plain pack / unpack. divisor >= 1: unpack and divide.
+int fusion_run(const ring_fusion_plan* p, void* fused, void* stream, bool pack, int divisor) {
   if (!p) return RING_ERR_ARGUMENT;
   if (p->total == 0) return RING_OK;
   if (!fused || (reinterpret_cast<uintptr_t>(fused) & 15u)) return RING_ERR_ARGUMENT;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (p->esz == 8) return pack ? launch_fusion<uint64_t, true>(p, fused, s) : launch_fusion<uint64_t, false>(p, fused, s);
-  return pack ? launch_fusion<uint32_t, true>(p, fused, s) : launch_fusion<uint32_t, false>(p, fused, s);
+  if (divisor > 0) {
+    if (p->dtype == RING_F32) return launch_fusion<float, false, true>(p, fused, s, divisor);
+    if (p->dtype == RING_I32) return launch_fusion<int32_t, false, true>(p, fused, s, divisor);
+    return launch_fusion<int64_t, false, true>(p, fused, s, divisor);
+  }
+  if (p->esz == 8)
+    return pack ? launch_fusion<uint64_t, true, false>(p, fused, s, 0) : launch_fusion<uint64_t, false, false>(p, fused, s, 0);
+  return pack ? launch_fusion<uint32_t, true, false>(p, fused, s, 0) : launch_fusion<uint32_t, false, false>(p, fused, s, 0);
 }
 
 }  // namespace
@@ -646,7 +691,7 @@ int ring_copy_bytes(void* dst, const void* src, size_t bytes, void* stream) {
   }
   uint64_t blocks = (bytes + kBlock - 1) / kBlock;
   if (blocks > 65536) blocks = 65536;
-  hipLaunchKernelGGL(bytes_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), 0, s,
+  launch(bytes_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(kBlock), s,
                      static_cast<uint8_t*>(dst), static_cast<const uint8_t*>(src),
                      static_cast<uint64_t>(bytes));
   RING_HIP(hipGetLastError());
@@ -712,18 +757,8 @@ int ring_scale(int dtype, void* data, size_t count, int divisor, void* stream) {
   if (divisor < 1) return RING_ERR_ARGUMENT;
   if (count == 0) return RING_OK;
   if (!data || (reinterpret_cast<uintptr_t>(data) & (dtype_size(dtype) - 1))) return RING_ERR_ARGUMENT;
-  const uint64_t vecs = count / (16 / dtype_size(dtype)) + 1;
-  uint64_t blocks = (vecs + kBlock - 1) / kBlock;
-  if (blocks > 16384) blocks = 16384;
-  const dim3 grid(static_cast<uint32_t>(blocks)), block(kBlock);
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  switch (dtype) {
-    case RING_F32: hipLaunchKernelGGL(scale_kernel<float>, grid, block, 0, s, static_cast<float*>(data), static_cast<uint64_t>(count), divisor); break;
-    case RING_I32: hipLaunchKernelGGL(scale_kernel<int32_t>, grid, block, 0, s, static_cast<int32_t*>(data), static_cast<uint64_t>(count), divisor); break;
-    default: hipLaunchKernelGGL(scale_kernel<int64_t>, grid, block, 0, s, static_cast<int64_t*>(data), static_cast<uint64_t>(count), divisor); break;
-  }
-  RING_HIP(hipGetLastError());
-  return RING_OK;
+  HostRow row{data, data, nullptr, count};
+  return launch_rows(&row, 1, dtype_size(dtype), dtype == RING_F32, static_cast<hipStream_t>(stream), divisor);
 }
 
 // ---- fusion ------------------------------------------------------------------------
@@ -809,11 +844,16 @@ int ring_fusion_plan_destroy(ring_fusion_plan* plan) {
 size_t ring_fusion_plan_elements(const ring_fusion_plan* plan) { return plan ? plan->total : 0; }
 
 int ring_fusion_pack(const ring_fusion_plan* plan, void* fused, void* stream) {
-  return fusion_run(plan, fused, stream, true);
+  return fusion_run(plan, fused, stream, true, 0);
 }
 
 int ring_fusion_unpack(const ring_fusion_plan* plan, const void* fused, void* stream) {
-  return fusion_run(plan, const_cast<void*>(fused), stream, false);
+  return fusion_run(plan, const_cast<void*>(fused), stream, false, 0);
+}
+
+int ring_fusion_unpack_scaled(const ring_fusion_plan* plan, const void* fused, int divisor, void* stream) {
+  if (divisor < 1) return RING_ERR_ARGUMENT;
+  return fusion_run(plan, const_cast<void*>(fused), stream, false, divisor);
 }
 
 }  // extern "C"

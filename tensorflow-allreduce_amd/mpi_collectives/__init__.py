@@ -420,12 +420,13 @@ class DistributedOptimizer:
         torch.cuda.current_stream().synchronize()      # the gradients' producers
         plan.pack(fused.data_ptr(), session.stream)
         ring_abi.stream_synchronize(session.stream)
-        handle = allreduce(fused, average=True)
+        handle = allreduce(fused, average=False)
         unpacked = {"done": False}
 
         def unpack(t):
             if not unpacked["done"]:
-                plan.unpack(t.data_ptr(), session.stream)
+                # the average's divide (tf.div by the size) rides on the unpack
+                plan.unpack_scaled(t.data_ptr(), session.size, session.stream)
                 ring_abi.stream_synchronize(session.stream)
                 unpacked["done"] = True
                 plan.close()

@@ -24,7 +24,7 @@ EXPORTS = (
     "ring_accumulate", "ring_reduce_scatter_steps", "ring_reduce_scatter_steps_from",
     "ring_allgather_steps", "ring_apply_rows",
     "ring_fusion_plan_create", "ring_fusion_plan_destroy", "ring_fusion_plan_elements",
-    "ring_fusion_pack", "ring_fusion_unpack", "ring_scale",
+    "ring_fusion_pack", "ring_fusion_unpack", "ring_fusion_unpack_scaled", "ring_scale",
 )
 
 
@@ -95,6 +95,7 @@ def lib():
             "ring_fusion_plan_elements": (sz, [vp]),
             "ring_fusion_pack": (ci, [vp, vp, vp]),
             "ring_fusion_unpack": (ci, [vp, vp, vp]),
+            "ring_fusion_unpack_scaled": (ci, [vp, vp, ci, vp]),
             "ring_scale": (ci, [ci, vp, sz, ci, vp]),
         }
         for name in EXPORTS:
@@ -251,6 +252,9 @@ class FusionPlan:
 
     def unpack(self, fused, stream):
         check(lib().ring_fusion_unpack(self._h, fused, stream), "ring_fusion_unpack")
+
+    def unpack_scaled(self, fused, divisor, stream):
+        check(lib().ring_fusion_unpack_scaled(self._h, fused, divisor, stream), "ring_fusion_unpack_scaled")
 
     def close(self):
         if self._h:

@@ -209,6 +209,17 @@ def _fusion_roundtrip(counts, dtype, rng, offsets=None):
         G.assert_same_bits(G.host(d), new[at:at + c], "unpack tensor %d" % j)
         assert int(torch.count_nonzero(base)) == int(np.count_nonzero(new[at:at + c]))  # nothing outside
         at += c
+    # unpack with the average folded in: tf.div by the number of ranks
+    for base in keep:
+        base.zero_()
+    plan.unpack_scaled(fused.data_ptr(), 6, None)
+    G.sync()
+    with np.errstate(all="ignore"):
+        want = new / np.float32(6) if np.dtype(dtype) == np.float32 else new // np.dtype(dtype).type(6)
+    at = 0
+    for j, (d, c) in enumerate(zip(devs, counts)):
+        G.assert_same_bits(G.host(d), want[at:at + c].astype(dtype), "unpack_scaled tensor %d" % j)
+        at += c
     plan.close()
 
 
