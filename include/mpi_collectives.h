@@ -79,6 +79,22 @@ void* mpic_world_stream(const mpic_world* world);
  * the stream has drained, 0: as soon as the work is enqueued). */
 int mpic_world_set_option(mpic_world* world, const char* name, int value);
 
+/* Tensor fusion in the coordinator (no counterpart in the reference, which runs
+ * one collective and one negotiation round per gradient, __init__.py:195-205).
+ * `buffer` is caller-owned device memory of size()*bytes_per_rank bytes, 16-byte
+ * aligned, rank r using slice r; bytes_per_rank (a multiple of 16) is the
+ * fusion threshold, 0 switches fusion off. While it is on, submitted
+ * collectives wait for mpic_world_flush(); at a flush, consecutive ready
+ * allreduces of one element type that fit the buffer together are packed per
+ * rank, reduced by ONE ring in place and unpacked into each op's output. Each
+ * tensor's result is then the reference ring applied to the packed buffer,
+ * which for float32 rounds differently from a ring per tensor (an element
+ * lands in another segment); grouping depends only on submission order and
+ * flush points, not on timing. Worlds with pre-staged peers never fuse. */
+int mpic_world_set_fusion_buffer(mpic_world* world, void* buffer, size_t bytes_per_rank);
+/* Start a tick now: everything submitted so far is negotiated and run. */
+int mpic_world_flush(mpic_world* world);
+
 /* Pre-staged peers for the op with node name `name`, consumed by the next
  * collective of that name: rs_segments[i] / ag_segments[i] are device pointers
  * to what the left neighbour sends at reduce-scatter / allgather step i

@@ -113,6 +113,13 @@ struct mpic_world {
   void* stream = nullptr;
   mpic::RingOptions ring_options;
   bool sync_on_done = true;
+  // Tensor fusion in the coordinator: allreduces that are ready in the same
+  // tick are packed, per rank, into that rank's slice of this caller-owned
+  // device buffer and reduced by one ring. Off while fusion_bytes == 0.
+  void* fusion_buffer = nullptr;
+  size_t fusion_bytes = 0;     // per rank
+  bool flush_requested = false;  // with fusion on, a tick starts when the embedder asks
+  std::map<std::string, ring_fusion_plan*> fusion_plans;  // keyed by the tensors' addresses and sizes
 
   int expected_requests() const { return real_rank >= 0 ? 1 : size; }
 };
@@ -297,6 +304,121 @@ void PerformCollectiveOp(mpic_world* w, const MPIResponse& response) {
   for (auto& kv : records) kv.second.callback(status);
 }
 
+// A fusion plan for these tensors, created on first use. Training loops reduce
+// the same gradient buffers every step, so plans are found again by the
+// tensors' addresses and sizes; the table is dropped when it grows large.
+ring_fusion_plan* FusionPlanFor(mpic_world* w, const std::vector<const void*>& ptrs,
+                                const std::vector<size_t>& counts, int ring_dtype) {
+  std::string key(reinterpret_cast<const char*>(ptrs.data()), ptrs.size() * sizeof(void*));
+  key.append(reinterpret_cast<const char*>(counts.data()), counts.size() * sizeof(size_t));
+  key.push_back(static_cast<char>(ring_dtype));
+  auto it = w->fusion_plans.find(key);
+  if (it != w->fusion_plans.end()) return it->second;
+  if (w->fusion_plans.size() >= 256) {
+    for (auto& kv : w->fusion_plans) ring_fusion_plan_destroy(kv.second);
+    w->fusion_plans.clear();
+  }
+  ring_fusion_plan* plan = nullptr;
+  if (ring_fusion_plan_create(ptrs.data(), counts.data(), static_cast<int>(ptrs.size()), ring_dtype, &plan) != RING_OK)
+    return nullptr;
+  w->fusion_plans[key] = plan;
+  return plan;
+}
+
+// Tensor fusion (no counterpart in the reference, where every gradient is its
+// own collective and its own negotiation round, __init__.py:195-205): the
+// allreduces `names`, all ready and valid, of one element type, are packed per
+// rank into that rank's fusion buffer in the order given, reduced by ONE ring
+// in place, and unpacked into each op's output. The result of each tensor is
+// the reference ring applied to the packed buffer.
+void PerformFusedAllreduce(mpic_world* w, const std::vector<std::string>& names) {
+  const int n = w->size;
+  std::vector<std::map<int, CollectiveOpRecord>> records;
+  {
+    std::lock_guard<std::mutex> guard(w->mu);
+    for (const std::string& name : names) {
+      auto it = w->tensor_table.find(name);
+      records.push_back(std::move(it->second));
+      w->tensor_table.erase(it);
+    }
+  }
+  Status status;
+  int code = 0;
+  const DataType dtype = records[0].begin()->second.in_t->dtype();
+  status = RingDataType(dtype, &code);
+  std::vector<size_t> counts;
+  size_t total = 0;
+  for (auto& rec : records) {
+    counts.push_back(static_cast<size_t>(rec.begin()->second.in_t->NumElements()));
+    total += counts.back();
+  }
+  std::vector<void*> bufs(static_cast<size_t>(n));
+  for (int r = 0; r < n && status.ok(); r++) {
+    bufs[static_cast<size_t>(r)] = static_cast<char*>(w->fusion_buffer) + static_cast<size_t>(r) * w->fusion_bytes;
+    std::vector<const void*> ins;
+    for (auto& rec : records) ins.push_back(rec.at(r).in_t->data());
+    ring_fusion_plan* plan = FusionPlanFor(w, ins, counts, code);
+    if (!plan || ring_fusion_pack(plan, bufs[static_cast<size_t>(r)], w->stream) != RING_OK)
+      status = errors::Unknown("MPI operation failed unexpectedly.");
+  }
+  if (status.ok()) {
+    std::vector<const void*> ins(bufs.begin(), bufs.end());
+    status = RingAllreduceAllRanks(n, dtype, ins.data(), bufs.data(), total, w->stream, w->ring_options);
+  }
+  for (int r = 0; r < n && status.ok(); r++) {
+    std::vector<const void*> outs;
+    for (auto& rec : records) outs.push_back(rec.at(r).out_t->data());
+    ring_fusion_plan* plan = FusionPlanFor(w, outs, counts, code);
+    if (!plan || ring_fusion_unpack(plan, bufs[static_cast<size_t>(r)], w->stream) != RING_OK)
+      status = errors::Unknown("MPI operation failed unexpectedly.");
+  }
+  if (status.ok() && w->sync_on_done && ring_stream_synchronize(w->stream) != RING_OK)
+    status = errors::Unknown("MPI operation failed unexpectedly.");
+  for (auto& rec : records)
+    for (auto& kv : rec) kv.second.callback(status);
+}
+
+// One tick's ready collectives, in the order they became ready. With fusion on,
+// runs of consecutive valid allreduces of one element type that fit the fusion
+// buffer together are reduced as one; everything else goes one by one.
+void PerformReady(mpic_world* w, const std::vector<std::string>& ready) {
+  std::vector<MPIResponse> responses;
+  for (const std::string& name : ready) responses.push_back(ConstructMPIResponse(&w->message_table, name));
+  const bool fusing = w->fusion_bytes > 0 && w->fusion_buffer && w->real_rank < 0 && w->size > 1;
+  size_t i = 0;
+  while (i < responses.size()) {
+    std::vector<std::string> group;
+    if (fusing && responses[i].response_type == MPIResponse::ALLREDUCE) {
+      size_t bytes = 0;
+      DataType group_dtype = DT_INVALID;
+      size_t j = i;
+      std::lock_guard<std::mutex> guard(w->mu);
+      for (; j < responses.size() && responses[j].response_type == MPIResponse::ALLREDUCE; j++) {
+        auto it = w->tensor_table.find(responses[j].tensor_name);
+        if (it == w->tensor_table.end() || static_cast<int>(it->second.size()) != w->size) break;
+        const CollectiveOpRecord& rec = it->second.begin()->second;
+        bool on_gpu = true;
+        for (auto& kv : it->second) on_gpu = on_gpu && kv.second.on_gpu;
+        const DataType dt = rec.in_t->dtype();
+        if (!on_gpu || DataTypeSize(dt) == 0 || dt == DT_DOUBLE) break;
+        if (group.empty()) group_dtype = dt;
+        // each tensor starts 16-byte aligned inside the buffer only by luck; the
+        // pack/unpack kernels handle any element alignment, so bytes just add up
+        if (dt != group_dtype || bytes + rec.in_t->TotalBytes() > w->fusion_bytes) break;
+        bytes += rec.in_t->TotalBytes();
+        group.push_back(responses[j].tensor_name);
+      }
+    }
+    if (group.size() >= 2) {
+      PerformFusedAllreduce(w, group);
+      i += group.size();
+    } else {
+      PerformCollectiveOp(w, responses[i]);
+      i++;
+    }
+  }
+}
+
 // mpi_ops.cc:572-795. Ticks are driven by arrivals, not by a 1 ms sleep.
 void BackgroundThreadLoop(mpic_world* w) {
   Status init;
@@ -319,8 +441,15 @@ void BackgroundThreadLoop(mpic_world* w) {
     std::queue<MPIRequest> message_queue;
     {
       std::unique_lock<std::mutex> lock(w->mu);
-      w->work_cv.wait(lock, [w] { return w->shut_down || !w->message_queue.empty(); });
+      // With fusion on a tick starts when the embedder asks for one (so the set of
+      // tensors fused together, and with it the rounding of the sums, does not
+      // depend on timing); otherwise every arrival starts one.
+      w->work_cv.wait(lock, [w] {
+        const bool hold = w->fusion_bytes > 0 && !w->flush_requested;
+        return w->shut_down || (!w->message_queue.empty() && !hold);
+      });
       std::swap(message_queue, w->message_queue);
+      w->flush_requested = false;
       should_shut_down = w->shut_down;
     }
     std::vector<std::string> ready_to_reduce;
@@ -330,10 +459,7 @@ void BackgroundThreadLoop(mpic_world* w) {
         ready_to_reduce.push_back(message.tensor_name);
       message_queue.pop();
     }
-    for (const std::string& name : ready_to_reduce) {
-      MPIResponse response = ConstructMPIResponse(&w->message_table, name);
-      PerformCollectiveOp(w, response);
-    }
+    PerformReady(w, ready_to_reduce);
   } while (!should_shut_down);
 
   // ops still waiting for absent ranks can never run: fail them
@@ -344,8 +470,10 @@ void BackgroundThreadLoop(mpic_world* w) {
   }
   for (auto& named : leftover)
     for (auto& kv : named.second) kv.second.callback(errors::Unknown("MPI was shut down before the collective ran."));
+  if (w->stream) ring_stream_synchronize(w->stream);
+  for (auto& kv : w->fusion_plans) ring_fusion_plan_destroy(kv.second);
+  w->fusion_plans.clear();
   if (w->stream) {
-    ring_stream_synchronize(w->stream);
     ring_stream_destroy(w->stream);
     w->stream = nullptr;
   }
@@ -747,6 +875,28 @@ int mpic_world_set_option(mpic_world* w, const char* name, int value) {
   else if (!strcmp(name, "fuse_copy")) w->ring_options.fuse_copy = value != 0;
   else if (!strcmp(name, "sync")) w->sync_on_done = value != 0;
   else return MPIC_INVALID_ARGUMENT;
+  return MPIC_OK;
+}
+
+int mpic_world_set_fusion_buffer(mpic_world* w, void* buffer, size_t bytes_per_rank) {
+  if (!w || (bytes_per_rank > 0 && (!buffer || (reinterpret_cast<uintptr_t>(buffer) & 15u) || (bytes_per_rank & 15u))))
+    return MPIC_INVALID_ARGUMENT;
+  {
+    std::lock_guard<std::mutex> guard(w->mu);
+    w->fusion_buffer = bytes_per_rank ? buffer : nullptr;
+    w->fusion_bytes = bytes_per_rank;
+  }
+  w->work_cv.notify_all();
+  return MPIC_OK;
+}
+
+int mpic_world_flush(mpic_world* w) {
+  if (!w) return MPIC_INVALID_ARGUMENT;
+  {
+    std::lock_guard<std::mutex> guard(w->mu);
+    w->flush_requested = true;
+  }
+  w->work_cv.notify_all();
   return MPIC_OK;
 }
 

@@ -165,7 +165,8 @@ Status RingAllreduceAllRanks(int n, DataType dt, const void* const* inputs, void
   // ring.h:146-148 on every rank
   for (int r = 0; r < n; r++) {
     if (!inputs[r] || !outputs[r]) return errors::InvalidArgument("null tensor with a non-zero element count");
-    rows[static_cast<size_t>(r)] = ring_row{outputs[r], inputs[r], nullptr, count};
+    // a rank reducing in place (a fusion buffer) has nothing to copy
+    rows[static_cast<size_t>(r)] = ring_row{outputs[r], inputs[r], nullptr, inputs[r] == outputs[r] ? 0 : count};
   }
   RING_RETURN_IF_ERROR(ring_apply_rows(rows.data(), n, code, stream), "ring_apply_rows");
 

@@ -101,9 +101,16 @@ class Session:
         real rank, whose peers are pre-staged with `stage_peers`.
       device: "GPU" (default when a GPU is present) or "CPU": where init() runs.
         Collectives have GPU kernels only.
+      fusion_threshold: bytes per rank of a fusion buffer (0 = off, the
+        reference's behaviour). When set, the allreduces submitted between two
+        `run` calls are packed, per element type and up to this many bytes, into
+        one buffer per rank and reduced by a single ring; each result is then
+        the ring applied to the packed buffer, which for float32 rounds
+        differently from one ring per tensor.
     """
 
-    def __init__(self, target='', graph=None, config=None, size=None, rank=None, device=None):
+    def __init__(self, target='', graph=None, config=None, size=None, rank=None, device=None,
+                 fusion_threshold=0):
         del target, graph, config
         L = _plugin.load_library('libmpi_collectives.so', mpi_ops._REQUIRED_OPS)
         self.size = int(size) if size is not None else _env_size()
@@ -123,10 +130,17 @@ class Session:
         self._counters = {}         # (rank, op) -> next auto-name index
         self._keep = []             # staged buffers kept alive until consumed
         self._prev = None
+        self._fusion_buffer = None
         self._enter_scope()
         try:
             # Initialize MPI on the relevant device (__init__.py:271-273).
             self.run(init())
+            if fusion_threshold and rank is None and self.size > 1:
+                per_rank = (int(fusion_threshold) + 15) // 16 * 16
+                self._fusion_buffer = torch.empty(per_rank * self.size, dtype=torch.uint8, device="cuda")
+                rc = L.mpic_world_set_fusion_buffer(self._world, self._fusion_buffer.data_ptr(), per_rank)
+                if rc != 0:
+                    raise InvalidArgumentError("could not install a fusion buffer of %d bytes per rank" % per_rank)
         except Exception:
             self.close()
             raise
@@ -273,6 +287,7 @@ class Session:
         first_error = None
         while self._pending:
             self._check_all_ranks_submitted()
+            _plugin.lib().mpic_world_flush(self._world)      # a tick: negotiate and run what was submitted
             batch, self._pending = self._pending, []
             for p in batch:
                 self._submitted.pop(p.node_name, None)

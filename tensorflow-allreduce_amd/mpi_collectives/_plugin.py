@@ -26,7 +26,8 @@ OK, UNKNOWN, INVALID_ARGUMENT, NOT_FOUND, FAILED_PRECONDITION, INTERNAL = 0, 2, 
 EXPORTS = (
     "mpic_op_count", "mpic_op_name", "mpic_op_signature", "mpic_op_doc", "mpic_op_has_kernel",
     "mpic_op_infer_shape", "mpic_world_create", "mpic_world_create_prestaged", "mpic_world_destroy",
-    "mpic_world_size", "mpic_world_stream", "mpic_world_set_option", "mpic_stage_peers",
+    "mpic_world_size", "mpic_world_stream", "mpic_world_set_option", "mpic_world_set_fusion_buffer",
+    "mpic_world_flush", "mpic_stage_peers",
     "mpic_context_create", "mpic_context_add_input", "mpic_context_compute", "mpic_context_wait",
     "mpic_context_message", "mpic_context_num_outputs", "mpic_context_output", "mpic_context_destroy",
     "mpic_ring_allreduce_prestaged", "mpic_ring_allgather_prestaged", "mpic_ring_allreduce_all_ranks",
@@ -110,6 +111,8 @@ def load_library(name="libmpi_collectives.so", op_list=None):
             "mpic_world_size": (ci, [vp]),
             "mpic_world_stream": (vp, [vp]),
             "mpic_world_set_option": (ci, [vp, cp, ci]),
+            "mpic_world_set_fusion_buffer": (ci, [vp, vp, sz]),
+            "mpic_world_flush": (ci, [vp]),
             "mpic_stage_peers": (ci, [vp, cp, pvp, pvp]),
             "mpic_context_create": (ci, [vp, ci, cp, cp, cp, ALLOC_FN, vp, pvp]),
             "mpic_context_add_input": (ci, [vp, ci, ci, p64, vp, ci]),

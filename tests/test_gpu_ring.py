@@ -399,3 +399,104 @@ def test_chained_allreduces_closed_form():
                 ours = cur * n + (spread * n * (n - 1) / 2 if i == 0 else 0)
         for s in state:
             assert np.allclose(G.host(s), np.float32(ours))
+
+
+def _expected_with_fusion(oracle, per_rank, groups):
+    """Per-tensor results when the tensors of each group are reduced as one
+    packed buffer (a group of one is a plain ring)."""
+    n = len(per_rank)
+    out = [None] * len(per_rank[0])
+    for g in groups:
+        packed = [np.concatenate([per_rank[r][j] for j in g]) for r in range(n)]
+        red = oracle.ring_allreduce(packed)[0]
+        at = 0
+        for j in g:
+            c = per_rank[0][j].size
+            out[j] = red[at:at + c]
+            at += c
+    return out
+
+
+@pytest.mark.parametrize("threshold,groups", [
+    (8 << 20, [[0, 1, 2, 3, 4, 5, 6]]),                    # everything fits: one ring
+    (20_000, [[0, 1, 2, 3], [4], [5, 6]]),                 # tensor 4 alone exceeds the buffer
+])
+def test_coordinator_fusion_matches_ring_on_packed_buffer(oracle, threshold, groups):
+    """Allreduces submitted between two runs are fused by the coordinator, in
+    submission order, up to the threshold; each tensor equals the reference
+    ring applied to the packed buffer of its group."""
+    n = 4
+    counts = [5, 4099, 64, 0, 100_003, 17, 2048]
+    per_rank = [[(np.random.default_rng(100 * r + j).standard_normal(c) * 10.0 ** (j - 3)).astype(np.float32)
+                 for j, c in enumerate(counts)] for r in range(n)]
+    want = _expected_with_fusion(oracle, per_rank, groups)
+    with mpi.Session(size=n, fusion_threshold=threshold) as session:
+        hs = [[None] * len(counts) for _ in range(n)]
+        for r in range(n):
+            with session.as_rank(r):
+                for j in range(len(counts)):
+                    hs[r][j] = mpi.allreduce(cuda(per_rank[r][j]), average=False)
+        outs = session.run(hs)
+    for r in range(n):
+        for j in range(len(counts)):
+            G.assert_same_bits(G.host(outs[r][j]), want[j], "fused by coordinator: rank %d tensor %d" % (r, j))
+
+
+def test_coordinator_fusion_groups_by_dtype_and_keeps_other_ops_apart(oracle):
+    n = 3
+    f = [[np.random.default_rng(r * 10 + j).standard_normal(1000 + j).astype(np.float32) for j in range(4)]
+         for r in range(n)]
+    i32 = [np.random.default_rng(50 + r).integers(-1000, 1001, 777).astype(np.int32) for r in range(n)]
+    rows = [2, 5, 1]
+    g = [np.random.default_rng(70 + r).standard_normal((rows[r], 3)).astype(np.float32) for r in range(n)]
+    with mpi.Session(size=n, fusion_threshold=1 << 20) as session:
+        hs = []
+        for r in range(n):
+            with session.as_rank(r):
+                hs.append([mpi.allreduce(cuda(f[r][0]), average=False), mpi.allreduce(cuda(f[r][1])),
+                           mpi.allreduce(cuda(i32[r]), average=False), mpi.allgather(cuda(g[r])),
+                           mpi.allreduce(cuda(f[r][2]), average=False), mpi.allreduce(cuda(f[r][3]), average=False)])
+        outs = session.run(hs)
+    first = _expected_with_fusion(oracle, [[f[r][0], f[r][1]] for r in range(n)], [[0, 1]])
+    # the int32 allreduce and the allgather's sizing pass are ready between the two
+    # float32 pairs, so each pair is its own group
+    second = _expected_with_fusion(oracle, [[f[r][2], f[r][3]] for r in range(n)], [[0, 1]])
+    ints = oracle.ring_allreduce(i32)[0]
+    for r in range(n):
+        G.assert_same_bits(G.host(outs[r][0]), first[0], "pair 1 a")
+        G.assert_same_bits(G.host(outs[r][1]), first[1] / np.float32(n), "pair 1 b (averaged)")
+        G.assert_same_bits(G.host(outs[r][2]), ints, "int32 between the groups")
+        G.assert_same_bits(G.host(outs[r][3]), np.concatenate(g), "allgather between the groups")
+        G.assert_same_bits(G.host(outs[r][4]), second[0], "pair 2 a")
+        G.assert_same_bits(G.host(outs[r][5]), second[1], "pair 2 b")
+
+
+def test_distributed_optimizer_over_coordinator_fusion(oracle):
+    """The reference's DistributedOptimizer issues one allreduce per gradient
+    (__init__.py:195-205); with a fusion threshold the coordinator reduces them
+    all with one ring."""
+    n = 3
+    torch.manual_seed(1)
+    base = torch.nn.Sequential(torch.nn.Linear(23, 31), torch.nn.ReLU(), torch.nn.Linear(31, 7)).cuda()
+    replicas, opts, local = [], [], []
+    with mpi.Session(size=n, fusion_threshold=1 << 20) as session:
+        gvs = []
+        for r in range(n):
+            m = torch.nn.Sequential(torch.nn.Linear(23, 31), torch.nn.ReLU(), torch.nn.Linear(31, 7)).cuda()
+            m.load_state_dict(base.state_dict())
+            replicas.append(m)
+            opts.append(mpi.DistributedOptimizer(torch.optim.SGD(m.parameters(), lr=0.05)))
+            x = torch.randn(9, 23, generator=torch.Generator().manual_seed(40 + r)).cuda()
+            with session.as_rank(r):
+                m(x).square().mean().backward()
+                local.append([G.host(p.grad).reshape(-1).copy() for p in m.parameters()])
+                gvs.append(opts[r].compute_gradients())
+        session.run()
+        for r in range(n):
+            with session.as_rank(r):
+                opts[r].apply_gradients(gvs[r])
+    k = len(local[0])
+    want = _expected_with_fusion(oracle, local, [list(range(k))])
+    for r in range(n):
+        for j, p in enumerate(replicas[r].parameters()):
+            G.assert_same_bits(G.host(p.grad).reshape(-1), want[j] / np.float32(n), "rank %d gradient %d" % (r, j))

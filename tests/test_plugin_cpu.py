@@ -282,3 +282,18 @@ def test_resnet50_shape_set():
     assert len(shapes) == 161 and sum(sizes) == 25_557_032
     assert min(sizes) == 64 and max(sizes) == 2_359_296
     assert sum(1 for s in sizes if s <= 2048) == 107
+
+
+def test_fusion_buffer_arguments_and_flush():
+    L = _plugin.load_library()
+    w = ctypes.c_void_p()
+    assert L.mpic_world_create(2, ctypes.byref(w)) == 0
+    try:
+        assert L.mpic_world_set_fusion_buffer(w.value, None, 1024) == 3        # a size without a buffer
+        assert L.mpic_world_set_fusion_buffer(w.value, 4096 + 8, 1024) == 3    # not 16-byte aligned
+        assert L.mpic_world_set_fusion_buffer(w.value, 4096, 1000) == 3        # not a multiple of 16
+        assert L.mpic_world_set_fusion_buffer(w.value, None, 0) == 0           # off
+        assert L.mpic_world_flush(w.value) == 0                                # harmless without pending work
+        assert L.mpic_world_flush(None) == 3
+    finally:
+        L.mpic_world_destroy(w.value)
