@@ -53,6 +53,25 @@ def test_accumulate_matches_oracle(oracle, dtype):
             G.assert_same_bits(G.host(db), b)
 
 
+def test_more_than_2_pow_32_elements():
+    """Counts are 64-bit end to end (the reference's CPU loop indexes with an
+    `unsigned int`, ring.cc:44, and passes size_t counts to MPI as int)."""
+    import torch
+    count = (1 << 32) + 12_345
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    a = torch.randint(-2**31, 2**31 - 1, (count + 3,), dtype=torch.int32, device="cuda", generator=gen)
+    b = torch.randint(-2**31, 2**31 - 1, (count + 1,), dtype=torch.int32, device="cuda", generator=gen)
+    want = a[3:] + b[1:]                                  # wraps like the ring's integer add
+    got = a.clone()
+    ring_abi.accumulate(ring_abi.I32, got.data_ptr() + 12, b.data_ptr() + 4, count, None)
+    G.sync()
+    assert torch.equal(got[3:], want) and torch.equal(got[:3], a[:3])
+    del want
+    ring_abi.copy_bytes(got.data_ptr(), b.data_ptr() + 4, count * 4, None)
+    G.sync()
+    assert torch.equal(got[:count], b[1:]) and torch.equal(got[count:], (a[3:] + b[1:])[count - 3:])
+
+
 def test_typed_entry_points_and_errors():
     L = ring_abi.lib()
     a, _ = G.dev(np.arange(10, dtype=np.float32))

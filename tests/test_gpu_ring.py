@@ -500,3 +500,37 @@ def test_distributed_optimizer_over_coordinator_fusion(oracle):
     for r in range(n):
         for j, p in enumerate(replicas[r].parameters()):
             G.assert_same_bits(G.host(p.grad).reshape(-1), want[j] / np.float32(n), "rank %d gradient %d" % (r, j))
+
+
+def test_per_rank_path_replays_from_a_hip_graph(oracle):
+    """The entry points only launch kernels (no allocation, no memset), so a
+    caller can capture a rank's whole data path in a HIP graph. Every replay,
+    with eager work and synchronisations in between, must reproduce the eager
+    result."""
+    n, r, count = 4, 1, 300_007
+    ins = make_inputs(n, count, np.float32, seed=21)
+    outs, rs, ag = oracle.ring_allreduce(ins, tap=True)
+    sizes, _ = ring_abi.segment_table(count, n)
+    L = _plugin.load_library()
+    din = cuda(ins[r])
+    dout = torch.zeros(count, device="cuda")
+    rs_t = [cuda(rs[r][i][:sizes[ring_abi.schedule(0, n, r, i)[1]]]) for i in range(n - 1)]
+    ag_t = [cuda(ag[r][i][:sizes[ring_abi.schedule(1, n, r, i)[1]]]) for i in range(n - 1)]
+    rs_p = (ctypes.c_void_p * (n - 1))(*[t.data_ptr() for t in rs_t])
+    ag_p = (ctypes.c_void_p * (n - 1))(*[t.data_ptr() for t in ag_t])
+    for flags in (1, 3):
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                rc = L.mpic_ring_allreduce_prestaged(n, r, _plugin.DT_FLOAT, din.data_ptr(), dout.data_ptr(), count,
+                                                     rs_p, ag_p, torch.cuda.current_stream().cuda_stream, flags)
+                assert rc == 0, L.mpic_last_error()
+        torch.cuda.current_stream().wait_stream(side)
+        for replay in range(4):
+            dout.zero_()                              # eager work between replays
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            G.assert_same_bits(G.host(dout), outs[r], "graph replay %d flags %d" % (replay, flags))
