@@ -33,6 +33,7 @@ collectives complete at once.
 """
 import contextlib
 import os
+import threading
 
 import torch
 
@@ -56,6 +57,7 @@ class PendingTensor:
         self._error = None
         self._ready = False
         self._post = []       # fn(tensor) -> tensor applied to the value when it arrives
+        self._first_op = None  # the op (chain) whose completion produces the value
 
     def _set(self, value=None, error=None):
         if error is None:
@@ -64,8 +66,23 @@ class PendingTensor:
         self._value, self._error, self._ready = value, error, True
 
     def result(self):
+        """The tensor. If it is not there yet, runs the session: every rank must
+        already have submitted the op (a single thread driving all ranks)."""
         if not self._ready:
             self._session.run()
+        if self._error is not None:
+            raise self._error
+        return self._value
+
+    def wait(self):
+        """The tensor, blocking until the collective has run. For ranks driven
+        from separate threads, as separate MPI processes would be: the call
+        returns once the other ranks' threads have submitted the op."""
+        op = self._first_op
+        while op is not None and not self._ready:
+            self._session._flush()
+            self._session._complete(op)
+            op = op.next_op
         if self._error is not None:
             raise self._error
         return self._value
@@ -125,6 +142,7 @@ class Session:
         if rc != 0:
             raise _plugin.error_for(rc, "could not create an MPI world of size %r, rank %r" % (size, rank))
         self._world = h.value
+        self._lock = threading.RLock()   # ranks may be driven from separate threads
         self._pending = []          # ops submitted and not yet waited for
         self._submitted = {}        # node name -> set of ranks, for the run() guard
         self._counters = {}         # (rank, op) -> next auto-name index
@@ -220,8 +238,9 @@ class Session:
         """TensorFlow uniquifies node names per graph: op, op_1, op_2, ... Every
         rank builds the same graph, so the k-th unnamed op matches across ranks."""
         base = name if name is not None else op
-        k = self._counters.get((r, base), 0)
-        self._counters[(r, base)] = k + 1
+        with self._lock:
+            k = self._counters.get((r, base), 0)
+            self._counters[(r, base)] = k + 1
         return base if k == 0 else "%s_%d" % (base, k)
 
     def _submit(self, r, op, node_name, inputs, device):
@@ -231,9 +250,14 @@ class Session:
             torch.cuda.current_stream().synchronize()
         pending = _plugin.PendingOp(self._world, r, op, node_name, inputs, device)
         pending.rank = r
+        pending.handle = pending.fail_handle = pending.on_done = pending.next_op = None
+        pending.lock = threading.Lock()
+        pending.completed = False
+        pending.error = None
         if op in ("MPIAllreduce", "MPIAllgather"):
-            self._submitted.setdefault(node_name, set()).add(r)
-            self._pending.append(pending)
+            with self._lock:
+                self._submitted.setdefault(node_name, set()).add(r)
+                self._pending.append(pending)
         return pending
 
     @property
@@ -242,15 +266,15 @@ class Session:
 
     def _result(self, pending):
         handle = PendingTensor(self)
+        handle._first_op = pending
         pending.handle = handle
-        pending.on_done = None
         if self._immediate:
             self._drain()
         return handle
 
     def _chain_allgather(self, r, sizing, tensor, name, dev):
         handle = PendingTensor(self)
-        sizing.handle = None
+        handle._first_op = sizing
 
         def after_sizing(outputs):
             sizes = outputs[0].cpu() if outputs[0].is_cuda else outputs[0]   # host-memory `sizes` input
@@ -258,7 +282,7 @@ class Session:
             with self.as_rank(r):
                 second = self._submit(r, 'MPIAllgather', node, [tensor, sizes], dev)
             second.handle = handle
-            second.on_done = None
+            sizing.next_op = second
 
         sizing.on_done = after_sizing
         sizing.fail_handle = handle
@@ -273,10 +297,44 @@ class Session:
         elif handle._error is None:
             handle._value = fn(handle._value)
 
-    def _check_all_ranks_submitted(self):
+    def _flush(self):
+        """Start a coordinator tick: negotiate and run what was submitted."""
+        _plugin.lib().mpic_world_flush(self._world)
+
+    def _complete(self, p):
+        """Wait for op p (blocks until every rank has submitted it), then run
+        its continuation and publish its result; once per op, from any thread."""
+        with p.lock:
+            if p.completed:
+                return p.error
+            try:
+                outputs = p.wait()
+                if p.on_done:
+                    p.on_done(outputs)
+                if p.handle is not None:
+                    p.handle._set(value=outputs[0])
+            except OpError as e:
+                p.error = e
+                for h in (p.handle, p.fail_handle):
+                    if h is not None:
+                        h._set(error=e)
+            p.completed = True
+        with self._lock:
+            if p in self._pending:
+                self._pending.remove(p)
+            ranks = self._submitted.get(p.node_name)
+            if ranks is not None:
+                ranks.discard(p.rank)
+                if not ranks:
+                    self._submitted.pop(p.node_name, None)
+        return p.error
+
+    def _check_all_ranks_submitted(self, batch):
         if self.real_rank is not None:
             return
-        for p in self._pending:
+        for p in batch:
+            if p.completed:
+                continue
             ranks = self._submitted.get(p.node_name, set())
             if len(ranks) != self.size:
                 raise FailedPreconditionError(
@@ -285,24 +343,15 @@ class Session:
 
     def _drain(self):
         first_error = None
-        while self._pending:
-            self._check_all_ranks_submitted()
-            _plugin.lib().mpic_world_flush(self._world)      # a tick: negotiate and run what was submitted
-            batch, self._pending = self._pending, []
+        while True:
+            with self._lock:
+                batch = list(self._pending)
+                if not batch:
+                    break
+                self._check_all_ranks_submitted(batch)
+            self._flush()
             for p in batch:
-                self._submitted.pop(p.node_name, None)
-            for p in batch:
-                try:
-                    outputs = p.wait()
-                    if getattr(p, "on_done", None):
-                        p.on_done(outputs)
-                    if getattr(p, "handle", None) is not None:
-                        p.handle._set(value=outputs[0])
-                except OpError as e:
-                    first_error = first_error or e
-                    for h in (getattr(p, "handle", None), getattr(p, "fail_handle", None)):
-                        if h is not None:
-                            h._set(error=e)
+                first_error = first_error or self._complete(p)
         if self.stream:
             ring_abi.stream_synchronize(self.stream)
         if first_error is not None:

@@ -534,3 +534,44 @@ def test_per_rank_path_replays_from_a_hip_graph(oracle):
             graph.replay()
             torch.cuda.synchronize()
             G.assert_same_bits(G.host(dout), outs[r], "graph replay %d flags %d" % (replay, flags))
+
+
+def test_ranks_driven_from_separate_threads(oracle):
+    """One thread per rank, as one MPI process per rank would run: every thread
+    submits its collectives and blocks on its own results; the readiness table
+    and the background thread see truly concurrent arrivals."""
+    import threading
+    n = 6
+    ins = make_inputs(n, 123_457, np.float32, seed=77)
+    ints = make_inputs(n, 1001, np.int64, seed=78)
+    rows = [3, 1, 4, 1, 5, 9]
+    parts = [np.random.default_rng(90 + r).standard_normal((rows[r], 7)).astype(np.float32) for r in range(n)]
+    want_sum = oracle.ring_allreduce(ins)[0]
+    want_int = oracle.ring_allreduce(ints)[0] // n
+    want_cat = np.concatenate(parts)
+    results, errors = [None] * n, []
+    with mpi.Session(size=n) as session:
+        def worker(r):
+            try:
+                with session.as_rank(r):
+                    out = []
+                    for rep in range(3):                       # the same ops again: node names must keep matching
+                        a = mpi.allreduce(cuda(ins[r]), average=False).wait()
+                        b = mpi.allreduce(cuda(ints[r])).wait()            # average: floor division
+                        c = mpi.allgather(cuda(parts[r])).wait()
+                        out.append((G.host(a), G.host(b), G.host(c)))
+                    results[r] = out
+            except Exception as e:                             # surfaced below, in the main thread
+                errors.append((r, e))
+        threads = [threading.Thread(target=worker, args=(r,)) for r in range(n)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(timeout=60)
+        assert not any(t.is_alive() for t in threads), "a rank is still waiting for its collective"
+    assert not errors, errors
+    for r in range(n):
+        for a, b, c in results[r]:
+            G.assert_same_bits(a, want_sum, "threaded allreduce rank %d" % r)
+            G.assert_same_bits(b, want_int, "threaded averaged int64 rank %d" % r)
+            G.assert_same_bits(c, want_cat, "threaded allgather rank %d" % r)
