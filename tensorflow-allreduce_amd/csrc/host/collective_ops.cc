@@ -28,6 +28,7 @@
 #include "mpi_collectives.h"
 #include "ring_abi.h"
 #include "ring_driver.h"
+#include "wire.h"
 
 namespace mpic {
 namespace {
@@ -37,35 +38,6 @@ using GPUDevice = struct GPUDeviceTag {};
 template <typename T> bool IsGPUDevice();
 template <> bool IsGPUDevice<GPUDevice>() { return true; }
 template <> bool IsGPUDevice<CPUDevice>() { return false; }
-
-// mpi_message.proto:12-17
-enum MPIDataType { TF_MPI_INVALID_TYPE = 0, TF_MPI_FLOAT32 = 1, TF_MPI_INT32 = 2, TF_MPI_INT64 = 3 };
-const char* MPIDataType_Name(MPIDataType t) {
-  switch (t) {
-    case TF_MPI_FLOAT32: return "TF_MPI_FLOAT32";
-    case TF_MPI_INT32: return "TF_MPI_INT32";
-    case TF_MPI_INT64: return "TF_MPI_INT64";
-    default: return "TF_MPI_INVALID_TYPE";
-  }
-}
-
-// mpi_message.proto:22-40
-struct MPIRequest {
-  enum RequestType { ALLREDUCE = 0, ALLGATHER = 1 };
-  int request_rank = 0;
-  RequestType request_type = ALLREDUCE;
-  MPIDataType tensor_type = TF_MPI_INVALID_TYPE;
-  std::string tensor_name;
-  std::vector<int64_t> tensor_shape;
-};
-
-// mpi_message.proto:49-63
-struct MPIResponse {
-  enum ResponseType { ALLREDUCE = 0, ALLGATHER = 1, ERROR = 2, DONE = 3, SHUTDOWN = 4 };
-  ResponseType response_type = DONE;
-  std::string tensor_name;
-  std::string error_message;
-};
 
 typedef std::function<void(const Status&)> CommunicationDoneCallback;
 
@@ -102,7 +74,9 @@ struct mpic_world {
   mpic::Status init_status;
   std::mutex mu;
   mpic::TensorTable tensor_table;
-  std::queue<mpic::MPIRequest> message_queue;
+  // requests on their way to the coordinator, in wire format (the bytes a rank
+  // in another process would send)
+  std::queue<std::string> message_queue;
   std::thread background_thread;
   bool shut_down = false;
   mpic::MessageTable message_table;  // coordinator side
@@ -382,8 +356,14 @@ void PerformFusedAllreduce(mpic_world* w, const std::vector<std::string>& names)
 // runs of consecutive valid allreduces of one element type that fit the fusion
 // buffer together are reduced as one; everything else goes one by one.
 void PerformReady(mpic_world* w, const std::vector<std::string>& ready) {
+  // Each response goes through its wire form, as it would to ranks in other
+  // processes (mpi_ops.cc:727-739).
   std::vector<MPIResponse> responses;
-  for (const std::string& name : ready) responses.push_back(ConstructMPIResponse(&w->message_table, name));
+  for (const std::string& name : ready) {
+    MPIResponse received;
+    if (received.ParseFromString(ConstructMPIResponse(&w->message_table, name).SerializeAsString()))
+      responses.push_back(received);
+  }
   const bool fusing = w->fusion_bytes > 0 && w->fusion_buffer && w->real_rank < 0 && w->size > 1;
   size_t i = 0;
   while (i < responses.size()) {
@@ -438,7 +418,7 @@ void BackgroundThreadLoop(mpic_world* w) {
 
   bool should_shut_down = false;
   do {
-    std::queue<MPIRequest> message_queue;
+    std::queue<std::string> message_queue;
     {
       std::unique_lock<std::mutex> lock(w->mu);
       // With fusion on a tick starts when the embedder asks for one (so the set of
@@ -454,8 +434,9 @@ void BackgroundThreadLoop(mpic_world* w) {
     }
     std::vector<std::string> ready_to_reduce;
     while (!message_queue.empty()) {
-      const MPIRequest& message = message_queue.front();
-      if (IncrementTensorCount(&w->message_table, message, w->expected_requests()))
+      MPIRequest message;
+      if (message.ParseFromString(message_queue.front()) &&
+          IncrementTensorCount(&w->message_table, message, w->expected_requests()))
         ready_to_reduce.push_back(message.tensor_name);
       message_queue.pop();
     }
@@ -521,7 +502,7 @@ void EnqueueTensorCollective(mpic_world* w, const CollectiveOpRecord& record, MP
   {
     std::lock_guard<std::mutex> guard(w->mu);
     w->tensor_table[record.name][record.rank] = record;
-    w->message_queue.push(message);
+    w->message_queue.push(message.SerializeAsString());
   }
   w->work_cv.notify_one();
 }

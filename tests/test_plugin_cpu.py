@@ -297,3 +297,18 @@ def test_fusion_buffer_arguments_and_flush():
         assert L.mpic_world_flush(None) == 3
     finally:
         L.mpic_world_destroy(w.value)
+
+
+def test_zero_sized_dimensions_survive_the_coordinator():
+    """A zero-sized dimension encodes as a zero byte; the reference's messages
+    are cut at the first one (mpi_ops.cc:703, 773). Here shapes with zeros are
+    compared, and reported, in full."""
+    with mpi.Session(size=2, device="CPU") as s:
+        errs = _errors(_submit_all(s, 'MPIAllreduce', [torch.zeros([0, 5]), torch.zeros([0, 6])], "z"))
+        assert errs[0].message == ("Mismatched allreduce tensor shapes: One rank reduced a tensor of shape [0,5], "
+                                   "but another rank sent a tensor of shape [0,6].")
+        s._pending.clear()
+        # equal empty shapes pass the checks (and are then refused for living in host memory)
+        errs = _errors(_submit_all(s, 'MPIAllreduce', [torch.zeros([0, 5]), torch.zeros([0, 5])], "z2"))
+        assert "GPU kernels only" in errs[0].message
+        s._pending.clear()
