@@ -929,10 +929,10 @@ int mpic_context_compute(mpic_context* c) {
   if (!c || c->started) return MPIC_INVALID_ARGUMENT;
   c->started = true;
   auto done = [c] {
-    {
-      std::lock_guard<std::mutex> guard(c->mu);
-      c->done = true;
-    }
+    // notify under the lock: the waiter may destroy the context as soon as it
+    // sees `done`, so nothing of the context is touched after the unlock
+    std::lock_guard<std::mutex> guard(c->mu);
+    c->done = true;
     c->cv.notify_all();
   };
   if (c->kernel->IsAsync()) {
