@@ -575,3 +575,20 @@ def test_ranks_driven_from_separate_threads(oracle):
             G.assert_same_bits(a, want_sum, "threaded allreduce rank %d" % r)
             G.assert_same_bits(b, want_int, "threaded averaged int64 rank %d" % r)
             G.assert_same_bits(c, want_cat, "threaded allgather rank %d" % r)
+
+
+@pytest.mark.parametrize("fusion", [False, True])
+def test_training_example_runs_and_learns(fusion, monkeypatch):
+    """The data-parallel example: replicas stay bit-identical and the loss falls."""
+    import importlib.util
+    import os
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
+                        "tensorflow-allreduce_amd", "examples", "train_virtual_ranks.py")
+    spec = importlib.util.spec_from_file_location("train_virtual_ranks", path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    monkeypatch.setattr("sys.argv", ["train_virtual_ranks.py", "--ranks", "3", "--steps", "2"] + (["--fusion"] if fusion else []))
+    first = mod.main()
+    monkeypatch.setattr("sys.argv", ["train_virtual_ranks.py", "--ranks", "3", "--steps", "30"] + (["--fusion"] if fusion else []))
+    last = mod.main()
+    assert last < first

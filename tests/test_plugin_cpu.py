@@ -312,3 +312,26 @@ def test_zero_sized_dimensions_survive_the_coordinator():
         errs = _errors(_submit_all(s, 'MPIAllreduce', [torch.zeros([0, 5]), torch.zeros([0, 5])], "z2"))
         assert "GPU kernels only" in errs[0].message
         s._pending.clear()
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="checks the behaviour on a machine without a GPU")
+def test_without_a_gpu_every_device_call_fails_and_nothing_is_computed_on_the_host():
+    L = ring_abi.lib()
+    a = numpy.ones(1024, dtype=numpy.float32)
+    b = numpy.full(1024, 2.0, dtype=numpy.float32)
+    assert L.ring_accumulate(ring_abi.F32, a.ctypes.data, b.ctypes.data, 1024, None) == 3      # RING_ERR_HIP
+    assert L.ring_last_hip_error() != 0
+    assert L.ring_copy_bytes(a.ctypes.data, b.ctypes.data, 4096, None) == 3
+    assert L.ring_scale(ring_abi.F32, a.ctypes.data, 1024, 2, None) == 3
+    stream = ctypes.c_void_p()
+    assert L.ring_stream_create(ctypes.byref(stream)) == 3
+    ptrs = (ctypes.c_void_p * 1)(a.ctypes.data)
+    counts = (ctypes.c_size_t * 1)(1024)
+    plan = ctypes.c_void_p()
+    assert L.ring_fusion_plan_create(ptrs, counts, 1, ring_abi.F32, ctypes.byref(plan)) == 3 and not plan.value
+    assert (a == 1.0).all()                                # the host never stood in for the device
+    with pytest.raises(ring_abi.RingError, match="HIP runtime call failed"):
+        ring_abi.accumulate(ring_abi.F32, a.ctypes.data, b.ctypes.data, 1024, None)
+    # a GPU session cannot even initialise: its dedicated stream cannot be created
+    with pytest.raises(mpi.UnknownError, match="Could not create the MPI stream"):
+        mpi.Session(size=2, device="GPU")
