@@ -188,9 +188,28 @@ MPIResponse ConstructMPIResponse(MessageTable* table, const std::string& name) {
   return response;
 }
 
+// The options an embedder may change while the background thread runs, read
+// once per collective under the world's mutex.
+struct WorldOptions {
+  RingOptions ring;
+  bool sync_on_done = true;
+  void* fusion_buffer = nullptr;
+  size_t fusion_bytes = 0;
+};
+WorldOptions SnapshotOptions(mpic_world* w) {
+  std::lock_guard<std::mutex> guard(w->mu);
+  WorldOptions o;
+  o.ring = w->ring_options;
+  o.sync_on_done = w->sync_on_done;
+  o.fusion_buffer = w->fusion_buffer;
+  o.fusion_bytes = w->fusion_bytes;
+  return o;
+}
+
 // mpi_ops.cc:435-515: run the collective for every rank that lives here, then
 // resume their ops.
 void PerformCollectiveOp(mpic_world* w, const MPIResponse& response) {
+  const WorldOptions opt = SnapshotOptions(w);
   std::map<int, CollectiveOpRecord> records;
   StagedPeers peers;
   bool have_peers = false;
@@ -236,12 +255,12 @@ void PerformCollectiveOp(mpic_world* w, const MPIResponse& response) {
     } else if (response.response_type == MPIResponse::ALLREDUCE) {
       status = RingAllreducePrestaged(n, r, dtype, first.in_t->data(), first.out_t->data(),
                                       static_cast<size_t>(first.in_t->NumElements()), peers.rs.data(),
-                                      peers.ag.data(), w->stream, w->ring_options);
+                                      peers.ag.data(), w->stream, opt.ring);
     } else {
       size_t epr = 1;
       for (int i = 1; i < first.in_t->shape().dims(); i++) epr *= static_cast<size_t>(first.in_t->dim_size(i));
       status = RingAllgatherPrestaged(n, r, dtype, first.in_t->data(), first.sizes_vec, epr, first.out_t->data(),
-                                      peers.ag.data(), w->stream, w->ring_options);
+                                      peers.ag.data(), w->stream, opt.ring);
     }
   } else {
     std::vector<const void*> ins(static_cast<size_t>(n));
@@ -252,7 +271,7 @@ void PerformCollectiveOp(mpic_world* w, const MPIResponse& response) {
     }
     if (response.response_type == MPIResponse::ALLREDUCE) {
       status = RingAllreduceAllRanks(n, dtype, ins.data(), outs.data(),
-                                     static_cast<size_t>(first.in_t->NumElements()), w->stream, w->ring_options);
+                                     static_cast<size_t>(first.in_t->NumElements()), w->stream, opt.ring);
     } else {
       size_t epr = 1;
       for (int i = 1; i < first.in_t->shape().dims(); i++) epr *= static_cast<size_t>(first.in_t->dim_size(i));
@@ -267,11 +286,11 @@ void PerformCollectiveOp(mpic_world* w, const MPIResponse& response) {
       }
       if (status.ok())
         status = RingAllgatherAllRanks(n, dtype, ins.data(), first.sizes_vec, epr, outs.data(), w->stream,
-                                       w->ring_options);
+                                       opt.ring);
     }
   }
 
-  if (status.ok() && w->sync_on_done && response.response_type != MPIResponse::ERROR) {
+  if (status.ok() && opt.sync_on_done && response.response_type != MPIResponse::ERROR) {
     const int rc = ring_stream_synchronize(w->stream);
     if (rc != RING_OK) status = errors::Unknown("MPI operation failed unexpectedly.");  // ring.h:36-39
   }
@@ -289,6 +308,7 @@ ring_fusion_plan* FusionPlanFor(mpic_world* w, const std::vector<const void*>& p
   auto it = w->fusion_plans.find(key);
   if (it != w->fusion_plans.end()) return it->second;
   if (w->fusion_plans.size() >= 256) {
+    ring_stream_synchronize(w->stream);  // launches in flight still read the plans' device tables
     for (auto& kv : w->fusion_plans) ring_fusion_plan_destroy(kv.second);
     w->fusion_plans.clear();
   }
@@ -305,7 +325,7 @@ ring_fusion_plan* FusionPlanFor(mpic_world* w, const std::vector<const void*>& p
 // rank into that rank's fusion buffer in the order given, reduced by ONE ring
 // in place, and unpacked into each op's output. The result of each tensor is
 // the reference ring applied to the packed buffer.
-void PerformFusedAllreduce(mpic_world* w, const std::vector<std::string>& names) {
+void PerformFusedAllreduce(mpic_world* w, const std::vector<std::string>& names, const WorldOptions& opt) {
   const int n = w->size;
   std::vector<std::map<int, CollectiveOpRecord>> records;
   {
@@ -328,7 +348,7 @@ void PerformFusedAllreduce(mpic_world* w, const std::vector<std::string>& names)
   }
   std::vector<void*> bufs(static_cast<size_t>(n));
   for (int r = 0; r < n && status.ok(); r++) {
-    bufs[static_cast<size_t>(r)] = static_cast<char*>(w->fusion_buffer) + static_cast<size_t>(r) * w->fusion_bytes;
+    bufs[static_cast<size_t>(r)] = static_cast<char*>(opt.fusion_buffer) + static_cast<size_t>(r) * opt.fusion_bytes;
     std::vector<const void*> ins;
     for (auto& rec : records) ins.push_back(rec.at(r).in_t->data());
     ring_fusion_plan* plan = FusionPlanFor(w, ins, counts, code);
@@ -337,7 +357,7 @@ void PerformFusedAllreduce(mpic_world* w, const std::vector<std::string>& names)
   }
   if (status.ok()) {
     std::vector<const void*> ins(bufs.begin(), bufs.end());
-    status = RingAllreduceAllRanks(n, dtype, ins.data(), bufs.data(), total, w->stream, w->ring_options);
+    status = RingAllreduceAllRanks(n, dtype, ins.data(), bufs.data(), total, w->stream, opt.ring);
   }
   for (int r = 0; r < n && status.ok(); r++) {
     std::vector<const void*> outs;
@@ -346,7 +366,7 @@ void PerformFusedAllreduce(mpic_world* w, const std::vector<std::string>& names)
     if (!plan || ring_fusion_unpack(plan, bufs[static_cast<size_t>(r)], w->stream) != RING_OK)
       status = errors::Unknown("MPI operation failed unexpectedly.");
   }
-  if (status.ok() && w->sync_on_done && ring_stream_synchronize(w->stream) != RING_OK)
+  if (status.ok() && opt.sync_on_done && ring_stream_synchronize(w->stream) != RING_OK)
     status = errors::Unknown("MPI operation failed unexpectedly.");
   for (auto& rec : records)
     for (auto& kv : rec) kv.second.callback(status);
@@ -364,7 +384,8 @@ void PerformReady(mpic_world* w, const std::vector<std::string>& ready) {
     if (received.ParseFromString(ConstructMPIResponse(&w->message_table, name).SerializeAsString()))
       responses.push_back(received);
   }
-  const bool fusing = w->fusion_bytes > 0 && w->fusion_buffer && w->real_rank < 0 && w->size > 1;
+  const WorldOptions opt = SnapshotOptions(w);
+  const bool fusing = opt.fusion_bytes > 0 && opt.fusion_buffer && w->real_rank < 0 && w->size > 1;
   size_t i = 0;
   while (i < responses.size()) {
     std::vector<std::string> group;
@@ -384,13 +405,13 @@ void PerformReady(mpic_world* w, const std::vector<std::string>& ready) {
         if (group.empty()) group_dtype = dt;
         // each tensor starts 16-byte aligned inside the buffer only by luck; the
         // pack/unpack kernels handle any element alignment, so bytes just add up
-        if (dt != group_dtype || bytes + rec.in_t->TotalBytes() > w->fusion_bytes) break;
+        if (dt != group_dtype || bytes + rec.in_t->TotalBytes() > opt.fusion_bytes) break;
         bytes += rec.in_t->TotalBytes();
         group.push_back(responses[j].tensor_name);
       }
     }
     if (group.size() >= 2) {
-      PerformFusedAllreduce(w, group);
+      PerformFusedAllreduce(w, group, opt);
       i += group.size();
     } else {
       PerformCollectiveOp(w, responses[i]);

@@ -9,18 +9,19 @@
 // Design, in the order it matters for an HBM-bound stream:
 //   * every lane moves 16 bytes per access (global_load/store_dwordx4), a
 //     wave64 touches 1 KiB of contiguous memory per instruction;
-//   * a workgroup is 4 waves; one tile is kUnroll x 256 x 16 B per operand, all
-//     loads of a tile are issued before the first add/store, so each wave
-//     keeps 2*kUnroll KiB in flight;
-//   * workgroups walk the tiles of ALL rows of a step table in one grid-stride
-//     loop, so the n-1 accumulates (or copies) of a rank are one launch, not
-//     n-1 launches and n-1 host syncs;
+//   * a workgroup is 4 waves; one tile is 4 x 256 x 16 B = 16 KiB per operand,
+//     all loads of a tile are issued before the first add/store, so each wave
+//     keeps 8 KiB in flight;
+//   * one launch carries a whole step table (up to 64 rows by value in the
+//     kernel arguments), so the n-1 accumulates (or copies) of a rank are one
+//     launch, not n-1 launches and n-1 host syncs. Rows with equal tile counts
+//     (the segments of an allreduce) use a 2-D grid (tiles, rows); unequal rows
+//     share a 1-D grid and a workgroup finds its row by a scalar binary search;
 //   * stores are 16-byte aligned: up to 3 head elements are peeled per row so
-//     the destination is aligned, the source is read with element-aligned
+//     the destination is aligned, the sources are read with element-aligned
 //     (possibly 16-byte-unaligned) dwordx4 loads. Ragged segment starts only
 //     cost those few scalar elements;
-//   * streams that are written once and not re-read by this launch use
-//     non-temporal stores;
+//   * every byte is touched once, so loads and stores are non-temporal;
 //   * LDS is used only by the fusion kernels, for the offset table of a tile
 //     that spans several small tensors.
 // No MFMA: the path is one add per 12 bytes.
