@@ -12,6 +12,10 @@
                           C++ (g++), no GPU code; calls libring_hip.so through
                           the C ABI.
 
+  tests/cpp/build/ring_gpu_test
+                          a C++ test of the C ABI (test code, linked with the
+                          oracle), run on the GPU by tests/test_gpu_cpp.py.
+
 hipcc cross-compiles for gfx950 without a GPU. Packed FP32 instructions are
 disabled for all device code.
 """
@@ -83,8 +87,35 @@ def build_plugin(verbose=True):
     return PLUGIN_SO
 
 
+def build_cpp_gpu_test(verbose=True):
+    """tests/cpp/build/ring_gpu_test: the C ABI exercised from C++ without Python
+    or torch, checked against the C oracle. Built here (on the CPU) so the GPU
+    run only has to execute it."""
+    cxx = shutil.which("g++") or shutil.which("c++")
+    out_dir = os.path.join(ROOT, "tests", "cpp", "build")
+    os.makedirs(out_dir, exist_ok=True)
+    exe = os.path.join(out_dir, "ring_gpu_test")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    obj = os.path.join(out_dir, "ring_oracle.o")
+    cmds = [
+        ["gcc", "-O2", "-std=gnu11", "-fno-fast-math", "-c", os.path.join(ROOT, "oracle", "ring_oracle.c"), "-o", obj],
+        [cxx, "-O2", "-std=c++17", "-Wall", "-Wextra", "-pthread", "-D__HIP_PLATFORM_AMD__",
+         "-I", os.path.join(rocm, "include"), "-I", os.path.join(ROOT, "include"), "-I", os.path.join(ROOT, "oracle"),
+         "-o", exe, os.path.join(ROOT, "tests", "cpp", "ring_gpu_test.cc"), obj,
+         "-L", LIB_DIR, "-lmpi_collectives", "-lring_hip", "-L", os.path.join(rocm, "lib"), "-lamdhip64",
+         "-Wl,-rpath," + LIB_DIR, "-Wl,-rpath," + os.path.join(rocm, "lib")],
+    ]
+    for cmd in cmds:
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if res.returncode != 0:
+            raise RuntimeError("building the C++ GPU test failed:\n" + res.stdout)
+    return exe
+
+
 def build_all(verbose=True):
-    return [build_ring_hip(verbose), build_plugin(verbose)]
+    return [build_ring_hip(verbose), build_plugin(verbose), build_cpp_gpu_test(verbose)]
 
 
 if __name__ == "__main__":
