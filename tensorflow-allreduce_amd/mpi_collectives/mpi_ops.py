@@ -97,6 +97,7 @@ def _allreduce(tensor, name=None):
     returned tensor holds the sum once every rank has submitted the op and the
     session has run (immediately, in a session with pre-staged peers).
     """
+    tensor = tensor.contiguous()            # the ring works on the flat buffer
     pending = _run('MPIAllreduce', [tensor], name, device="GPU" if tensor.is_cuda else "CPU")
     return _current()[0]._result(pending)
 
@@ -110,6 +111,7 @@ def allgather(tensor, name=None):
     whose result is the host-side `sizes` input of the gather proper.
     """
     session, r = _current()
+    tensor = tensor.contiguous()
     if name is None:
         name = "allgather"
     sizing_name = "{}_sizing".format(name)

@@ -592,3 +592,38 @@ def test_training_example_runs_and_learns(fusion, monkeypatch):
     monkeypatch.setattr("sys.argv", ["train_virtual_ranks.py", "--ranks", "3", "--steps", "30"] + (["--fusion"] if fusion else []))
     last = mod.main()
     assert last < first
+
+
+def test_reference_cpu_case_two_ranks_one_mebi_elements():
+    """The reference's own CPU-runnable case: MPIAllreduce (sum) of one float32
+    tensor of 1,048,576 elements at 2 ranks, values uniform[-1,1] from
+    seed=1234+rank. With two ranks the sum is a single commutative add."""
+    xs = [np.random.default_rng(1234 + r).uniform(-1, 1, 1_048_576).astype(np.float32) for r in range(2)]
+    with mpi.Session(size=2) as session:
+        hs = []
+        for r in range(2):
+            with session.as_rank(r):
+                hs.append(mpi.allreduce(cuda(xs[r]), average=False))
+        outs = session.run(hs)
+    for o in outs:
+        G.assert_same_bits(G.host(o), xs[0] + xs[1], "two-rank allreduce")
+
+
+def test_non_contiguous_and_multi_dimensional_tensors(oracle):
+    n = 3
+    base = [np.random.default_rng(r).standard_normal((40, 50)).astype(np.float32) for r in range(n)]
+    want = oracle.ring_allreduce([np.ascontiguousarray(b.T) for b in base])[0].reshape(50, 40)
+    gathered = np.concatenate([np.ascontiguousarray(b.T) for b in base])
+    with mpi.Session(size=n) as session:
+        hs, gs = [], []
+        for r in range(n):
+            with session.as_rank(r):
+                t = cuda(base[r]).t()                       # a transposed view: not contiguous
+                assert not t.is_contiguous()
+                hs.append(mpi.allreduce(t, average=False))
+                gs.append(mpi.allgather(t))
+        outs, cats = session.run([hs, gs])
+    for o, c in zip(outs, cats):
+        assert list(o.shape) == [50, 40] and list(c.shape) == [150, 40]
+        G.assert_same_bits(G.host(o), want, "transposed input")
+        G.assert_same_bits(G.host(c), gathered, "transposed gather")
