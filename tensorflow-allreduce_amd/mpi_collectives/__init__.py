@@ -83,6 +83,8 @@ class PendingTensor:
             self._session._flush()
             self._session._complete(op)
             op = op.next_op
+        if self._session.stream:
+            ring_abi.stream_synchronize(self._session.stream)     # post-processing (the average) is asynchronous
         if self._error is not None:
             raise self._error
         return self._value
@@ -247,7 +249,9 @@ class Session:
         if any(t.is_cuda for t in inputs):
             # the inputs' producers must have finished before the ring reads them (the
             # reference defers the enqueue with a stream host callback, mpi_ops.cc:1099-1105)
-            torch.cuda.current_stream().synchronize()
+            producers = torch.cuda.current_stream()
+            if not producers.query():
+                producers.synchronize()
         pending = _plugin.PendingOp(self._world, r, op, node_name, inputs, device)
         pending.rank = r
         pending.handle = pending.fail_handle = pending.on_done = pending.next_op = None
@@ -296,6 +300,8 @@ class Session:
             handle._post.append(fn)
         elif handle._error is None:
             handle._value = fn(handle._value)
+            if self.stream:
+                ring_abi.stream_synchronize(self.stream)
 
     def _flush(self):
         """Start a coordinator tick: negotiate and run what was submitted."""
@@ -385,8 +391,8 @@ def _div(session, handle):
 
     def fn(t):
         if t.numel():
+            # asynchronous on the session's stream; run() and wait() drain it
             ring_abi.scale(_TORCH2RING[t.dtype], t.data_ptr(), t.numel(), n, session.stream)
-            ring_abi.stream_synchronize(session.stream)
         return t
 
     session._after(handle, fn)
