@@ -249,7 +249,7 @@ class Session:
         if any(t.is_cuda for t in inputs):
             # the inputs' producers must have finished before the ring reads them (the
             # reference defers the enqueue with a stream host callback, mpi_ops.cc:1099-1105)
-            producers = torch.cuda.current_stream()
+            producers = torch.cuda.current_stream(inputs[0].device)
             if not producers.query():
                 producers.synchronize()
         pending = _plugin.PendingOp(self._world, r, op, node_name, inputs, device)

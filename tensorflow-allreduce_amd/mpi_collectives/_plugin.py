@@ -168,6 +168,39 @@ def infer_shape(op, shape):
     return [None if out[i] < 0 else int(out[i]) for i in range(n)]
 
 
+# One allocator callback serves every op: `user` carries the op's key. (Creating a
+# ctypes callback per op costs more than the rest of the submission.)
+_live_ops = {}
+_next_key = [1]
+_have_gpu = []      # torch.cuda.is_available(), asked once
+
+
+def have_gpu():
+    if not _have_gpu:
+        _have_gpu.append(torch.cuda.is_available())
+    return _have_gpu[0]
+
+
+def _alloc_for_op(user, dtype, ndims, dims, host_memory):
+    # Device outputs go to the GPU. On a machine without one the memory is host
+    # memory and no collective can run on it (the ops have GPU kernels only); the
+    # cross-rank checks, which need no device, still can.
+    op = _live_ops.get(user)
+    try:
+        shape = [dims[i] for i in range(ndims)]
+        on_gpu = not host_memory and have_gpu()
+        t = torch.empty(shape, dtype=DT2TORCH[dtype], device="cuda" if on_gpu else "cpu")
+        op._outputs.append(t)
+        return t.data_ptr() if t.numel() or host_memory else None
+    except Exception as e:            # never let an exception cross the C boundary
+        if op is not None:
+            op._alloc_error = e
+        return None
+
+
+_ALLOC_CB = ALLOC_FN(_alloc_for_op)
+
+
 class PendingOp:
     """One op instance in flight: keeps inputs, outputs and the C context alive
     until the op's done() has run."""
@@ -178,26 +211,16 @@ class PendingOp:
         self._inputs = inputs       # keep-alive
         self._finalizers = []
         self._waited = False
+        self._alloc_error = None
         self.op, self.node_name = op, node_name
-
-        def _alloc(_user, dtype, ndims, dims, host_memory):
-            # Device outputs go to the GPU. On a machine without one the memory is
-            # host memory and no collective can run on it (the ops have GPU kernels
-            # only); the cross-rank checks, which need no device, still can.
-            try:
-                shape = [dims[i] for i in range(ndims)]
-                on_gpu = not host_memory and torch.cuda.is_available()
-                t = torch.empty(shape, dtype=DT2TORCH[dtype], device="cuda" if on_gpu else "cpu")
-                self._outputs.append(t)
-                return t.data_ptr() if t.numel() or host_memory else None
-            except Exception as e:            # never let an exception cross the C boundary
-                self._alloc_error = e
-                return None
-
-        self._alloc_cb = ALLOC_FN(_alloc)
+        self._key = _next_key[0]
+        _next_key[0] += 1
+        _live_ops[self._key] = self
         h = ctypes.c_void_p()
         rc = L.mpic_context_create(world, rank, op.encode(), (node_name or "").encode(), device.encode(),
-                                   self._alloc_cb, None, ctypes.byref(h))
+                                   _ALLOC_CB, self._key, ctypes.byref(h))
+        if rc != OK:
+            _live_ops.pop(self._key, None)
         if rc == NOT_FOUND:
             raise NotFoundError("No OpKernel was registered to support Op '%s' on device %s" % (op, device))
         if rc != OK:
@@ -213,7 +236,8 @@ class PendingOp:
             rc = L.mpic_context_add_input(self._h, dt, t.dim(), dims, t.data_ptr() if t.numel() else None, int(host))
             if rc != OK:
                 raise error_for(rc, "bad input for %s" % op)
-        rc = L.mpic_context_compute(self._h)
+        rc = L.mpic_context_compute(self._h)       # outputs are allocated during this call
+        _live_ops.pop(self._key, None)
         if rc != OK:
             raise error_for(rc, "could not start %s" % op)
 
