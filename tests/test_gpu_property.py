@@ -1,0 +1,126 @@
+"""Property tests on the GPU (hypothesis, derandomised): random ring sizes,
+element counts, element types, buffer misalignments and step-table shapes,
+always compared bit for bit with the CPU oracle."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+from hypothesis import HealthCheck, given, settings, strategies as st
+
+import gpu_util as G
+from gpu_util import ring_abi
+from mpi_collectives import _plugin
+
+pytestmark = pytest.mark.gpu
+
+COMMON = dict(deadline=None, derandomize=True, suppress_health_check=list(HealthCheck))
+DT = {np.dtype(np.float32): _plugin.DT_FLOAT, np.dtype(np.int32): _plugin.DT_INT32,
+      np.dtype(np.int64): _plugin.DT_INT64}
+counts = st.one_of(st.integers(0, 40), st.integers(0, 70_000), st.sampled_from([4095, 4096, 4097, 8191, 65_536]))
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _gpu():
+    G.require_gpu()
+
+
+@settings(max_examples=60, **COMMON)
+@given(n=st.integers(1, 9), count=counts, dtype=st.sampled_from(G.DTYPES), seed=st.integers(0, 2**31),
+       offs=st.lists(st.integers(0, 3), min_size=2, max_size=2))
+def test_all_ranks_ring_equals_oracle(oracle, n, count, dtype, seed, offs):
+    ins = [G.random_array(np.random.default_rng(seed + r), count, dtype, wide=True) for r in range(n)]
+    want = oracle.ring_allreduce_lockstep(ins)
+    L = _plugin.load_library()
+    dins, douts, keep = [], [], []
+    for r in range(n):
+        a, ka = G.dev(ins[r], offs[0])
+        b, kb = G.dev(np.zeros(count, dtype=dtype), offs[1])
+        dins.append(a)
+        douts.append(b)
+        keep += [ka, kb]
+    pin = (ctypes.c_void_p * n)(*[t.data_ptr() if count else None for t in dins])
+    pout = (ctypes.c_void_p * n)(*[t.data_ptr() if count else None for t in douts])
+    rc = L.mpic_ring_allreduce_all_ranks(n, DT[np.dtype(dtype)], pin, pout, count,
+                                         torch.cuda.current_stream().cuda_stream, 1)
+    assert rc == 0, L.mpic_last_error()
+    torch.cuda.synchronize()
+    for r in range(n):
+        G.assert_same_bits(G.host(douts[r]), want[r], "n=%d count=%d %s rank %d" % (n, count, dtype.__name__, r))
+
+
+@settings(max_examples=40, **COMMON)
+@given(n=st.integers(2, 9), count=counts, dtype=st.sampled_from(G.DTYPES), seed=st.integers(0, 2**31),
+       r_pick=st.integers(0, 8), flags=st.sampled_from([0, 1, 3]))
+def test_prestaged_rank_equals_oracle(oracle, n, count, dtype, seed, r_pick, flags):
+    r = r_pick % n
+    ins = [G.random_array(np.random.default_rng(seed + k), count, dtype, wide=True) for k in range(n)]
+    outs, rs, ag = oracle.ring_allreduce(ins, tap=True)
+    sizes, _ = ring_abi.segment_table(count, n)
+    L = _plugin.load_library()
+    din, _k1 = G.dev(ins[r], seed % 4)
+    dout, _k2 = G.dev(np.zeros(count, dtype=dtype), (seed >> 2) % 4)
+    keep = []
+    rs_p = (ctypes.c_void_p * (n - 1))()
+    ag_p = (ctypes.c_void_p * (n - 1))()
+    for i in range(n - 1):
+        a, ka = G.dev(rs[r][i][:sizes[ring_abi.schedule(0, n, r, i)[1]]], (seed + i) % 4)
+        b, kb = G.dev(ag[r][i][:sizes[ring_abi.schedule(1, n, r, i)[1]]], (seed + 2 * i) % 4)
+        keep += [ka, kb]
+        rs_p[i] = a.data_ptr() if a.numel() else None
+        ag_p[i] = b.data_ptr() if b.numel() else None
+    rc = L.mpic_ring_allreduce_prestaged(n, r, DT[np.dtype(dtype)], din.data_ptr() if count else None,
+                                         dout.data_ptr() if count else None, count, rs_p, ag_p,
+                                         torch.cuda.current_stream().cuda_stream, flags)
+    assert rc == 0, L.mpic_last_error()
+    torch.cuda.synchronize()
+    G.assert_same_bits(G.host(dout), outs[r], "n=%d r=%d count=%d flags=%d" % (n, r, count, flags))
+
+
+@settings(max_examples=40, **COMMON)
+@given(rows=st.lists(st.integers(0, 5000), min_size=1, max_size=12), epr=st.sampled_from([1, 3, 17, 256]),
+       dtype=st.sampled_from(G.DTYPES), seed=st.integers(0, 2**31))
+def test_all_ranks_allgather_is_the_concatenation(rows, epr, dtype, seed):
+    n = len(rows)
+    parts = [G.random_array(np.random.default_rng(seed + r), rows[r] * epr, dtype) for r in range(n)]
+    want = np.concatenate(parts) if parts else np.empty(0, dtype=dtype)
+    L = _plugin.load_library()
+    dins = [G.dev(p, r % 4) for r, p in enumerate(parts)]
+    douts = [G.dev(np.zeros(want.size, dtype=dtype), (r + 1) % 4) for r in range(n)]
+    pin = (ctypes.c_void_p * n)(*[d[0].data_ptr() if d[0].numel() else None for d in dins])
+    pout = (ctypes.c_void_p * n)(*[d[0].data_ptr() if want.size else None for d in douts])
+    rows_c = (ctypes.c_size_t * n)(*rows)
+    rc = L.mpic_ring_allgather_all_ranks(n, DT[np.dtype(dtype)], pin, rows_c, epr, pout,
+                                         torch.cuda.current_stream().cuda_stream, 1)
+    assert rc == 0, L.mpic_last_error()
+    torch.cuda.synchronize()
+    for r in range(n):
+        G.assert_same_bits(G.host(douts[r][0]), want, "allgather rows=%r epr=%d rank %d" % (rows, epr, r))
+
+
+@settings(max_examples=30, **COMMON)
+@given(sizes=st.lists(st.integers(0, 9000), min_size=0, max_size=40), dtype=st.sampled_from(G.DTYPES),
+       seed=st.integers(0, 2**31), divisor=st.integers(1, 9))
+def test_fusion_pack_unpack_roundtrip(sizes, dtype, seed, divisor):
+    rng = np.random.default_rng(seed)
+    hosts = [G.random_array(rng, c, dtype, wide=True) for c in sizes]
+    devs = [G.dev(h, int(rng.integers(0, 4))) for h in hosts]
+    plan = ring_abi.FusionPlan([d[0].data_ptr() if c else None for d, c in zip(devs, sizes)], sizes,
+                               G.NP2ABI[np.dtype(dtype)])
+    total = sum(sizes)
+    fused = torch.zeros(total + 4, dtype=G.NP2TORCH[np.dtype(dtype)], device="cuda")
+    plan.pack(fused.data_ptr(), None)
+    torch.cuda.synchronize()
+    want = np.concatenate(hosts) if hosts else np.empty(0, dtype=dtype)
+    G.assert_same_bits(G.host(fused)[:total], want, "pack")
+    for d in devs:
+        d[1].zero_()
+    plan.unpack_scaled(fused.data_ptr(), divisor, None)
+    torch.cuda.synchronize()
+    with np.errstate(all="ignore"):
+        scaled = want / np.float32(divisor) if dtype == np.float32 else want // dtype(divisor)
+    at = 0
+    for d, c in zip(devs, sizes):
+        G.assert_same_bits(G.host(d[0]), scaled[at:at + c].astype(dtype), "unpack_scaled")
+        at += c
+    plan.close()
