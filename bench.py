@@ -359,6 +359,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--workload", default=WORKLOADS[0], choices=WORKLOADS)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="launch option of the kernel library (unroll, blocks_per_cu, nontemporal[_copy|_accumulate|"
+                         "_allgather|_pack|_unpack]), "
+                         "for comparing launch shapes under a profiler")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures the per-rank data path on ONE GPU (the ring's N ranks are virtual); "
@@ -372,6 +376,11 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs the MI355X; no GPU is visible")
     ring_abi.lib()
+    options = {}
+    for item in args.option:
+        name, _, value = item.partition("=")
+        ring_abi.set_option(name, int(value))
+        options[name] = int(value)
     w = make_workload(args.workload)
     torch.cuda.synchronize()
 
@@ -428,7 +437,7 @@ def main():
         "dtype": w.dtype,
         "data": "synthetic",
         "config": {"workload": w.description, "name": w.name, "bytes_per_step": w.bytes_per_step,
-                   "launches_per_step": nph},
+                   "launches_per_step": nph, **({"launch_options": options} if options else {})},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "roofline": {
             "bound": "hbm",
@@ -441,6 +450,9 @@ def main():
             "algorithmic_bytes_per_launch": dom[1],
             "avg_launch_us": round(phase_us[w.dominant], 3),
             "launches_timed": len(samples),
+            "note": "achieved = algorithmic bytes / launch duration; in an allreduce step the accumulate reads the "
+                    "buffer the in->out copy has just written, so part of its reads can come from the last-level "
+                    "cache instead of HBM",
         },
         "phases": {p[0]: {"us": round(t, 3), "GBps": round(p[1] / t / 1e3, 1), "bytes": p[1]}
                    for p, t in zip(w.phases, phase_us)},

@@ -66,10 +66,16 @@ size_t ring_dtype_size(int dtype);
 
 /* Launch-shape knobs for measurement runs (process-wide; not needed for
  * normal use): "unroll" = 16-byte vectors per lane per tile (2, 4, 8),
- * "nontemporal" = non-temporal stores (0, 1), "blocks_per_cu" = 0 for one
- * workgroup per tile, k > 0 for a persistent grid of CUs x k workgroups that
- * stride over the tiles. No counterpart in the reference, whose launch shape
- * is the constant <<<32, 256>>> (ring.cu.cc:64). */
+ * "blocks_per_cu" = 0 for one workgroup per tile, k > 0 for a persistent grid
+ * of CUs x k workgroups that stride over the tiles. Cache policy per kind of
+ * launch: "nontemporal_copy" (ring_copy_bytes), "nontemporal_accumulate"
+ * (accumulates, reduce-scatter tables, row tables, scale),
+ * "nontemporal_allgather" (copy tables), "nontemporal_pack",
+ * "nontemporal_unpack"; value bit 0 = non-temporal stores, bit 1 =
+ * non-temporal loads, -1 = the default (3, except ordinary stores for the copy
+ * and the pack, whose output the next kernel reads, and loads by size for the
+ * copy). "nontemporal" sets all five. No counterpart in the reference, whose
+ * launch shape is the constant <<<32, 256>>> (ring.cu.cc:64). */
 int ring_set_option(const char* name, int value);
 
 /* Timing of single launches, for benchmarks (no counterpart in the

@@ -143,17 +143,22 @@ struct RowTable {
   Row row[kMaxRows];
 };
 
-template <typename T, bool NT>
+// NT: bit 0 = non-temporal stores, bit 1 = non-temporal loads (3, both, is the
+// default: every byte is touched once).
+template <typename T, int NT>
 __device__ __forceinline__ void store_vec(typename VecOf<T>::type* p, typename VecOf<T>::type v) {
-  if (NT) __builtin_nontemporal_store(v, p); else *p = v;
+  if (NT & 1) __builtin_nontemporal_store(v, p); else *p = v;
 }
+// A macro, not a function template: the operand's type carries a reduced
+// alignment (element-aligned 16-byte loads) that template deduction would drop.
+#define RING_LOAD_VEC(NT, p) (((NT) & 2) ? __builtin_nontemporal_load(p) : *(p))
 
 // One workgroup-tile of a row: vectors [v0, v0 + 256*UNROLL) of the aligned
 // body, plus the row's scalar head (tile 0) and tail (last tile). dst is
 // brought to 16-byte alignment by the head; a and b are read with
 // element-aligned 16-byte loads. a == dst (divide) and b == dst (add) are
 // allowed: every element is read before it is written, by the same lane.
-template <typename T, int OP, int UNROLL, bool NT>
+template <typename T, int OP, int UNROLL, int NT>
 __device__ __forceinline__ void row_tile(T* dst, const T* a, const T* b, uint64_t count, uint32_t tile,
                                          uint32_t tiles_in_row, int n) {
   typedef typename VecOf<T>::type V;
@@ -180,10 +185,10 @@ __device__ __forceinline__ void row_tile(T* dst, const T* a, const T* b, uint64_
   if (static_cast<uint64_t>(tile + 1) * kTileVecs <= nvec) {
     V x[UNROLL], y[UNROLL];
 #pragma unroll
-    for (int j = 0; j < UNROLL; j++) x[j] = __builtin_nontemporal_load(&av[v0 + j * kBlock]);
+    for (int j = 0; j < UNROLL; j++) x[j] = RING_LOAD_VEC(NT, &av[v0 + j * kBlock]);
     if (OP == kOpAdd) {
 #pragma unroll
-      for (int j = 0; j < UNROLL; j++) y[j] = __builtin_nontemporal_load(&bv[v0 + j * kBlock]);
+      for (int j = 0; j < UNROLL; j++) y[j] = RING_LOAD_VEC(NT, &bv[v0 + j * kBlock]);
     }
 #pragma unroll
     for (int j = 0; j < UNROLL; j++) x[j] = apply_vec<T, OP>(x[j], y[j], n);
@@ -194,16 +199,16 @@ __device__ __forceinline__ void row_tile(T* dst, const T* a, const T* b, uint64_
     for (int j = 0; j < UNROLL; j++) {
       const uint64_t v = v0 + j * kBlock;
       if (v < nvec) {
-        V x = __builtin_nontemporal_load(&av[v]);
+        V x = RING_LOAD_VEC(NT, &av[v]);
         V y = x;
-        if (OP == kOpAdd) y = __builtin_nontemporal_load(&bv[v]);
+        if (OP == kOpAdd) y = RING_LOAD_VEC(NT, &bv[v]);
         store_vec<T, NT>(&dv[v], apply_vec<T, OP>(x, y, n));
       }
     }
   }
 }
 
-template <typename T, int MODE, int UNROLL, bool NT>
+template <typename T, int MODE, int UNROLL, int NT>
 __device__ __forceinline__ void run_row(const Row& r, uint32_t tile, uint32_t tiles, int divisor) {
   T* dst = static_cast<T*>(r.dst);
   const T* a = static_cast<const T*>(r.a);
@@ -213,7 +218,7 @@ __device__ __forceinline__ void run_row(const Row& r, uint32_t tile, uint32_t ti
   else row_tile<T, kOpCopy, UNROLL, NT>(dst, a, nullptr, r.count, tile, tiles, 0);
 }
 
-template <typename T, int MODE, int UNROLL, bool NT>
+template <typename T, int MODE, int UNROLL, int NT>
 __global__ void __launch_bounds__(kBlock) rows_kernel(const RowTable tab) {
   if (tab.uniform_tiles) {
     const Row r = tab.row[blockIdx.y];  // one scalar load, no search
@@ -255,7 +260,7 @@ __global__ void __launch_bounds__(kBlock) bytes_kernel(uint8_t* __restrict__ dst
 constexpr uint32_t kFusionTileVecs = 1024;
 constexpr uint32_t kFusionLdsCap = 512;  // tensors of one tile staged in LDS
 
-template <typename T, bool PACK, bool NT, bool DIV>
+template <typename T, bool PACK, int NT, bool DIV>
 __global__ void __launch_bounds__(kBlock)
 fusion_kernel(T* __restrict__ fused, const uint64_t* __restrict__ offsets, T* const* __restrict__ ptrs,
               const uint32_t* __restrict__ tile_first, const uint32_t* __restrict__ tile_last,
@@ -321,9 +326,20 @@ fusion_kernel(T* __restrict__ fused, const uint64_t* __restrict__ offsets, T* co
 
 // ---- launch configuration -----------------------------------------------------
 
+constexpr uint64_t kCacheResidentBytes = 128ull << 20;
+
+enum Role { kRoleCopy, kRoleAccumulate, kRoleAllgather, kRolePack, kRoleUnpack, kRoles };
+
 struct Tuning {
   int unroll = 4;          // 16-byte vectors per lane per tile: 2, 4 or 8
-  int nontemporal = 1;     // non-temporal stores
+  // Cache policy per role; bit 0: non-temporal stores, bit 1: non-temporal
+  // loads, -1: chosen by size. Accumulates, allgather copies and the unpack
+  // touch their bytes once. The in->out copy and the pack write the buffer the
+  // reduce-scatter reads next, so their stores stay ordinary (measured 2-5 %
+  // of a step on tensors up to 128 MiB, which the last-level cache can hold);
+  // the copy's loads turn non-temporal above that size, where ordinary ones
+  // only evict what the next kernel wants.
+  int nt[kRoles] = {-1, 3, 3, 2, 3};
   int blocks_per_cu = 0;   // 0: one workgroup per tile; >0: persistent grid of CUs x this
 };
 Tuning g_tuning;
@@ -350,14 +366,21 @@ int device_info(DeviceInfo* out) {
 }
 
 template <typename T, int MODE>
-int launch_rows_typed(const RowTable& tab, dim3 grid, hipStream_t stream) {
-  const bool nt = g_tuning.nontemporal != 0;
+int launch_rows_typed(const RowTable& tab, dim3 grid, hipStream_t stream, int nt) {
 #define RING_LAUNCH(U, N) launch(rows_kernel<T, MODE, U, N>, grid, dim3(kBlock), stream, tab)
-  switch (g_tuning.unroll) {
-    case 2: if (nt) RING_LAUNCH(2, true); else RING_LAUNCH(2, false); break;
-    case 8: if (nt) RING_LAUNCH(8, true); else RING_LAUNCH(8, false); break;
-    default: if (nt) RING_LAUNCH(4, true); else RING_LAUNCH(4, false); break;
+#define RING_LAUNCH_NT(U)                       \
+  switch (nt & 3) {                             \
+    case 0: RING_LAUNCH(U, 0); break;           \
+    case 1: RING_LAUNCH(U, 1); break;           \
+    case 2: RING_LAUNCH(U, 2); break;           \
+    default: RING_LAUNCH(U, 3); break;          \
   }
+  switch (g_tuning.unroll) {
+    case 2: RING_LAUNCH_NT(2); break;
+    case 8: RING_LAUNCH_NT(8); break;
+    default: RING_LAUNCH_NT(4); break;
+  }
+#undef RING_LAUNCH_NT
 #undef RING_LAUNCH
   RING_HIP(hipGetLastError());
   return RING_OK;
@@ -375,7 +398,13 @@ struct HostRow {
 // divisor > 0: every row is divided in place / out of place by it (kDiv) and
 // the element type is signed.
 int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, hipStream_t stream,
-                int divisor = 0) {
+                Role role, int divisor = 0) {
+  int nt = g_tuning.nt[role];
+  if (nt < 0) {
+    uint64_t bytes = 0;
+    for (size_t k = 0; k < n_rows; k++) bytes += rows[k].count * esz;
+    nt = bytes <= kCacheResidentBytes ? 0 : 2;
+  }
   const int unroll = (g_tuning.unroll == 2 || g_tuning.unroll == 8) ? g_tuning.unroll : 4;
   const uint64_t tile_vecs = static_cast<uint64_t>(kBlock) * unroll;
   const uint64_t vec = 16 / esz;
@@ -431,18 +460,18 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
     }
     int rc;
     if (divisor > 0) {
-      rc = esz == 8 ? launch_rows_typed<int64_t, kDiv>(tab, grid, stream)
-           : is_float ? launch_rows_typed<float, kDiv>(tab, grid, stream)
-                      : launch_rows_typed<int32_t, kDiv>(tab, grid, stream);
+      rc = esz == 8 ? launch_rows_typed<int64_t, kDiv>(tab, grid, stream, nt)
+           : is_float ? launch_rows_typed<float, kDiv>(tab, grid, stream, nt)
+                      : launch_rows_typed<int32_t, kDiv>(tab, grid, stream, nt);
     } else if (!any_add) {
-      rc = esz == 8 ? launch_rows_typed<uint64_t, kCopy>(tab, grid, stream)
-                    : launch_rows_typed<uint32_t, kCopy>(tab, grid, stream);
+      rc = esz == 8 ? launch_rows_typed<uint64_t, kCopy>(tab, grid, stream, nt)
+                    : launch_rows_typed<uint32_t, kCopy>(tab, grid, stream, nt);
     } else if (esz == 8) {
-      rc = launch_rows_typed<uint64_t, kAdd>(tab, grid, stream);
+      rc = launch_rows_typed<uint64_t, kAdd>(tab, grid, stream, nt);
     } else if (is_float) {
-      rc = launch_rows_typed<float, kAdd>(tab, grid, stream);
+      rc = launch_rows_typed<float, kAdd>(tab, grid, stream, nt);
     } else {
-      rc = launch_rows_typed<uint32_t, kAdd>(tab, grid, stream);
+      rc = launch_rows_typed<uint32_t, kAdd>(tab, grid, stream, nt);
     }
     if (rc != RING_OK) return rc;
   }
@@ -474,7 +503,8 @@ int steps_common(const void* input, void* buffer, const ring_step* steps, int n_
       return RING_ERR_ARGUMENT;
     rows.push_back(HostRow{d, steps[i].src, kind == kStepCopy ? nullptr : local, steps[i].count});
   }
-  return launch_rows(rows.data(), rows.size(), esz, dtype == RING_F32, static_cast<hipStream_t>(stream));
+  return launch_rows(rows.data(), rows.size(), esz, dtype == RING_F32, static_cast<hipStream_t>(stream),
+                     kind == kStepCopy ? kRoleAllgather : kRoleAccumulate);
 }
 
 }  // namespace
@@ -507,16 +537,20 @@ int launch_fusion(const ring_fusion_plan* p, void* fused, hipStream_t stream, in
     const uint64_t cap = static_cast<uint64_t>(info.cus) * g_tuning.blocks_per_cu;
     if (grid > cap) grid = static_cast<uint32_t>(cap);
   }
-  if (g_tuning.nontemporal)
-    launch(fusion_kernel<T, PACK, true, DIV>, dim3(grid), dim3(kBlock), stream, static_cast<T*>(fused),
-           static_cast<const uint64_t*>(p->d_offsets), reinterpret_cast<T* const*>(p->d_ptrs),
-           static_cast<const uint32_t*>(p->d_tile_first), static_cast<const uint32_t*>(p->d_tile_last), p->ntiles,
-           p->total, divisor);
-  else
-    launch(fusion_kernel<T, PACK, false, DIV>, dim3(grid), dim3(kBlock), stream, static_cast<T*>(fused),
-           static_cast<const uint64_t*>(p->d_offsets), reinterpret_cast<T* const*>(p->d_ptrs),
-           static_cast<const uint32_t*>(p->d_tile_first), static_cast<const uint32_t*>(p->d_tile_last), p->ntiles,
-           p->total, divisor);
+#define RING_FUSION(N)                                                                                   \
+  launch(fusion_kernel<T, PACK, N, DIV>, dim3(grid), dim3(kBlock), stream, static_cast<T*>(fused),       \
+         static_cast<const uint64_t*>(p->d_offsets), reinterpret_cast<T* const*>(p->d_ptrs),             \
+         static_cast<const uint32_t*>(p->d_tile_first), static_cast<const uint32_t*>(p->d_tile_last),    \
+         p->ntiles, p->total, divisor)
+  int nt = g_tuning.nt[PACK ? kRolePack : kRoleUnpack];
+  if (nt < 0) nt = 2;
+  switch (nt & 3) {
+    case 0: RING_FUSION(0); break;
+    case 1: RING_FUSION(1); break;
+    case 2: RING_FUSION(2); break;
+    default: RING_FUSION(3); break;
+  }
+#undef RING_FUSION
   RING_HIP(hipGetLastError());
   return RING_OK;
 }
@@ -562,15 +596,26 @@ int ring_last_hip_error(void) { return g_last_hip_error; }
 size_t ring_dtype_size(int dtype) { return dtype_size(dtype); }
 
 // Tuning knobs for measurement runs; not part of the drop-in surface.
-// name: "unroll" (2|4|8), "nontemporal" (0|1), "blocks_per_cu" (0 = one
-// workgroup per tile).
+// name: "unroll" (2|4|8), "blocks_per_cu" (0 = one workgroup per tile),
+// "nontemporal" (bit 0 stores, bit 1 loads; sets every role) and
+// "nontemporal_copy" / "_accumulate" / "_allgather" / "_pack" / "_unpack".
 int ring_set_option(const char* name, int value) {
   if (!name) return RING_ERR_ARGUMENT;
   if (!strcmp(name, "unroll")) {
     if (value != 2 && value != 4 && value != 8) return RING_ERR_ARGUMENT;
     g_tuning.unroll = value;
-  } else if (!strcmp(name, "nontemporal")) {
-    g_tuning.nontemporal = value ? 1 : 0;
+  } else if (!strncmp(name, "nontemporal", 11)) {
+    static const char* const kSuffix[kRoles] = {"_copy", "_accumulate", "_allgather", "_pack", "_unpack"};
+    if (value < -1 || value > 3) return RING_ERR_ARGUMENT;
+    const Tuning defaults;
+    bool known = name[11] == 0;
+    for (int r = 0; r < kRoles; r++) {
+      if (name[11] == 0 || !strcmp(name + 11, kSuffix[r])) {
+        g_tuning.nt[r] = value < 0 ? defaults.nt[r] : value;  // -1: back to the default
+        known = true;
+      }
+    }
+    if (!known) return RING_ERR_ARGUMENT;
   } else if (!strcmp(name, "blocks_per_cu")) {
     if (value < 0 || value > 64) return RING_ERR_ARGUMENT;
     g_tuning.blocks_per_cu = value;
@@ -688,7 +733,7 @@ int ring_copy_bytes(void* dst, const void* src, size_t bytes, void* stream) {
   const uintptr_t all = reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src) | bytes;
   if ((all & 3u) == 0) {
     HostRow row{dst, src, nullptr, bytes / 4};
-    return launch_rows(&row, 1, 4, false, s);
+    return launch_rows(&row, 1, 4, false, s, kRoleCopy);
   }
   uint64_t blocks = (bytes + kBlock - 1) / kBlock;
   if (blocks > 65536) blocks = 65536;
@@ -707,7 +752,7 @@ int ring_accumulate(int dtype, void* dst, const void* src, size_t count, void* s
   if ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & (esz - 1))
     return RING_ERR_ARGUMENT;
   HostRow row{dst, src, dst, count};
-  return launch_rows(&row, 1, esz, dtype == RING_F32, static_cast<hipStream_t>(stream));
+  return launch_rows(&row, 1, esz, dtype == RING_F32, static_cast<hipStream_t>(stream), kRoleAccumulate);
 }
 
 int ring_accumulate_f32(float* dst, const float* src, size_t count, void* stream) {
@@ -746,7 +791,8 @@ int ring_apply_rows(const ring_row* rows, int n_rows, int dtype, void* stream) {
       return RING_ERR_ARGUMENT;
     host.push_back(HostRow{rows[i].dst, rows[i].a, rows[i].b, rows[i].count});
   }
-  return launch_rows(host.data(), host.size(), esz, dtype == RING_F32, static_cast<hipStream_t>(stream));
+  return launch_rows(host.data(), host.size(), esz, dtype == RING_F32, static_cast<hipStream_t>(stream),
+                     kRoleAccumulate);
 }
 
 int ring_allgather_steps(void* buffer, const ring_step* steps, int n_steps, int dtype, void* stream) {
@@ -759,7 +805,8 @@ int ring_scale(int dtype, void* data, size_t count, int divisor, void* stream) {
   if (count == 0) return RING_OK;
   if (!data || (reinterpret_cast<uintptr_t>(data) & (dtype_size(dtype) - 1))) return RING_ERR_ARGUMENT;
   HostRow row{data, data, nullptr, count};
-  return launch_rows(&row, 1, dtype_size(dtype), dtype == RING_F32, static_cast<hipStream_t>(stream), divisor);
+  return launch_rows(&row, 1, dtype_size(dtype), dtype == RING_F32, static_cast<hipStream_t>(stream),
+                     kRoleAccumulate, divisor);
 }
 
 // ---- fusion ------------------------------------------------------------------------

@@ -19,7 +19,7 @@ COUNTS = [0, 1, 2, 3, 4, 5, 7, 8, 1023, 1024, 1025, 4096, 4097, 3 * 4096 + 7, 26
 def _gpu():
     G.require_gpu()
     yield
-    for k, v in (("unroll", 4), ("nontemporal", 1), ("blocks_per_cu", 0)):
+    for k, v in (("unroll", 4), ("nontemporal", -1), ("blocks_per_cu", 0)):
         ring_abi.set_option(k, v)
 
 
@@ -156,6 +156,7 @@ def test_step_tables_match_oracle(oracle, dtype, n_rows):
 
 
 @pytest.mark.parametrize("opt", [("unroll", 2), ("unroll", 8), ("nontemporal", 0),
+                                 ("nontemporal", 1), ("nontemporal", 2), ("nontemporal", 3),
                                  ("blocks_per_cu", 1), ("blocks_per_cu", 8)])
 def test_launch_options_do_not_change_results(oracle, opt):
     ring_abi.set_option(*opt)
@@ -173,8 +174,9 @@ def test_launch_options_do_not_change_results(oracle, opt):
                 G.sync()
                 G.assert_same_bits(G.host(da), oracle.accumulate(a.copy(), b), str(opt))
                 G.assert_same_bits(G.host(dc), b, str(opt))
+            _fusion_roundtrip([5, 0, 4096, 1, 0, 3, 8191, 2, 70_001], dtype, rng)
     finally:
-        for k, v in (("unroll", 4), ("nontemporal", 1), ("blocks_per_cu", 0)):
+        for k, v in (("unroll", 4), ("nontemporal", -1), ("blocks_per_cu", 0)):
             ring_abi.set_option(k, v)
 
 
