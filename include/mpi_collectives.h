@@ -116,6 +116,17 @@ int mpic_context_create(mpic_world* world, int rank, const char* op, const char*
                         const char* device, mpic_alloc_fn alloc, void* user, mpic_context** ctx);
 int mpic_context_add_input(mpic_context* ctx, int dtype, int ndims, const int64_t* dims,
                            const void* data, int host_memory);
+/* Fuses the graph's tf.div(output, divisor) consumer into this node: the
+ * reference's allreduce(average=True) is MPIAllreduce followed by
+ * tf.div(summed_tensor, size()) (__init__.py:160-164; :153-157 divides the
+ * gathered values of an IndexedSlices). With a divisor > 0 an MPIAllreduce /
+ * MPIAllgather node delivers exactly that quotient (true division for float32,
+ * floor division for the integers) without a pass of its own: the divide rides
+ * on the last accumulate of each segment (on the unpack for fused tensors, on
+ * the own-slice copy of an allgather). Every rank must ask for the same
+ * divisor. In a world with pre-staged peers the allgather-phase segments are
+ * what a peer would send: already divided. Call before mpic_context_compute. */
+int mpic_context_set_divisor(mpic_context* ctx, int divisor);
 /* Runs Compute / ComputeAsync on the calling thread and returns. */
 int mpic_context_compute(mpic_context* ctx);
 /* Blocks until the op's done() ran; returns its status code. */
@@ -129,7 +140,8 @@ int mpic_context_destroy(mpic_context* ctx);
 /* ---- the ring driver, callable without the op layer ------------------------
  * RingAllreduce (ring.h:136-228) for rank r of n whose incoming segments are
  * already in device memory. `flags`: bit 0 = batched, bit 1 = fuse the
- * in->out copy. Asynchronous on `stream`. `dtype` is an mpic_dtype. */
+ * in->out copy, bits 8-30 = divisor (0: none; see mpic_context_set_divisor).
+ * Asynchronous on `stream`. `dtype` is an mpic_dtype. */
 int mpic_ring_allreduce_prestaged(int n, int r, int dtype, const void* input, void* output,
                                   size_t count, const void* const* rs_segments,
                                   const void* const* ag_segments, void* stream, int flags);

@@ -192,6 +192,18 @@ typedef struct ring_row {
   uint64_t count; /* elements */
 } ring_row;
 int ring_apply_rows(const ring_row* rows, int n_rows, int dtype, void* stream);
+/* The same launch with the divide of allreduce(average=True) folded in
+ * (the reference divides in a separate graph op after the collective,
+ * __init__.py:160-164 `tf.div(summed_tensor, size())`): rows with divide[k] != 0
+ * (all rows when `divide` is NULL) store (b[i] + a[i]) / divisor, or
+ * a[i] / divisor without b, with ring_scale's division (true division for
+ * float32, floor division for the integers) applied to the already rounded
+ * sum, so the result equals the two passes done one after the other. A ring
+ * divides once, where a segment's sum becomes complete: at the last
+ * reduce-scatter step of the rank that owns it. divisor 0 = ring_apply_rows.
+ * `rows` and `divide` are HOST arrays. */
+int ring_apply_rows_avg(const ring_row* rows, int n_rows, const unsigned char* divide, int divisor,
+                        int dtype, void* stream);
 
 /* ---- tensor fusion (no counterpart in the reference, which issues one
  * MPIAllreduce per gradient, __init__.py:195-205): k tensors are packed back

@@ -52,6 +52,7 @@ struct CollectiveOpRecord {
   size_t temp_elements = 0;       // what the reference's temp tensor would hold (mpi_ops.cc:1073-1077)
   Tensor* out_t = nullptr;
   bool on_gpu = false;
+  int divisor = 0;                // > 0: deliver tf.div(result, divisor) (a fused consumer)
   CommunicationDoneCallback callback;
 };
 
@@ -232,11 +233,19 @@ void PerformCollectiveOp(mpic_world* w, const MPIResponse& response) {
   const CollectiveOpRecord& first = records.begin()->second;
   const DataType dtype = first.in_t->dtype();
   const int n = w->size;
-  bool on_gpu = true;
-  for (auto& kv : records) on_gpu = on_gpu && kv.second.on_gpu;
+  bool on_gpu = true, same_divisor = true;
+  for (auto& kv : records) {
+    on_gpu = on_gpu && kv.second.on_gpu;
+    same_divisor = same_divisor && kv.second.divisor == first.divisor;
+  }
+  RingOptions ring = opt.ring;
+  ring.divisor = first.divisor;
 
   if (response.response_type == MPIResponse::ERROR) {
     status = errors::FailedPrecondition(response.error_message);
+  } else if (!same_divisor) {
+    status = errors::FailedPrecondition("Mismatched fused divisors: ranks asked for different divisions of " +
+                                        response.tensor_name + ".");
   } else if (dtype != DT_FLOAT && dtype != DT_INT32 && dtype != DT_INT64) {
     status = errors::Unknown(response.response_type == MPIResponse::ALLGATHER
                                  ? "Invalid tensor type for MPI allgather."
@@ -255,12 +264,12 @@ void PerformCollectiveOp(mpic_world* w, const MPIResponse& response) {
     } else if (response.response_type == MPIResponse::ALLREDUCE) {
       status = RingAllreducePrestaged(n, r, dtype, first.in_t->data(), first.out_t->data(),
                                       static_cast<size_t>(first.in_t->NumElements()), peers.rs.data(),
-                                      peers.ag.data(), w->stream, opt.ring);
+                                      peers.ag.data(), w->stream, ring);
     } else {
       size_t epr = 1;
       for (int i = 1; i < first.in_t->shape().dims(); i++) epr *= static_cast<size_t>(first.in_t->dim_size(i));
       status = RingAllgatherPrestaged(n, r, dtype, first.in_t->data(), first.sizes_vec, epr, first.out_t->data(),
-                                      peers.ag.data(), w->stream, opt.ring);
+                                      peers.ag.data(), w->stream, ring);
     }
   } else {
     std::vector<const void*> ins(static_cast<size_t>(n));
@@ -271,7 +280,7 @@ void PerformCollectiveOp(mpic_world* w, const MPIResponse& response) {
     }
     if (response.response_type == MPIResponse::ALLREDUCE) {
       status = RingAllreduceAllRanks(n, dtype, ins.data(), outs.data(),
-                                     static_cast<size_t>(first.in_t->NumElements()), w->stream, opt.ring);
+                                     static_cast<size_t>(first.in_t->NumElements()), w->stream, ring);
     } else {
       size_t epr = 1;
       for (int i = 1; i < first.in_t->shape().dims(); i++) epr *= static_cast<size_t>(first.in_t->dim_size(i));
@@ -286,7 +295,7 @@ void PerformCollectiveOp(mpic_world* w, const MPIResponse& response) {
       }
       if (status.ok())
         status = RingAllgatherAllRanks(n, dtype, ins.data(), first.sizes_vec, epr, outs.data(), w->stream,
-                                       opt.ring);
+                                       ring);
     }
   }
 
@@ -355,6 +364,20 @@ void PerformFusedAllreduce(mpic_world* w, const std::vector<std::string>& names,
     if (!plan || ring_fusion_pack(plan, bufs[static_cast<size_t>(r)], w->stream) != RING_OK)
       status = errors::Unknown("MPI operation failed unexpectedly.");
   }
+  // fused tf.div consumers: when the whole group asks for the same division it
+  // rides on the unpack, otherwise each tensor that asks for one is divided
+  // after the unpack
+  int divisor = records[0].begin()->second.divisor;
+  bool uniform = true;
+  for (auto& rec : records) {
+    for (auto& kv : rec) {
+      if (kv.second.divisor != rec.begin()->second.divisor)
+        status = errors::FailedPrecondition("Mismatched fused divisors: ranks asked for different divisions of " +
+                                            kv.second.name + ".");
+    }
+    uniform = uniform && rec.begin()->second.divisor == divisor;
+  }
+  if (!uniform) divisor = 0;
   if (status.ok()) {
     std::vector<const void*> ins(bufs.begin(), bufs.end());
     status = RingAllreduceAllRanks(n, dtype, ins.data(), bufs.data(), total, w->stream, opt.ring);
@@ -363,8 +386,16 @@ void PerformFusedAllreduce(mpic_world* w, const std::vector<std::string>& names,
     std::vector<const void*> outs;
     for (auto& rec : records) outs.push_back(rec.at(r).out_t->data());
     ring_fusion_plan* plan = FusionPlanFor(w, outs, counts, code);
-    if (!plan || ring_fusion_unpack(plan, bufs[static_cast<size_t>(r)], w->stream) != RING_OK)
+    if (!plan || (divisor > 0 ? ring_fusion_unpack_scaled(plan, bufs[static_cast<size_t>(r)], divisor, w->stream)
+                              : ring_fusion_unpack(plan, bufs[static_cast<size_t>(r)], w->stream)) != RING_OK)
       status = errors::Unknown("MPI operation failed unexpectedly.");
+    for (auto& rec : records) {
+      const CollectiveOpRecord& op = rec.at(r);
+      if (uniform || op.divisor <= 0 || !status.ok()) continue;
+      if (ring_scale(code, op.out_t->data(), static_cast<size_t>(op.out_t->NumElements()), op.divisor, w->stream) !=
+          RING_OK)
+        status = errors::Unknown("MPI operation failed unexpectedly.");
+    }
   }
   if (status.ok() && opt.sync_on_done && ring_stream_synchronize(w->stream) != RING_OK)
     status = errors::Unknown("MPI operation failed unexpectedly.");
@@ -657,6 +688,7 @@ class MPIAllreduceOp : public AsyncOpKernel {
     record.out_t = output_tensor;
     record.on_gpu = IsGPUDevice<Device>() && !input_tensor->host_memory();
     record.temp_elements = ring_temp_elements(static_cast<size_t>(input_tensor->NumElements()), world->size);
+    record.divisor = context->fused_divisor();
     record.callback = [done, context](const Status& status) {
       context->SetStatus(status);
       done();
@@ -743,6 +775,7 @@ class MPIAllgatherOp : public AsyncOpKernel {
     OP_REQUIRES_OK_ASYNC(context,
                          context->allocate_output(0, output_shape, input_tensor->dtype(), false, &output_tensor), done);
     record.out_t = output_tensor;
+    record.divisor = context->fused_divisor();
     record.callback = [done, context](const Status& status) {
       context->SetStatus(status);
       done();
@@ -943,6 +976,12 @@ int mpic_context_add_input(mpic_context* c, int dtype, int ndims, const int64_t*
   std::vector<int64_t> d(dims, dims + ndims);
   c->ctx->AddInput(mpic::Tensor(static_cast<mpic::DataType>(dtype), mpic::TensorShape(d), const_cast<void*>(data),
                                 host_memory != 0));
+  return MPIC_OK;
+}
+
+int mpic_context_set_divisor(mpic_context* c, int divisor) {
+  if (!c || c->started || divisor < 0) return MPIC_INVALID_ARGUMENT;
+  c->ctx->set_fused_divisor(divisor);
   return MPIC_OK;
 }
 

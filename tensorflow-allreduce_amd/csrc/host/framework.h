@@ -215,7 +215,15 @@ class OpKernelContext {
   int rank() const { return rank_; }
   bool on_gpu() const { return on_gpu_; }
 
+  // Set by an executor that has fused the graph's tf.div(output, n) consumer
+  // into this node (the reference's allreduce(average=True) is MPIAllreduce
+  // followed by tf.div, __init__.py:160-164): the kernel then delivers
+  // output / n. 0: no consumer fused.
+  void set_fused_divisor(int n) { fused_divisor_ = n; }
+  int fused_divisor() const { return fused_divisor_; }
+
  private:
+  int fused_divisor_ = 0;
   void* world_;
   int rank_;
   bool on_gpu_;

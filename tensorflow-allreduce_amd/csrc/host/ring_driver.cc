@@ -58,10 +58,24 @@ Status RingAllreducePrestaged(int n, int r, DataType dt, const void* input, void
   std::vector<size_t> sizes(static_cast<size_t>(n)), starts(static_cast<size_t>(n));
   RING_RETURN_IF_ERROR(ring_segment_table(count, n, sizes.data(), starts.data()), "ring_segment_table");
 
-  const bool fuse = opts.fuse_copy && opts.batched && input != output && n > 1;
+  const int divisor = opts.divisor;
+  if (divisor < 0) return errors::InvalidArgument("negative divisor");
+  if (n == 1) {  // ring.h:146-148 is all there is; a lone rank owns every element
+    if (divisor > 0) {
+      ring_row row{output, input, nullptr, count};
+      RING_RETURN_IF_ERROR(ring_apply_rows_avg(&row, 1, nullptr, divisor, code, stream), "ring_apply_rows_avg");
+    } else if (input != output) {
+      RING_RETURN_IF_ERROR(ring_copy_bytes(output, input, count * esz, stream), "ring_copy_bytes");
+    }
+    return Status::OK();
+  }
+  const bool fuse = opts.fuse_copy && opts.batched && input != output;
   if (!fuse && input != output)  // ring.h:146-148
     RING_RETURN_IF_ERROR(ring_copy_bytes(output, input, count * esz, stream), "ring_copy_bytes");
-  if (n == 1) return Status::OK();
+  // the segment whose sum completes at the last step (n-2) is the one this rank
+  // owns and sends first in the allgather: the only one it divides
+  std::vector<unsigned char> divide(static_cast<size_t>(n), 0);
+  divide[static_cast<size_t>(n - 2)] = 1;
 
   // ring.h:183-205: step i receives segment (r-i-1) and adds it into the buffer
   if (fuse) {
@@ -73,8 +87,18 @@ Status RingAllreducePrestaged(int n, int r, DataType dt, const void* input, void
     // segment r is only ever sent, never accumulated: plain copy
     const size_t own = static_cast<size_t>(r);
     rows.push_back(ring_row{at(output, starts[own], esz), at(input, starts[own], esz), nullptr, sizes[own]});
-    RING_RETURN_IF_ERROR(ring_apply_rows(rows.data(), static_cast<int>(rows.size()), code, stream),
-                         "ring_apply_rows");
+    RING_RETURN_IF_ERROR(ring_apply_rows_avg(rows.data(), static_cast<int>(rows.size()), divide.data(), divisor,
+                                             code, stream),
+                         "ring_apply_rows_avg");
+  } else if (opts.batched && divisor > 0) {
+    std::vector<ring_row> rows;
+    for (int i = 0; i < n - 1; i++) {
+      const size_t seg = static_cast<size_t>(Seg(RING_PHASE_REDUCE_SCATTER, n, r, i, true));
+      char* dst = at(output, starts[seg], esz);
+      rows.push_back(ring_row{dst, rs_recv[i], dst, sizes[seg]});
+    }
+    RING_RETURN_IF_ERROR(ring_apply_rows_avg(rows.data(), n - 1, divide.data(), divisor, code, stream),
+                         "ring_apply_rows_avg");
   } else if (opts.batched) {
     std::vector<ring_step> steps;
     for (int i = 0; i < n - 1; i++) {
@@ -86,8 +110,14 @@ Status RingAllreducePrestaged(int n, int r, DataType dt, const void* input, void
   } else {
     for (int i = 0; i < n - 1; i++) {
       const size_t seg = static_cast<size_t>(Seg(RING_PHASE_REDUCE_SCATTER, n, r, i, true));
-      RING_RETURN_IF_ERROR(ring_accumulate(code, at(output, starts[seg], esz), rs_recv[i], sizes[seg], stream),
-                           "ring_accumulate");
+      if (divisor > 0 && i == n - 2) {
+        char* dst = at(output, starts[seg], esz);
+        ring_row row{dst, rs_recv[i], dst, sizes[seg]};
+        RING_RETURN_IF_ERROR(ring_apply_rows_avg(&row, 1, nullptr, divisor, code, stream), "ring_apply_rows_avg");
+      } else {
+        RING_RETURN_IF_ERROR(ring_accumulate(code, at(output, starts[seg], esz), rs_recv[i], sizes[seg], stream),
+                             "ring_accumulate");
+      }
     }
   }
 
@@ -128,7 +158,20 @@ Status RingAllgatherPrestaged(int n, int r, DataType dt, const void* input, cons
 
   // ring.h:279-298: step i receives segment (r-i-1) in place. With a step table
   // the own-slice copy is one more row of the same launch.
-  if (opts.batched) {
+  if (opts.divisor < 0) return errors::InvalidArgument("negative divisor");
+  if (opts.batched && opts.divisor > 0) {
+    std::vector<ring_row> table;
+    std::vector<unsigned char> divide(static_cast<size_t>(n), 0);
+    divide[0] = 1;  // the own slice; what arrives was divided by its owner
+    table.push_back(ring_row{own ? at(output, starts[static_cast<size_t>(r)], esz) : nullptr, input, nullptr, own});
+    for (int i = 0; i < n - 1; i++) {
+      const size_t seg = static_cast<size_t>(Seg(RING_PHASE_GATHER, n, r, i, true));
+      const size_t cnt = elems_per_row * rows[seg];
+      table.push_back(ring_row{cnt ? at(output, starts[seg], esz) : nullptr, recv[i], nullptr, cnt});
+    }
+    RING_RETURN_IF_ERROR(ring_apply_rows_avg(table.data(), n, divide.data(), opts.divisor, code, stream),
+                         "ring_apply_rows_avg");
+  } else if (opts.batched) {
     std::vector<ring_step> steps;
     steps.push_back(ring_step{starts[static_cast<size_t>(r)], input, own});
     for (int i = 0; i < n - 1; i++) {
@@ -137,6 +180,10 @@ Status RingAllgatherPrestaged(int n, int r, DataType dt, const void* input, cons
     }
     RING_RETURN_IF_ERROR(ring_allgather_steps(output, steps.data(), n, code, stream), "ring_allgather_steps");
   } else {
+    if (opts.divisor > 0) {
+      ring_row row{own ? at(output, starts[static_cast<size_t>(r)], esz) : nullptr, input, nullptr, own};
+      RING_RETURN_IF_ERROR(ring_apply_rows_avg(&row, 1, nullptr, opts.divisor, code, stream), "ring_apply_rows_avg");
+    } else
     RING_RETURN_IF_ERROR(ring_copy_bytes(at(output, starts[static_cast<size_t>(r)], esz), input, own * esz, stream),
                          "ring_copy_bytes");
     for (int i = 0; i < n - 1; i++) {
@@ -151,11 +198,11 @@ Status RingAllgatherPrestaged(int n, int r, DataType dt, const void* input, cons
 
 Status RingAllreduceAllRanks(int n, DataType dt, const void* const* inputs, void* const* outputs, size_t count,
                              void* stream, const RingOptions& opts) {
-  (void)opts;
   int code = 0;
   Status s = RingDataType(dt, &code);
   if (!s.ok()) return s;
   if (n < 1) return errors::InvalidArgument("empty ring");
+  if (opts.divisor < 0) return errors::InvalidArgument("negative divisor");
   if (count == 0) return Status::OK();
   const size_t esz = ring_dtype_size(code);
   std::vector<size_t> sizes(static_cast<size_t>(n)), starts(static_cast<size_t>(n));
@@ -166,9 +213,12 @@ Status RingAllreduceAllRanks(int n, DataType dt, const void* const* inputs, void
   for (int r = 0; r < n; r++) {
     if (!inputs[r] || !outputs[r]) return errors::InvalidArgument("null tensor with a non-zero element count");
     // a rank reducing in place (a fusion buffer) has nothing to copy
-    rows[static_cast<size_t>(r)] = ring_row{outputs[r], inputs[r], nullptr, inputs[r] == outputs[r] ? 0 : count};
+    const bool nothing = inputs[r] == outputs[r] && !(n == 1 && opts.divisor > 0);
+    rows[static_cast<size_t>(r)] = ring_row{outputs[r], inputs[r], nullptr, nothing ? 0 : count};
   }
-  RING_RETURN_IF_ERROR(ring_apply_rows(rows.data(), n, code, stream), "ring_apply_rows");
+  // a lone rank owns every element: its copy is where the divide happens
+  RING_RETURN_IF_ERROR(ring_apply_rows_avg(rows.data(), n, nullptr, n == 1 ? opts.divisor : 0, code, stream),
+                       "ring_apply_rows");
 
   // ring.h:183-205: at step i rank r adds its left neighbour's segment (r-i-1)
   for (int i = 0; i < n - 1; i++) {
@@ -178,7 +228,9 @@ Status RingAllreduceAllRanks(int n, DataType dt, const void* const* inputs, void
       char* dst = at(outputs[r], starts[seg], esz);
       rows[static_cast<size_t>(r)] = ring_row{dst, at(static_cast<const void*>(outputs[left]), starts[seg], esz), dst, sizes[seg]};
     }
-    RING_RETURN_IF_ERROR(ring_apply_rows(rows.data(), n, code, stream), "ring_apply_rows");
+    // the last step completes every rank's owned segment: all of its rows divide
+    RING_RETURN_IF_ERROR(ring_apply_rows_avg(rows.data(), n, nullptr, i == n - 2 ? opts.divisor : 0, code, stream),
+                         "ring_apply_rows");
   }
   // ring.h:211-225: at step i rank r receives segment (r-i) from the left
   for (int i = 0; i < n - 1; i++) {
@@ -195,7 +247,7 @@ Status RingAllreduceAllRanks(int n, DataType dt, const void* const* inputs, void
 
 Status RingAllgatherAllRanks(int n, DataType dt, const void* const* inputs, const std::vector<size_t>& rows_per_rank,
                              size_t elems_per_row, void* const* outputs, void* stream, const RingOptions& opts) {
-  (void)opts;
+  if (opts.divisor < 0) return errors::InvalidArgument("negative divisor");
   int code = 0;
   Status s = RingDataType(dt, &code);
   if (!s.ok()) return s;
@@ -210,7 +262,8 @@ Status RingAllgatherAllRanks(int n, DataType dt, const void* const* inputs, cons
     if (own && (!inputs[r] || !outputs[r])) return errors::InvalidArgument("null tensor with a non-zero element count");
     rows[static_cast<size_t>(r)] = ring_row{own ? at(outputs[r], starts[static_cast<size_t>(r)], esz) : nullptr, inputs[r], nullptr, own};
   }
-  RING_RETURN_IF_ERROR(ring_apply_rows(rows.data(), n, code, stream), "ring_apply_rows");
+  // every rank divides its own slice on the way into its output
+  RING_RETURN_IF_ERROR(ring_apply_rows_avg(rows.data(), n, nullptr, opts.divisor, code, stream), "ring_apply_rows");
   for (int i = 0; i < n - 1; i++) {  // ring.h:279-298
     for (int r = 0; r < n; r++) {
       const int left = (r - 1 + n) % n;

@@ -22,10 +22,19 @@ struct RingOptions {
   // Fold the in->out copy (ring.h:146-148) into the reduce-scatter:
   // out[seg] = in[seg] + received, the same single add per element.
   bool fuse_copy = false;
+  // > 0: the result is tf.div(result, divisor), the average of
+  // allreduce(average=True) (__init__.py:160-164, 153-157 of the reference),
+  // computed where a value becomes final instead of in a pass of its own: the
+  // owner of a segment divides in its last reduce-scatter accumulate (the
+  // owner of an allgather slice, when it copies the slice into its output), and
+  // what then travels round the ring is already divided. Pre-staged allgather
+  // segments are therefore expected divided, as a peer would send them.
+  int divisor = 0;
   static RingOptions FromFlags(int flags) {
     RingOptions o;
     o.batched = (flags & 1) != 0;
     o.fuse_copy = (flags & 2) != 0;
+    o.divisor = (flags >> 8) & 0x7fffff;
     return o;
   }
 };

@@ -98,30 +98,44 @@ __device__ __forceinline__ int64_t div_one(int64_t x, int n) {
 __device__ __forceinline__ uint32_t div_one(uint32_t x, int) { return x; }
 __device__ __forceinline__ uint64_t div_one(uint64_t x, int) { return x; }
 
+// The add of the accumulate; signed integers wrap like the unsigned carriers.
+__device__ __forceinline__ float add_one(float a, float b) { return b + a; }
+__device__ __forceinline__ uint32_t add_one(uint32_t a, uint32_t b) { return b + a; }
+__device__ __forceinline__ uint64_t add_one(uint64_t a, uint64_t b) { return b + a; }
+__device__ __forceinline__ int32_t add_one(int32_t a, int32_t b) {
+  return static_cast<int32_t>(static_cast<uint32_t>(b) + static_cast<uint32_t>(a));
+}
+__device__ __forceinline__ int64_t add_one(int64_t a, int64_t b) {
+  return static_cast<int64_t>(static_cast<uint64_t>(b) + static_cast<uint64_t>(a));
+}
+
 // kOpCopy: dst = a.  kOpAdd: dst = b + a (b may be dst itself: the in-place
 // accumulate of the reference).  kOpDiv: dst = a / n (a may be dst itself).
-enum Op { kOpCopy = 0, kOpAdd = 1, kOpDiv = 2 };
+// kOpAddDiv: dst = (b + a) / n, the last accumulate of an averaged allreduce:
+// the sum is rounded exactly as kOpAdd rounds it and then divided exactly as
+// kOpDiv divides it, so the result equals the two passes done separately.
+enum Op { kOpCopy = 0, kOpAdd = 1, kOpDiv = 2, kOpAddDiv = 3 };
 
 template <typename T, int OP>
 __device__ __forceinline__ T apply_one(T a, T b, int n) {
-  if (OP == kOpAdd) return b + a;
+  if (OP == kOpAdd) return add_one(a, b);
   if (OP == kOpDiv) return div_one(a, n);
+  if (OP == kOpAddDiv) return div_one(add_one(a, b), n);
   return a;
 }
 template <typename T, int OP>
 __device__ __forceinline__ typename VecOf<T>::type apply_vec(typename VecOf<T>::type a, typename VecOf<T>::type b, int n) {
-  if (OP == kOpAdd) return b + a;
-  if (OP == kOpDiv) {
+  if (OP == kOpCopy) return a;
 #pragma unroll
-    for (uint32_t c = 0; c < 16 / sizeof(T); c++) a[c] = div_one(a[c], n);
-  }
+  for (uint32_t c = 0; c < 16 / sizeof(T); c++) a[c] = apply_one<T, OP>(a[c], b[c], n);
   return a;
 }
 
 // Launch modes of rows_kernel. kCopy: every row is a copy. kAdd: a row with a
 // second operand is an add, a row without one is still a copy, so one launch
-// can mix both. kDiv: every row is divided by the table's divisor.
-enum Mode { kCopy = 0, kAdd = 1, kDiv = 2 };
+// can mix both. kAvg: as kAdd on the signed element types, and the rows whose
+// bit is set in the table's div_mask also divide by the table's divisor.
+enum Mode { kCopy = 0, kAdd = 1, kAvg = 2 };
 
 // Rows of one launch, passed by value in the kernel arguments (read with
 // scalar loads; uniform per workgroup).
@@ -138,7 +152,8 @@ struct RowTable {
   // segments of an allreduce). 0: rows differ; the grid is 1-D over all tiles
   // and a workgroup finds its row by binary search over tile_begin.
   uint32_t uniform_tiles;
-  int divisor;                        // kDiv only
+  int divisor;                        // kAvg only
+  uint64_t div_mask;                  // kAvg only: bit k set = row k divides
   uint32_t tile_begin[kMaxRows + 1];  // prefix sum of tiles per row
   Row row[kMaxRows];
 };
@@ -171,10 +186,11 @@ __device__ __forceinline__ void row_tile(T* dst, const T* a, const T* b, uint64_
   const uint64_t nvec = (count - head) / VEC;
   const uint32_t tid = threadIdx.x;
 
-  if (tile == 0 && tid < head) dst[tid] = apply_one<T, OP>(a[tid], OP == kOpAdd ? b[tid] : T(), n);
+  constexpr bool kTwo = OP == kOpAdd || OP == kOpAddDiv;  // reads b as well
+  if (tile == 0 && tid < head) dst[tid] = apply_one<T, OP>(a[tid], kTwo ? b[tid] : T(), n);
   if (tile + 1 == tiles_in_row) {
     const uint64_t e = head + nvec * VEC + tid;
-    if (e < count) dst[e] = apply_one<T, OP>(a[e], OP == kOpAdd ? b[e] : T(), n);
+    if (e < count) dst[e] = apply_one<T, OP>(a[e], kTwo ? b[e] : T(), n);
   }
 
   V* dv = reinterpret_cast<V*>(dst + head);
@@ -186,7 +202,7 @@ __device__ __forceinline__ void row_tile(T* dst, const T* a, const T* b, uint64_
     V x[UNROLL], y[UNROLL];
 #pragma unroll
     for (int j = 0; j < UNROLL; j++) x[j] = RING_LOAD_VEC(NT, &av[v0 + j * kBlock]);
-    if (OP == kOpAdd) {
+    if (kTwo) {
 #pragma unroll
       for (int j = 0; j < UNROLL; j++) y[j] = RING_LOAD_VEC(NT, &bv[v0 + j * kBlock]);
     }
@@ -201,7 +217,7 @@ __device__ __forceinline__ void row_tile(T* dst, const T* a, const T* b, uint64_
       if (v < nvec) {
         V x = RING_LOAD_VEC(NT, &av[v]);
         V y = x;
-        if (OP == kOpAdd) y = RING_LOAD_VEC(NT, &bv[v]);
+        if (kTwo) y = RING_LOAD_VEC(NT, &bv[v]);
         store_vec<T, NT>(&dv[v], apply_vec<T, OP>(x, y, n));
       }
     }
@@ -209,21 +225,28 @@ __device__ __forceinline__ void row_tile(T* dst, const T* a, const T* b, uint64_
 }
 
 template <typename T, int MODE, int UNROLL, int NT>
-__device__ __forceinline__ void run_row(const Row& r, uint32_t tile, uint32_t tiles, int divisor) {
+__device__ __forceinline__ void run_row(const Row& r, uint32_t tile, uint32_t tiles, int divisor, bool divide) {
   T* dst = static_cast<T*>(r.dst);
   const T* a = static_cast<const T*>(r.a);
   const T* b = static_cast<const T*>(r.b);
-  if (MODE == kDiv) row_tile<T, kOpDiv, UNROLL, NT>(dst, a, nullptr, r.count, tile, tiles, divisor);
-  else if (MODE == kAdd && b != nullptr) row_tile<T, kOpAdd, UNROLL, NT>(dst, a, b, r.count, tile, tiles, 0);
-  else row_tile<T, kOpCopy, UNROLL, NT>(dst, a, nullptr, r.count, tile, tiles, 0);
+  // every condition is uniform over the workgroup (kernel arguments only)
+  if (MODE == kAvg && divide) {
+    if (b != nullptr) row_tile<T, kOpAddDiv, UNROLL, NT>(dst, a, b, r.count, tile, tiles, divisor);
+    else row_tile<T, kOpDiv, UNROLL, NT>(dst, a, nullptr, r.count, tile, tiles, divisor);
+  } else if (MODE != kCopy && b != nullptr) {
+    row_tile<T, kOpAdd, UNROLL, NT>(dst, a, b, r.count, tile, tiles, 0);
+  } else {
+    row_tile<T, kOpCopy, UNROLL, NT>(dst, a, nullptr, r.count, tile, tiles, 0);
+  }
 }
 
 template <typename T, int MODE, int UNROLL, int NT>
 __global__ void __launch_bounds__(kBlock) rows_kernel(const RowTable tab) {
   if (tab.uniform_tiles) {
     const Row r = tab.row[blockIdx.y];  // one scalar load, no search
+    const bool divide = MODE == kAvg && ((tab.div_mask >> blockIdx.y) & 1u);
     for (uint32_t t = blockIdx.x; t < tab.uniform_tiles; t += gridDim.x)
-      run_row<T, MODE, UNROLL, NT>(r, t, tab.uniform_tiles, tab.divisor);
+      run_row<T, MODE, UNROLL, NT>(r, t, tab.uniform_tiles, tab.divisor, divide);
     return;
   }
   const uint32_t total = tab.tile_begin[tab.n_rows];
@@ -235,7 +258,8 @@ __global__ void __launch_bounds__(kBlock) rows_kernel(const RowTable tab) {
       if (tab.tile_begin[mid] <= t) lo = mid; else hi = mid;
     }
     const uint32_t first = tab.tile_begin[lo];
-    run_row<T, MODE, UNROLL, NT>(tab.row[lo], t - first, tab.tile_begin[lo + 1] - first, tab.divisor);
+    run_row<T, MODE, UNROLL, NT>(tab.row[lo], t - first, tab.tile_begin[lo + 1] - first, tab.divisor,
+                                 MODE == kAvg && ((tab.div_mask >> lo) & 1u));
   }
 }
 
@@ -391,12 +415,13 @@ struct HostRow {
   const void* a;
   const void* b;   // null: copy row
   uint64_t count;  // elements of `esz` bytes
+  bool divide;     // with a divisor: this row also divides
 };
 
 // Launches rows (any number) in groups of kMaxRows. esz: 4 or 8. A table with
 // no add row runs the copy-only kernel.
-// divisor > 0: every row is divided in place / out of place by it (kDiv) and
-// the element type is signed.
+// divisor > 0: rows marked `divide` also divide by it (kAvg) and the element
+// type is signed.
 int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, hipStream_t stream,
                 Role role, int divisor = 0) {
   int nt = g_tuning.nt[role];
@@ -414,6 +439,7 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
     RowTable tab;
     tab.n_rows = 0;
     tab.divisor = divisor;
+    tab.div_mask = 0;
     tab.tile_begin[0] = 0;
     uint64_t tiles = 0;
     uint64_t first_tiles = 0;
@@ -433,6 +459,7 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
       }
       const int k = tab.n_rows++;
       tab.row[k] = Row{r.dst, r.a, r.b, r.count};
+      if (divisor > 0 && r.divide) tab.div_mask |= 1ull << k;
       any_add = any_add || r.b != nullptr;
       if (k == 0) first_tiles = t;
       uniform = uniform && t == first_tiles;
@@ -459,10 +486,10 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
       grid = dim3(static_cast<uint32_t>(tiles < cap ? tiles : cap));
     }
     int rc;
-    if (divisor > 0) {
-      rc = esz == 8 ? launch_rows_typed<int64_t, kDiv>(tab, grid, stream, nt)
-           : is_float ? launch_rows_typed<float, kDiv>(tab, grid, stream, nt)
-                      : launch_rows_typed<int32_t, kDiv>(tab, grid, stream, nt);
+    if (tab.div_mask != 0) {
+      rc = esz == 8 ? launch_rows_typed<int64_t, kAvg>(tab, grid, stream, nt)
+           : is_float ? launch_rows_typed<float, kAvg>(tab, grid, stream, nt)
+                      : launch_rows_typed<int32_t, kAvg>(tab, grid, stream, nt);
     } else if (!any_add) {
       rc = esz == 8 ? launch_rows_typed<uint64_t, kCopy>(tab, grid, stream, nt)
                     : launch_rows_typed<uint32_t, kCopy>(tab, grid, stream, nt);
@@ -501,7 +528,7 @@ int steps_common(const void* input, void* buffer, const ring_step* steps, int n_
     if ((reinterpret_cast<uintptr_t>(d) | reinterpret_cast<uintptr_t>(steps[i].src) |
          reinterpret_cast<uintptr_t>(local)) & (esz - 1))
       return RING_ERR_ARGUMENT;
-    rows.push_back(HostRow{d, steps[i].src, kind == kStepCopy ? nullptr : local, steps[i].count});
+    rows.push_back(HostRow{d, steps[i].src, kind == kStepCopy ? nullptr : local, steps[i].count, false});
   }
   return launch_rows(rows.data(), rows.size(), esz, dtype == RING_F32, static_cast<hipStream_t>(stream),
                      kind == kStepCopy ? kRoleAllgather : kRoleAccumulate);
@@ -732,7 +759,7 @@ int ring_copy_bytes(void* dst, const void* src, size_t bytes, void* stream) {
   hipStream_t s = static_cast<hipStream_t>(stream);
   const uintptr_t all = reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src) | bytes;
   if ((all & 3u) == 0) {
-    HostRow row{dst, src, nullptr, bytes / 4};
+    HostRow row{dst, src, nullptr, bytes / 4, false};
     return launch_rows(&row, 1, 4, false, s, kRoleCopy);
   }
   uint64_t blocks = (bytes + kBlock - 1) / kBlock;
@@ -751,7 +778,7 @@ int ring_accumulate(int dtype, void* dst, const void* src, size_t count, void* s
   const size_t esz = dtype_size(dtype);
   if ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & (esz - 1))
     return RING_ERR_ARGUMENT;
-  HostRow row{dst, src, dst, count};
+  HostRow row{dst, src, dst, count, false};
   return launch_rows(&row, 1, esz, dtype == RING_F32, static_cast<hipStream_t>(stream), kRoleAccumulate);
 }
 
@@ -776,8 +803,13 @@ int ring_reduce_scatter_steps_from(const void* input, void* buffer, const ring_s
 }
 
 int ring_apply_rows(const ring_row* rows, int n_rows, int dtype, void* stream) {
+  return ring_apply_rows_avg(rows, n_rows, nullptr, 0, dtype, stream);
+}
+
+int ring_apply_rows_avg(const ring_row* rows, int n_rows, const unsigned char* divide, int divisor, int dtype,
+                        void* stream) {
   if (!dtype_ok(dtype)) return RING_ERR_DTYPE;
-  if (n_rows < 0) return RING_ERR_ARGUMENT;
+  if (n_rows < 0 || divisor < 0) return RING_ERR_ARGUMENT;
   if (n_rows == 0) return RING_OK;
   if (!rows) return RING_ERR_ARGUMENT;
   const size_t esz = dtype_size(dtype);
@@ -789,10 +821,11 @@ int ring_apply_rows(const ring_row* rows, int n_rows, int dtype, void* stream) {
     if ((reinterpret_cast<uintptr_t>(rows[i].dst) | reinterpret_cast<uintptr_t>(rows[i].a) |
          reinterpret_cast<uintptr_t>(rows[i].b)) & (esz - 1))
       return RING_ERR_ARGUMENT;
-    host.push_back(HostRow{rows[i].dst, rows[i].a, rows[i].b, rows[i].count});
+    host.push_back(HostRow{rows[i].dst, rows[i].a, rows[i].b, rows[i].count,
+                           divisor > 0 && (!divide || divide[i] != 0)});
   }
   return launch_rows(host.data(), host.size(), esz, dtype == RING_F32, static_cast<hipStream_t>(stream),
-                     kRoleAccumulate);
+                     kRoleAccumulate, divisor);
 }
 
 int ring_allgather_steps(void* buffer, const ring_step* steps, int n_steps, int dtype, void* stream) {
@@ -804,7 +837,7 @@ int ring_scale(int dtype, void* data, size_t count, int divisor, void* stream) {
   if (divisor < 1) return RING_ERR_ARGUMENT;
   if (count == 0) return RING_OK;
   if (!data || (reinterpret_cast<uintptr_t>(data) & (dtype_size(dtype) - 1))) return RING_ERR_ARGUMENT;
-  HostRow row{data, data, nullptr, count};
+  HostRow row{data, data, nullptr, count, true};
   return launch_rows(&row, 1, dtype_size(dtype), dtype == RING_F32, static_cast<hipStream_t>(stream),
                      kRoleAccumulate, divisor);
 }

@@ -245,14 +245,14 @@ class Session:
             self._counters[(r, base)] = k + 1
         return base if k == 0 else "%s_%d" % (base, k)
 
-    def _submit(self, r, op, node_name, inputs, device):
+    def _submit(self, r, op, node_name, inputs, device, divisor=0):
         if any(t.is_cuda for t in inputs):
             # the inputs' producers must have finished before the ring reads them (the
             # reference defers the enqueue with a stream host callback, mpi_ops.cc:1099-1105)
             producers = torch.cuda.current_stream(inputs[0].device)
             if not producers.query():
                 producers.synchronize()
-        pending = _plugin.PendingOp(self._world, r, op, node_name, inputs, device)
+        pending = _plugin.PendingOp(self._world, r, op, node_name, inputs, device, divisor)
         pending.rank = r
         pending.handle = pending.fail_handle = pending.on_done = pending.next_op = None
         pending.lock = threading.Lock()
@@ -276,7 +276,7 @@ class Session:
             self._drain()
         return handle
 
-    def _chain_allgather(self, r, sizing, tensor, name, dev):
+    def _chain_allgather(self, r, sizing, tensor, name, dev, divisor=0):
         handle = PendingTensor(self)
         handle._first_op = sizing
 
@@ -284,7 +284,7 @@ class Session:
             sizes = outputs[0].cpu() if outputs[0].is_cuda else outputs[0]   # host-memory `sizes` input
             node = self._node_name(r, 'MPIAllgather', name)
             with self.as_rank(r):
-                second = self._submit(r, 'MPIAllgather', node, [tensor, sizes], dev)
+                second = self._submit(r, 'MPIAllgather', node, [tensor, sizes], dev, divisor)
             second.handle = handle
             sizing.next_op = second
 
@@ -357,7 +357,8 @@ class Session:
                 self._check_all_ranks_submitted(batch)
             self._flush()
             for p in batch:
-                first_error = first_error or self._complete(p)
+                error = self._complete(p)          # every op is completed, also after a failure
+                first_error = first_error or error
         if self.stream:
             ring_abi.stream_synchronize(self.stream)
         if first_error is not None:
@@ -414,15 +415,20 @@ def allreduce(tensor, average=True):
     the represented tensor.
     """
     session, _ = mpi_ops._current()
+    # With every rank in this process the average's tf.div is fused into the
+    # collective (the owner of a segment divides in its last accumulate). A
+    # session with pre-staged peers keeps the reference's order, collective
+    # then division, so that what is staged is the reference's wire traffic.
+    fold = session.size if average and session.real_rank is None else 0
     if isinstance(tensor, IndexedSlices):
         # For IndexedSlices, do two allgathers instead of an allreduce.
-        values = allgather(tensor.values)
+        values = allgather(tensor.values, divisor=fold)
         indices = allgather(tensor.indices)
         # To make this operation into an average, divide all gathered values by the MPI size.
-        new_values = _div(session, values) if average else values
+        new_values = _div(session, values) if average and not fold else values
         return IndexedSlices(new_values, indices, dense_shape=tensor.dense_shape)
-    summed_tensor = _allreduce(tensor)
-    return _div(session, summed_tensor) if average else summed_tensor
+    summed_tensor = _allreduce(tensor, divisor=fold)
+    return _div(session, summed_tensor) if average and not fold else summed_tensor
 
 
 class DistributedOptimizer:

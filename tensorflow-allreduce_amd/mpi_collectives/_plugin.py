@@ -28,7 +28,7 @@ EXPORTS = (
     "mpic_op_infer_shape", "mpic_world_create", "mpic_world_create_prestaged", "mpic_world_destroy",
     "mpic_world_size", "mpic_world_stream", "mpic_world_set_option", "mpic_world_set_fusion_buffer",
     "mpic_world_flush", "mpic_stage_peers",
-    "mpic_context_create", "mpic_context_add_input", "mpic_context_compute", "mpic_context_wait",
+    "mpic_context_create", "mpic_context_add_input", "mpic_context_set_divisor", "mpic_context_compute", "mpic_context_wait",
     "mpic_context_message", "mpic_context_num_outputs", "mpic_context_output", "mpic_context_destroy",
     "mpic_ring_allreduce_prestaged", "mpic_ring_allgather_prestaged", "mpic_ring_allreduce_all_ranks",
     "mpic_ring_allgather_all_ranks", "mpic_last_error",
@@ -116,6 +116,7 @@ def load_library(name="libmpi_collectives.so", op_list=None):
             "mpic_stage_peers": (ci, [vp, cp, pvp, pvp]),
             "mpic_context_create": (ci, [vp, ci, cp, cp, cp, ALLOC_FN, vp, pvp]),
             "mpic_context_add_input": (ci, [vp, ci, ci, p64, vp, ci]),
+            "mpic_context_set_divisor": (ci, [vp, ci]),
             "mpic_context_compute": (ci, [vp]),
             "mpic_context_wait": (ci, [vp]),
             "mpic_context_message": (cp, [vp]),
@@ -205,7 +206,7 @@ class PendingOp:
     """One op instance in flight: keeps inputs, outputs and the C context alive
     until the op's done() has run."""
 
-    def __init__(self, world, rank, op, node_name, inputs, device):
+    def __init__(self, world, rank, op, node_name, inputs, device, divisor=0):
         L = lib()
         self._outputs = []          # torch tensors the op allocated, in allocation order
         self._inputs = inputs       # keep-alive
@@ -236,6 +237,10 @@ class PendingOp:
             rc = L.mpic_context_add_input(self._h, dt, t.dim(), dims, t.data_ptr() if t.numel() else None, int(host))
             if rc != OK:
                 raise error_for(rc, "bad input for %s" % op)
+        if divisor:
+            rc = L.mpic_context_set_divisor(self._h, divisor)
+            if rc != OK:
+                raise error_for(rc, "bad divisor for %s" % op)
         rc = L.mpic_context_compute(self._h)       # outputs are allocated during this call
         _live_ops.pop(self._key, None)
         if rc != OK:

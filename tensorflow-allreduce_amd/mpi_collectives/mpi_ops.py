@@ -49,12 +49,12 @@ def _current():
     return _scope.session, _scope.rank
 
 
-def _run(op, inputs, name, device=None):
+def _run(op, inputs, name, device=None, divisor=0):
     session, rank = _current()
     node_name = session._node_name(rank, op, name)
     if device is None:
         device = "GPU" if any(t.is_cuda for t in inputs) or not inputs else "CPU"
-    return session._submit(rank, op, node_name, inputs, device)
+    return session._submit(rank, op, node_name, inputs, device, divisor)
 
 
 def _scalar(op, name):
@@ -88,7 +88,7 @@ def local_rank(name=None):
     return _scalar('MPILocalRank', name)
 
 
-def _allreduce(tensor, name=None):
+def _allreduce(tensor, name=None, divisor=0):
     """Sums `tensor` over all the MPI processes.
 
     The reduction is keyed by the name of the op. The tensor type and shape
@@ -96,19 +96,25 @@ def _allreduce(tensor, name=None):
     start until all ranks are ready to send and receive the tensor, so the
     returned tensor holds the sum once every rank has submitted the op and the
     session has run (immediately, in a session with pre-staged peers).
+
+    divisor > 0 (not in the reference): the op delivers tf.div(sum, divisor),
+    the consumer `allreduce(average=True)` appends, without a pass of its own.
     """
     tensor = tensor.contiguous()            # the ring works on the flat buffer
-    pending = _run('MPIAllreduce', [tensor], name, device="GPU" if tensor.is_cuda else "CPU")
+    pending = _run('MPIAllreduce', [tensor], name, device="GPU" if tensor.is_cuda else "CPU", divisor=divisor)
     return _current()[0]._result(pending)
 
 
-def allgather(tensor, name=None):
+def allgather(tensor, name=None, divisor=0):
     """Concatenates `tensor` with the same tensor on all other MPI processes
     along the first dimension, which may differ between ranks.
 
     As in the reference (mpi_ops.py:152-160) this is two collectives: a gather
     of every rank's first-dimension size, flagged by a scalar `sizes` input,
     whose result is the host-side `sizes` input of the gather proper.
+
+    divisor > 0 (not in the reference): the gathered values arrive divided by
+    it (tf.div), each rank dividing its own slice on the way into the ring.
     """
     session, r = _current()
     tensor = tensor.contiguous()
@@ -120,4 +126,4 @@ def allgather(tensor, name=None):
     first = tensor.shape[0] if tensor.dim() > 0 else 0
     my_size = torch.tensor([first], dtype=torch.int64, device=tensor.device)
     sizing = _run('MPIAllgather', [my_size, sizes_flag], sizing_name, device=dev)
-    return session._chain_allgather(r, sizing, tensor, name, dev)
+    return session._chain_allgather(r, sizing, tensor, name, dev, divisor)

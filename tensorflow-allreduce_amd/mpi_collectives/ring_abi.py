@@ -22,7 +22,7 @@ EXPORTS = (
     "ring_schedule", "ring_stream_create", "ring_stream_destroy", "ring_stream_synchronize",
     "ring_copy_bytes", "ring_accumulate_f32", "ring_accumulate_i32", "ring_accumulate_i64",
     "ring_accumulate", "ring_reduce_scatter_steps", "ring_reduce_scatter_steps_from",
-    "ring_allgather_steps", "ring_apply_rows",
+    "ring_allgather_steps", "ring_apply_rows", "ring_apply_rows_avg",
     "ring_fusion_plan_create", "ring_fusion_plan_destroy", "ring_fusion_plan_elements",
     "ring_fusion_pack", "ring_fusion_unpack", "ring_fusion_unpack_scaled", "ring_scale",
 )
@@ -90,6 +90,7 @@ def lib():
             "ring_reduce_scatter_steps_from": (ci, [vp, vp, ctypes.POINTER(Step), ci, ci, vp]),
             "ring_allgather_steps": (ci, [vp, ctypes.POINTER(Step), ci, ci, vp]),
             "ring_apply_rows": (ci, [ctypes.POINTER(Row), ci, ci, vp]),
+            "ring_apply_rows_avg": (ci, [ctypes.POINTER(Row), ci, ctypes.POINTER(ctypes.c_ubyte), ci, ci, vp]),
             "ring_fusion_plan_create": (ci, [ctypes.POINTER(vp), psz, ci, ci, ctypes.POINTER(vp)]),
             "ring_fusion_plan_destroy": (ci, [vp]),
             "ring_fusion_plan_elements": (sz, [vp]),
@@ -227,6 +228,17 @@ def apply_rows(rows, dtype, stream):
     for i, (d, a, b, cnt) in enumerate(rows):
         arr[i].dst, arr[i].a, arr[i].b, arr[i].count = d, a, b, cnt
     check(lib().ring_apply_rows(arr, len(rows), dtype, stream), "ring_apply_rows")
+
+
+def apply_rows_avg(rows, divide, divisor, dtype, stream):
+    """As apply_rows; rows with divide[k] true (all rows when divide is None)
+    also divide by `divisor` (tf.div semantics)."""
+    rows = list(rows)
+    arr = (Row * max(len(rows), 1))()
+    for i, (d, a, b, cnt) in enumerate(rows):
+        arr[i].dst, arr[i].a, arr[i].b, arr[i].count = d, a, b, cnt
+    flags = None if divide is None else (ctypes.c_ubyte * max(len(rows), 1))(*[1 if f else 0 for f in divide])
+    check(lib().ring_apply_rows_avg(arr, len(rows), flags, divisor, dtype, stream), "ring_apply_rows_avg")
 
 
 def scale(dtype, data, count, divisor, stream):

@@ -181,6 +181,65 @@ def test_launch_options_do_not_change_results(oracle, opt):
 
 
 @pytest.mark.parametrize("dtype", G.DTYPES)
+def test_rows_with_the_divide_folded_in(dtype):
+    """ring_apply_rows_avg: flagged rows store (b + a) / n or a / n, the others
+    b + a or a; equal to the accumulate followed by ring_scale's division,
+    negative integers floored, any alignment, more rows than one table holds."""
+    import torch
+    rng = np.random.default_rng(77)
+    code = G.NP2ABI[np.dtype(dtype)]
+    for n_rows, divisor in ((1, 1), (4, 8), (7, 3), (70, 6)):
+        counts = [int(c) for c in rng.integers(0, 9000, n_rows)]
+        counts[0] = 20_011
+        rows, wants, devs, flags = [], [], [], []
+        for k, c in enumerate(counts):
+            a = G.random_array(rng, c, dtype)
+            b = G.random_array(rng, c, dtype)
+            if dtype != np.float32 and c:
+                a[: c // 2] = -np.abs(a[: c // 2])          # negative sums with remainders
+                b[: c // 2] = -np.abs(b[: c // 2])
+            da, _ = G.dev(a, k % 4)
+            kind = k % 3                                        # in-place add, out-of-place add, copy
+            flag = bool((k * 7 + 1) % 2)
+            if kind == 0:
+                db, _ = G.dev(b, (k + 1) % 4)
+                dst, bptr = db, db.data_ptr()
+            elif kind == 1:
+                db, _ = G.dev(b, (k + 2) % 4)
+                dst, _ = G.dev(np.zeros(c, dtype=dtype), (k + 3) % 4)
+                bptr = db.data_ptr()
+            else:
+                db = None
+                dst, _ = G.dev(np.zeros(c, dtype=dtype), (k + 1) % 4)
+                bptr = None
+            with np.errstate(all="ignore"):
+                w = a if kind == 2 else (b + a).astype(dtype)
+                if flag:
+                    w = w / np.float32(divisor) if dtype == np.float32 else w // dtype(divisor)
+            rows.append((dst.data_ptr() if c else None, da.data_ptr() if c else None, bptr if c else None, c))
+            wants.append(np.asarray(w, dtype=dtype))
+            devs.append((dst, da, db))
+            flags.append(flag)
+        ring_abi.apply_rows_avg(rows, flags, divisor, code, None)
+        G.sync()
+        for k, (dst, _, _) in enumerate(devs):
+            G.assert_same_bits(G.host(dst), wants[k], "row %d of %d, /%d, flag %s" % (k, n_rows, divisor, flags[k]))
+    # divide=None flags every row; divisor 0 is plain ring_apply_rows
+    a = G.random_array(rng, 1000, dtype)
+    da, _ = G.dev(a, 1)
+    out, _ = G.dev(np.zeros(1000, dtype=dtype), 2)
+    ring_abi.apply_rows_avg([(out.data_ptr(), da.data_ptr(), None, 1000)], None, 5, code, None)
+    G.sync()
+    with np.errstate(all="ignore"):
+        G.assert_same_bits(G.host(out), (a / np.float32(5) if dtype == np.float32 else a // dtype(5)).astype(dtype), "all rows")
+    ring_abi.apply_rows_avg([(out.data_ptr(), da.data_ptr(), None, 1000)], [True], 0, code, None)
+    G.sync()
+    G.assert_same_bits(G.host(out), a, "divisor 0")
+    with pytest.raises(ring_abi.RingError):
+        ring_abi.apply_rows_avg([(out.data_ptr(), da.data_ptr(), None, 1000)], None, -1, code, None)
+
+
+@pytest.mark.parametrize("dtype", G.DTYPES)
 def test_scale_is_tf_div(dtype):
     """allreduce(average=True) divides with tf.div (__init__.py:160-164): true
     division for float32, floor division for integers."""

@@ -224,6 +224,78 @@ def test_prestaged_rank_matches_oracle_small(oracle, dtype):
                 G.assert_same_bits(G.host(got), outs[r], "prestaged n=%d r=%d flags=%d" % (n, r, flags))
 
 
+def _tf_div(x, n):
+    with np.errstate(all="ignore"):
+        return (x / np.float32(n) if x.dtype == np.float32 else x // x.dtype.type(n)).astype(x.dtype)
+
+
+@pytest.mark.parametrize("dtype", G.DTYPES)
+def test_prestaged_rank_with_the_average_folded_in(oracle, dtype):
+    """Divisor in the flags: the rank divides the segment it owns in its last
+    accumulate and receives the other segments already divided (what its
+    peers, doing the same, send): the output is tf.div(sum, divisor)."""
+    for n, count, divisor in ((1, 9, 1), (1, 10, 3), (2, 7, 2), (3, 3, 3), (6, 4099, 6), (8, 100_003, 8), (4, 50, 7)):
+        ins = make_inputs(n, count, dtype, seed=20 + n)
+        outs, rs, ag = oracle.ring_allreduce(ins, tap=True)
+        sizes, _ = ring_abi.segment_table(count, n)
+        ag_div = [[_tf_div(seg, divisor) for seg in per_rank] for per_rank in ag]
+        for r in sorted({0, n // 2, n - 1}):
+            for flags in (0, 1, 3):
+                got = _prestaged(n, r, ins, rs, ag_div, flags | (divisor << 8), dtype)
+                G.assert_same_bits(G.host(got), _tf_div(outs[r], divisor),
+                                   "folded average n=%d r=%d flags=%d /%d" % (n, r, flags, divisor))
+
+
+def test_average_costs_no_extra_launch():
+    """allreduce(average=True) over resident ranks: as many kernel launches as
+    the sum alone (the divide rides on the last reduce-scatter step)."""
+    L = _plugin.load_library()
+    n, count = 4, 10_000
+    ins = [cuda(np.full(count, r + 1, dtype=np.float32)) for r in range(n)]
+    outs = [torch.empty(count, device="cuda") for _ in range(n)]
+    ip = (ctypes.c_void_p * n)(*[t.data_ptr() for t in ins])
+    op = (ctypes.c_void_p * n)(*[t.data_ptr() for t in outs])
+    stream = torch.cuda.current_stream().cuda_stream
+    assert L.mpic_ring_allreduce_all_ranks(n, _plugin.DT_FLOAT, ip, op, count, stream, 1 | (n << 8)) == 0
+    torch.cuda.synchronize()
+    for o in outs:
+        assert torch.equal(o, torch.full((count,), 2.5, device="cuda"))     # (1+2+3+4)/4
+
+
+def test_mismatched_divisors_are_refused():
+    """Every rank must fuse the same division (FailedPrecondition otherwise)."""
+    with mpi.Session(size=2) as session:
+        hs = []
+        for r in range(2):
+            with session.as_rank(r):
+                hs.append(mpi._allreduce(cuda(np.ones(8, dtype=np.float32)), name="x", divisor=2 if r else 0))
+        with pytest.raises(mpi.FailedPreconditionError, match="Mismatched fused divisors"):
+            session.run(hs)
+
+
+def test_coordinator_fusion_with_average(oracle):
+    """Averaged allreduces fused by the coordinator; sums and averages submitted
+    together still form one group (each averaged tensor is divided after the
+    unpack), a group of averages only has the divide ride on the unpack."""
+    n = 3
+    counts = [1000, 37, 5000, 64]
+    per_rank = [[np.random.default_rng(10 * r + j).standard_normal(c).astype(np.float32) for j, c in enumerate(counts)]
+                for r in range(n)]
+    want = _expected_with_fusion(oracle, per_rank, [[0, 1, 2, 3]])
+    for averaged in ((0, 1), (0, 1, 2, 3)):
+        with mpi.Session(size=n, fusion_threshold=1 << 20) as session:
+            hs = [[None] * 4 for _ in range(n)]
+            for r in range(n):
+                with session.as_rank(r):
+                    for j in range(4):
+                        hs[r][j] = mpi.allreduce(cuda(per_rank[r][j]), average=j in averaged)
+            outs = session.run(hs)
+        for r in range(n):
+            for j in range(4):
+                G.assert_same_bits(G.host(outs[r][j]), _tf_div(want[j], n) if j in averaged else want[j],
+                                   "coordinator fusion + average %s: rank %d tensor %d" % (averaged, r, j))
+
+
 def test_prestaged_64mib_float32_n8(oracle):
     """The headline shape: 16,777,216 float32, N=8, values N(0,1) from seed=rank,
     peers' segments staged from the oracle's full ring."""

@@ -247,6 +247,21 @@ def test_run_refuses_to_wait_for_ranks_that_never_submitted():
         pending.wait()
 
 
+def test_fused_divisor_arguments_and_failure_drain():
+    """A negative divisor is refused before the op starts; when several ops of
+    one run fail, every one of them is completed and the first error raised."""
+    with mpi.Session(size=2, device="CPU") as s:
+        with pytest.raises(mpi.InvalidArgumentError, match="bad divisor"):
+            _plugin.PendingOp(s._world, 0, 'MPIAllreduce', 'neg', [torch.zeros(4)], 'GPU', divisor=-1)
+        for r in range(2):
+            for name in ("a", "b"):
+                # host tensors: both collectives are refused ("GPU kernels only")
+                s._submit(r, 'MPIAllreduce', name, [torch.zeros(4)], "GPU", 2)
+        with pytest.raises(mpi.FailedPreconditionError, match="GPU kernels only"):
+            s.run()
+        assert not s._pending and not s._submitted
+
+
 def test_node_names_are_uniquified_like_graph_nodes():
     with mpi.Session(size=2, device="CPU") as s:
         assert [s._node_name(0, 'MPIAllreduce', None) for _ in range(3)] == \
