@@ -81,9 +81,12 @@ class Workload:
     def check(self, k):
         return True
 
+    step_bytes = None    # algorithmic bytes of one step when it is not the sum of the phases
+    step_launches = None  # kernel launches of one step when it is not one per phase
+
     @property
     def bytes_per_step(self):
-        return sum(p[1] for p in self.phases)
+        return self.step_bytes if self.step_bytes is not None else sum(p[1] for p in self.phases)
 
 
 class RingAllreduce(Workload):
@@ -167,6 +170,42 @@ class RingAllreduce(Workload):
         for g, t in zip(s["ag_seg"], s["ag"]):
             ok = ok and torch.equal(s["out"][self.starts[g]:self.starts[g] + self.sizes[g]], t)
         return bool(ok)
+
+
+class RingAllreducePerStep(RingAllreduce):
+    """The same allreduce with one launch per ring step, the structure of the
+    reference's loop (ring.h:183-225): copy, n-1 accumulates of one segment,
+    n-1 copies of one segment, all asynchronous on the stream. The phases timed
+    are single launches: the copy, one accumulate, one segment copy."""
+
+    def __init__(self, *args):
+        super().__init__(*args)
+        self.step_bytes = sum(p[1] for p in self.phases)
+        self.step_launches = 2 * self.n - 1
+        seg = self.sizes[self.sets[0]["rs_seg"][0]]
+        self.phases = (self.phases[0],
+                       ("accumulate_one_step", seg * self.esz * 3, "rows_kernel<float, kAdd> (one segment, %d elements)" % seg),
+                       ("copy_one_step", seg * self.esz * 2, "rows_kernel<unsigned int, kCopy> (one segment, %d elements)" % seg))
+
+    def launch_step(self, k, stream, fused=False):
+        s = self.sets[k % self.nsets]
+        rc = self.L.mpic_ring_allreduce_prestaged(self.n, s["r"], self.pdt, s["inp"].data_ptr(), s["out"].data_ptr(),
+                                                  self.count, s["rs_ptrs"], s["ag_ptrs"], stream, 0)
+        if rc != 0:
+            raise RuntimeError("mpic_ring_allreduce_prestaged failed: %s" % self.L.mpic_last_error().decode())
+
+    def launch_phase(self, k, i, stream):
+        s, A, R = self.sets[k % self.nsets], self.ring_abi, self.R
+        if i == 0:
+            return super().launch_phase(k, i, stream)
+        # all n-1 launches of the phase, so that a sampled step does a whole step's
+        # work; the armed events time the first of them
+        for g, t in zip(s["rs_seg"], s["rs"]) if i == 1 else zip(s["ag_seg"], s["ag"]):
+            dst = s["out"].data_ptr() + self.starts[g] * self.esz
+            if i == 1:
+                A.check(R.ring_accumulate(self.code, dst, t.data_ptr(), self.sizes[g], stream), "accumulate")
+            else:
+                A.check(R.ring_copy_bytes(dst, t.data_ptr(), self.sizes[g] * self.esz, stream), "copy")
 
 
 class FusedResnet50(Workload):
@@ -272,6 +311,11 @@ def make_workload(name):
                              "float32 ring allreduce of one 16,777,216-element (64 MiB) tensor, N=8 virtual ranks: "
                              "in->out copy + 7 reduce-scatter accumulates + 7 allgather copies on 2,097,152-element "
                              "segments per step, peers pre-staged in HBM, buffers rotated over 8 virtual ranks (cold)")
+    if name == "allreduce_f32_64MiB_n8_per_step":
+        return RingAllreducePerStep(name, "f32", 16 * 1024 * 1024, 8, 8,
+                                    "float32 ring allreduce of one 64 MiB tensor, N=8 virtual ranks, ONE LAUNCH PER RING "
+                                    "STEP as in the reference's loop: copy + 7 accumulate launches + 7 copy launches "
+                                    "(15 per step), peers pre-staged, buffers rotated over 8 virtual ranks")
     if name in ("allreduce_i32_10000019_n6", "allreduce_i64_10000019_n6"):
         dt = name.split("_")[1]
         return RingAllreduce(name, dt, 10_000_019, 6, 12,
@@ -291,7 +335,7 @@ def make_workload(name):
 
 
 WORKLOADS = ("allreduce_f32_64MiB_n8", "allreduce_i32_10000019_n6", "allreduce_i64_10000019_n6",
-             "fused_resnet50_n8", "allgather_f32_n16", "allreduce_f32_1GiB_n64")
+             "fused_resnet50_n8", "allgather_f32_n16", "allreduce_f32_1GiB_n64", "allreduce_f32_64MiB_n8_per_step")
 
 
 def cpu_baseline(w):
@@ -437,7 +481,7 @@ def main():
         "dtype": w.dtype,
         "data": "synthetic",
         "config": {"workload": w.description, "name": w.name, "bytes_per_step": w.bytes_per_step,
-                   "launches_per_step": nph, **({"launch_options": options} if options else {})},
+                   "launches_per_step": w.step_launches or nph, **({"launch_options": options} if options else {})},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "roofline": {
             "bound": "hbm",
@@ -458,7 +502,7 @@ def main():
                    for p, t in zip(w.phases, phase_us)},
         "phases_note": "HIP events carried by each launch of every %dth step of the timed region" % SAMPLE_EVERY,
     }
-    if isinstance(w, RingAllreduce):
+    if isinstance(w, RingAllreduce) and not isinstance(w, RingAllreducePerStep):
         # the same job with the in->out copy folded into the accumulate (fewer bytes, same result)
         fused_elapsed, _ = timed(steps, min(warmup, 50), fused=True)
         if not w.check(steps - 1):
