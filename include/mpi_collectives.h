@@ -156,6 +156,58 @@ int mpic_ring_allreduce_all_ranks(int n, int dtype, const void* const* inputs,
                                   void* const* outputs, size_t count, void* stream, int flags);
 int mpic_ring_allgather_all_ranks(int n, int dtype, const void* const* inputs, const size_t* rows,
                                   size_t elems_per_row, void* const* outputs, void* stream, int flags);
+/* ---- the ring over a real transport ------------------------------------------
+ * The reference's loops exchange segments with MPI_Irecv / MPI_Send / MPI_Wait
+ * (reduce-scatter, ring.h:189-200) and MPI_Sendrecv (allgather, ring.h:221-224,
+ * 291-295) on tag TAG_TENSOR (ring.h:19). A transport supplies those calls for
+ * DEVICE buffers (GPU-aware MPI, a peer-to-peer copy engine, ...): each returns
+ * 0 on success, and all are host-blocking in MPI's sense, i.e. when `send`
+ * returns the buffer may be reused and when `wait` returns the data is in
+ * `buf`, visible to work enqueued on any stream afterwards. MPI_Sendrecv is
+ * irecv + send + wait. */
+typedef struct mpic_transport {
+  void* user;
+  int (*irecv)(void* user, void* buf, size_t bytes, int source, int tag, void** request);
+  int (*send)(void* user, const void* buf, size_t bytes, int dest, int tag);
+  int (*wait)(void* user, void* request);
+} mpic_transport;
+
+/* RingAllreduce (ring.h:136-228) for rank r of n over `transport`. `temp` is
+ * the reference's temp tensor (mpi_ops.cc:1073-1077): device memory for
+ * temp_elements elements, at least ring_temp_elements(count, n). `flags`:
+ * bits 4-7 = chunks-1 (0: every segment travels whole, the reference's
+ * structure, with the stream synchronised before each send as ring.cu.cc:69
+ * does); with 2..16 chunks a segment travels in pieces, the accumulate of a
+ * piece is enqueued as soon as it has arrived and a piece is forwarded as soon
+ * as ITS accumulate has finished, so transfers overlap the accumulates of the
+ * other pieces. When temp_elements holds two segments the pieces of successive
+ * steps alternate between the halves (a receive is posted without waiting for
+ * the previous step's accumulates). Bits 8-30 = divisor
+ * (mpic_context_set_divisor). The per-element additions and their order are
+ * those of the reference for any chunk count. Blocks the calling thread; the
+ * output is complete on return. */
+int mpic_ring_allreduce_transport(int n, int r, int dtype, const void* input, void* output, void* temp,
+                                  size_t temp_elements, size_t count, const mpic_transport* transport,
+                                  void* stream, int flags);
+/* RingAllgather (ring.h:236-301) over `transport`; `flags` as above (chunks,
+ * divisor: the own slice is divided before it is first sent). */
+int mpic_ring_allgather_transport(int n, int r, int dtype, const void* input, const size_t* rows,
+                                  size_t elems_per_row, void* output, const mpic_transport* transport,
+                                  void* stream, int flags);
+
+/* A transport between the virtual ranks of ONE process, each driven by its own
+ * thread, all on the current GPU: a send blocks until the matching receive was
+ * posted, then copies device to device. Messages between one pair of ranks on
+ * one tag match in order, as MPI's do. Every blocking call gives up after
+ * timeout_seconds (a peer that died) and returns non-zero. It stands in for
+ * xGMI / MPI where there is one GPU; it is not a fast path. */
+typedef struct mpic_loopback mpic_loopback;
+int mpic_loopback_create(int n, double timeout_seconds, mpic_loopback** loopback);
+int mpic_loopback_destroy(mpic_loopback* loopback);
+/* Fills *transport with rank `rank`'s endpoint (owned by the loopback). Call on
+ * the thread that will drive the rank, with the GPU current. */
+int mpic_loopback_endpoint(mpic_loopback* loopback, int rank, mpic_transport* transport);
+
 /* Message of the last failing mpic_ring_* call on this thread. */
 const char* mpic_last_error(void);
 

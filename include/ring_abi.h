@@ -89,6 +89,14 @@ int ring_event_create(void** event);
 int ring_event_destroy(void* event);
 int ring_event_elapsed_us(void* start, void* stop, double* us);
 int ring_time_next_launch(void* start_event, void* stop_event);
+/* Ordering between the stream and the host at a finer grain than
+ * ring_stream_synchronize: record marks the work enqueued on `stream` so far,
+ * synchronize blocks the host until that work has finished. A ring driver
+ * that hands a freshly accumulated chunk to a host-driven transport (the
+ * reference synchronises the whole stream after every kernel, ring.cu.cc:69)
+ * waits for that chunk only. */
+int ring_event_record(void* event, void* stream);
+int ring_event_synchronize(void* event);
 
 /* ---- host-side tables (no GPU involved) ---------------------------------- */
 

@@ -29,7 +29,7 @@ ROOT = os.path.dirname(HERE)
 LIB_DIR = os.path.join(HERE, "lib")
 RING_HIP_SO = os.path.join(LIB_DIR, "libring_hip.so")
 PLUGIN_SO = os.path.join(LIB_DIR, "libmpi_collectives.so")
-HOST_SOURCES = ["framework.cc", "wire.cc", "ring_driver.cc", "collective_ops.cc"]
+HOST_SOURCES = ["framework.cc", "wire.cc", "ring_driver.cc", "transport.cc", "collective_ops.cc"]
 CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-pthread", "-Wall", "-Wextra"]
 
 HIP_FLAGS = [

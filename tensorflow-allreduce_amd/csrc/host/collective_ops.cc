@@ -28,6 +28,7 @@
 #include "mpi_collectives.h"
 #include "ring_abi.h"
 #include "ring_driver.h"
+#include "transport.h"
 #include "wire.h"
 
 namespace mpic {
@@ -1055,6 +1056,25 @@ int mpic_ring_allgather_prestaged(int n, int r, int dtype, const void* input, co
   std::vector<size_t> rv(rows, rows + n);
   mpic::Status s = mpic::RingAllgatherPrestaged(n, r, static_cast<mpic::DataType>(dtype), input, rv, elems_per_row,
                                                 output, segments, stream, mpic::RingOptions::FromFlags(flags));
+  return s.ok() ? MPIC_OK : mpic::Fail(s);
+}
+
+int mpic_ring_allreduce_transport(int n, int r, int dtype, const void* input, void* output, void* temp,
+                                  size_t temp_elements, size_t count, const mpic_transport* transport, void* stream,
+                                  int flags) {
+  mpic::Status s = mpic::RingAllreduceTransport(n, r, static_cast<mpic::DataType>(dtype), input, output, temp,
+                                                temp_elements, count, transport, stream,
+                                                mpic::RingOptions::FromFlags(flags));
+  return s.ok() ? MPIC_OK : mpic::Fail(s);
+}
+
+int mpic_ring_allgather_transport(int n, int r, int dtype, const void* input, const size_t* rows,
+                                  size_t elems_per_row, void* output, const mpic_transport* transport, void* stream,
+                                  int flags) {
+  if (n < 1 || !rows) return MPIC_INVALID_ARGUMENT;
+  std::vector<size_t> rv(rows, rows + n);
+  mpic::Status s = mpic::RingAllgatherTransport(n, r, static_cast<mpic::DataType>(dtype), input, rv, elems_per_row,
+                                                output, transport, stream, mpic::RingOptions::FromFlags(flags));
   return s.ok() ? MPIC_OK : mpic::Fail(s);
 }
 

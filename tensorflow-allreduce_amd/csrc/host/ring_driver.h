@@ -30,10 +30,13 @@ struct RingOptions {
   // what then travels round the ring is already divided. Pre-staged allgather
   // segments are therefore expected divided, as a peer would send them.
   int divisor = 0;
+  // Transport-driven rings only: pieces a segment travels in (1..16).
+  int chunks = 1;
   static RingOptions FromFlags(int flags) {
     RingOptions o;
     o.batched = (flags & 1) != 0;
     o.fuse_copy = (flags & 2) != 0;
+    o.chunks = ((flags >> 4) & 15) + 1;
     o.divisor = (flags >> 8) & 0x7fffff;
     return o;
   }

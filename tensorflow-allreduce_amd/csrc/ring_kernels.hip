@@ -676,6 +676,18 @@ int ring_event_elapsed_us(void* start, void* stop, double* us) {
   return RING_OK;
 }
 
+int ring_event_record(void* event, void* stream) {
+  if (!event) return RING_ERR_ARGUMENT;
+  RING_HIP(hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream)));
+  return RING_OK;
+}
+
+int ring_event_synchronize(void* event) {
+  if (!event) return RING_ERR_ARGUMENT;
+  RING_HIP(hipEventSynchronize(static_cast<hipEvent_t>(event)));
+  return RING_OK;
+}
+
 int ring_time_next_launch(void* start_event, void* stop_event) {
   g_time_start = static_cast<hipEvent_t>(start_event);
   g_time_stop = static_cast<hipEvent_t>(stop_event);

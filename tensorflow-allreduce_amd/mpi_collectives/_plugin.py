@@ -31,8 +31,20 @@ EXPORTS = (
     "mpic_context_create", "mpic_context_add_input", "mpic_context_set_divisor", "mpic_context_compute", "mpic_context_wait",
     "mpic_context_message", "mpic_context_num_outputs", "mpic_context_output", "mpic_context_destroy",
     "mpic_ring_allreduce_prestaged", "mpic_ring_allgather_prestaged", "mpic_ring_allreduce_all_ranks",
-    "mpic_ring_allgather_all_ranks", "mpic_last_error",
+    "mpic_ring_allgather_all_ranks", "mpic_ring_allreduce_transport", "mpic_ring_allgather_transport",
+    "mpic_loopback_create", "mpic_loopback_destroy", "mpic_loopback_endpoint", "mpic_last_error",
 )
+
+
+class Transport(ctypes.Structure):
+    """mpic_transport: the MPI point-to-point calls of the reference's ring for
+    device buffers; each callback returns 0 on success."""
+    IRECV = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int,
+                             ctypes.c_int, ctypes.POINTER(ctypes.c_void_p))
+    SEND = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int,
+                            ctypes.c_int)
+    WAIT = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p)
+    _fields_ = [("user", ctypes.c_void_p), ("irecv", IRECV), ("send", SEND), ("wait", WAIT)]
 
 
 class OpError(RuntimeError):
@@ -127,6 +139,11 @@ def load_library(name="libmpi_collectives.so", op_list=None):
             "mpic_ring_allgather_prestaged": (ci, [ci, ci, ci, vp, psz, sz, vp, pvp, vp, ci]),
             "mpic_ring_allreduce_all_ranks": (ci, [ci, ci, pvp, pvp, sz, vp, ci]),
             "mpic_ring_allgather_all_ranks": (ci, [ci, ci, pvp, psz, sz, pvp, vp, ci]),
+            "mpic_ring_allreduce_transport": (ci, [ci, ci, ci, vp, vp, vp, sz, sz, ctypes.POINTER(Transport), vp, ci]),
+            "mpic_ring_allgather_transport": (ci, [ci, ci, ci, vp, psz, sz, vp, ctypes.POINTER(Transport), vp, ci]),
+            "mpic_loopback_create": (ci, [ci, ctypes.c_double, pvp]),
+            "mpic_loopback_destroy": (ci, [vp]),
+            "mpic_loopback_endpoint": (ci, [vp, ci, ctypes.POINTER(Transport)]),
             "mpic_last_error": (cp, []),
         }
         for sym in EXPORTS:

@@ -120,6 +120,33 @@ int main() {
     mpic_context_destroy(cs[r]);
   }
   CHECK(mpic_world_destroy(w) == MPIC_OK);
+
+  // the in-process transport under concurrent ranks: every rank posts its
+  // receives, sends to the right and waits, as the ring's steps do (zero-byte
+  // messages: no device is touched)
+  {
+    mpic_loopback* lb = nullptr;
+    CHECK(mpic_loopback_create(kRanks, 30.0, &lb) == MPIC_OK);
+    std::atomic<int> exchanged{0};
+    std::vector<std::thread> ranks;
+    for (int r = 0; r < kRanks; r++) {
+      ranks.emplace_back([lb, r, kRanks, &exchanged] {
+        mpic_transport t;
+        CHECK(mpic_loopback_endpoint(lb, r, &t) == MPIC_OK);
+        const int left = (r - 1 + kRanks) % kRanks, right = (r + 1) % kRanks;
+        for (int step = 0; step < 300; step++) {
+          void* reqs[3];
+          for (int c = 0; c < 3; c++) CHECK(t.irecv(t.user, nullptr, 0, left, 12, &reqs[c]) == 0);
+          for (int c = 0; c < 3; c++) CHECK(t.send(t.user, nullptr, 0, right, 12) == 0);
+          for (int c = 0; c < 3; c++) CHECK(t.wait(t.user, reqs[c]) == 0);
+          exchanged++;
+        }
+      });
+    }
+    for (auto& t : ranks) t.join();
+    CHECK(exchanged == kRanks * 300);
+    CHECK(mpic_loopback_destroy(lb) == MPIC_OK);
+  }
   std::printf("ok\n");
   return 0;
 }

@@ -24,7 +24,7 @@ def test_coordinator_under_thread_sanitizer(tmp_path):
     submitted collectives fail the cross-rank checks before any device work."""
     exe = str(tmp_path / "coordinator_test")
     lib_dir = os.path.join(ROOT, "tensorflow-allreduce_amd", "lib")
-    sources = [os.path.join(HOST, f) for f in ("framework.cc", "wire.cc", "ring_driver.cc", "collective_ops.cc")]
+    sources = [os.path.join(HOST, f) for f in ("framework.cc", "wire.cc", "ring_driver.cc", "transport.cc", "collective_ops.cc")]
     subprocess.run(["g++", "-std=c++17", "-O1", "-g", "-Wall", "-Wextra", "-fsanitize=thread", "-pthread",
                     "-I", HOST, "-I", os.path.join(ROOT, "include"), "-o", exe,
                     os.path.join(ROOT, "tests", "cpp", "coordinator_test.cc")] + sources +

@@ -262,6 +262,47 @@ def test_fused_divisor_arguments_and_failure_drain():
         assert not s._pending and not s._submitted
 
 
+def test_loopback_transport_matches_messages_and_times_out():
+    """Host-side behaviour of the in-process transport: argument checks, a wait
+    or a send without a peer gives up after the timeout, zero-byte messages
+    match in order without touching a device."""
+    import time
+    L = _plugin.load_library()
+    h = ctypes.c_void_p()
+    assert L.mpic_loopback_create(0, 1.0, ctypes.byref(h)) == 3
+    assert L.mpic_loopback_create(2, 0.0, ctypes.byref(h)) == 3
+    assert L.mpic_loopback_create(2, 0.2, ctypes.byref(h)) == 0
+    try:
+        t0, t1 = _plugin.Transport(), _plugin.Transport()
+        assert L.mpic_loopback_endpoint(h.value, 2, ctypes.byref(t0)) == 3
+        assert L.mpic_loopback_endpoint(h.value, 0, ctypes.byref(t0)) == 0
+        assert L.mpic_loopback_endpoint(h.value, 1, ctypes.byref(t1)) == 0
+        req = ctypes.c_void_p()
+        assert t0.irecv(t0.user, None, 8, 1, 12, ctypes.byref(req)) != 0          # bytes without a buffer
+        assert t0.irecv(t0.user, None, 0, 5, 12, ctypes.byref(req)) != 0          # no such rank
+        began = time.perf_counter()
+        assert t0.send(t0.user, None, 0, 1, 12) != 0                              # nobody receives
+        assert 0.15 < time.perf_counter() - began < 5.0
+        assert t1.irecv(t1.user, None, 0, 0, 12, ctypes.byref(req)) == 0
+        first = req.value
+        assert t1.irecv(t1.user, None, 0, 0, 12, ctypes.byref(req)) == 0
+        assert t1.wait(t1.user, req.value) != 0                                   # second message never sent
+        assert t0.send(t0.user, None, 0, 1, 12) == 0
+        assert t1.wait(t1.user, first) == 0
+        assert t0.send(t0.user, None, 0, 1, 7) != 0                               # other tag: no match
+    finally:
+        L.mpic_loopback_destroy(h.value)
+    # the ring over a transport checks its arguments before it touches the device
+    bad = _plugin.Transport()
+    x = ctypes.create_string_buffer(64)
+    addr = ctypes.addressof(x)
+    assert L.mpic_ring_allreduce_transport(2, 0, _plugin.DT_FLOAT, addr, addr, addr, 8, 16, None, None, 0) == 3
+    assert L.mpic_ring_allreduce_transport(2, 0, _plugin.DT_FLOAT, addr, addr, addr, 8, 16, ctypes.byref(bad), None, 0) == 3
+    assert L.mpic_ring_allreduce_transport(2, 2, _plugin.DT_FLOAT, addr, addr, addr, 8, 16, ctypes.byref(bad), None, 0) == 3
+    assert L.mpic_ring_allreduce_transport(2, 0, _plugin.DT_DOUBLE, addr, addr, addr, 8, 16, ctypes.byref(bad), None, 0) == 9
+    assert b"Invalid tensor type" in L.mpic_last_error()
+
+
 def test_node_names_are_uniquified_like_graph_nodes():
     with mpi.Session(size=2, device="CPU") as s:
         assert [s._node_name(0, 'MPIAllreduce', None) for _ in range(3)] == \
