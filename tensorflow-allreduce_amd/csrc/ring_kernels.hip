@@ -21,7 +21,11 @@
 //     the destination is aligned, the sources are read with element-aligned
 //     (possibly 16-byte-unaligned) dwordx4 loads. Ragged segment starts only
 //     cost those few scalar elements;
-//   * every byte is touched once, so loads and stores are non-temporal;
+//   * what is touched once (accumulates, allgather copies, unpack) is loaded
+//     and stored non-temporally; the in->out copy and the fusion pack, whose
+//     output the reduce-scatter reads next, store with the ordinary policy;
+//   * the average's divide rides on the accumulate that completes a segment
+//     (or on the unpack), never on a pass of its own;
 //   * LDS is used only by the fusion kernels, for the offset table of a tile
 //     that spans several small tensors.
 // No MFMA: the path is one add per 12 bytes.
