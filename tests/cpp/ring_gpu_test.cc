@@ -9,7 +9,9 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <atomic>
 #include <random>
+#include <thread>
 #include <vector>
 
 #include "mpi_collectives.h"
@@ -111,6 +113,40 @@ static void ring_case(int n, size_t count, void* stream) {
   }
   CHECK(mpic_ring_allreduce_all_ranks(n, Code<T>::mpic, d_ins.data(), d_outs.data(), count, stream, 1) == MPIC_OK);
   CHECK(ring_stream_synchronize(stream) == RING_OK);
+  for (int r = 0; r < n; r++)
+    CHECK(std::memcmp(to_host(static_cast<T*>(d_outs[r]), count).data(), want[r].data(), count * sizeof(T)) == 0);
+
+  // (3) one thread per rank, segments exchanged through the loopback transport
+  // in 4 pieces with a two-segment temp: the reference's loop, pipelined
+  mpic_loopback* lb = nullptr;
+  CHECK(mpic_loopback_create(n, 30.0, &lb) == MPIC_OK);
+  std::vector<T*> d_temp(n);
+  for (int r = 0; r < n; r++) {
+    HIP_OK(hipMemset(d_outs[r], 0, count * sizeof(T)));
+    d_temp[r] = to_device(std::vector<T>(2 * slot + 1));
+  }
+  HIP_OK(hipDeviceSynchronize());
+  std::atomic<int> failures{0};
+  std::vector<std::thread> threads;
+  for (int r = 0; r < n; r++) {
+    threads.emplace_back([&, r] {
+      mpic_transport t;
+      void* own_stream = nullptr;
+      if (mpic_loopback_endpoint(lb, r, &t) != MPIC_OK || ring_stream_create(&own_stream) != RING_OK) {
+        failures++;
+        return;
+      }
+      if (mpic_ring_allreduce_transport(n, r, Code<T>::mpic, d_ins[r], d_outs[r], d_temp[r], 2 * slot, count, &t,
+                                        own_stream, (4 - 1) << 4) != MPIC_OK) {
+        std::fprintf(stderr, "rank %d: %s\n", r, mpic_last_error());
+        failures++;
+      }
+      ring_stream_destroy(own_stream);
+    });
+  }
+  for (auto& th : threads) th.join();
+  CHECK(failures == 0);
+  CHECK(mpic_loopback_destroy(lb) == MPIC_OK);
   for (int r = 0; r < n; r++)
     CHECK(std::memcmp(to_host(static_cast<T*>(d_outs[r]), count).data(), want[r].data(), count * sizeof(T)) == 0);
 }
