@@ -27,10 +27,15 @@ def _gpu():
 
 @settings(max_examples=60, **COMMON)
 @given(n=st.integers(1, 9), count=counts, dtype=st.sampled_from(G.DTYPES), seed=st.integers(0, 2**31),
-       offs=st.lists(st.integers(0, 3), min_size=2, max_size=2))
-def test_all_ranks_ring_equals_oracle(oracle, n, count, dtype, seed, offs):
+       offs=st.lists(st.integers(0, 3), min_size=2, max_size=2), divisor=st.sampled_from([0, 0, 1, 2, 3, 7, 8, 64]))
+def test_all_ranks_ring_equals_oracle(oracle, n, count, dtype, seed, offs, divisor):
+    """Sum, or (divisor > 0) the average folded into the last accumulate:
+    tf.div of the oracle's sum."""
     ins = [G.random_array(np.random.default_rng(seed + r), count, dtype, wide=True) for r in range(n)]
     want = oracle.ring_allreduce_lockstep(ins)
+    if divisor:
+        with np.errstate(all="ignore"):
+            want = [(w / np.float32(divisor) if dtype == np.float32 else w // dtype(divisor)).astype(dtype) for w in want]
     L = _plugin.load_library()
     dins, douts, keep = [], [], []
     for r in range(n):
@@ -42,11 +47,12 @@ def test_all_ranks_ring_equals_oracle(oracle, n, count, dtype, seed, offs):
     pin = (ctypes.c_void_p * n)(*[t.data_ptr() if count else None for t in dins])
     pout = (ctypes.c_void_p * n)(*[t.data_ptr() if count else None for t in douts])
     rc = L.mpic_ring_allreduce_all_ranks(n, DT[np.dtype(dtype)], pin, pout, count,
-                                         torch.cuda.current_stream().cuda_stream, 1)
+                                         torch.cuda.current_stream().cuda_stream, 1 | (divisor << 8))
     assert rc == 0, L.mpic_last_error()
     torch.cuda.synchronize()
     for r in range(n):
-        G.assert_same_bits(G.host(douts[r]), want[r], "n=%d count=%d %s rank %d" % (n, count, dtype.__name__, r))
+        G.assert_same_bits(G.host(douts[r]), want[r],
+                           "n=%d count=%d %s rank %d /%d" % (n, count, dtype.__name__, r, divisor))
 
 
 @settings(max_examples=40, **COMMON)
