@@ -435,9 +435,16 @@ def main():
     # let the queue drain and the sampled launches start on an idle GPU
     event_pool = [[ring_abi.event_create() for _ in range(2 * nph)] for _ in range(steps // SAMPLE_EVERY + 1)]
 
-    def timed(nsteps, nwarm, fused=False, with_samples=False):
+    def timed(nsteps, nwarm, fused=False, with_samples=False, hot=False):
+        # hot: the same buffer set every step (what fits stays in the last-level
+        # cache); otherwise the sets rotate and every step starts cold
+        if hot:
+            def launch_step(k, stream, fused):
+                w.launch_step(0, stream, fused)
+        else:
+            launch_step = w.launch_step
         for k in range(nwarm):
-            w.launch_step(k, stream, fused)
+            launch_step(k, stream, fused)
         ring_abi.stream_synchronize(stream)
         torch.cuda.synchronize()
         samples = []
@@ -452,7 +459,7 @@ def main():
                     w.launch_phase(k, i, stream)
                 samples.append(e)
             else:
-                w.launch_step(k, stream, fused)
+                launch_step(k, stream, fused)
         ring_abi.stream_synchronize(stream)
         torch.cuda.synchronize()
         return time.perf_counter() - t0, samples
@@ -462,8 +469,8 @@ def main():
         sys.exit("bench.py: the output of the timed path is wrong; refusing to report a number")
     ms_per_step = elapsed / steps * 1e3
     value = w.bytes_per_step * steps / elapsed / 1e9
-    phase_us = [statistics.mean(ring_abi.event_elapsed_us(e[2 * i], e[2 * i + 1]) for e in samples)
-                for i in range(nph)]
+    phase_times = [[ring_abi.event_elapsed_us(e[2 * i], e[2 * i + 1]) for e in samples] for i in range(nph)]
+    phase_us = [statistics.mean(t) for t in phase_times]
     dom = w.phases[w.dominant]
     achieved = dom[1] / phase_us[w.dominant] / 1e3
 
@@ -498,10 +505,21 @@ def main():
                     "buffer the in->out copy has just written, so part of its reads can come from the last-level "
                     "cache instead of HBM",
         },
-        "phases": {p[0]: {"us": round(t, 3), "GBps": round(p[1] / t / 1e3, 1), "bytes": p[1]}
-                   for p, t in zip(w.phases, phase_us)},
-        "phases_note": "HIP events carried by each launch of every %dth step of the timed region" % SAMPLE_EVERY,
+        "phases": {p[0]: {"us": round(t, 3), "median_us": round(statistics.median(phase_times[i]), 3),
+                          "min_us": round(min(phase_times[i]), 3), "GBps": round(p[1] / t / 1e3, 1),
+                          "bytes": p[1]}
+                   for i, (p, t) in enumerate(zip(w.phases, phase_us))},
+        "phases_note": "HIP events carried by each launch of every %dth step of the timed region; us = mean"
+                       % SAMPLE_EVERY,
     }
+    # the same steps on ONE buffer set: at the headline size the working set fits the
+    # last-level cache, so this is the cache-resident rate, not the HBM one
+    hot_steps = max(steps // 4, 1)
+    hot_elapsed, _ = timed(hot_steps, min(warmup, 50), hot=True)
+    result["hot"] = {"ms_per_step": round(hot_elapsed / hot_steps * 1e3, 5),
+                     "GBps": round(w.bytes_per_step * hot_steps / hot_elapsed / 1e9, 1),
+                     "note": "every step on the same buffers (%.0f MiB touched per step); `value` is the cold rate, "
+                             "buffer sets rotated" % (w.bytes_per_step / 2**20)}
     if isinstance(w, RingAllreduce) and not isinstance(w, RingAllreducePerStep):
         # the same job with the in->out copy folded into the accumulate (fewer bytes, same result)
         fused_elapsed, _ = timed(steps, min(warmup, 50), fused=True)
