@@ -164,12 +164,17 @@ int mpic_ring_allgather_all_ranks(int n, int dtype, const void* const* inputs, c
  * 0 on success, and all are host-blocking in MPI's sense, i.e. when `send`
  * returns the buffer may be reused and when `wait` returns the data is in
  * `buf`, visible to work enqueued on any stream afterwards. MPI_Sendrecv is
- * irecv + send + wait. */
+ * irecv + send + wait. `wait` consumes the request whether it succeeds or not.
+ * `cancel` (MPI_Cancel + MPI_Request_free; may be NULL) abandons a request that
+ * will not be waited for: when a collective ends early with an error the
+ * driver cancels what it had posted, and after the call the transport must no
+ * longer write to that receive's buffer. */
 typedef struct mpic_transport {
   void* user;
   int (*irecv)(void* user, void* buf, size_t bytes, int source, int tag, void** request);
   int (*send)(void* user, const void* buf, size_t bytes, int dest, int tag);
   int (*wait)(void* user, void* request);
+  int (*cancel)(void* user, void* request);
 } mpic_transport;
 
 /* RingAllreduce (ring.h:136-228) for rank r of n over `transport`. `temp` is

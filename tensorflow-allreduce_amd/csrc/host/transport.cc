@@ -77,6 +77,32 @@ class PieceEvents {
   std::vector<void*> events_;
 };
 
+// Receives posted and not yet waited for. A wait consumes its request whether
+// it succeeds or not; whatever is still outstanding when the collective ends
+// early is cancelled, so the transport stops touching the caller's buffers.
+class Requests {
+ public:
+  Requests(const mpic_transport* t, int n) : t_(t), reqs_(static_cast<size_t>(n), nullptr) {}
+  ~Requests() {
+    for (void* r : reqs_)
+      if (r && t_ && t_->cancel) t_->cancel(t_->user, r);
+  }
+  Requests(const Requests&) = delete;
+  Requests& operator=(const Requests&) = delete;
+  void** slot(int c) { return &reqs_[static_cast<size_t>(c)]; }
+  bool pending(int c) const { return reqs_[static_cast<size_t>(c)] != nullptr; }
+  int Wait(int c) {
+    void* r = reqs_[static_cast<size_t>(c)];
+    reqs_[static_cast<size_t>(c)] = nullptr;
+    return t_->wait(t_->user, r);
+  }
+  void swap(Requests& other) { reqs_.swap(other.reqs_); }
+
+ private:
+  const mpic_transport* t_;
+  std::vector<void*> reqs_;
+};
+
 inline char* At(void* base, size_t elems, size_t esz) { return static_cast<char*>(base) + elems * esz; }
 inline void* OrNull(char* p, size_t count) { return count ? p : nullptr; }
 
@@ -135,7 +161,7 @@ Status RingAllreduceTransport(int n, int r, DataType dt, const void* input, void
   const bool two_halves = pieces && temp_elements >= 2 * max_seg;
   PieceEvents done;
   if (pieces) DEVICE_REQUIRES_OK(done.Create(chunks), "ring_event_create");
-  std::vector<void*> requests(static_cast<size_t>(chunks), nullptr);
+  Requests requests(t, chunks);
 
   // ring.h:183-205: at step i send segment (r-i), receive segment (r-i-1) into
   // temp and add it into the buffer.
@@ -154,7 +180,7 @@ Status RingAllreduceTransport(int n, int r, DataType dt, const void* input, void
     for (int c = 0; c < chunks; c++) {
       const Piece& p = recv_pieces[static_cast<size_t>(c)];
       MPI_REQUIRES_OK(t->irecv(t->user, OrNull(At(half, p.offset, esz), p.count), p.count * esz, recv_from,
-                               kTagTensor, &requests[static_cast<size_t>(c)]),
+                               kTagTensor, requests.slot(c)),
                       "MPI_Irecv", i);
     }
     for (int c = 0; c < chunks; c++) {
@@ -168,8 +194,7 @@ Status RingAllreduceTransport(int n, int r, DataType dt, const void* input, void
     }
     for (int c = 0; c < chunks; c++) {
       const Piece& p = recv_pieces[static_cast<size_t>(c)];
-      MPI_REQUIRES_OK(t->wait(t->user, requests[static_cast<size_t>(c)]), "MPI_Wait", i);
-      requests[static_cast<size_t>(c)] = nullptr;
+      MPI_REQUIRES_OK(requests.Wait(c), "MPI_Wait", i);
       if (p.count) {
         char* dst = At(output, starts[recv_seg] + p.offset, esz);
         // the last step completes the segment this rank owns: the average's divide rides on it
@@ -189,7 +214,7 @@ Status RingAllreduceTransport(int n, int r, DataType dt, const void* input, void
   // straight into the buffer (MPI_Sendrecv = receive posted, send, wait). A
   // piece is forwarded once it has arrived; the wait for step i's pieces is
   // therefore made at step i+1, just before each is sent on.
-  std::vector<void*> previous(static_cast<size_t>(chunks), nullptr);
+  Requests previous(t, chunks);
   for (int i = 0; i < n - 1; i++) {
     const size_t send_seg = static_cast<size_t>(((r - i + 1) % n + n) % n);
     const size_t recv_seg = static_cast<size_t>(((r - i) % n + n) % n);
@@ -198,7 +223,7 @@ Status RingAllreduceTransport(int n, int r, DataType dt, const void* input, void
     for (int c = 0; c < chunks; c++) {
       const Piece& p = recv_pieces[static_cast<size_t>(c)];
       MPI_REQUIRES_OK(t->irecv(t->user, OrNull(At(output, starts[recv_seg] + p.offset, esz), p.count),
-                               p.count * esz, recv_from, kTagTensor, &requests[static_cast<size_t>(c)]),
+                               p.count * esz, recv_from, kTagTensor, requests.slot(c)),
                       "MPI_Sendrecv", i);
     }
     for (int c = 0; c < chunks; c++) {
@@ -208,8 +233,7 @@ Status RingAllreduceTransport(int n, int r, DataType dt, const void* input, void
         if (two_halves)
           DEVICE_REQUIRES_OK(ring_event_synchronize(done[static_cast<size_t>(c)]), "ring_event_synchronize");
       } else {
-        MPI_REQUIRES_OK(t->wait(t->user, previous[static_cast<size_t>(c)]), "MPI_Sendrecv", i - 1);
-        previous[static_cast<size_t>(c)] = nullptr;
+        MPI_REQUIRES_OK(previous.Wait(c), "MPI_Sendrecv", i - 1);
       }
       MPI_REQUIRES_OK(t->send(t->user, OrNull(At(output, starts[send_seg] + p.offset, esz), p.count),
                               p.count * esz, send_to, kTagTensor),
@@ -218,8 +242,7 @@ Status RingAllreduceTransport(int n, int r, DataType dt, const void* input, void
     previous.swap(requests);
   }
   for (int c = 0; c < chunks; c++) {
-    if (previous[static_cast<size_t>(c)])
-      MPI_REQUIRES_OK(t->wait(t->user, previous[static_cast<size_t>(c)]), "MPI_Sendrecv", n - 2);
+    if (previous.pending(c)) MPI_REQUIRES_OK(previous.Wait(c), "MPI_Sendrecv", n - 2);
   }
   return Status::OK();
 }
@@ -259,7 +282,7 @@ Status RingAllgatherTransport(int n, int r, DataType dt, const void* input, cons
   const int recv_from = (r - 1 + n) % n;
   const int send_to = (r + 1) % n;
   // ring.h:279-298: at step i send segment (r-i), receive segment (r-i-1).
-  std::vector<void*> requests(static_cast<size_t>(chunks), nullptr), previous(static_cast<size_t>(chunks), nullptr);
+  Requests requests(t, chunks), previous(t, chunks);
   for (int i = 0; i < n - 1; i++) {
     const size_t send_seg = static_cast<size_t>(((r - i) % n + n) % n);
     const size_t recv_seg = static_cast<size_t>(((r - i - 1) % n + n) % n);
@@ -268,14 +291,13 @@ Status RingAllgatherTransport(int n, int r, DataType dt, const void* input, cons
     for (int c = 0; c < chunks; c++) {
       const Piece& p = recv_pieces[static_cast<size_t>(c)];
       MPI_REQUIRES_OK(t->irecv(t->user, OrNull(At(output, starts[recv_seg] + p.offset, esz), p.count),
-                               p.count * esz, recv_from, kTagTensor, &requests[static_cast<size_t>(c)]),
+                               p.count * esz, recv_from, kTagTensor, requests.slot(c)),
                       "MPI_Sendrecv", i);
     }
     for (int c = 0; c < chunks; c++) {
       const Piece& p = send_pieces[static_cast<size_t>(c)];
       if (i > 0) {
-        MPI_REQUIRES_OK(t->wait(t->user, previous[static_cast<size_t>(c)]), "MPI_Sendrecv", i - 1);
-        previous[static_cast<size_t>(c)] = nullptr;
+        MPI_REQUIRES_OK(previous.Wait(c), "MPI_Sendrecv", i - 1);
       }
       MPI_REQUIRES_OK(t->send(t->user, OrNull(At(output, starts[send_seg] + p.offset, esz), p.count),
                               p.count * esz, send_to, kTagTensor),
@@ -284,8 +306,7 @@ Status RingAllgatherTransport(int n, int r, DataType dt, const void* input, cons
     previous.swap(requests);
   }
   for (int c = 0; c < chunks; c++) {
-    if (previous[static_cast<size_t>(c)])
-      MPI_REQUIRES_OK(t->wait(t->user, previous[static_cast<size_t>(c)]), "MPI_Sendrecv", n - 2);
+    if (previous.pending(c)) MPI_REQUIRES_OK(previous.Wait(c), "MPI_Sendrecv", n - 2);
   }
   return Status::OK();
 }
@@ -306,6 +327,7 @@ constexpr int kLoopbackArgument = 4;
 struct PostedReceive {
   void* buf = nullptr;
   size_t bytes = 0;
+  std::tuple<int, int, int> key;  // (source, destination, tag): the queue it waits in
   bool done = false;
   int status = 0;
 };
@@ -337,6 +359,21 @@ std::chrono::system_clock::time_point Deadline(const mpic_loopback* w) {
          std::chrono::duration_cast<std::chrono::system_clock::duration>(w->timeout);
 }
 
+// Takes a receive nobody will wait for out of its queue. If a sender has already
+// claimed it, its copy is under way: wait (bounded) until that has finished, so
+// that on return the buffer is no longer written.
+void Withdraw(mpic_loopback* w, const std::shared_ptr<PostedReceive>& p, std::unique_lock<std::mutex>* lock) {
+  if (p->done) return;
+  auto& queue = w->posted[p->key];
+  for (auto it = queue.begin(); it != queue.end(); ++it) {
+    if (it->get() == p.get()) {
+      queue.erase(it);
+      return;
+    }
+  }
+  w->cv.wait_until(*lock, Deadline(w), [&] { return p->done; });
+}
+
 int LoopbackIrecv(void* user, void* buf, size_t bytes, int source, int tag, void** request) {
   LoopbackEndpoint* ep = static_cast<LoopbackEndpoint*>(user);
   mpic_loopback* w = ep->world;
@@ -344,9 +381,10 @@ int LoopbackIrecv(void* user, void* buf, size_t bytes, int source, int tag, void
   auto p = std::make_shared<PostedReceive>();
   p->buf = buf;
   p->bytes = bytes;
+  p->key = std::make_tuple(source, ep->rank, tag);
   {
     std::lock_guard<std::mutex> guard(w->mu);
-    w->posted[std::make_tuple(source, ep->rank, tag)].push_back(p);
+    w->posted[p->key].push_back(p);
   }
   w->cv.notify_all();
   *request = new std::shared_ptr<PostedReceive>(p);
@@ -390,8 +428,20 @@ int LoopbackWait(void* user, void* request) {
   std::unique_ptr<std::shared_ptr<PostedReceive>> holder(static_cast<std::shared_ptr<PostedReceive>*>(request));
   std::shared_ptr<PostedReceive> p = *holder;
   std::unique_lock<std::mutex> lock(w->mu);
-  if (!w->cv.wait_until(lock, Deadline(w), [&] { return p->done; })) return kLoopbackTimeout;
-  return p->status;
+  if (w->cv.wait_until(lock, Deadline(w), [&] { return p->done; })) return p->status;
+  Withdraw(w, p, &lock);
+  return kLoopbackTimeout;
+}
+
+// MPI_Cancel + MPI_Request_free for a receive that will not be waited for.
+int LoopbackCancel(void* user, void* request) {
+  LoopbackEndpoint* ep = static_cast<LoopbackEndpoint*>(user);
+  mpic_loopback* w = ep->world;
+  if (!request) return kLoopbackArgument;
+  std::unique_ptr<std::shared_ptr<PostedReceive>> holder(static_cast<std::shared_ptr<PostedReceive>*>(request));
+  std::unique_lock<std::mutex> lock(w->mu);
+  Withdraw(w, *holder, &lock);
+  return 0;
 }
 
 }  // namespace
@@ -429,6 +479,7 @@ int mpic_loopback_endpoint(mpic_loopback* w, int rank, mpic_transport* transport
   transport->irecv = LoopbackIrecv;
   transport->send = LoopbackSend;
   transport->wait = LoopbackWait;
+  transport->cancel = LoopbackCancel;
   return MPIC_OK;
 }
 

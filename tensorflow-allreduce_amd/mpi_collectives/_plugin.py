@@ -44,7 +44,7 @@ class Transport(ctypes.Structure):
     SEND = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int,
                             ctypes.c_int)
     WAIT = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p)
-    _fields_ = [("user", ctypes.c_void_p), ("irecv", IRECV), ("send", SEND), ("wait", WAIT)]
+    _fields_ = [("user", ctypes.c_void_p), ("irecv", IRECV), ("send", SEND), ("wait", WAIT), ("cancel", WAIT)]
 
 
 class OpError(RuntimeError):

@@ -290,6 +290,14 @@ def test_loopback_transport_matches_messages_and_times_out():
         assert t0.send(t0.user, None, 0, 1, 12) == 0
         assert t1.wait(t1.user, first) == 0
         assert t0.send(t0.user, None, 0, 1, 7) != 0                               # other tag: no match
+        # a cancelled receive is gone: the next send finds nothing to match
+        assert t1.irecv(t1.user, None, 0, 0, 12, ctypes.byref(req)) == 0
+        assert t1.cancel(t1.user, req.value) == 0
+        assert t0.send(t0.user, None, 0, 1, 12) != 0
+        # so is one whose wait timed out
+        assert t1.irecv(t1.user, None, 0, 0, 12, ctypes.byref(req)) == 0
+        assert t1.wait(t1.user, req.value) != 0
+        assert t0.send(t0.user, None, 0, 1, 12) != 0
     finally:
         L.mpic_loopback_destroy(h.value)
     # the ring over a transport checks its arguments before it touches the device
