@@ -74,8 +74,9 @@ int mpic_world_size(const mpic_world* world);
  * a hipStream_t. Valid after MPIInit has run. */
 void* mpic_world_stream(const mpic_world* world);
 /* Options: "batched" (1: one launch per ring phase, 0: one launch per ring
- * step as in ring.h:183-225), "fuse_copy" (1: fold the in->out copy of
- * ring.h:146-148 into the reduce-scatter), "sync" (1: done() is called after
+ * step as in ring.h:183-225; default 1), "fuse_copy" (1: fold the in->out copy
+ * of ring.h:146-148 into the reduce-scatter, out[seg] = in[seg] + received, the
+ * same single add; default 1), "sync" (1: done() is called after
  * the stream has drained, 0: as soon as the work is enqueued). */
 int mpic_world_set_option(mpic_world* world, const char* name, int value);
 

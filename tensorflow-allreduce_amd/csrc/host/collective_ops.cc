@@ -87,7 +87,9 @@ struct mpic_world {
   int real_rank = -1;  // -1: every rank lives in this process
   int device = -1;     // -1 for no GPU
   void* stream = nullptr;
-  mpic::RingOptions ring_options;
+  // a world folds the in->out copy into the reduce-scatter unless told otherwise
+  // (same results, a third fewer bytes)
+  mpic::RingOptions ring_options = [] { mpic::RingOptions o; o.fuse_copy = true; return o; }();
   bool sync_on_done = true;
   // Tensor fusion in the coordinator: allreduces that are ready in the same
   // tick are packed, per rank, into that rank's slice of this caller-owned

@@ -209,16 +209,26 @@ Status RingAllreduceAllRanks(int n, DataType dt, const void* const* inputs, void
   RING_RETURN_IF_ERROR(ring_segment_table(count, n, sizes.data(), starts.data()), "ring_segment_table");
 
   std::vector<ring_row> rows(static_cast<size_t>(n));
-  // ring.h:146-148 on every rank
-  for (int r = 0; r < n; r++) {
+  for (int r = 0; r < n; r++)
     if (!inputs[r] || !outputs[r]) return errors::InvalidArgument("null tensor with a non-zero element count");
-    // a rank reducing in place (a fusion buffer) has nothing to copy
-    const bool nothing = inputs[r] == outputs[r] && !(n == 1 && opts.divisor > 0);
-    rows[static_cast<size_t>(r)] = ring_row{outputs[r], inputs[r], nullptr, nothing ? 0 : count};
+  // Without the in->out copy (ring.h:146-148): every segment of a rank's output
+  // is written by one of the 2(n-1) steps anyway (the reduce-scatter writes all
+  // but segment r, the allgather all but segment r+1), and a rank accumulates
+  // into each segment once, so the local operand of that add is still the
+  // untouched input: out[seg] = in[seg] + received is the same single add. What
+  // is received at step 0 is the neighbour's own segment, which it never
+  // accumulates into: its input. n == 1 has no steps and keeps the copy.
+  const bool fuse = opts.fuse_copy && n > 1;
+  if (!fuse) {
+    for (int r = 0; r < n; r++) {
+      // a rank reducing in place (a fusion buffer) has nothing to copy
+      const bool nothing = inputs[r] == outputs[r] && !(n == 1 && opts.divisor > 0);
+      rows[static_cast<size_t>(r)] = ring_row{outputs[r], inputs[r], nullptr, nothing ? 0 : count};
+    }
+    // a lone rank owns every element: its copy is where the divide happens
+    RING_RETURN_IF_ERROR(ring_apply_rows_avg(rows.data(), n, nullptr, n == 1 ? opts.divisor : 0, code, stream),
+                         "ring_apply_rows");
   }
-  // a lone rank owns every element: its copy is where the divide happens
-  RING_RETURN_IF_ERROR(ring_apply_rows_avg(rows.data(), n, nullptr, n == 1 ? opts.divisor : 0, code, stream),
-                       "ring_apply_rows");
 
   // ring.h:183-205: at step i rank r adds its left neighbour's segment (r-i-1)
   for (int i = 0; i < n - 1; i++) {
@@ -226,7 +236,10 @@ Status RingAllreduceAllRanks(int n, DataType dt, const void* const* inputs, void
       const int left = (r - 1 + n) % n;
       const size_t seg = static_cast<size_t>(Seg(RING_PHASE_REDUCE_SCATTER, n, r, i, true));
       char* dst = at(outputs[r], starts[seg], esz);
-      rows[static_cast<size_t>(r)] = ring_row{dst, at(static_cast<const void*>(outputs[left]), starts[seg], esz), dst, sizes[seg]};
+      const void* local = fuse ? static_cast<const void*>(at(inputs[r], starts[seg], esz)) : dst;
+      const void* received = (fuse && i == 0) ? at(inputs[left], starts[seg], esz)
+                                              : at(static_cast<const void*>(outputs[left]), starts[seg], esz);
+      rows[static_cast<size_t>(r)] = ring_row{dst, received, local, sizes[seg]};
     }
     // the last step completes every rank's owned segment: all of its rows divide
     RING_RETURN_IF_ERROR(ring_apply_rows_avg(rows.data(), n, nullptr, i == n - 2 ? opts.divisor : 0, code, stream),

@@ -46,15 +46,19 @@ def test_allreduce_all_ranks_matches_oracle(oracle, dtype, n):
     for count in sorted({0, 1, max(n - 1, 0), n, n + 1, 17, 4913, 1_000_003}):
         ins = make_inputs(n, count, dtype, seed=31 * n + count)
         want = oracle.ring_allreduce(ins)
-        with mpi.Session(size=n) as session:
-            handles = []
+        for fuse in (1, 0):          # without / with the in->out copy as a launch of its own
+            with mpi.Session(size=n) as session:
+                session.set_option("fuse_copy", fuse)
+                handles, dins = [], [cuda(x) for x in ins]
+                for r in range(n):
+                    with session.as_rank(r):
+                        assert mpi.rank() == r
+                        handles.append(mpi.allreduce(dins[r], average=False))
+                outs = session.run(handles)
             for r in range(n):
-                with session.as_rank(r):
-                    assert mpi.rank() == r
-                    handles.append(mpi.allreduce(cuda(ins[r]), average=False))
-            outs = session.run(handles)
-        for r in range(n):
-            G.assert_same_bits(G.host(outs[r]), want[r], "allreduce %s n=%d count=%d rank %d" % (dtype.__name__, n, count, r))
+                G.assert_same_bits(G.host(outs[r]), want[r], "allreduce %s n=%d count=%d rank %d fuse=%d"
+                                   % (dtype.__name__, n, count, r, fuse))
+                G.assert_same_bits(G.host(dins[r]), ins[r], "the input is never written")
 
 
 @pytest.mark.parametrize("size", [1, 2, 3, 4, 7, 9, 12, 14])
