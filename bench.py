@@ -139,7 +139,7 @@ class RingAllreduce(Workload):
             ("allgather", ag_elems * esz * 2,
              "rows_kernel<%s, kCopy> (batched allgather copies, %d rows, %d elements)" % (carrier, n - 1, ag_elems)))
         self.dominant = 1
-        self.fused_bytes = rs_elems * esz * 3 + self.sizes[s0["r"]] * esz * 2 + ag_elems * esz * 2
+        self.fused_bytes = rs_elems * esz * 3 + ag_elems * esz * 2
         self.description = what
 
     def launch_step(self, k, stream, fused=False):
@@ -403,6 +403,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--workload", default=WORKLOADS[0], choices=WORKLOADS)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--variant", choices=("all", "reference", "fused"), default="all",
+                    help="all: the reference-shaped path (the reported value), then the extras: the same job with "
+                         "the in->out copy folded into the accumulate, and the hot (one buffer set) rate. "
+                         "reference / fused: that path alone, for kernel traces (kernel names do not tell the two "
+                         "accumulates apart, and the extras would mix into the per-kernel averages)")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="launch option of the kernel library (unroll, blocks_per_cu, nontemporal[_copy|_accumulate|"
                          "_allgather|_pack|_unpack]), "
@@ -464,6 +469,19 @@ def main():
         torch.cuda.synchronize()
         return time.perf_counter() - t0, samples
 
+    if args.variant == "fused":
+        if not isinstance(w, RingAllreduce) or isinstance(w, RingAllreducePerStep):
+            sys.exit("bench.py: --variant fused applies to the allreduce workloads")
+        fused_elapsed, _ = timed(steps, warmup, fused=True)
+        if not w.check(steps - 1):
+            sys.exit("bench.py: the output of the fused-copy path is wrong; refusing to report a number")
+        print(json.dumps({"metric": "per-rank ring data path GB/s, %s, in->out copy folded into the accumulate" % w.name,
+                          "value": round(w.fused_bytes * steps / fused_elapsed / 1e9, 1), "unit": "GB/s", "n_gpus": 1,
+                          "steps": steps, "warmup": warmup, "ms_per_step": round(fused_elapsed / steps * 1e3, 5),
+                          "higher_is_better": True, "dtype": w.dtype, "data": "synthetic",
+                          "config": {"workload": w.description, "name": w.name, "bytes_per_step": w.fused_bytes,
+                                     "launches_per_step": 2}}))
+        return
     elapsed, samples = timed(steps, warmup, with_samples=True)
     if not w.check(steps - 1):
         sys.exit("bench.py: the output of the timed path is wrong; refusing to report a number")
@@ -514,24 +532,27 @@ def main():
     }
     # the same steps on ONE buffer set: at the headline size the working set fits the
     # last-level cache, so this is the cache-resident rate, not the HBM one
-    hot_steps = max(steps // 4, 1)
-    hot_elapsed, _ = timed(hot_steps, min(warmup, 50), hot=True)
-    result["hot"] = {"ms_per_step": round(hot_elapsed / hot_steps * 1e3, 5),
-                     "GBps": round(w.bytes_per_step * hot_steps / hot_elapsed / 1e9, 1),
-                     "note": "every step on the same buffers (%.0f MiB touched per step); `value` is the cold rate, "
-                             "buffer sets rotated" % (w.bytes_per_step / 2**20)}
+    if args.variant == "all":
+        hot_steps = max(steps // 4, 1)
+        hot_elapsed, _ = timed(hot_steps, min(warmup, 50), hot=True)
+        result["hot"] = {"ms_per_step": round(hot_elapsed / hot_steps * 1e3, 5),
+                         "GBps": round(w.bytes_per_step * hot_steps / hot_elapsed / 1e9, 1),
+                         "note": "every step on the same buffers (%.0f MiB touched per step); `value` is the cold "
+                                 "rate, buffer sets rotated" % (w.bytes_per_step / 2**20)}
     if isinstance(w, RingAllreduce) and not isinstance(w, RingAllreducePerStep):
         # the same job with the in->out copy folded into the accumulate (fewer bytes, same result)
-        fused_elapsed, _ = timed(steps, min(warmup, 50), fused=True)
-        if not w.check(steps - 1):
-            sys.exit("bench.py: the output of the fused-copy path is wrong; refusing to report a number")
-        result["fused_copy"] = {
-            "ms_per_step": round(fused_elapsed / steps * 1e3, 5),
-            "bytes_per_step": w.fused_bytes,
-            "GBps": round(w.fused_bytes * steps / fused_elapsed / 1e9, 1),
-            "launches_per_step": 2,
-            "note": "same allreduce with the in->out copy folded into the accumulate (out = in + received)",
-        }
+        if args.variant == "all":
+            fused_elapsed, _ = timed(steps, min(warmup, 50), fused=True)
+            if not w.check(steps - 1):
+                sys.exit("bench.py: the output of the fused-copy path is wrong; refusing to report a number")
+            result["fused_copy"] = {
+                "ms_per_step": round(fused_elapsed / steps * 1e3, 5),
+                "bytes_per_step": w.fused_bytes,
+                "GBps": round(w.fused_bytes * steps / fused_elapsed / 1e9, 1),
+                "launches_per_step": 2,
+                "note": "same allreduce with the in->out copy folded into the accumulate (out = in + received; the "
+                        "segment that is only sent is written by the first allgather step and never copied)",
+            }
         if not args.no_cpu_baseline:
             try:
                 result["cpu_baseline"] = cpu_baseline(w)

@@ -84,9 +84,9 @@ Status RingAllreducePrestaged(int n, int r, DataType dt, const void* input, void
       const size_t seg = static_cast<size_t>(Seg(RING_PHASE_REDUCE_SCATTER, n, r, i, true));
       rows.push_back(ring_row{at(output, starts[seg], esz), rs_recv[i], at(input, starts[seg], esz), sizes[seg]});
     }
-    // segment r is only ever sent, never accumulated: plain copy
-    const size_t own = static_cast<size_t>(r);
-    rows.push_back(ring_row{at(output, starts[own], esz), at(input, starts[own], esz), nullptr, sizes[own]});
+    // Segment r is only ever sent, never accumulated, and the first allgather
+    // step overwrites it with its final value (ring.h:211-225 receives segment
+    // r at step 0): a transport would send it from the input, nothing copies it.
     RING_RETURN_IF_ERROR(ring_apply_rows_avg(rows.data(), static_cast<int>(rows.size()), divide.data(), divisor,
                                              code, stream),
                          "ring_apply_rows_avg");
