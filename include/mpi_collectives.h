@@ -76,7 +76,9 @@ void* mpic_world_stream(const mpic_world* world);
 /* Options: "batched" (1: one launch per ring phase, 0: one launch per ring
  * step as in ring.h:183-225; default 1), "fuse_copy" (1: fold the in->out copy
  * of ring.h:146-148 into the reduce-scatter, out[seg] = in[seg] + received, the
- * same single add; default 1), "sync" (1: done() is called after
+ * same single add; default 1), "direct" (worlds that hold all ranks: 1 = the
+ * direct form of mpic_ring_allreduce_all_ranks, default; 0 = the lockstep
+ * ring), "sync" (1: done() is called after
  * the stream has drained, 0: as soon as the work is enqueued). */
 int mpic_world_set_option(mpic_world* world, const char* name, int value);
 
@@ -146,13 +148,27 @@ int mpic_context_destroy(mpic_context* ctx);
 int mpic_ring_allreduce_prestaged(int n, int r, int dtype, const void* input, void* output,
                                   size_t count, const void* const* rs_segments,
                                   const void* const* ag_segments, void* stream, int flags);
+/* The same allreduce where every rank's copy of a segment can be addressed at
+ * once (peers push into staging slots over their own links instead of passing
+ * partial sums round the ring): rank r owns segment s = (r+1) mod n;
+ * peer_segments[k], k = 0..n-2, is rank (s+k) mod n's copy of segment s, and
+ * they are folded with the rank's own copy in ring order, one pass
+ * (ring_fold_rows), into output[s]; ag_segments[i] is the finished segment
+ * (r-i) mod n. The output is bit-identical to mpic_ring_allreduce_prestaged
+ * fed with the ring's traffic. `flags`: bits 8-30 = divisor. No counterpart in
+ * the reference. */
+int mpic_ring_allreduce_direct_prestaged(int n, int r, int dtype, const void* input, void* output,
+                                         size_t count, const void* const* peer_segments,
+                                         const void* const* ag_segments, void* stream, int flags);
 /* RingAllgather (ring.h:236-301) for rank r: rows[k] = rank k's first
  * dimension, segments[i] = what arrives at step i. */
 int mpic_ring_allgather_prestaged(int n, int r, int dtype, const void* input, const size_t* rows,
                                   size_t elems_per_row, void* output,
                                   const void* const* segments, void* stream, int flags);
 /* All n ranks resident on this GPU: inputs[k] / outputs[k] are rank k's
- * tensors; a neighbour's buffer is read in place of a transfer. */
+ * tensors; a neighbour's buffer is read in place of a transfer. `flags` bit 2:
+ * the direct form (every segment folded by its owner in one launch, every
+ * finished segment copied straight from its owner in a second). */
 int mpic_ring_allreduce_all_ranks(int n, int dtype, const void* const* inputs,
                                   void* const* outputs, size_t count, void* stream, int flags);
 int mpic_ring_allgather_all_ranks(int n, int dtype, const void* const* inputs, const size_t* rows,

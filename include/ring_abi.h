@@ -71,10 +71,10 @@ size_t ring_dtype_size(int dtype);
  * launch: "nontemporal_copy" (ring_copy_bytes), "nontemporal_accumulate"
  * (accumulates, reduce-scatter tables, row tables, scale),
  * "nontemporal_allgather" (copy tables), "nontemporal_pack",
- * "nontemporal_unpack"; value bit 0 = non-temporal stores, bit 1 =
+ * "nontemporal_unpack", "nontemporal_fold"; value bit 0 = non-temporal stores, bit 1 =
  * non-temporal loads, -1 = the default (3, except ordinary stores for the copy
  * and the pack, whose output the next kernel reads, and loads by size for the
- * copy). "nontemporal" sets all five. No counterpart in the reference, whose
+ * copy). "nontemporal" sets all six. No counterpart in the reference, whose
  * launch shape is the constant <<<32, 256>>> (ring.cu.cc:64). */
 int ring_set_option(const char* name, int value);
 
@@ -212,6 +212,25 @@ int ring_apply_rows(const ring_row* rows, int n_rows, int dtype, void* stream);
  * `rows` and `divide` are HOST arrays. */
 int ring_apply_rows_avg(const ring_row* rows, int n_rows, const unsigned char* divide, int divisor,
                         int dtype, void* stream);
+
+/* A segment reduced in one pass. After its n-1 reduce-scatter steps the ring
+ * holds in segment s the left fold over the ranks in ring order,
+ *   acc = x_s; acc = x_{s+1} + acc; ...; acc = x_{s+n-1} + acc
+ * (ring.h:183-205: at step i rank r adds what it received, the running sum of
+ * segment (r-i-1), into its own copy). Where every rank's copy of the segment
+ * is addressable at once, the owner computes that fold directly: for every
+ * row, dst[i] = srcs[m-1][i] + (... + (srcs[1][i] + srcs[0][i])), the same
+ * additions in the same order, with m reads and one write per element instead
+ * of 3(m-1) accesses. divisor > 0: the fold is divided as ring_scale divides
+ * (the average) before it is stored. dst may be one of the row's own sources.
+ * `rows` and each `srcs` are HOST arrays; every row has m sources, 1 <= m <=
+ * 256. No counterpart in the reference. */
+typedef struct ring_fold_row {
+  void* dst;
+  const void* const* srcs; /* m device pointers, in fold order */
+  uint64_t count;          /* elements */
+} ring_fold_row;
+int ring_fold_rows(const ring_fold_row* rows, int n_rows, int m, int divisor, int dtype, void* stream);
 
 /* ---- tensor fusion (no counterpart in the reference, which issues one
  * MPIAllreduce per gradient, __init__.py:195-205): k tensors are packed back

@@ -89,7 +89,7 @@ struct mpic_world {
   void* stream = nullptr;
   // a world folds the in->out copy into the reduce-scatter unless told otherwise
   // (same results, a third fewer bytes)
-  mpic::RingOptions ring_options = [] { mpic::RingOptions o; o.fuse_copy = true; return o; }();
+  mpic::RingOptions ring_options = [] { mpic::RingOptions o; o.fuse_copy = true; o.direct = true; return o; }();
   bool sync_on_done = true;
   // Tensor fusion in the coordinator: allreduces that are ready in the same
   // tick are packed, per rank, into that rank's slice of this caller-owned
@@ -911,6 +911,7 @@ int mpic_world_set_option(mpic_world* w, const char* name, int value) {
   std::lock_guard<std::mutex> guard(w->mu);
   if (!strcmp(name, "batched")) w->ring_options.batched = value != 0;
   else if (!strcmp(name, "fuse_copy")) w->ring_options.fuse_copy = value != 0;
+  else if (!strcmp(name, "direct")) w->ring_options.direct = value != 0;
   else if (!strcmp(name, "sync")) w->sync_on_done = value != 0;
   else return MPIC_INVALID_ARGUMENT;
   return MPIC_OK;
@@ -1048,6 +1049,15 @@ int mpic_ring_allreduce_prestaged(int n, int r, int dtype, const void* input, vo
                                   int flags) {
   mpic::Status s = mpic::RingAllreducePrestaged(n, r, static_cast<mpic::DataType>(dtype), input, output, count,
                                                 rs_segments, ag_segments, stream, mpic::RingOptions::FromFlags(flags));
+  return s.ok() ? MPIC_OK : mpic::Fail(s);
+}
+
+int mpic_ring_allreduce_direct_prestaged(int n, int r, int dtype, const void* input, void* output, size_t count,
+                                         const void* const* peer_segments, const void* const* ag_segments,
+                                         void* stream, int flags) {
+  mpic::Status s = mpic::RingAllreduceDirectPrestaged(n, r, static_cast<mpic::DataType>(dtype), input, output, count,
+                                                      peer_segments, ag_segments, stream,
+                                                      mpic::RingOptions::FromFlags(flags));
   return s.ok() ? MPIC_OK : mpic::Fail(s);
 }
 

@@ -139,6 +139,44 @@ Status RingAllreducePrestaged(int n, int r, DataType dt, const void* input, void
   return Status::OK();
 }
 
+Status RingAllreduceDirectPrestaged(int n, int r, DataType dt, const void* input, void* output, size_t count,
+                                    const void* const* peers, const void* const* ag_recv, void* stream,
+                                    const RingOptions& opts) {
+  int code = 0;
+  Status s = RingDataType(dt, &code);
+  if (!s.ok()) return s;
+  if (n < 1 || r < 0 || r >= n) return errors::InvalidArgument("rank out of range for the ring");
+  if (opts.divisor < 0) return errors::InvalidArgument("negative divisor");
+  const size_t esz = ring_dtype_size(code);
+  if (count == 0) return Status::OK();
+  if (!input || !output) return errors::InvalidArgument("null tensor with a non-zero element count");
+  if (n > 1 && (!peers || !ag_recv)) return errors::InvalidArgument("no staged peer segments");
+  std::vector<size_t> sizes(static_cast<size_t>(n)), starts(static_cast<size_t>(n));
+  RING_RETURN_IF_ERROR(ring_segment_table(count, n, sizes.data(), starts.data()), "ring_segment_table");
+
+  // the owned segment: x_s, x_{s+1}, ..., x_{s+n-1} = this rank's own, folded in that order
+  const size_t own = static_cast<size_t>((r + 1) % n);
+  if (sizes[own]) {
+    std::vector<const void*> srcs;
+    for (int k = 0; k < n - 1; k++) {
+      if (!peers[k]) return errors::InvalidArgument("null staged peer segment");
+      srcs.push_back(peers[k]);
+    }
+    srcs.push_back(at(input, starts[own], esz));
+    ring_fold_row row{at(output, starts[own], esz), srcs.data(), sizes[own]};
+    RING_RETURN_IF_ERROR(ring_fold_rows(&row, 1, n, opts.divisor, code, stream), "ring_fold_rows");
+  }
+  // every other segment arrives finished (ring.h:211-225 delivers the same values step by step)
+  std::vector<ring_step> steps;
+  for (int i = 0; i < n - 1; i++) {
+    const size_t seg = static_cast<size_t>(Seg(RING_PHASE_ALLGATHER, n, r, i, true));
+    steps.push_back(ring_step{starts[seg], ag_recv[i], sizes[seg]});
+  }
+  if (n > 1)
+    RING_RETURN_IF_ERROR(ring_allgather_steps(output, steps.data(), n - 1, code, stream), "ring_allgather_steps");
+  return Status::OK();
+}
+
 Status RingAllgatherPrestaged(int n, int r, DataType dt, const void* input, const std::vector<size_t>& rows,
                               size_t elems_per_row, void* output, const void* const* recv, void* stream,
                               const RingOptions& opts) {
@@ -211,6 +249,34 @@ Status RingAllreduceAllRanks(int n, DataType dt, const void* const* inputs, void
   std::vector<ring_row> rows(static_cast<size_t>(n));
   for (int r = 0; r < n; r++)
     if (!inputs[r] || !outputs[r]) return errors::InvalidArgument("null tensor with a non-zero element count");
+
+  if (opts.direct) {
+    // One launch: the owner of every segment folds the n copies in ring order.
+    std::vector<std::vector<const void*>> srcs(static_cast<size_t>(n));
+    std::vector<ring_fold_row> folds;
+    for (int j = 0; j < n; j++) {
+      const size_t seg = static_cast<size_t>((j + 1) % n);
+      for (int k = 0; k < n; k++)
+        srcs[static_cast<size_t>(j)].push_back(at(inputs[(static_cast<int>(seg) + k) % n], starts[seg], esz));
+      folds.push_back(ring_fold_row{at(outputs[j], starts[seg], esz), srcs[static_cast<size_t>(j)].data(), sizes[seg]});
+    }
+    if (!(n == 1 && inputs[0] == outputs[0] && opts.divisor == 0))
+      RING_RETURN_IF_ERROR(ring_fold_rows(folds.data(), n, n, opts.divisor, code, stream), "ring_fold_rows");
+    // One more: every rank copies each finished segment from its owner.
+    std::vector<ring_row> copies;
+    for (int r = 0; r < n; r++) {
+      for (int seg = 0; seg < n; seg++) {
+        const int owner = (seg - 1 + n) % n;
+        if (owner == r) continue;
+        const size_t sg = static_cast<size_t>(seg);
+        copies.push_back(ring_row{at(outputs[r], starts[sg], esz),
+                                  at(static_cast<const void*>(outputs[owner]), starts[sg], esz), nullptr, sizes[sg]});
+      }
+    }
+    RING_RETURN_IF_ERROR(ring_apply_rows(copies.data(), static_cast<int>(copies.size()), code, stream),
+                         "ring_apply_rows");
+    return Status::OK();
+  }
   // Without the in->out copy (ring.h:146-148): every segment of a rank's output
   // is written by one of the 2(n-1) steps anyway (the reduce-scatter writes all
   // but segment r, the allgather all but segment r+1), and a rank accumulates

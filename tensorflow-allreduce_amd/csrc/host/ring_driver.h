@@ -30,12 +30,19 @@ struct RingOptions {
   // what then travels round the ring is already divided. Pre-staged allgather
   // segments are therefore expected divided, as a peer would send them.
   int divisor = 0;
+  // Where every rank's copy of a segment is addressable at once: its owner
+  // folds the n copies in ring order in one pass (ring_fold_rows) instead of
+  // n-1 accumulate steps, and every rank copies each finished segment straight
+  // from its owner instead of passing it round. Same additions in the same
+  // order, so the same bits; 2 launches instead of 2(n-1)+1.
+  bool direct = false;
   // Transport-driven rings only: pieces a segment travels in (1..16).
   int chunks = 1;
   static RingOptions FromFlags(int flags) {
     RingOptions o;
     o.batched = (flags & 1) != 0;
     o.fuse_copy = (flags & 2) != 0;
+    o.direct = (flags & 4) != 0;
     o.chunks = ((flags >> 4) & 15) + 1;
     o.divisor = (flags >> 8) & 0x7fffff;
     return o;
@@ -52,6 +59,16 @@ Status RingDataType(DataType dt, int* ring_dtype);
 Status RingAllreducePrestaged(int n, int r, DataType dt, const void* input, void* output, size_t count,
                               const void* const* rs_recv, const void* const* ag_recv, void* stream,
                               const RingOptions& opts);
+
+// The direct form for rank r of n, which owns segment s = (r+1) mod n: peers[k]
+// (k = 0..n-2) is rank (s+k) mod n's copy of segment s, as that rank would push
+// it into this rank's staging slot; they and the rank's own copy are folded in
+// ring order into output[s]. ag_recv[i]: the finished segment (r-i) mod n, as
+// its owner would push it. Bit-identical to RingAllreducePrestaged fed with
+// the ring's own traffic.
+Status RingAllreduceDirectPrestaged(int n, int r, DataType dt, const void* input, void* output, size_t count,
+                                    const void* const* peers, const void* const* ag_recv, void* stream,
+                                    const RingOptions& opts);
 
 // ring.h:236-301 for rank r of n. recv[i]: the segment received at step i
 // (segment (r-i-1) mod n).

@@ -276,6 +276,128 @@ __global__ void __launch_bounds__(kBlock) bytes_kernel(uint8_t* __restrict__ dst
     dst[i] = src[i];
 }
 
+// ---- fold: a segment reduced in one pass, in ring order ---------------------------
+// The ring leaves in segment s the left fold acc = x_s; acc = x_{s+1} + acc; ...
+// over the ranks in ring order (ring.h:183-205 unrolled over its n-1 steps).
+// Where every rank's copy of the segment is addressable at once (all ranks on
+// one GPU, or peers that pushed their copies into staging slots over their own
+// links) the owner computes that fold directly: m reads and one write per
+// element instead of 3(m-1) accesses, the same additions in the same order.
+
+constexpr int kMaxFoldRows = 32;
+constexpr int kMaxFoldPtrs = 256;
+
+struct FoldRow {
+  void* dst;
+  uint64_t count;      // elements
+  uint32_t first_ptr;  // index of the row's first source in FoldTable::src
+  uint32_t pad;
+};
+struct FoldTable {
+  int n_rows;
+  int m;                   // sources per row, folded in the order they are listed
+  int divisor;             // > 0: the fold is divided (tf.div) before it is stored
+  uint32_t uniform_tiles;  // as RowTable
+  uint32_t tile_begin[kMaxFoldRows + 1];
+  FoldRow row[kMaxFoldRows];
+  const void* src[kMaxFoldPtrs];
+};
+
+// One tile of a fold row. dst may be one of the row's own sources: a lane reads
+// every source of its elements before it stores them.
+template <typename T, int UNROLL, bool DIV, int NT>
+__device__ __forceinline__ void fold_tile(T* dst, const void* const* src, int m, uint64_t count, uint32_t tile,
+                                          uint32_t tiles_in_row, int n) {
+  typedef typename VecOf<T>::type V;
+  typedef V VU __attribute__((aligned(sizeof(T))));
+  constexpr uint32_t VEC = 16 / sizeof(T);
+  constexpr uint32_t kTileVecs = kBlock * UNROLL;
+  constexpr int kGroup = 4;  // sources whose loads are issued together
+
+  uint64_t head = ((16u - (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(dst)) & 15u)) & 15u) / sizeof(T);
+  if (head > count) head = count;
+  const uint64_t nvec = (count - head) / VEC;
+  const uint32_t tid = threadIdx.x;
+
+  // scalar head (tile 0) and tail (last tile)
+  auto scalar = [&](uint64_t e) {
+    T acc = static_cast<const T*>(src[0])[e];
+    for (int k = 1; k < m; k++) acc = add_one(acc, static_cast<const T*>(src[k])[e]);
+    dst[e] = DIV ? div_one(acc, n) : acc;
+  };
+  if (tile == 0 && tid < head) scalar(tid);
+  if (tile + 1 == tiles_in_row) {
+    const uint64_t e = head + nvec * VEC + tid;
+    if (e < count) scalar(e);
+  }
+
+  V* dv = reinterpret_cast<V*>(dst + head);
+  const uint64_t v0 = static_cast<uint64_t>(tile) * kTileVecs + tid;
+  const bool full = static_cast<uint64_t>(tile + 1) * kTileVecs <= nvec;
+  bool ok[UNROLL];
+  V acc[UNROLL];
+  {
+    const VU* sv = reinterpret_cast<const VU*>(static_cast<const T*>(src[0]) + head);
+#pragma unroll
+    for (int j = 0; j < UNROLL; j++) {
+      ok[j] = full || v0 + j * kBlock < nvec;
+      if (ok[j]) acc[j] = RING_LOAD_VEC(NT, &sv[v0 + j * kBlock]);
+    }
+  }
+  for (int k = 1; k < m; k += kGroup) {
+    const int group = m - k < kGroup ? m - k : kGroup;  // uniform
+    V x[kGroup][UNROLL];
+#pragma unroll
+    for (int g = 0; g < kGroup; g++) {
+      if (g < group) {
+        const VU* sv = reinterpret_cast<const VU*>(static_cast<const T*>(src[k + g]) + head);
+#pragma unroll
+        for (int j = 0; j < UNROLL; j++)
+          if (ok[j]) x[g][j] = RING_LOAD_VEC(NT, &sv[v0 + j * kBlock]);
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < kGroup; g++) {
+      if (g < group) {
+#pragma unroll
+        for (int j = 0; j < UNROLL; j++)
+          if (ok[j]) acc[j] = apply_vec<T, kOpAdd>(acc[j], x[g][j], 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < UNROLL; j++) {
+    if (ok[j]) {
+      if (DIV) acc[j] = apply_vec<T, kOpDiv>(acc[j], acc[j], n);
+      store_vec<T, NT>(&dv[v0 + j * kBlock], acc[j]);
+    }
+  }
+}
+
+template <typename T, bool DIV, int NT>
+__global__ void __launch_bounds__(kBlock) fold_kernel(const FoldTable tab) {
+  constexpr int UNROLL = 2;
+  if (tab.uniform_tiles) {
+    const FoldRow r = tab.row[blockIdx.y];
+    for (uint32_t t = blockIdx.x; t < tab.uniform_tiles; t += gridDim.x)
+      fold_tile<T, UNROLL, DIV, NT>(static_cast<T*>(r.dst), tab.src + r.first_ptr, tab.m, r.count, t,
+                                    tab.uniform_tiles, tab.divisor);
+    return;
+  }
+  const uint32_t total = tab.tile_begin[tab.n_rows];
+  for (uint32_t t = blockIdx.x; t < total; t += gridDim.x) {
+    int lo = 0, hi = tab.n_rows;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (tab.tile_begin[mid] <= t) lo = mid; else hi = mid;
+    }
+    const FoldRow r = tab.row[lo];
+    const uint32_t first = tab.tile_begin[lo];
+    fold_tile<T, UNROLL, DIV, NT>(static_cast<T*>(r.dst), tab.src + r.first_ptr, tab.m, r.count, t - first,
+                                  tab.tile_begin[lo + 1] - first, tab.divisor);
+  }
+}
+
 // ---- tensor fusion: pack / unpack -----------------------------------------------
 // The fused buffer is cut into tiles of 1024 16-byte groups. A tile that lies
 // inside one tensor (all of the bytes of a ResNet-sized gradient set, bar a few
@@ -356,7 +478,7 @@ fusion_kernel(T* __restrict__ fused, const uint64_t* __restrict__ offsets, T* co
 
 constexpr uint64_t kCacheResidentBytes = 128ull << 20;
 
-enum Role { kRoleCopy, kRoleAccumulate, kRoleAllgather, kRolePack, kRoleUnpack, kRoles };
+enum Role { kRoleCopy, kRoleAccumulate, kRoleAllgather, kRolePack, kRoleUnpack, kRoleFold, kRoles };
 
 struct Tuning {
   int unroll = 4;          // 16-byte vectors per lane per tile: 2, 4 or 8
@@ -367,7 +489,7 @@ struct Tuning {
   // of a step on tensors up to 128 MiB, which the last-level cache can hold);
   // the copy's loads turn non-temporal above that size, where ordinary ones
   // only evict what the next kernel wants.
-  int nt[kRoles] = {-1, 3, 3, 2, 3};
+  int nt[kRoles] = {-1, 3, 3, 2, 3, 2};  // the fold's result is what the allgather reads next
   int blocks_per_cu = 0;   // 0: one workgroup per tile; >0: persistent grid of CUs x this
 };
 Tuning g_tuning;
@@ -636,7 +758,8 @@ int ring_set_option(const char* name, int value) {
     if (value != 2 && value != 4 && value != 8) return RING_ERR_ARGUMENT;
     g_tuning.unroll = value;
   } else if (!strncmp(name, "nontemporal", 11)) {
-    static const char* const kSuffix[kRoles] = {"_copy", "_accumulate", "_allgather", "_pack", "_unpack"};
+    static const char* const kSuffix[kRoles] = {"_copy", "_accumulate", "_allgather", "_pack", "_unpack",
+                                                "_fold"};
     if (value < -1 || value > 3) return RING_ERR_ARGUMENT;
     const Tuning defaults;
     bool known = name[11] == 0;
@@ -846,6 +969,83 @@ int ring_apply_rows_avg(const ring_row* rows, int n_rows, const unsigned char* d
 
 int ring_allgather_steps(void* buffer, const ring_step* steps, int n_steps, int dtype, void* stream) {
   return steps_common(nullptr, buffer, steps, n_steps, dtype, stream, kStepCopy);
+}
+
+int ring_fold_rows(const ring_fold_row* rows, int n_rows, int m, int divisor, int dtype, void* stream) {
+  if (!dtype_ok(dtype)) return RING_ERR_DTYPE;
+  if (n_rows < 0 || m < 1 || m > kMaxFoldPtrs || divisor < 0) return RING_ERR_ARGUMENT;
+  if (n_rows == 0) return RING_OK;
+  if (!rows) return RING_ERR_ARGUMENT;
+  const size_t esz = dtype_size(dtype);
+  constexpr uint64_t kTileVecs = static_cast<uint64_t>(kBlock) * 2;
+  const uint64_t vec = 16 / esz;
+  const int rows_per_launch = kMaxFoldPtrs / m < kMaxFoldRows ? kMaxFoldPtrs / m : kMaxFoldRows;
+  int nt = g_tuning.nt[kRoleFold];
+  if (nt < 0) nt = 2;
+  int i = 0;
+  while (i < n_rows) {
+    FoldTable tab;
+    tab.n_rows = 0;
+    tab.m = m;
+    tab.divisor = divisor;
+    tab.tile_begin[0] = 0;
+    uint64_t tiles = 0, first_tiles = 0;
+    bool uniform = true;
+    while (i < n_rows && tab.n_rows < rows_per_launch) {
+      const ring_fold_row& r = rows[i];
+      if (r.count == 0) { i++; continue; }
+      if (!r.dst || !r.srcs || (reinterpret_cast<uintptr_t>(r.dst) & (esz - 1))) return RING_ERR_ARGUMENT;
+      const uintptr_t d = reinterpret_cast<uintptr_t>(r.dst);
+      uint64_t head = ((16u - (d & 15u)) & 15u) / esz;
+      if (head > r.count) head = r.count;
+      uint64_t t = ((r.count - head) / vec + kTileVecs - 1) / kTileVecs;
+      if (t == 0) t = 1;
+      if (tiles + t > 0x7fffffffull) {
+        if (tab.n_rows == 0) return RING_ERR_ARGUMENT;
+        break;
+      }
+      const int k = tab.n_rows++;
+      tab.row[k] = FoldRow{r.dst, r.count, static_cast<uint32_t>(k * m), 0};
+      for (int j = 0; j < m; j++) {
+        if (!r.srcs[j] || (reinterpret_cast<uintptr_t>(r.srcs[j]) & (esz - 1))) return RING_ERR_ARGUMENT;
+        tab.src[k * m + j] = r.srcs[j];
+      }
+      if (k == 0) first_tiles = t;
+      uniform = uniform && t == first_tiles;
+      tiles += t;
+      tab.tile_begin[k + 1] = static_cast<uint32_t>(tiles);
+      i++;
+    }
+    if (tab.n_rows == 0) continue;
+    dim3 grid;
+    if (uniform) {
+      tab.uniform_tiles = static_cast<uint32_t>(first_tiles);
+      grid = dim3(static_cast<uint32_t>(first_tiles), static_cast<uint32_t>(tab.n_rows));
+    } else {
+      tab.uniform_tiles = 0;
+      grid = dim3(static_cast<uint32_t>(tiles));
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+#define RING_FOLD(T, D)                                                              \
+  switch (nt & 3) {                                                                  \
+    case 0: launch(fold_kernel<T, D, 0>, grid, dim3(kBlock), s, tab); break;         \
+    case 1: launch(fold_kernel<T, D, 1>, grid, dim3(kBlock), s, tab); break;         \
+    case 2: launch(fold_kernel<T, D, 2>, grid, dim3(kBlock), s, tab); break;         \
+    default: launch(fold_kernel<T, D, 3>, grid, dim3(kBlock), s, tab); break;        \
+  }
+    if (divisor > 0) {
+      if (dtype == RING_F32) { RING_FOLD(float, true) }
+      else if (dtype == RING_I32) { RING_FOLD(int32_t, true) }
+      else { RING_FOLD(int64_t, true) }
+    } else {
+      if (dtype == RING_F32) { RING_FOLD(float, false) }
+      else if (dtype == RING_I32) { RING_FOLD(int32_t, false) }
+      else { RING_FOLD(int64_t, false) }
+    }
+#undef RING_FOLD
+    RING_HIP(hipGetLastError());
+  }
+  return RING_OK;
 }
 
 int ring_scale(int dtype, void* data, size_t count, int divisor, void* stream) {

@@ -211,7 +211,7 @@ class Session:
         return _plugin.lib().mpic_world_stream(self._world)
 
     def set_option(self, name, value):
-        """"batched", "fuse_copy" or "sync": see mpic_world_set_option."""
+        """"batched", "fuse_copy", "direct" or "sync": see mpic_world_set_option."""
         rc = _plugin.lib().mpic_world_set_option(self._world, name.encode(), int(value))
         if rc != 0:
             raise InvalidArgumentError("unknown session option %r" % name)

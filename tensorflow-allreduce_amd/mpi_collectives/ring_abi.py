@@ -22,7 +22,7 @@ EXPORTS = (
     "ring_schedule", "ring_stream_create", "ring_stream_destroy", "ring_stream_synchronize",
     "ring_copy_bytes", "ring_accumulate_f32", "ring_accumulate_i32", "ring_accumulate_i64",
     "ring_accumulate", "ring_reduce_scatter_steps", "ring_reduce_scatter_steps_from",
-    "ring_allgather_steps", "ring_apply_rows", "ring_apply_rows_avg",
+    "ring_allgather_steps", "ring_apply_rows", "ring_apply_rows_avg", "ring_fold_rows",
     "ring_fusion_plan_create", "ring_fusion_plan_destroy", "ring_fusion_plan_elements",
     "ring_fusion_pack", "ring_fusion_unpack", "ring_fusion_unpack_scaled", "ring_scale",
 )
@@ -50,6 +50,11 @@ class Row(ctypes.Structure):
 
 
 _lib = None
+
+
+class FoldRow(ctypes.Structure):
+    """ring_fold_row: dst = srcs[m-1] + (... + (srcs[1] + srcs[0]))."""
+    _fields_ = [("dst", ctypes.c_void_p), ("srcs", ctypes.POINTER(ctypes.c_void_p)), ("count", ctypes.c_uint64)]
 
 
 def lib():
@@ -93,6 +98,7 @@ def lib():
             "ring_allgather_steps": (ci, [vp, ctypes.POINTER(Step), ci, ci, vp]),
             "ring_apply_rows": (ci, [ctypes.POINTER(Row), ci, ci, vp]),
             "ring_apply_rows_avg": (ci, [ctypes.POINTER(Row), ci, ctypes.POINTER(ctypes.c_ubyte), ci, ci, vp]),
+            "ring_fold_rows": (ci, [ctypes.POINTER(FoldRow), ci, ci, ci, ci, vp]),
             "ring_fusion_plan_create": (ci, [ctypes.POINTER(vp), psz, ci, ci, ctypes.POINTER(vp)]),
             "ring_fusion_plan_destroy": (ci, [vp]),
             "ring_fusion_plan_elements": (sz, [vp]),
@@ -241,6 +247,18 @@ def apply_rows_avg(rows, divide, divisor, dtype, stream):
         arr[i].dst, arr[i].a, arr[i].b, arr[i].count = d, a, b, cnt
     flags = None if divide is None else (ctypes.c_ubyte * max(len(rows), 1))(*[1 if f else 0 for f in divide])
     check(lib().ring_apply_rows_avg(arr, len(rows), flags, divisor, dtype, stream), "ring_apply_rows_avg")
+
+
+def fold_rows(rows, m, divisor, dtype, stream):
+    """rows: iterable of (dst, [m source pointers in fold order], count)."""
+    rows = list(rows)
+    arr = (FoldRow * max(len(rows), 1))()
+    keep = []
+    for i, (d, srcs, cnt) in enumerate(rows):
+        ptrs = (ctypes.c_void_p * m)(*srcs)
+        keep.append(ptrs)
+        arr[i].dst, arr[i].srcs, arr[i].count = d, ctypes.cast(ptrs, ctypes.POINTER(ctypes.c_void_p)), cnt
+    check(lib().ring_fold_rows(arr, len(rows), m, divisor, dtype, stream), "ring_fold_rows")
 
 
 def scale(dtype, data, count, divisor, stream):

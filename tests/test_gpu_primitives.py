@@ -239,6 +239,57 @@ def test_rows_with_the_divide_folded_in(dtype):
         ring_abi.apply_rows_avg([(out.data_ptr(), da.data_ptr(), None, 1000)], None, -1, code, None)
 
 
+def _fold_reference(srcs, divisor, dtype):
+    """acc = s0; acc = s_k + acc, one rounded add per step, then tf.div."""
+    acc = srcs[0].copy()
+    with np.errstate(all="ignore"):
+        for s in srcs[1:]:
+            acc = (s + acc).astype(dtype)
+        if divisor:
+            acc = (acc / np.float32(divisor) if dtype == np.float32 else acc // dtype(divisor)).astype(dtype)
+    return acc
+
+
+@pytest.mark.parametrize("dtype", G.DTYPES)
+def test_fold_rows_is_the_sequential_fold(dtype):
+    """ring_fold_rows against a numpy fold in the same order: any number of
+    sources, rows of equal and unequal length, any alignment, the divide, a
+    destination that is one of the sources, more rows than one launch holds."""
+    rng = np.random.default_rng(99)
+    code = G.NP2ABI[np.dtype(dtype)]
+    cases = [(1, 1, [10]), (2, 1, [4099]), (3, 2, [7, 0]), (8, 8, [30_011] * 8), (8, 3, [5, 9000, 123]),
+             (9, 40, [int(c) for c in rng.integers(0, 3000, 40)]), (64, 2, [2049, 2049]), (256, 1, [1500])]
+    for m, n_rows, counts in cases:
+        for divisor in (0, 6):
+            rows, wants, dsts, keep = [], [], [], []
+            for k, c in enumerate(counts):
+                hs = [G.random_array(rng, c, dtype, wide=dtype == np.float32) for _ in range(m)]
+                if dtype != np.float32 and c:
+                    hs[0][: c // 2] = -np.abs(hs[0][: c // 2]) - 7        # negative sums for the floor division
+                ds = [G.dev(h, (k + j) % 4) for j, h in enumerate(hs)]
+                keep.append(ds)
+                in_place = k % 2 == 1                                     # dst is the last source
+                if in_place:
+                    dst = ds[-1][0]
+                else:
+                    dst, base = G.dev(np.zeros(c, dtype=dtype), (k + 2) % 4)
+                    keep.append(base)
+                rows.append((dst.data_ptr() if c else None, [d[0].data_ptr() if c else None for d in ds], c))
+                wants.append(_fold_reference(hs, divisor, dtype))
+                dsts.append(dst)
+            ring_abi.fold_rows(rows, m, divisor, code, None)
+            G.sync()
+            for k in range(n_rows):
+                G.assert_same_bits(G.host(dsts[k]), wants[k], "fold m=%d row %d of %d /%d" % (m, k, n_rows, divisor))
+    x, _ = G.dev(np.ones(8, dtype=dtype), 0)
+    with pytest.raises(ring_abi.RingError):
+        ring_abi.fold_rows([(x.data_ptr(), [x.data_ptr()] * 257, 8)], 257, 0, code, None)
+    with pytest.raises(ring_abi.RingError):
+        ring_abi.fold_rows([(x.data_ptr(), [None, x.data_ptr()], 8)], 2, 0, code, None)
+    with pytest.raises(ring_abi.RingError):
+        ring_abi.fold_rows([(x.data_ptr(), [x.data_ptr()], 8)], 1, -1, code, None)
+
+
 @pytest.mark.parametrize("dtype", G.DTYPES)
 def test_scale_is_tf_div(dtype):
     """allreduce(average=True) divides with tf.div (__init__.py:160-164): true

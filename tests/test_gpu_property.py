@@ -27,8 +27,9 @@ def _gpu():
 
 @settings(max_examples=60, **COMMON)
 @given(n=st.integers(1, 9), count=counts, dtype=st.sampled_from(G.DTYPES), seed=st.integers(0, 2**31),
-       offs=st.lists(st.integers(0, 3), min_size=2, max_size=2), divisor=st.sampled_from([0, 0, 1, 2, 3, 7, 8, 64]), fuse=st.booleans())
-def test_all_ranks_ring_equals_oracle(oracle, n, count, dtype, seed, offs, divisor, fuse):
+       offs=st.lists(st.integers(0, 3), min_size=2, max_size=2), divisor=st.sampled_from([0, 0, 1, 2, 3, 7, 8, 64]), fuse=st.booleans(),
+       direct=st.booleans())
+def test_all_ranks_ring_equals_oracle(oracle, n, count, dtype, seed, offs, divisor, fuse, direct):
     """Sum, or (divisor > 0) the average folded into the last accumulate:
     tf.div of the oracle's sum."""
     ins = [G.random_array(np.random.default_rng(seed + r), count, dtype, wide=True) for r in range(n)]
@@ -47,12 +48,12 @@ def test_all_ranks_ring_equals_oracle(oracle, n, count, dtype, seed, offs, divis
     pin = (ctypes.c_void_p * n)(*[t.data_ptr() if count else None for t in dins])
     pout = (ctypes.c_void_p * n)(*[t.data_ptr() if count else None for t in douts])
     rc = L.mpic_ring_allreduce_all_ranks(n, DT[np.dtype(dtype)], pin, pout, count,
-                                         torch.cuda.current_stream().cuda_stream, 1 | (2 if fuse else 0) | (divisor << 8))
+                                         torch.cuda.current_stream().cuda_stream, 1 | (2 if fuse else 0) | (4 if direct else 0) | (divisor << 8))
     assert rc == 0, L.mpic_last_error()
     torch.cuda.synchronize()
     for r in range(n):
         G.assert_same_bits(G.host(douts[r]), want[r],
-                           "n=%d count=%d %s rank %d /%d" % (n, count, dtype.__name__, r, divisor))
+                           "n=%d count=%d %s rank %d /%d fuse=%s direct=%s" % (n, count, dtype.__name__, r, divisor, fuse, direct))
 
 
 @settings(max_examples=40, **COMMON)

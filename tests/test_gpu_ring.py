@@ -46,8 +46,11 @@ def test_allreduce_all_ranks_matches_oracle(oracle, dtype, n):
     for count in sorted({0, 1, max(n - 1, 0), n, n + 1, 17, 4913, 1_000_003}):
         ins = make_inputs(n, count, dtype, seed=31 * n + count)
         want = oracle.ring_allreduce(ins)
-        for fuse in (1, 0):          # without / with the in->out copy as a launch of its own
+        # the direct form (a world's default), then the lockstep ring without / with
+        # the in->out copy as a launch of its own
+        for direct, fuse in ((1, 1), (0, 1), (0, 0)):
             with mpi.Session(size=n) as session:
+                session.set_option("direct", direct)
                 session.set_option("fuse_copy", fuse)
                 handles, dins = [], [cuda(x) for x in ins]
                 for r in range(n):
@@ -56,8 +59,8 @@ def test_allreduce_all_ranks_matches_oracle(oracle, dtype, n):
                         handles.append(mpi.allreduce(dins[r], average=False))
                 outs = session.run(handles)
             for r in range(n):
-                G.assert_same_bits(G.host(outs[r]), want[r], "allreduce %s n=%d count=%d rank %d fuse=%d"
-                                   % (dtype.__name__, n, count, r, fuse))
+                G.assert_same_bits(G.host(outs[r]), want[r], "allreduce %s n=%d count=%d rank %d direct=%d fuse=%d"
+                                   % (dtype.__name__, n, count, r, direct, fuse))
                 G.assert_same_bits(G.host(dins[r]), ins[r], "the input is never written")
 
 
@@ -248,6 +251,35 @@ def test_prestaged_rank_with_the_average_folded_in(oracle, dtype):
                 got = _prestaged(n, r, ins, rs, ag_div, flags | (divisor << 8), dtype)
                 G.assert_same_bits(G.host(got), _tf_div(outs[r], divisor),
                                    "folded average n=%d r=%d flags=%d /%d" % (n, r, flags, divisor))
+
+
+@pytest.mark.parametrize("dtype", G.DTYPES)
+def test_direct_form_for_one_rank_matches_the_ring(oracle, dtype):
+    """mpic_ring_allreduce_direct_prestaged: the owner folds every rank's raw
+    copy of its segment in ring order; the other segments arrive finished.
+    Bit-identical to the oracle's ring, with and without the divide."""
+    L = _plugin.load_library()
+    for n, count, divisor in ((1, 9, 0), (2, 7, 0), (3, 2, 0), (6, 4099, 6), (8, 100_003, 0), (8, 50_000, 8), (5, 0, 0)):
+        ins = make_inputs(n, count, dtype, seed=40 + n)
+        want = oracle.ring_allreduce(ins)[0]
+        if divisor:
+            want = _tf_div(want, divisor)
+        sizes, starts = ring_abi.segment_table(count, n)
+        for r in sorted({0, n // 2, n - 1}):
+            s = (r + 1) % n
+            peers = [cuda(ins[(s + k) % n][starts[s]:starts[s] + sizes[s]]) for k in range(n - 1)]
+            ag_segs = [ring_abi.schedule(ring_abi.PHASE_ALLGATHER, n, r, i)[1] for i in range(n - 1)]
+            ags = [cuda(want[starts[g]:starts[g] + sizes[g]]) for g in ag_segs]
+            pp = (ctypes.c_void_p * max(n - 1, 1))(*[t.data_ptr() if t.numel() else None for t in peers])
+            ap = (ctypes.c_void_p * max(n - 1, 1))(*[t.data_ptr() if t.numel() else None for t in ags])
+            din = cuda(ins[r])
+            dout = torch.zeros(count + 4, dtype=G.NP2TORCH[np.dtype(dtype)], device="cuda")[:count]
+            rc = L.mpic_ring_allreduce_direct_prestaged(n, r, DT[np.dtype(dtype)], din.data_ptr() if count else None,
+                                                        dout.data_ptr() if count else None, count, pp, ap,
+                                                        torch.cuda.current_stream().cuda_stream, divisor << 8)
+            assert rc == 0, L.mpic_last_error()
+            torch.cuda.synchronize()
+            G.assert_same_bits(G.host(dout), want, "direct n=%d r=%d count=%d /%d" % (n, r, count, divisor))
 
 
 def test_average_costs_no_extra_launch():
