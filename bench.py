@@ -208,6 +208,75 @@ class RingAllreducePerStep(RingAllreduce):
                 A.check(R.ring_copy_bytes(dst, t.data_ptr(), self.sizes[g] * self.esz, stream), "copy")
 
 
+class RingAllreduceDirect(Workload):
+    """The direct form of the same allreduce for one rank of n: the n-1 peers'
+    raw copies of the rank's own segment lie in staging slots (as peers pushing
+    over their own links would leave them) and are folded with the rank's copy
+    in ring order in ONE pass; the other n-1 segments arrive finished and are
+    copied in. Same result as the ring, bit for bit."""
+
+    def __init__(self, name, count, n, nsets, what):
+        import torch
+        from mpi_collectives import _plugin, ring_abi
+        self.torch, self.ring_abi = torch, ring_abi
+        self.L = _plugin.load_library('libmpi_collectives.so', ['MPIAllreduce', 'MPIAllgather'])
+        self.R = ring_abi.lib()
+        self.pdt = _plugin.DT_FLOAT
+        self.name, self.dtype, self.count, self.n, self.nsets, self.esz = name, "f32", count, n, nsets, 4
+        self.sizes, self.starts = ring_abi.segment_table(count, n)
+        self.sets = []
+        for s in range(nsets):
+            r = s % n
+            own = (r + 1) % n
+            gen = torch.Generator(device="cuda").manual_seed(r)
+            inp = torch.randn(count, device="cuda", generator=gen)
+            out = torch.empty(count, device="cuda")
+            peers = [torch.randn(self.sizes[own], device="cuda", generator=gen) for _ in range(n - 1)]
+            ag_seg = [ring_abi.schedule(ring_abi.PHASE_ALLGATHER, n, r, i)[1] for i in range(n - 1)]
+            ag = [torch.randn(self.sizes[g], device="cuda", generator=gen) for g in ag_seg]
+            srcs = [t.data_ptr() for t in peers] + [inp.data_ptr() + self.starts[own] * 4]
+            self.sets.append(dict(
+                r=r, own=own, inp=inp, out=out, peers=peers, ag=ag, ag_seg=ag_seg, srcs=srcs,
+                peer_ptrs=(ctypes.c_void_p * max(n - 1, 1))(*[t.data_ptr() for t in peers]),
+                ag_ptrs=(ctypes.c_void_p * max(n - 1, 1))(*[t.data_ptr() for t in ag]),
+                ag_steps=ring_abi.make_steps([(self.starts[g], t.data_ptr(), self.sizes[g]) for g, t in zip(ag_seg, ag)])))
+        seg = self.sizes[self.sets[0]["own"]]
+        ag_elems = sum(self.sizes[g] for g in self.sets[0]["ag_seg"])
+        self.phases = (
+            ("fold", seg * 4 * (n + 1), "fold_kernel<float> (%d sources -> 1 segment of %d elements)" % (n, seg)),
+            ("allgather", ag_elems * 8, "rows_kernel<unsigned int, kCopy> (%d rows, %d elements)" % (n - 1, ag_elems)))
+        self.dominant = 1
+        self.description = what
+
+    def launch_step(self, k, stream, fused=False):
+        s = self.sets[k % self.nsets]
+        rc = self.L.mpic_ring_allreduce_direct_prestaged(self.n, s["r"], self.pdt, s["inp"].data_ptr(),
+                                                         s["out"].data_ptr(), self.count, s["peer_ptrs"], s["ag_ptrs"],
+                                                         stream, 0)
+        if rc != 0:
+            raise RuntimeError("mpic_ring_allreduce_direct_prestaged failed: %s" % self.L.mpic_last_error().decode())
+
+    def launch_phase(self, k, i, stream):
+        s, A = self.sets[k % self.nsets], self.ring_abi
+        if i == 0:
+            own = s["own"]
+            A.fold_rows([(s["out"].data_ptr() + self.starts[own] * 4, s["srcs"], self.sizes[own])], self.n, 0, A.F32, stream)
+        else:
+            A.check(self.R.ring_allgather_steps(s["out"].data_ptr(), s["ag_steps"][0], s["ag_steps"][1], A.F32, stream),
+                    "allgather")
+
+    def check(self, k):
+        s, torch = self.sets[k % self.nsets], self.torch
+        a, b = self.starts[s["own"]], self.starts[s["own"]] + self.sizes[s["own"]]
+        acc = s["peers"][0].clone()
+        for t in s["peers"][1:]:
+            acc = t + acc
+        ok = torch.equal(s["out"][a:b], s["inp"][a:b] + acc)
+        for g, t in zip(s["ag_seg"], s["ag"]):
+            ok = ok and torch.equal(s["out"][self.starts[g]:self.starts[g] + self.sizes[g]], t)
+        return bool(ok)
+
+
 class FusedResnet50(Workload):
     """161 float32 gradients packed into one fusion buffer, ring-reduced in
     place at N=8 (peers pre-staged), unpacked with the average's divide."""
@@ -311,6 +380,12 @@ def make_workload(name):
                              "float32 ring allreduce of one 16,777,216-element (64 MiB) tensor, N=8 virtual ranks: "
                              "in->out copy + 7 reduce-scatter accumulates + 7 allgather copies on 2,097,152-element "
                              "segments per step, peers pre-staged in HBM, buffers rotated over 8 virtual ranks (cold)")
+    if name == "allreduce_f32_64MiB_n8_direct":
+        return RingAllreduceDirect(name, 16 * 1024 * 1024, 8, 8,
+                                   "float32 allreduce of one 64 MiB tensor, N=8 virtual ranks, DIRECT form: the rank's own "
+                                   "2,097,152-element segment folded in ring order from the 7 peers' staged raw copies "
+                                   "and its own (8 reads, 1 write per element, one launch) + 7 copies of finished "
+                                   "segments; buffers rotated over 8 virtual ranks")
     if name == "allreduce_f32_64MiB_n8_per_step":
         return RingAllreducePerStep(name, "f32", 16 * 1024 * 1024, 8, 8,
                                     "float32 ring allreduce of one 64 MiB tensor, N=8 virtual ranks, ONE LAUNCH PER RING "
@@ -335,7 +410,8 @@ def make_workload(name):
 
 
 WORKLOADS = ("allreduce_f32_64MiB_n8", "allreduce_i32_10000019_n6", "allreduce_i64_10000019_n6",
-             "fused_resnet50_n8", "allgather_f32_n16", "allreduce_f32_1GiB_n64", "allreduce_f32_64MiB_n8_per_step")
+             "fused_resnet50_n8", "allgather_f32_n16", "allreduce_f32_1GiB_n64", "allreduce_f32_64MiB_n8_per_step",
+             "allreduce_f32_64MiB_n8_direct")
 
 
 def cpu_baseline(w):

@@ -71,10 +71,12 @@ size_t ring_dtype_size(int dtype);
  * launch: "nontemporal_copy" (ring_copy_bytes), "nontemporal_accumulate"
  * (accumulates, reduce-scatter tables, row tables, scale),
  * "nontemporal_allgather" (copy tables), "nontemporal_pack",
- * "nontemporal_unpack", "nontemporal_fold"; value bit 0 = non-temporal stores, bit 1 =
- * non-temporal loads, -1 = the default (3, except ordinary stores for the copy
- * and the pack, whose output the next kernel reads, and loads by size for the
- * copy). "nontemporal" sets all six. No counterpart in the reference, whose
+ * "nontemporal_unpack", "nontemporal_fold", "nontemporal_broadcast" (copy
+ * rows of one call that share a source); value bit 0 = non-temporal stores,
+ * bit 1 = non-temporal loads, -1 = the default: 3, except ordinary stores
+ * where the next kernel reads the output (copy, pack, fold), ordinary loads
+ * for a source several rows share (broadcast), and loads by size for the copy.
+ * "nontemporal" sets all seven. No counterpart in the reference, whose
  * launch shape is the constant <<<32, 256>>> (ring.cu.cc:64). */
 int ring_set_option(const char* name, int value);
 

@@ -36,6 +36,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <new>
 #include <vector>
 
@@ -286,6 +287,12 @@ __global__ void __launch_bounds__(kBlock) bytes_kernel(uint8_t* __restrict__ dst
 
 constexpr int kMaxFoldRows = 32;
 constexpr int kMaxFoldPtrs = 256;
+// Tile shape, from a sweep on 8 sources of 8 MiB (the 64 MiB, N=8 segment):
+// 2 vectors per lane per source with the loads of 8 sources in flight at once
+// took 12.7 us; 4 sources at once 13.1; 1 vector per lane 14.2-14.9; 4 vectors
+// per lane (half as many workgroups) 17.3-18.0.
+constexpr int kFoldUnroll = 2;
+constexpr int kFoldGroup = 8;
 
 struct FoldRow {
   void* dst;
@@ -305,14 +312,14 @@ struct FoldTable {
 
 // One tile of a fold row. dst may be one of the row's own sources: a lane reads
 // every source of its elements before it stores them.
-template <typename T, int UNROLL, bool DIV, int NT>
+template <typename T, int UNROLL, int GROUP, bool DIV, int NT>
 __device__ __forceinline__ void fold_tile(T* dst, const void* const* src, int m, uint64_t count, uint32_t tile,
                                           uint32_t tiles_in_row, int n) {
   typedef typename VecOf<T>::type V;
   typedef V VU __attribute__((aligned(sizeof(T))));
   constexpr uint32_t VEC = 16 / sizeof(T);
   constexpr uint32_t kTileVecs = kBlock * UNROLL;
-  constexpr int kGroup = 4;  // sources whose loads are issued together
+  constexpr int kGroup = GROUP;  // sources whose loads are issued together
 
   uint64_t head = ((16u - (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(dst)) & 15u)) & 15u) / sizeof(T);
   if (head > count) head = count;
@@ -374,13 +381,12 @@ __device__ __forceinline__ void fold_tile(T* dst, const void* const* src, int m,
   }
 }
 
-template <typename T, bool DIV, int NT>
+template <typename T, bool DIV, int NT, int UNROLL, int GROUP>
 __global__ void __launch_bounds__(kBlock) fold_kernel(const FoldTable tab) {
-  constexpr int UNROLL = 2;
   if (tab.uniform_tiles) {
     const FoldRow r = tab.row[blockIdx.y];
     for (uint32_t t = blockIdx.x; t < tab.uniform_tiles; t += gridDim.x)
-      fold_tile<T, UNROLL, DIV, NT>(static_cast<T*>(r.dst), tab.src + r.first_ptr, tab.m, r.count, t,
+      fold_tile<T, UNROLL, GROUP, DIV, NT>(static_cast<T*>(r.dst), tab.src + r.first_ptr, tab.m, r.count, t,
                                     tab.uniform_tiles, tab.divisor);
     return;
   }
@@ -393,7 +399,7 @@ __global__ void __launch_bounds__(kBlock) fold_kernel(const FoldTable tab) {
     }
     const FoldRow r = tab.row[lo];
     const uint32_t first = tab.tile_begin[lo];
-    fold_tile<T, UNROLL, DIV, NT>(static_cast<T*>(r.dst), tab.src + r.first_ptr, tab.m, r.count, t - first,
+    fold_tile<T, UNROLL, GROUP, DIV, NT>(static_cast<T*>(r.dst), tab.src + r.first_ptr, tab.m, r.count, t - first,
                                   tab.tile_begin[lo + 1] - first, tab.divisor);
   }
 }
@@ -478,7 +484,7 @@ fusion_kernel(T* __restrict__ fused, const uint64_t* __restrict__ offsets, T* co
 
 constexpr uint64_t kCacheResidentBytes = 128ull << 20;
 
-enum Role { kRoleCopy, kRoleAccumulate, kRoleAllgather, kRolePack, kRoleUnpack, kRoleFold, kRoles };
+enum Role { kRoleCopy, kRoleAccumulate, kRoleAllgather, kRolePack, kRoleUnpack, kRoleFold, kRoleBroadcast, kRoles };
 
 struct Tuning {
   int unroll = 4;          // 16-byte vectors per lane per tile: 2, 4 or 8
@@ -489,7 +495,10 @@ struct Tuning {
   // of a step on tensors up to 128 MiB, which the last-level cache can hold);
   // the copy's loads turn non-temporal above that size, where ordinary ones
   // only evict what the next kernel wants.
-  int nt[kRoles] = {-1, 3, 3, 2, 3, 2};  // the fold's result is what the allgather reads next
+  // the fold's result is what the allgather reads next; a source that several
+  // rows copy (a finished segment fetched by every other rank) is loaded with
+  // the ordinary policy so that it is fetched from HBM once
+  int nt[kRoles] = {-1, 3, 3, 2, 3, 2, 1};
   int blocks_per_cu = 0;   // 0: one workgroup per tile; >0: persistent grid of CUs x this
 };
 Tuning g_tuning;
@@ -759,7 +768,7 @@ int ring_set_option(const char* name, int value) {
     g_tuning.unroll = value;
   } else if (!strncmp(name, "nontemporal", 11)) {
     static const char* const kSuffix[kRoles] = {"_copy", "_accumulate", "_allgather", "_pack", "_unpack",
-                                                "_fold"};
+                                                "_fold", "_broadcast"};
     if (value < -1 || value > 3) return RING_ERR_ARGUMENT;
     const Tuning defaults;
     bool known = name[11] == 0;
@@ -963,8 +972,22 @@ int ring_apply_rows_avg(const ring_row* rows, int n_rows, const unsigned char* d
     host.push_back(HostRow{rows[i].dst, rows[i].a, rows[i].b, rows[i].count,
                            divisor > 0 && (!divide || divide[i] != 0)});
   }
-  return launch_rows(host.data(), host.size(), esz, dtype == RING_F32, static_cast<hipStream_t>(stream),
-                     kRoleAccumulate, divisor);
+  // copy rows that share a source: one buffer handed to several destinations
+  Role role = kRoleAccumulate;
+  if (divisor == 0 && host.size() > 1) {
+    std::vector<const void*> sources;
+    bool copies_only = true;
+    for (const HostRow& r : host) {
+      copies_only = copies_only && r.b == nullptr;
+      sources.push_back(r.a);
+    }
+    if (copies_only) {
+      std::sort(sources.begin(), sources.end());
+      if (std::adjacent_find(sources.begin(), sources.end()) != sources.end()) role = kRoleBroadcast;
+    }
+  }
+  return launch_rows(host.data(), host.size(), esz, dtype == RING_F32, static_cast<hipStream_t>(stream), role,
+                     divisor);
 }
 
 int ring_allgather_steps(void* buffer, const ring_step* steps, int n_steps, int dtype, void* stream) {
@@ -977,7 +1000,7 @@ int ring_fold_rows(const ring_fold_row* rows, int n_rows, int m, int divisor, in
   if (n_rows == 0) return RING_OK;
   if (!rows) return RING_ERR_ARGUMENT;
   const size_t esz = dtype_size(dtype);
-  constexpr uint64_t kTileVecs = static_cast<uint64_t>(kBlock) * 2;
+  constexpr uint64_t kTileVecs = static_cast<uint64_t>(kBlock) * kFoldUnroll;
   const uint64_t vec = 16 / esz;
   const int rows_per_launch = kMaxFoldPtrs / m < kMaxFoldRows ? kMaxFoldPtrs / m : kMaxFoldRows;
   int nt = g_tuning.nt[kRoleFold];
@@ -1026,12 +1049,13 @@ int ring_fold_rows(const ring_fold_row* rows, int n_rows, int m, int divisor, in
       grid = dim3(static_cast<uint32_t>(tiles));
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
-#define RING_FOLD(T, D)                                                              \
-  switch (nt & 3) {                                                                  \
-    case 0: launch(fold_kernel<T, D, 0>, grid, dim3(kBlock), s, tab); break;         \
-    case 1: launch(fold_kernel<T, D, 1>, grid, dim3(kBlock), s, tab); break;         \
-    case 2: launch(fold_kernel<T, D, 2>, grid, dim3(kBlock), s, tab); break;         \
-    default: launch(fold_kernel<T, D, 3>, grid, dim3(kBlock), s, tab); break;        \
+#define RING_FOLD_UG(T, D, N) launch(fold_kernel<T, D, N, kFoldUnroll, kFoldGroup>, grid, dim3(kBlock), s, tab);
+#define RING_FOLD(T, D)                          \
+  switch (nt & 3) {                              \
+    case 0: RING_FOLD_UG(T, D, 0) break;         \
+    case 1: RING_FOLD_UG(T, D, 1) break;         \
+    case 2: RING_FOLD_UG(T, D, 2) break;         \
+    default: RING_FOLD_UG(T, D, 3) break;        \
   }
     if (divisor > 0) {
       if (dtype == RING_F32) { RING_FOLD(float, true) }
@@ -1042,6 +1066,7 @@ int ring_fold_rows(const ring_fold_row* rows, int n_rows, int m, int divisor, in
       else if (dtype == RING_I32) { RING_FOLD(int32_t, false) }
       else { RING_FOLD(int64_t, false) }
     }
+#undef RING_FOLD_UG
 #undef RING_FOLD
     RING_HIP(hipGetLastError());
   }
