@@ -168,7 +168,9 @@ int mpic_ring_allgather_prestaged(int n, int r, int dtype, const void* input, co
 /* All n ranks resident on this GPU: inputs[k] / outputs[k] are rank k's
  * tensors; a neighbour's buffer is read in place of a transfer. `flags` bit 2:
  * the direct form (every segment folded by its owner in one launch, every
- * finished segment copied straight from its owner in a second). */
+ * finished segment copied straight from its owner in a second; for the
+ * allgather, every slice copied from its owner's input into every output in
+ * one launch). */
 int mpic_ring_allreduce_all_ranks(int n, int dtype, const void* const* inputs,
                                   void* const* outputs, size_t count, void* stream, int flags);
 int mpic_ring_allgather_all_ranks(int n, int dtype, const void* const* inputs, const size_t* rows,

@@ -335,6 +335,26 @@ Status RingAllgatherAllRanks(int n, DataType dt, const void* const* inputs, cons
   std::vector<size_t> starts(static_cast<size_t>(n));
   RING_RETURN_IF_ERROR(ring_allgather_table(rows_per_rank.data(), n, elems_per_row, starts.data()), "ring_allgather_table");
 
+  if (opts.direct) {
+    // Every slice straight from its owner's input into every rank's output, one
+    // launch: the values a ring allgather delivers after n-1 steps (it only
+    // moves bytes). A divisor divides every copy, which gives each rank what
+    // the owner's one division would have sent round.
+    std::vector<ring_row> all;
+    for (int r = 0; r < n; r++) {
+      for (int k = 0; k < n; k++) {
+        const size_t cnt = elems_per_row * rows_per_rank[static_cast<size_t>(k)];
+        if (cnt == 0) continue;
+        if (!inputs[k] || !outputs[r]) return errors::InvalidArgument("null tensor with a non-zero element count");
+        all.push_back(ring_row{at(outputs[r], starts[static_cast<size_t>(k)], esz), inputs[k], nullptr, cnt});
+      }
+    }
+    RING_RETURN_IF_ERROR(ring_apply_rows_avg(all.data(), static_cast<int>(all.size()), nullptr, opts.divisor, code,
+                                             stream),
+                         "ring_apply_rows");
+    return Status::OK();
+  }
+
   std::vector<ring_row> rows(static_cast<size_t>(n));
   for (int r = 0; r < n; r++) {  // ring.h:263-266
     const size_t own = elems_per_row * rows_per_rank[static_cast<size_t>(r)];

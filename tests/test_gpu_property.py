@@ -86,11 +86,15 @@ def test_prestaged_rank_equals_oracle(oracle, n, count, dtype, seed, r_pick, fla
 
 @settings(max_examples=40, **COMMON)
 @given(rows=st.lists(st.integers(0, 5000), min_size=1, max_size=12), epr=st.sampled_from([1, 3, 17, 256]),
-       dtype=st.sampled_from(G.DTYPES), seed=st.integers(0, 2**31))
-def test_all_ranks_allgather_is_the_concatenation(rows, epr, dtype, seed):
+       dtype=st.sampled_from(G.DTYPES), seed=st.integers(0, 2**31), direct=st.booleans(),
+       divisor=st.sampled_from([0, 0, 3, 8]))
+def test_all_ranks_allgather_is_the_concatenation(rows, epr, dtype, seed, direct, divisor):
     n = len(rows)
     parts = [G.random_array(np.random.default_rng(seed + r), rows[r] * epr, dtype) for r in range(n)]
     want = np.concatenate(parts) if parts else np.empty(0, dtype=dtype)
+    if divisor:
+        with np.errstate(all="ignore"):
+            want = (want / np.float32(divisor) if dtype == np.float32 else want // dtype(divisor)).astype(dtype)
     L = _plugin.load_library()
     dins = [G.dev(p, r % 4) for r, p in enumerate(parts)]
     douts = [G.dev(np.zeros(want.size, dtype=dtype), (r + 1) % 4) for r in range(n)]
@@ -98,11 +102,13 @@ def test_all_ranks_allgather_is_the_concatenation(rows, epr, dtype, seed):
     pout = (ctypes.c_void_p * n)(*[d[0].data_ptr() if want.size else None for d in douts])
     rows_c = (ctypes.c_size_t * n)(*rows)
     rc = L.mpic_ring_allgather_all_ranks(n, DT[np.dtype(dtype)], pin, rows_c, epr, pout,
-                                         torch.cuda.current_stream().cuda_stream, 1)
+                                         torch.cuda.current_stream().cuda_stream,
+                                         1 | (4 if direct else 0) | (divisor << 8))
     assert rc == 0, L.mpic_last_error()
     torch.cuda.synchronize()
     for r in range(n):
-        G.assert_same_bits(G.host(douts[r][0]), want, "allgather rows=%r epr=%d rank %d" % (rows, epr, r))
+        G.assert_same_bits(G.host(douts[r][0]), want,
+                           "allgather rows=%r epr=%d rank %d direct=%s /%d" % (rows, epr, r, direct, divisor))
 
 
 @settings(max_examples=30, **COMMON)

@@ -110,14 +110,16 @@ def test_allreduce_average_is_tf_div(oracle, n):
             G.assert_same_bits(G.host(o), want.astype(dtype), "average %s n=%d" % (dtype.__name__, n))
 
 
+@pytest.mark.parametrize("direct", [1, 0])
 @pytest.mark.parametrize("size", [1, 2, 3, 7, 16])
-def test_reference_allgather_tests(size):
+def test_reference_allgather_tests(size, direct):
     """mpi_ops_test.py:204-263: rank-stamped tensors, equal and variable first
     dimension, 1-3 dims, int32 and float32 (int64 added)."""
     tensor_sizes = ([17, 32, 81, 12, 15, 23, 22] * 5)[:size]
     for dtype, dim, variable in itertools.product((torch.int32, torch.float32, torch.int64), (1, 2, 3), (False, True)):
         rows = tensor_sizes if variable else [17] * size
         with mpi.Session(size=size) as session:
+            session.set_option("direct", direct)        # every slice from its owner at once / the lockstep ring
             hs = []
             for r in range(size):
                 with session.as_rank(r):
@@ -132,7 +134,8 @@ def test_reference_allgather_tests(size):
                 assert bool((part == i).all()), "mpi.allgather produces incorrect gathered tensor"
 
 
-def test_allgather_variable_rows_n16_matches_oracle(oracle):
+@pytest.mark.parametrize("direct", [1, 0])
+def test_allgather_variable_rows_n16_matches_oracle(oracle, direct):
     """Rank i contributes [rows_i, 1024] float32 with rows_i uniform in [1, 4096]."""
     n = 16
     rows = [int(np.random.default_rng(i).integers(1, 4097)) for i in range(n)]
@@ -140,6 +143,7 @@ def test_allgather_variable_rows_n16_matches_oracle(oracle):
     want = np.concatenate(ins, axis=0)
     assert np.array_equal(oracle.ring_allgather([x[:3] for x in ins])[5], np.concatenate([x[:3] for x in ins]))
     with mpi.Session(size=n) as session:
+        session.set_option("direct", direct)
         hs = []
         for r in range(n):
             with session.as_rank(r):
@@ -153,12 +157,14 @@ def test_allgather_variable_rows_n16_matches_oracle(oracle):
         assert torch.equal(outs[r], outs[0])
 
 
-def test_allgather_with_empty_ranks_and_indexed_slices(oracle):
+@pytest.mark.parametrize("direct", [1, 0])
+def test_allgather_with_empty_ranks_and_indexed_slices(oracle, direct):
     n = 4
     rows = [3, 0, 5, 1]
     vals = [np.random.default_rng(r).standard_normal((rows[r], 6)).astype(np.float32) for r in range(n)]
     idx = [np.arange(rows[r], dtype=np.int64) * 10 + r for r in range(n)]
     with mpi.Session(size=n) as session:
+        session.set_option("direct", direct)
         hs = []
         for r in range(n):
             with session.as_rank(r):
