@@ -743,10 +743,12 @@ def test_non_contiguous_and_multi_dimensional_tensors(oracle):
         G.assert_same_bits(G.host(c), gathered, "transposed gather")
 
 
-def test_committed_known_answer_vectors_on_the_gpu():
+@pytest.mark.parametrize("direct", [0, 1])
+def test_committed_known_answer_vectors_on_the_gpu(direct):
     """tests/golden/ring_kats.json (order-sensitive inputs, expected values from
     a pure-Python mailbox simulation of the reference schedule) through the op
-    layer: every rank's output equals the committed answer bit for bit."""
+    layer, as the lockstep ring and in the direct form: every rank's output
+    equals the committed answer bit for bit."""
     import json
     import os
     with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ring_kats.json")) as f:
@@ -762,10 +764,12 @@ def test_committed_known_answer_vectors_on_the_gpu():
             want = np.array(case["expected"], dtype=dt)
         n = case["n"]
         with mpi.Session(size=n) as session:
+            session.set_option("direct", direct)
             hs = []
             for r in range(n):
                 with session.as_rank(r):
                     hs.append(mpi.allreduce(cuda(ins[r]), average=False))
             outs = session.run(hs)
         for r in range(n):
-            G.assert_same_bits(G.host(outs[r]), want, "KAT %s n=%d count=%d rank %d" % (case["dtype"], n, case["count"], r))
+            G.assert_same_bits(G.host(outs[r]), want,
+                               "KAT %s n=%d count=%d rank %d direct=%d" % (case["dtype"], n, case["count"], r, direct))
