@@ -288,6 +288,27 @@ def test_direct_form_for_one_rank_matches_the_ring(oracle, dtype):
             G.assert_same_bits(G.host(dout), want, "direct n=%d r=%d count=%d /%d" % (n, r, count, divisor))
 
 
+@pytest.mark.parametrize("n", [33, 64])
+def test_direct_form_with_more_sources_than_one_launch_holds(oracle, n):
+    """n*n source pointers exceed one fold launch's table: the rows are spread
+    over several launches; float32 and int64 against the oracle."""
+    L = _plugin.load_library()
+    for dtype in (np.float32, np.int64):
+        count = 10 * n + 7
+        ins = make_inputs(n, count, dtype, seed=n)
+        want = oracle.ring_allreduce_lockstep(ins)
+        dins = [cuda(x) for x in ins]
+        douts = [torch.zeros(count, dtype=G.NP2TORCH[np.dtype(dtype)], device="cuda") for _ in range(n)]
+        ip = (ctypes.c_void_p * n)(*[t.data_ptr() for t in dins])
+        op = (ctypes.c_void_p * n)(*[t.data_ptr() for t in douts])
+        rc = L.mpic_ring_allreduce_all_ranks(n, DT[np.dtype(dtype)], ip, op, count,
+                                             torch.cuda.current_stream().cuda_stream, 7)
+        assert rc == 0, L.mpic_last_error()
+        torch.cuda.synchronize()
+        for r in range(n):
+            G.assert_same_bits(G.host(douts[r]), want[r], "direct n=%d rank %d" % (n, r))
+
+
 def test_average_costs_no_extra_launch():
     """allreduce(average=True) over resident ranks: as many kernel launches as
     the sum alone (the divide rides on the last reduce-scatter step)."""
