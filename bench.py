@@ -243,27 +243,26 @@ class RingAllreduceDirect(Workload):
         seg = self.sizes[self.sets[0]["own"]]
         ag_elems = sum(self.sizes[g] for g in self.sets[0]["ag_seg"])
         self.phases = (
-            ("fold", seg * 4 * (n + 1), "fold_kernel<float> (%d sources -> 1 segment of %d elements)" % (n, seg)),
-            ("allgather", ag_elems * 8, "rows_kernel<unsigned int, kCopy> (%d rows, %d elements)" % (n - 1, ag_elems)))
-        self.dominant = 1
+            ("fold_and_copies", seg * 4 * (n + 1) + ag_elems * 8,
+             "fold_kernel<float> (1 row folding %d sources into %d elements + %d copy rows, %d elements)"
+             % (n, seg, n - 1, ag_elems)),)
+        self.dominant = 0
         self.description = what
 
     def launch_step(self, k, stream, fused=False):
         s = self.sets[k % self.nsets]
         rc = self.L.mpic_ring_allreduce_direct_prestaged(self.n, s["r"], self.pdt, s["inp"].data_ptr(),
                                                          s["out"].data_ptr(), self.count, s["peer_ptrs"], s["ag_ptrs"],
-                                                         stream, 0)
+                                                         stream, 1)
         if rc != 0:
             raise RuntimeError("mpic_ring_allreduce_direct_prestaged failed: %s" % self.L.mpic_last_error().decode())
 
     def launch_phase(self, k, i, stream):
         s, A = self.sets[k % self.nsets], self.ring_abi
-        if i == 0:
-            own = s["own"]
-            A.fold_rows([(s["out"].data_ptr() + self.starts[own] * 4, s["srcs"], self.sizes[own])], self.n, 0, A.F32, stream)
-        else:
-            A.check(self.R.ring_allgather_steps(s["out"].data_ptr(), s["ag_steps"][0], s["ag_steps"][1], A.F32, stream),
-                    "allgather")
+        own, out = s["own"], s["out"].data_ptr()
+        A.fold_and_copy_rows([(out + self.starts[own] * 4, s["srcs"], self.sizes[own])], self.n, 0,
+                             [(out + self.starts[g] * 4, t.data_ptr(), self.sizes[g]) for g, t in zip(s["ag_seg"], s["ag"])],
+                             A.F32, stream)
 
     def check(self, k):
         s, torch = self.sets[k % self.nsets], self.torch
@@ -384,8 +383,8 @@ def make_workload(name):
         return RingAllreduceDirect(name, 16 * 1024 * 1024, 8, 8,
                                    "float32 allreduce of one 64 MiB tensor, N=8 virtual ranks, DIRECT form: the rank's own "
                                    "2,097,152-element segment folded in ring order from the 7 peers' staged raw copies "
-                                   "and its own (8 reads, 1 write per element, one launch) + 7 copies of finished "
-                                   "segments; buffers rotated over 8 virtual ranks")
+                                   "and its own (8 reads, 1 write per element) + 7 copies of finished segments, all in "
+                                   "one launch; buffers rotated over 8 virtual ranks")
     if name == "allreduce_f32_64MiB_n8_per_step":
         return RingAllreducePerStep(name, "f32", 16 * 1024 * 1024, 8, 8,
                                     "float32 ring allreduce of one 64 MiB tensor, N=8 virtual ranks, ONE LAUNCH PER RING "

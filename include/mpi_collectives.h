@@ -155,8 +155,9 @@ int mpic_ring_allreduce_prestaged(int n, int r, int dtype, const void* input, vo
  * they are folded with the rank's own copy in ring order, one pass
  * (ring_fold_rows), into output[s]; ag_segments[i] is the finished segment
  * (r-i) mod n. The output is bit-identical to mpic_ring_allreduce_prestaged
- * fed with the ring's traffic. `flags`: bits 8-30 = divisor. No counterpart in
- * the reference. */
+ * fed with the ring's traffic. `flags`: bit 0 = fold and copies in one launch
+ * (they write disjoint segments), bits 8-30 = divisor. No counterpart in the
+ * reference. */
 int mpic_ring_allreduce_direct_prestaged(int n, int r, int dtype, const void* input, void* output,
                                          size_t count, const void* const* peer_segments,
                                          const void* const* ag_segments, void* stream, int flags);

@@ -233,6 +233,13 @@ typedef struct ring_fold_row {
   uint64_t count;          /* elements */
 } ring_fold_row;
 int ring_fold_rows(const ring_fold_row* rows, int n_rows, int m, int divisor, int dtype, void* stream);
+/* The fold rows and, in the SAME launch, plain copy rows (b must be NULL; never
+ * divided): a rank's whole direct step, its own segment folded from the
+ * pushed copies while the other ranks' finished segments are copied in. The
+ * two kinds of row write disjoint memory, so one launch saves the start-up and
+ * drain of a second. */
+int ring_fold_and_copy_rows(const ring_fold_row* fold_rows, int n_fold, int m, int divisor,
+                            const ring_row* copy_rows, int n_copy, int dtype, void* stream);
 
 /* ---- tensor fusion (no counterpart in the reference, which issues one
  * MPIAllreduce per gradient, __init__.py:195-205): k tensors are packed back

@@ -156,24 +156,27 @@ Status RingAllreduceDirectPrestaged(int n, int r, DataType dt, const void* input
 
   // the owned segment: x_s, x_{s+1}, ..., x_{s+n-1} = this rank's own, folded in that order
   const size_t own = static_cast<size_t>((r + 1) % n);
-  if (sizes[own]) {
-    std::vector<const void*> srcs;
-    for (int k = 0; k < n - 1; k++) {
-      if (!peers[k]) return errors::InvalidArgument("null staged peer segment");
-      srcs.push_back(peers[k]);
-    }
-    srcs.push_back(at(input, starts[own], esz));
-    ring_fold_row row{at(output, starts[own], esz), srcs.data(), sizes[own]};
-    RING_RETURN_IF_ERROR(ring_fold_rows(&row, 1, n, opts.divisor, code, stream), "ring_fold_rows");
+  std::vector<const void*> srcs;
+  for (int k = 0; k < n - 1; k++) {
+    if (sizes[own] && !peers[k]) return errors::InvalidArgument("null staged peer segment");
+    srcs.push_back(peers[k]);
   }
+  srcs.push_back(at(input, starts[own], esz));
+  ring_fold_row fold{at(output, starts[own], esz), srcs.data(), sizes[own]};
   // every other segment arrives finished (ring.h:211-225 delivers the same values step by step)
-  std::vector<ring_step> steps;
+  std::vector<ring_row> copies;
   for (int i = 0; i < n - 1; i++) {
     const size_t seg = static_cast<size_t>(Seg(RING_PHASE_ALLGATHER, n, r, i, true));
-    steps.push_back(ring_step{starts[seg], ag_recv[i], sizes[seg]});
+    copies.push_back(ring_row{at(output, starts[seg], esz), ag_recv[i], nullptr, sizes[seg]});
   }
-  if (n > 1)
-    RING_RETURN_IF_ERROR(ring_allgather_steps(output, steps.data(), n - 1, code, stream), "ring_allgather_steps");
+  if (opts.batched) {
+    // fold and copies write disjoint segments: one launch
+    RING_RETURN_IF_ERROR(ring_fold_and_copy_rows(&fold, 1, n, opts.divisor, copies.data(), n - 1, code, stream),
+                         "ring_fold_and_copy_rows");
+  } else {
+    RING_RETURN_IF_ERROR(ring_fold_rows(&fold, 1, n, opts.divisor, code, stream), "ring_fold_rows");
+    RING_RETURN_IF_ERROR(ring_apply_rows(copies.data(), n - 1, code, stream), "ring_apply_rows");
+  }
   return Status::OK();
 }
 

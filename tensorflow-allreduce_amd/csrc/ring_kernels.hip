@@ -298,12 +298,12 @@ struct FoldRow {
   void* dst;
   uint64_t count;      // elements
   uint32_t first_ptr;  // index of the row's first source in FoldTable::src
-  uint32_t pad;
+  uint32_t m;          // sources, folded in the order they are listed; 1 = a copy row
 };
 struct FoldTable {
   int n_rows;
-  int m;                   // sources per row, folded in the order they are listed
-  int divisor;             // > 0: the fold is divided (tf.div) before it is stored
+  int divisor;             // > 0: rows whose bit is set in div_mask are divided (tf.div) before they are stored
+  uint32_t div_mask;
   uint32_t uniform_tiles;  // as RowTable
   uint32_t tile_begin[kMaxFoldRows + 1];
   FoldRow row[kMaxFoldRows];
@@ -311,10 +311,11 @@ struct FoldTable {
 };
 
 // One tile of a fold row. dst may be one of the row's own sources: a lane reads
-// every source of its elements before it stores them.
+// every source of its elements before it stores them. DIV && divide: the fold
+// is divided by n before it is stored (divide is uniform over the workgroup).
 template <typename T, int UNROLL, int GROUP, bool DIV, int NT>
 __device__ __forceinline__ void fold_tile(T* dst, const void* const* src, int m, uint64_t count, uint32_t tile,
-                                          uint32_t tiles_in_row, int n) {
+                                          uint32_t tiles_in_row, int n, bool divide) {
   typedef typename VecOf<T>::type V;
   typedef V VU __attribute__((aligned(sizeof(T))));
   constexpr uint32_t VEC = 16 / sizeof(T);
@@ -330,7 +331,7 @@ __device__ __forceinline__ void fold_tile(T* dst, const void* const* src, int m,
   auto scalar = [&](uint64_t e) {
     T acc = static_cast<const T*>(src[0])[e];
     for (int k = 1; k < m; k++) acc = add_one(acc, static_cast<const T*>(src[k])[e]);
-    dst[e] = DIV ? div_one(acc, n) : acc;
+    dst[e] = (DIV && divide) ? div_one(acc, n) : acc;
   };
   if (tile == 0 && tid < head) scalar(tid);
   if (tile + 1 == tiles_in_row) {
@@ -375,19 +376,32 @@ __device__ __forceinline__ void fold_tile(T* dst, const void* const* src, int m,
 #pragma unroll
   for (int j = 0; j < UNROLL; j++) {
     if (ok[j]) {
-      if (DIV) acc[j] = apply_vec<T, kOpDiv>(acc[j], acc[j], n);
+      if (DIV && divide) acc[j] = apply_vec<T, kOpDiv>(acc[j], acc[j], n);
       store_vec<T, NT>(&dv[v0 + j * kBlock], acc[j]);
     }
   }
 }
 
+// A row with one source and no divide is a plain copy (the finished segments a
+// rank takes in next to the fold of its own): touched once, so non-temporal
+// both ways whatever the fold rows use.
+template <typename T, bool DIV, int NT, int UNROLL, int GROUP>
+__device__ __forceinline__ void fold_row_tile(const FoldTable& tab, int row, uint32_t tile, uint32_t tiles_in_row) {
+  const FoldRow r = tab.row[row];
+  const bool divide = DIV && ((tab.div_mask >> row) & 1u);
+  if (r.m == 1 && !divide)
+    fold_tile<T, UNROLL, GROUP, false, 3>(static_cast<T*>(r.dst), tab.src + r.first_ptr, 1, r.count, tile, tiles_in_row,
+                                          0, false);
+  else
+    fold_tile<T, UNROLL, GROUP, DIV, NT>(static_cast<T*>(r.dst), tab.src + r.first_ptr, static_cast<int>(r.m), r.count,
+                                         tile, tiles_in_row, tab.divisor, divide);
+}
+
 template <typename T, bool DIV, int NT, int UNROLL, int GROUP>
 __global__ void __launch_bounds__(kBlock) fold_kernel(const FoldTable tab) {
   if (tab.uniform_tiles) {
-    const FoldRow r = tab.row[blockIdx.y];
     for (uint32_t t = blockIdx.x; t < tab.uniform_tiles; t += gridDim.x)
-      fold_tile<T, UNROLL, GROUP, DIV, NT>(static_cast<T*>(r.dst), tab.src + r.first_ptr, tab.m, r.count, t,
-                                    tab.uniform_tiles, tab.divisor);
+      fold_row_tile<T, DIV, NT, UNROLL, GROUP>(tab, static_cast<int>(blockIdx.y), t, tab.uniform_tiles);
     return;
   }
   const uint32_t total = tab.tile_begin[tab.n_rows];
@@ -397,10 +411,8 @@ __global__ void __launch_bounds__(kBlock) fold_kernel(const FoldTable tab) {
       const int mid = (lo + hi) >> 1;
       if (tab.tile_begin[mid] <= t) lo = mid; else hi = mid;
     }
-    const FoldRow r = tab.row[lo];
     const uint32_t first = tab.tile_begin[lo];
-    fold_tile<T, UNROLL, GROUP, DIV, NT>(static_cast<T*>(r.dst), tab.src + r.first_ptr, tab.m, r.count, t - first,
-                                  tab.tile_begin[lo + 1] - first, tab.divisor);
+    fold_row_tile<T, DIV, NT, UNROLL, GROUP>(tab, lo, t - first, tab.tile_begin[lo + 1] - first);
   }
 }
 
@@ -994,29 +1006,39 @@ int ring_allgather_steps(void* buffer, const ring_step* steps, int n_steps, int 
   return steps_common(nullptr, buffer, steps, n_steps, dtype, stream, kStepCopy);
 }
 
-int ring_fold_rows(const ring_fold_row* rows, int n_rows, int m, int divisor, int dtype, void* stream) {
-  if (!dtype_ok(dtype)) return RING_ERR_DTYPE;
-  if (n_rows < 0 || m < 1 || m > kMaxFoldPtrs || divisor < 0) return RING_ERR_ARGUMENT;
-  if (n_rows == 0) return RING_OK;
-  if (!rows) return RING_ERR_ARGUMENT;
+namespace {
+
+struct HostFoldRow {
+  void* dst;
+  const void* const* srcs;
+  int m;
+  uint64_t count;
+  bool divide;
+};
+
+// Launches fold rows (any number, any mix of source counts) in tables of at most
+// kMaxFoldRows rows and kMaxFoldPtrs source pointers.
+int launch_fold(const HostFoldRow* rows, size_t n_rows, int divisor, int dtype, hipStream_t s) {
   const size_t esz = dtype_size(dtype);
   constexpr uint64_t kTileVecs = static_cast<uint64_t>(kBlock) * kFoldUnroll;
   const uint64_t vec = 16 / esz;
-  const int rows_per_launch = kMaxFoldPtrs / m < kMaxFoldRows ? kMaxFoldPtrs / m : kMaxFoldRows;
   int nt = g_tuning.nt[kRoleFold];
   if (nt < 0) nt = 2;
-  int i = 0;
+  size_t i = 0;
   while (i < n_rows) {
     FoldTable tab;
     tab.n_rows = 0;
-    tab.m = m;
     tab.divisor = divisor;
+    tab.div_mask = 0;
     tab.tile_begin[0] = 0;
     uint64_t tiles = 0, first_tiles = 0;
+    uint32_t ptrs = 0;
     bool uniform = true;
-    while (i < n_rows && tab.n_rows < rows_per_launch) {
-      const ring_fold_row& r = rows[i];
+    while (i < n_rows && tab.n_rows < kMaxFoldRows) {
+      const HostFoldRow& r = rows[i];
       if (r.count == 0) { i++; continue; }
+      if (r.m < 1 || r.m > kMaxFoldPtrs) return RING_ERR_ARGUMENT;
+      if (ptrs + static_cast<uint32_t>(r.m) > static_cast<uint32_t>(kMaxFoldPtrs)) break;  // next table
       if (!r.dst || !r.srcs || (reinterpret_cast<uintptr_t>(r.dst) & (esz - 1))) return RING_ERR_ARGUMENT;
       const uintptr_t d = reinterpret_cast<uintptr_t>(r.dst);
       uint64_t head = ((16u - (d & 15u)) & 15u) / esz;
@@ -1028,11 +1050,12 @@ int ring_fold_rows(const ring_fold_row* rows, int n_rows, int m, int divisor, in
         break;
       }
       const int k = tab.n_rows++;
-      tab.row[k] = FoldRow{r.dst, r.count, static_cast<uint32_t>(k * m), 0};
-      for (int j = 0; j < m; j++) {
+      tab.row[k] = FoldRow{r.dst, r.count, ptrs, static_cast<uint32_t>(r.m)};
+      for (int j = 0; j < r.m; j++) {
         if (!r.srcs[j] || (reinterpret_cast<uintptr_t>(r.srcs[j]) & (esz - 1))) return RING_ERR_ARGUMENT;
-        tab.src[k * m + j] = r.srcs[j];
+        tab.src[ptrs++] = r.srcs[j];
       }
+      if (divisor > 0 && r.divide) tab.div_mask |= 1u << k;
       if (k == 0) first_tiles = t;
       uniform = uniform && t == first_tiles;
       tiles += t;
@@ -1048,7 +1071,6 @@ int ring_fold_rows(const ring_fold_row* rows, int n_rows, int m, int divisor, in
       tab.uniform_tiles = 0;
       grid = dim3(static_cast<uint32_t>(tiles));
     }
-    hipStream_t s = static_cast<hipStream_t>(stream);
 #define RING_FOLD_UG(T, D, N) launch(fold_kernel<T, D, N, kFoldUnroll, kFoldGroup>, grid, dim3(kBlock), s, tab);
 #define RING_FOLD(T, D)                          \
   switch (nt & 3) {                              \
@@ -1057,7 +1079,7 @@ int ring_fold_rows(const ring_fold_row* rows, int n_rows, int m, int divisor, in
     case 2: RING_FOLD_UG(T, D, 2) break;         \
     default: RING_FOLD_UG(T, D, 3) break;        \
   }
-    if (divisor > 0) {
+    if (tab.div_mask != 0) {
       if (dtype == RING_F32) { RING_FOLD(float, true) }
       else if (dtype == RING_I32) { RING_FOLD(int32_t, true) }
       else { RING_FOLD(int64_t, true) }
@@ -1071,6 +1093,29 @@ int ring_fold_rows(const ring_fold_row* rows, int n_rows, int m, int divisor, in
     RING_HIP(hipGetLastError());
   }
   return RING_OK;
+}
+
+}  // namespace
+
+int ring_fold_rows(const ring_fold_row* rows, int n_rows, int m, int divisor, int dtype, void* stream) {
+  return ring_fold_and_copy_rows(rows, n_rows, m, divisor, nullptr, 0, dtype, stream);
+}
+
+int ring_fold_and_copy_rows(const ring_fold_row* fold_rows, int n_fold, int m, int divisor, const ring_row* copy_rows,
+                            int n_copy, int dtype, void* stream) {
+  if (!dtype_ok(dtype)) return RING_ERR_DTYPE;
+  if (n_fold < 0 || n_copy < 0 || divisor < 0) return RING_ERR_ARGUMENT;
+  if (n_fold > 0 && (m < 1 || m > kMaxFoldPtrs || !fold_rows)) return RING_ERR_ARGUMENT;
+  if (n_copy > 0 && !copy_rows) return RING_ERR_ARGUMENT;
+  std::vector<HostFoldRow> host;
+  host.reserve(static_cast<size_t>(n_fold) + static_cast<size_t>(n_copy));
+  for (int i = 0; i < n_fold; i++)
+    host.push_back(HostFoldRow{fold_rows[i].dst, fold_rows[i].srcs, m, fold_rows[i].count, true});
+  for (int i = 0; i < n_copy; i++) {
+    if (copy_rows[i].b != nullptr) return RING_ERR_ARGUMENT;  // copy rows only
+    host.push_back(HostFoldRow{copy_rows[i].dst, &copy_rows[i].a, 1, copy_rows[i].count, false});
+  }
+  return launch_fold(host.data(), host.size(), divisor, dtype, static_cast<hipStream_t>(stream));
 }
 
 int ring_scale(int dtype, void* data, size_t count, int divisor, void* stream) {

@@ -22,7 +22,7 @@ EXPORTS = (
     "ring_schedule", "ring_stream_create", "ring_stream_destroy", "ring_stream_synchronize",
     "ring_copy_bytes", "ring_accumulate_f32", "ring_accumulate_i32", "ring_accumulate_i64",
     "ring_accumulate", "ring_reduce_scatter_steps", "ring_reduce_scatter_steps_from",
-    "ring_allgather_steps", "ring_apply_rows", "ring_apply_rows_avg", "ring_fold_rows",
+    "ring_allgather_steps", "ring_apply_rows", "ring_apply_rows_avg", "ring_fold_rows", "ring_fold_and_copy_rows",
     "ring_fusion_plan_create", "ring_fusion_plan_destroy", "ring_fusion_plan_elements",
     "ring_fusion_pack", "ring_fusion_unpack", "ring_fusion_unpack_scaled", "ring_scale",
 )
@@ -99,6 +99,7 @@ def lib():
             "ring_apply_rows": (ci, [ctypes.POINTER(Row), ci, ci, vp]),
             "ring_apply_rows_avg": (ci, [ctypes.POINTER(Row), ci, ctypes.POINTER(ctypes.c_ubyte), ci, ci, vp]),
             "ring_fold_rows": (ci, [ctypes.POINTER(FoldRow), ci, ci, ci, ci, vp]),
+            "ring_fold_and_copy_rows": (ci, [ctypes.POINTER(FoldRow), ci, ci, ci, ctypes.POINTER(Row), ci, ci, vp]),
             "ring_fusion_plan_create": (ci, [ctypes.POINTER(vp), psz, ci, ci, ctypes.POINTER(vp)]),
             "ring_fusion_plan_destroy": (ci, [vp]),
             "ring_fusion_plan_elements": (sz, [vp]),
@@ -249,8 +250,7 @@ def apply_rows_avg(rows, divide, divisor, dtype, stream):
     check(lib().ring_apply_rows_avg(arr, len(rows), flags, divisor, dtype, stream), "ring_apply_rows_avg")
 
 
-def fold_rows(rows, m, divisor, dtype, stream):
-    """rows: iterable of (dst, [m source pointers in fold order], count)."""
+def _fold_array(rows, m):
     rows = list(rows)
     arr = (FoldRow * max(len(rows), 1))()
     keep = []
@@ -258,7 +258,24 @@ def fold_rows(rows, m, divisor, dtype, stream):
         ptrs = (ctypes.c_void_p * m)(*srcs)
         keep.append(ptrs)
         arr[i].dst, arr[i].srcs, arr[i].count = d, ctypes.cast(ptrs, ctypes.POINTER(ctypes.c_void_p)), cnt
-    check(lib().ring_fold_rows(arr, len(rows), m, divisor, dtype, stream), "ring_fold_rows")
+    return arr, len(rows), keep
+
+
+def fold_rows(rows, m, divisor, dtype, stream):
+    """rows: iterable of (dst, [m source pointers in fold order], count)."""
+    arr, n, _keep = _fold_array(rows, m)
+    check(lib().ring_fold_rows(arr, n, m, divisor, dtype, stream), "ring_fold_rows")
+
+
+def fold_and_copy_rows(fold, m, divisor, copies, dtype, stream):
+    """fold: as fold_rows; copies: iterable of (dst, src, count); one launch."""
+    arr, n, _keep = _fold_array(fold, m)
+    copies = list(copies)
+    carr = (Row * max(len(copies), 1))()
+    for i, (d, a, cnt) in enumerate(copies):
+        carr[i].dst, carr[i].a, carr[i].b, carr[i].count = d, a, None, cnt
+    check(lib().ring_fold_and_copy_rows(arr, n, m, divisor, carr, len(copies), dtype, stream),
+          "ring_fold_and_copy_rows")
 
 
 def scale(dtype, data, count, divisor, stream):

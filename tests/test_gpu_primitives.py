@@ -291,6 +291,41 @@ def test_fold_rows_is_the_sequential_fold(dtype):
 
 
 @pytest.mark.parametrize("dtype", G.DTYPES)
+def test_fold_and_copy_rows_in_one_call(dtype):
+    """Fold rows (divided) and plain copy rows (never divided) of one call; more
+    source pointers and rows than one launch's table holds."""
+    rng = np.random.default_rng(123)
+    code = G.NP2ABI[np.dtype(dtype)]
+    for m, fold_counts, copy_counts, divisor in ((8, [20_003], [5000, 7, 0, 9001, 4096, 33, 12_345], 8),
+                                                 (100, [700, 1300, 5], [int(c) for c in rng.integers(0, 2000, 45)], 0),
+                                                 (3, [], [10, 20], 4), (2, [9], [], 2)):
+        keep, fold, copies, checks = [], [], [], []
+        for k, c in enumerate(fold_counts):
+            hs = [G.random_array(rng, c, dtype) for _ in range(m)]
+            ds = [G.dev(h, (k + j) % 4) for j, h in enumerate(hs)]
+            dst, base = G.dev(np.zeros(c, dtype=dtype), (k + 1) % 4)
+            keep += [ds, base]
+            fold.append((dst.data_ptr(), [d[0].data_ptr() for d in ds], c))
+            checks.append((dst, _fold_reference(hs, divisor, dtype), "fold row %d" % k))
+        for k, c in enumerate(copy_counts):
+            h = G.random_array(rng, c, dtype)
+            d, b1 = G.dev(h, k % 4)
+            dst, b2 = G.dev(np.zeros(c, dtype=dtype), (k + 3) % 4)
+            keep += [b1, b2]
+            copies.append((dst.data_ptr() if c else None, d.data_ptr() if c else None, c))
+            checks.append((dst, h, "copy row %d" % k))
+        ring_abi.fold_and_copy_rows(fold, m, divisor, copies, code, None)
+        G.sync()
+        for dst, want, what in checks:
+            G.assert_same_bits(G.host(dst), want, "%s (m=%d, /%d)" % (what, m, divisor))
+    x, _ = G.dev(np.ones(8, dtype=dtype), 0)
+    L = ring_abi.lib()
+    bad = (ring_abi.Row * 1)()
+    bad[0].dst, bad[0].a, bad[0].b, bad[0].count = x.data_ptr(), x.data_ptr(), x.data_ptr(), 8      # an add row
+    assert L.ring_fold_and_copy_rows(None, 0, 1, 0, bad, 1, code, None) == 2      # RING_ERR_ARGUMENT
+
+
+@pytest.mark.parametrize("dtype", G.DTYPES)
 def test_scale_is_tf_div(dtype):
     """allreduce(average=True) divides with tf.div (__init__.py:160-164): true
     division for float32, floor division for integers."""

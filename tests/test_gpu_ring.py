@@ -279,13 +279,16 @@ def test_direct_form_for_one_rank_matches_the_ring(oracle, dtype):
             pp = (ctypes.c_void_p * max(n - 1, 1))(*[t.data_ptr() if t.numel() else None for t in peers])
             ap = (ctypes.c_void_p * max(n - 1, 1))(*[t.data_ptr() if t.numel() else None for t in ags])
             din = cuda(ins[r])
-            dout = torch.zeros(count + 4, dtype=G.NP2TORCH[np.dtype(dtype)], device="cuda")[:count]
-            rc = L.mpic_ring_allreduce_direct_prestaged(n, r, DT[np.dtype(dtype)], din.data_ptr() if count else None,
-                                                        dout.data_ptr() if count else None, count, pp, ap,
-                                                        torch.cuda.current_stream().cuda_stream, divisor << 8)
-            assert rc == 0, L.mpic_last_error()
-            torch.cuda.synchronize()
-            G.assert_same_bits(G.host(dout), want, "direct n=%d r=%d count=%d /%d" % (n, r, count, divisor))
+            for one_launch in (1, 0):
+                dout = torch.zeros(count + 4, dtype=G.NP2TORCH[np.dtype(dtype)], device="cuda")[:count]
+                rc = L.mpic_ring_allreduce_direct_prestaged(n, r, DT[np.dtype(dtype)], din.data_ptr() if count else None,
+                                                            dout.data_ptr() if count else None, count, pp, ap,
+                                                            torch.cuda.current_stream().cuda_stream,
+                                                            one_launch | (divisor << 8))
+                assert rc == 0, L.mpic_last_error()
+                torch.cuda.synchronize()
+                G.assert_same_bits(G.host(dout), want, "direct n=%d r=%d count=%d /%d one launch=%d"
+                                   % (n, r, count, divisor, one_launch))
 
 
 @pytest.mark.parametrize("n", [33, 64])
