@@ -102,6 +102,18 @@ static void ring_case(int n, size_t count, void* stream) {
     CHECK(mpic_ring_allreduce_prestaged(n, r, Code<T>::mpic, d_in, d_out, count, rs_p.data(), ag_p.data(), stream, 3) == MPIC_OK);
     CHECK(ring_stream_synchronize(stream) == RING_OK);
     CHECK(std::memcmp(to_host(d_out, count).data(), want[r].data(), count * sizeof(T)) == 0);
+    // the direct form: every peer's raw copy of the owned segment, folded in ring order in one pass
+    const int own = (r + 1) % n;
+    std::vector<const void*> raw;
+    for (int k = 0; k < n - 1; k++) {
+      const std::vector<T>& peer = in[(own + k) % n];
+      raw.push_back(to_device(std::vector<T>(peer.begin() + starts[own], peer.begin() + starts[own] + sizes[own]), k % 4));
+    }
+    HIP_OK(hipMemset(d_out, 0, count * sizeof(T)));
+    CHECK(mpic_ring_allreduce_direct_prestaged(n, r, Code<T>::mpic, d_in, d_out, count, raw.data(), ag_p.data(), stream,
+                                               r % 2) == MPIC_OK);
+    CHECK(ring_stream_synchronize(stream) == RING_OK);
+    CHECK(std::memcmp(to_host(d_out, count).data(), want[r].data(), count * sizeof(T)) == 0);
   }
 
   // (2) all ranks resident: the neighbour's buffer is the transport
