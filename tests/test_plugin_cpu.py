@@ -393,6 +393,15 @@ def test_without_a_gpu_every_device_call_fails_and_nothing_is_computed_on_the_ho
     counts = (ctypes.c_size_t * 1)(1024)
     plan = ctypes.c_void_p()
     assert L.ring_fusion_plan_create(ptrs, counts, 1, ring_abi.F32, ctypes.byref(plan)) == 3 and not plan.value
+    srcs = (ctypes.c_void_p * 2)(a.ctypes.data, b.ctypes.data)
+    fold = (ring_abi.FoldRow * 1)()
+    fold[0].dst, fold[0].srcs, fold[0].count = a.ctypes.data, ctypes.cast(srcs, ctypes.POINTER(ctypes.c_void_p)), 1024
+    assert L.ring_fold_rows(fold, 1, 2, 0, ring_abi.F32, None) == 3
+    assert L.ring_fold_rows(fold, 1, 2, 0, 7, None) == 1                                        # RING_ERR_DTYPE
+    assert L.ring_fold_rows(fold, 1, 0, 0, ring_abi.F32, None) == 2                             # no sources
+    assert L.ring_fold_rows(fold, 1, 257, 0, ring_abi.F32, None) == 2                           # too many sources
+    assert L.ring_fold_rows(fold, 0, 2, 0, ring_abi.F32, None) == 0                             # nothing to do
+    assert L.ring_event_record(None, None) == 2 and L.ring_event_synchronize(None) == 2
     assert (a == 1.0).all()                                # the host never stood in for the device
     with pytest.raises(ring_abi.RingError, match="HIP runtime call failed"):
         ring_abi.accumulate(ring_abi.F32, a.ctypes.data, b.ctypes.data, 1024, None)
