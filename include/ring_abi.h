@@ -267,6 +267,27 @@ int ring_fusion_unpack(const ring_fusion_plan* plan, const void* fused, void* st
 int ring_fusion_unpack_scaled(const ring_fusion_plan* plan, const void* fused, int divisor,
                               void* stream);
 
+/* Fusion without passes of its own. A span is `count` elements of the plan's
+ * fused element space starting at `begin` (a ring segment of the packed
+ * buffer). Gather: out[i] = tensor_element(begin + i) + incoming[i], or a plain
+ * pack of the span when incoming is NULL: the first accumulate of a segment
+ * takes its local operand straight from the tensors and leaves the sum in the
+ * wire buffer the next rank is sent from. Scatter: tensor_element(begin + i) =
+ * incoming[i], divided by divisor when divisor > 0: a finished segment goes
+ * straight to the tensors. Elements outside the spans are not touched. Spans
+ * must be sorted by `begin` and disjoint; `spans` is a HOST array. Together
+ * the two calls do what pack, n-1 accumulates, and unpack do, minus one read
+ * and one write of the whole set. */
+typedef struct ring_fusion_span {
+  uint64_t begin;       /* first element in the fused space */
+  uint64_t count;       /* elements */
+  const void* incoming; /* element 0 of the span's incoming data */
+  void* out;            /* gather: element 0 of the span's destination; scatter: unused */
+} ring_fusion_span;
+int ring_fusion_gather(const ring_fusion_plan* plan, const ring_fusion_span* spans, int n_spans, void* stream);
+int ring_fusion_scatter(const ring_fusion_plan* plan, const ring_fusion_span* spans, int n_spans, int divisor,
+                        void* stream);
+
 #ifdef __cplusplus
 }
 #endif

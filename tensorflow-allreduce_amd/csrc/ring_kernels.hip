@@ -492,6 +492,122 @@ fusion_kernel(T* __restrict__ fused, const uint64_t* __restrict__ offsets, T* co
   }
 }
 
+// ---- tensor fusion without passes of its own -------------------------------------
+// The pack before a fused allreduce and the unpack after it read and write the
+// whole set once each for nothing but a change of layout. Both fold into the
+// ring's own work: the first touch of a segment by the reduce-scatter can take
+// its local operand straight from the tensors (gather: out = tensor + incoming,
+// written to the wire buffer the next rank is sent from), and the allgather's
+// finished segments can go straight to the tensors (scatter: tensor = incoming,
+// optionally divided). A launch works on spans of the fused element space, one
+// per ring segment; a tile of the space meets at most a few spans and, as in
+// the pack / unpack kernel, either lies inside one tensor or finds its tensors
+// through an offset table staged in LDS.
+
+constexpr int kMaxFusionSpans = 64;
+struct FusionSpan {
+  uint64_t begin, end;  // elements of the fused space
+  const void* in;       // element `begin` of what arrives (gather: may be null, then a plain pack)
+  void* out;            // gather only: element `begin` of the linear destination
+};
+struct FusionSpanTable {
+  int n;
+  int divisor;  // scatter: > 0 divides
+  FusionSpan span[kMaxFusionSpans];
+};
+
+template <typename T, bool GATHER, int NT, bool DIV>
+__global__ void __launch_bounds__(kBlock)
+fusion_span_kernel(const uint64_t* __restrict__ offsets, T* const* __restrict__ ptrs,
+                   const uint32_t* __restrict__ tile_first, const uint32_t* __restrict__ tile_last, uint32_t tile_lo,
+                   uint32_t tile_hi, uint64_t total, const FusionSpanTable tab) {
+  typedef typename VecOf<T>::type V;
+  typedef V VU __attribute__((aligned(sizeof(T))));
+  constexpr uint32_t VEC = 16 / sizeof(T);
+  constexpr uint64_t kTileElems = static_cast<uint64_t>(kFusionTileVecs) * VEC;
+  constexpr int SOP = DIV ? kOpDiv : kOpCopy;  // scatter
+  __shared__ uint64_t s_off[kFusionLdsCap + 1];
+  __shared__ T* s_ptr[kFusionLdsCap];
+
+  for (uint32_t tile = tile_lo + blockIdx.x; tile < tile_hi; tile += gridDim.x) {
+    const uint64_t e0 = static_cast<uint64_t>(tile) * kTileElems;
+    const uint64_t e1 = (e0 + kTileElems < total) ? e0 + kTileElems : total;
+    const uint32_t t0 = tile_first[tile];
+    const uint32_t t1 = tile_last[tile];
+    const uint32_t tensors = t1 - t0 + 1;
+    const uint64_t* off_tab = offsets + t0;
+    T* const* ptr_tab = ptrs + t0;
+    const bool staged = tensors > 1 && tensors <= kFusionLdsCap;  // uniform per workgroup
+    if (staged) {
+      for (uint32_t i = threadIdx.x; i <= tensors; i += kBlock) s_off[i] = offsets[t0 + i];
+      for (uint32_t i = threadIdx.x; i < tensors; i += kBlock) s_ptr[i] = ptrs[t0 + i];
+      __syncthreads();
+      off_tab = s_off;
+      ptr_tab = s_ptr;
+    }
+    // first span that ends after e0 (spans are sorted and disjoint)
+    int lo = 0, hi = tab.n;
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (tab.span[mid].end <= e0) lo = mid + 1; else hi = mid;
+    }
+    for (int sp = lo; sp < tab.n && tab.span[sp].begin < e1; sp++) {
+      const FusionSpan span = tab.span[sp];
+      const uint64_t b0 = span.begin > e0 ? span.begin : e0;
+      const uint64_t b1 = span.end < e1 ? span.end : e1;
+      if (b0 >= b1) continue;
+      const T* lin_in = span.in ? static_cast<const T*>(span.in) + (b0 - span.begin) : nullptr;
+      T* lin_out = GATHER ? static_cast<T*>(span.out) + (b0 - span.begin) : nullptr;
+      // the tensor holding b0 (uniform scalar walk over the tile's few tensors)
+      uint32_t ta = 0;
+      while (off_tab[ta + 1] <= b0) ta++;
+      if (b1 <= off_tab[ta + 1]) {
+        // the piece lies inside one tensor: the aligned-store span code of the step tables
+        T* tensor = ptr_tab[ta] + (b0 - off_tab[ta]);
+        if (GATHER) {
+          if (lin_in) row_tile<T, kOpAdd, 4, NT>(lin_out, lin_in, tensor, b1 - b0, 0, 1, 0);
+          else row_tile<T, kOpCopy, 4, NT>(lin_out, tensor, nullptr, b1 - b0, 0, 1, 0);
+        } else {
+          row_tile<T, SOP, 4, NT>(tensor, lin_in, nullptr, b1 - b0, 0, 1, tab.divisor);
+        }
+        continue;
+      }
+      // several tensors: every lane finds the tensor of its 16-byte group
+      const uint32_t ngroups = static_cast<uint32_t>((b1 - b0 + VEC - 1) / VEC);
+      for (uint32_t g = threadIdx.x; g < ngroups; g += kBlock) {
+        uint64_t e = b0 + static_cast<uint64_t>(g) * VEC;
+        uint32_t l = ta, h = tensors;  // off_tab[l] <= e < off_tab[h]
+        while (h - l > 1) {
+          const uint32_t mid = (l + h) >> 1;
+          if (off_tab[mid] <= e) l = mid; else h = mid;
+        }
+        const uint64_t i = e - b0;
+        if (e + VEC <= off_tab[l + 1] && e + VEC <= b1) {
+          VU* tv = reinterpret_cast<VU*>(ptr_tab[l] + (e - off_tab[l]));
+          if (GATHER) {
+            V x = *tv;
+            if (lin_in) x = apply_vec<T, kOpAdd>(*reinterpret_cast<const VU*>(lin_in + i), x, 0);
+            *reinterpret_cast<VU*>(lin_out + i) = x;
+          } else {
+            const V x = *reinterpret_cast<const VU*>(lin_in + i);
+            *tv = apply_vec<T, SOP>(x, x, tab.divisor);
+          }
+        } else {
+          const uint64_t end = (e + VEC < b1) ? e + VEC : b1;
+          for (; e < end; e++) {
+            while (e >= off_tab[l + 1]) l++;
+            T* tp = ptr_tab[l] + (e - off_tab[l]);
+            const uint64_t k = e - b0;
+            if (GATHER) lin_out[k] = lin_in ? apply_one<T, kOpAdd>(lin_in[k], *tp, 0) : *tp;
+            else *tp = apply_one<T, SOP>(lin_in[k], T(), tab.divisor);
+          }
+        }
+      }
+    }
+    if (staged) __syncthreads();  // before the next tile overwrites the table
+  }
+}
+
 // ---- launch configuration -----------------------------------------------------
 
 constexpr uint64_t kCacheResidentBytes = 128ull << 20;
@@ -1221,6 +1337,93 @@ int ring_fusion_unpack(const ring_fusion_plan* plan, const void* fused, void* st
 int ring_fusion_unpack_scaled(const ring_fusion_plan* plan, const void* fused, int divisor, void* stream) {
   if (divisor < 1) return RING_ERR_ARGUMENT;
   return fusion_run(plan, const_cast<void*>(fused), stream, false, divisor);
+}
+
+}  // extern "C"
+
+namespace {
+
+template <typename T, bool GATHER, bool DIV>
+int launch_fusion_spans(const ring_fusion_plan* p, const FusionSpanTable& tab, uint32_t tile_lo, uint32_t tile_hi,
+                        hipStream_t stream) {
+  uint32_t grid = tile_hi - tile_lo;
+  int nt = g_tuning.nt[GATHER ? kRolePack : kRoleUnpack];
+  if (nt < 0) nt = GATHER ? 2 : 3;
+#define RING_SPANS(N)                                                                                        \
+  launch(fusion_span_kernel<T, GATHER, N, DIV>, dim3(grid), dim3(kBlock), stream,                            \
+         static_cast<const uint64_t*>(p->d_offsets), reinterpret_cast<T* const*>(p->d_ptrs),                 \
+         static_cast<const uint32_t*>(p->d_tile_first), static_cast<const uint32_t*>(p->d_tile_last),        \
+         tile_lo, tile_hi, p->total, tab)
+  switch (nt & 3) {
+    case 0: RING_SPANS(0); break;
+    case 1: RING_SPANS(1); break;
+    case 2: RING_SPANS(2); break;
+    default: RING_SPANS(3); break;
+  }
+#undef RING_SPANS
+  RING_HIP(hipGetLastError());
+  return RING_OK;
+}
+
+// Checks the spans (sorted, disjoint, inside the plan, operands present and
+// element-aligned) and launches them in tables of kMaxFusionSpans.
+int fusion_spans_run(const ring_fusion_plan* p, const ring_fusion_span* spans, int n, bool gather, int divisor,
+                     void* stream) {
+  if (!p || n < 0 || (n > 0 && !spans) || divisor < 0) return RING_ERR_ARGUMENT;
+  const uint64_t tile_elems = static_cast<uint64_t>(kFusionTileVecs) * (16 / p->esz);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  uint64_t previous_end = 0;
+  int i = 0;
+  while (i < n) {
+    FusionSpanTable tab;
+    tab.n = 0;
+    tab.divisor = divisor;
+    bool any_in = false;
+    while (i < n && tab.n < kMaxFusionSpans) {
+      const ring_fusion_span& sp = spans[i++];
+      if (sp.count == 0) continue;
+      const uint64_t end = sp.begin + sp.count;
+      if (sp.begin < previous_end || end < sp.begin || end > p->total) return RING_ERR_ARGUMENT;
+      if (gather ? !sp.out : !sp.incoming) return RING_ERR_ARGUMENT;
+      if ((reinterpret_cast<uintptr_t>(sp.incoming) | reinterpret_cast<uintptr_t>(sp.out)) & (p->esz - 1))
+        return RING_ERR_ARGUMENT;
+      previous_end = end;
+      any_in = any_in || sp.incoming != nullptr;
+      tab.span[tab.n++] = FusionSpan{sp.begin, end, sp.incoming, gather ? sp.out : nullptr};
+    }
+    if (tab.n == 0) continue;
+    const uint32_t tile_lo = static_cast<uint32_t>(tab.span[0].begin / tile_elems);
+    const uint32_t tile_hi = static_cast<uint32_t>((tab.span[tab.n - 1].end + tile_elems - 1) / tile_elems);
+    int rc;
+    if (gather) {
+      // adds wrap on the unsigned carriers; a table without arrivals is a plain pack
+      if (p->dtype == RING_F32 && any_in) rc = launch_fusion_spans<float, true, false>(p, tab, tile_lo, tile_hi, s);
+      else if (p->esz == 8) rc = launch_fusion_spans<uint64_t, true, false>(p, tab, tile_lo, tile_hi, s);
+      else rc = launch_fusion_spans<uint32_t, true, false>(p, tab, tile_lo, tile_hi, s);
+    } else if (divisor > 0) {
+      if (p->dtype == RING_F32) rc = launch_fusion_spans<float, false, true>(p, tab, tile_lo, tile_hi, s);
+      else if (p->dtype == RING_I32) rc = launch_fusion_spans<int32_t, false, true>(p, tab, tile_lo, tile_hi, s);
+      else rc = launch_fusion_spans<int64_t, false, true>(p, tab, tile_lo, tile_hi, s);
+    } else {
+      if (p->esz == 8) rc = launch_fusion_spans<uint64_t, false, false>(p, tab, tile_lo, tile_hi, s);
+      else rc = launch_fusion_spans<uint32_t, false, false>(p, tab, tile_lo, tile_hi, s);
+    }
+    if (rc != RING_OK) return rc;
+  }
+  return RING_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ring_fusion_gather(const ring_fusion_plan* plan, const ring_fusion_span* spans, int n_spans, void* stream) {
+  return fusion_spans_run(plan, spans, n_spans, true, 0, stream);
+}
+
+int ring_fusion_scatter(const ring_fusion_plan* plan, const ring_fusion_span* spans, int n_spans, int divisor,
+                        void* stream) {
+  return fusion_spans_run(plan, spans, n_spans, false, divisor, stream);
 }
 
 }  // extern "C"

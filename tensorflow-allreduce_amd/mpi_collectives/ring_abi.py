@@ -24,7 +24,8 @@ EXPORTS = (
     "ring_accumulate", "ring_reduce_scatter_steps", "ring_reduce_scatter_steps_from",
     "ring_allgather_steps", "ring_apply_rows", "ring_apply_rows_avg", "ring_fold_rows", "ring_fold_and_copy_rows",
     "ring_fusion_plan_create", "ring_fusion_plan_destroy", "ring_fusion_plan_elements",
-    "ring_fusion_pack", "ring_fusion_unpack", "ring_fusion_unpack_scaled", "ring_scale",
+    "ring_fusion_pack", "ring_fusion_unpack", "ring_fusion_unpack_scaled", "ring_fusion_gather",
+    "ring_fusion_scatter", "ring_scale",
 )
 
 
@@ -55,6 +56,21 @@ _lib = None
 class FoldRow(ctypes.Structure):
     """ring_fold_row: dst = srcs[m-1] + (... + (srcs[1] + srcs[0]))."""
     _fields_ = [("dst", ctypes.c_void_p), ("srcs", ctypes.POINTER(ctypes.c_void_p)), ("count", ctypes.c_uint64)]
+
+
+class FusionSpan(ctypes.Structure):
+    """ring_fusion_span: `count` elements of a plan's fused space from `begin`."""
+    _fields_ = [("begin", ctypes.c_uint64), ("count", ctypes.c_uint64), ("incoming", ctypes.c_void_p),
+                ("out", ctypes.c_void_p)]
+
+
+def make_spans(spans):
+    """spans: iterable of (begin, count, incoming_or_None, out_or_None) -> ctypes array, length."""
+    spans = list(spans)
+    arr = (FusionSpan * max(len(spans), 1))()
+    for i, (b, c, inc, out) in enumerate(spans):
+        arr[i].begin, arr[i].count, arr[i].incoming, arr[i].out = b, c, inc, out
+    return arr, len(spans)
 
 
 def lib():
@@ -106,6 +122,8 @@ def lib():
             "ring_fusion_pack": (ci, [vp, vp, vp]),
             "ring_fusion_unpack": (ci, [vp, vp, vp]),
             "ring_fusion_unpack_scaled": (ci, [vp, vp, ci, vp]),
+            "ring_fusion_gather": (ci, [vp, ctypes.POINTER(FusionSpan), ci, vp]),
+            "ring_fusion_scatter": (ci, [vp, ctypes.POINTER(FusionSpan), ci, ci, vp]),
             "ring_scale": (ci, [ci, vp, sz, ci, vp]),
         }
         for name in EXPORTS:
@@ -304,6 +322,14 @@ class FusionPlan:
 
     def unpack_scaled(self, fused, divisor, stream):
         check(lib().ring_fusion_unpack_scaled(self._h, fused, divisor, stream), "ring_fusion_unpack_scaled")
+
+    def gather(self, spans, stream):
+        """spans: (ctypes array, n) from make_spans: out = tensors (+ incoming) per span."""
+        check(lib().ring_fusion_gather(self._h, spans[0], spans[1], stream), "ring_fusion_gather")
+
+    def scatter(self, spans, divisor, stream):
+        """tensors = incoming (/ divisor) per span."""
+        check(lib().ring_fusion_scatter(self._h, spans[0], spans[1], divisor, stream), "ring_fusion_scatter")
 
     def close(self):
         if self._h:

@@ -402,6 +402,67 @@ def test_fusion_pack_unpack(dtype):
     _fusion_roundtrip([int(c) for c in rng.integers(1, 200, 700)], dtype, rng)
 
 
+@pytest.mark.parametrize("dtype", G.DTYPES)
+def test_fusion_gather_and_scatter_spans(dtype):
+    """Spans of the fused element space: gather = tensors (+ incoming) into a
+    linear buffer, scatter = incoming (/ divisor) into the tensors; spans that
+    start and end inside tensors, cover many tiny tensors, leave gaps; against
+    numpy on the concatenation."""
+    import torch
+    rng = np.random.default_rng(31)
+    code = G.NP2ABI[np.dtype(dtype)]
+    tdt = G.NP2TORCH[np.dtype(dtype)]
+    for counts in ([int(np.prod(s)) for s in G.resnet50_shapes()][:40], [5, 0, 4096, 1, 0, 3, 8191, 2, 70_001],
+                   [int(c) for c in rng.integers(0, 4, 3000)] + [10_000], [int(c) for c in rng.integers(1, 200, 700)]):
+        hosts = [G.random_array(rng, c, dtype) for c in counts]
+        devs = [G.dev(h, int(rng.integers(0, 4))) for h in hosts]
+        plan = ring_abi.FusionPlan([d[0].data_ptr() if c else None for d, c in zip(devs, counts)], counts, code)
+        total = sum(counts)
+        flat = np.concatenate(hosts)
+        # 5 spans with gaps, boundaries anywhere
+        cuts = sorted(int(c) for c in rng.integers(0, total + 1, 10))
+        spans = [(cuts[2 * k], cuts[2 * k + 1] - cuts[2 * k]) for k in range(5)]
+        incoming = [G.random_array(rng, c, dtype) for _, c in spans]
+        d_in = [G.dev(x, k % 4) for k, x in enumerate(incoming)]
+        d_out = [G.dev(np.zeros(c, dtype=dtype), (k + 1) % 4) for k, (_, c) in enumerate(spans)]
+        with_in = [k % 2 == 0 for k in range(5)]                     # every other span is a plain pack
+        ring_abi_spans = ring_abi.make_spans(
+            [(b, c, d_in[k][0].data_ptr() if (with_in[k] and c) else None, d_out[k][0].data_ptr() if c else None)
+             for k, (b, c) in enumerate(spans)])
+        plan.gather(ring_abi_spans, None)
+        G.sync()
+        for k, (b, c) in enumerate(spans):
+            with np.errstate(all="ignore"):
+                want = (flat[b:b + c] + incoming[k]).astype(dtype) if with_in[k] else flat[b:b + c]
+            G.assert_same_bits(G.host(d_out[k][0]), want, "gather span %d [%d,+%d)" % (k, b, c))
+        for d, h in zip(devs, hosts):                               # gather never writes the tensors
+            G.assert_same_bits(G.host(d[0]), h, "tensor after gather")
+        for divisor in (0, 6):
+            for d, h in zip(devs, hosts):
+                d[0].copy_(torch.from_numpy(h))
+            plan.scatter(ring_abi.make_spans([(b, c, d_in[k][0].data_ptr() if c else None, None)
+                                              for k, (b, c) in enumerate(spans)]), divisor, None)
+            G.sync()
+            want = flat.copy()
+            for k, (b, c) in enumerate(spans):
+                with np.errstate(all="ignore"):
+                    x = incoming[k]
+                    if divisor:
+                        x = (x / np.float32(divisor) if dtype == np.float32 else x // dtype(divisor)).astype(dtype)
+                want[b:b + c] = x
+            got = np.concatenate([G.host(d[0]) for d in devs]) if devs else np.empty(0, dtype=dtype)
+            G.assert_same_bits(got, want, "scatter /%d" % divisor)
+        # spans out of order, overlapping or beyond the plan are refused
+        if total > 10:
+            a = d_in[0][0].data_ptr()
+            for bad in ([(5, 3, a, a), (2, 2, a, a)], [(0, 6, a, a), (5, 3, a, a)], [(total - 1, 2, a, a)]):
+                with pytest.raises(ring_abi.RingError):
+                    plan.gather(ring_abi.make_spans(bad), None)
+            with pytest.raises(ring_abi.RingError):
+                plan.scatter(ring_abi.make_spans([(0, 4, None, None)]), 0, None)
+        plan.close()
+
+
 def test_fusion_errors():
     L = ring_abi.lib()
     h = ctypes.c_void_p()
