@@ -332,6 +332,60 @@ class FusedResnet50(Workload):
             self.launch_phase(k, i, stream)
 
 
+class FusedResnet50NoPasses(FusedResnet50):
+    """The same fused allreduce without pack and unpack passes: the
+    reduce-scatter's accumulates gather their local operand from the 161
+    tensors (the segment that is only sent is packed alongside), the finished
+    segments scatter straight into the tensors with the divide. Two launches."""
+
+    def __init__(self, nsets=4):
+        super().__init__(nsets)
+        from mpi_collectives import _plugin
+        self.L = _plugin.load_library('libmpi_collectives.so', ['MPIAllreduce', 'MPIAllgather'])
+        self.name = "fused_resnet50_n8_no_passes"
+        A = self.ring_abi
+        sizes, starts = A.segment_table(self.total, 8)
+        for s, st in enumerate(self.sets):
+            r = s % 8
+            rs_seg = [A.schedule(0, 8, r, i)[1] for i in range(7)]
+            ag_seg = [A.schedule(1, 8, r, i)[1] for i in range(7)]
+            rs_of = {g: t for g, t in zip(rs_seg, st["rs"])}
+            ag_of = {g: t for g, t in zip(ag_seg, st["ag"])}
+            own, wire = (r + 1) % 8, st["fused"].data_ptr()
+            st["r"] = r
+            st["rs_ptrs"] = (ctypes.c_void_p * 7)(*[t.data_ptr() for t in st["rs"]])
+            st["ag_ptrs"] = (ctypes.c_void_p * 7)(*[t.data_ptr() for t in st["ag"]])
+            st["gather"] = A.make_spans([(starts[g], sizes[g], rs_of[g].data_ptr() if g in rs_of else None,
+                                          wire + starts[g] * 4) for g in range(8)])
+            st["scatter"] = A.make_spans([(starts[g], sizes[g],
+                                           wire + starts[g] * 4 if g == own else ag_of[g].data_ptr(), None)
+                                          for g in range(8)])
+        seg = self.total // 8
+        self.phases = (
+            ("gather_accumulate", 7 * seg * 12 + seg * 8,
+             "fusion_span_kernel<float, gather> (7 segments tensors + received -> wire, 1 segment packed)"),
+            ("scatter_scaled", 8 * seg * 8, "fusion_span_kernel<float, scatter, divide> (8 finished segments -> 161 tensors, /8)"))
+        self.dominant = 0
+        self.description = ("tensor-fusion allreduce of a ResNet-50 v1 gradient set (161 float32 tensors, 25,557,032 "
+                            "elements, values ~N(0,1e-3)) at N=8 virtual ranks WITHOUT pack and unpack passes: the 7 "
+                            "accumulates read their local operand from the tensors and write the wire buffer, the 8 "
+                            "finished segments go straight into the tensors with the divide by 8; 2 launches per step")
+
+    def launch_phase(self, k, i, stream):
+        s = self.sets[k % self.nsets]
+        if i == 0:
+            s["plan"].gather(s["gather"], stream)
+        else:
+            s["plan"].scatter(s["scatter"], 8, stream)
+
+    def launch_step(self, k, stream, fused=False):
+        s = self.sets[k % self.nsets]
+        rc = self.L.mpic_ring_allreduce_fused_prestaged(s["plan"]._h, 8, s["r"], s["fused"].data_ptr(), s["rs_ptrs"],
+                                                        s["ag_ptrs"], stream, 8 << 8)
+        if rc != 0:
+            raise RuntimeError("mpic_ring_allreduce_fused_prestaged failed: %s" % self.L.mpic_last_error().decode())
+
+
 class AllgatherN16(Workload):
     """RingAllgather at N=16: rank i contributes [rows_i, 1024] float32,
     rows_i uniform in [1, 4096] from seed=i; one launch per step gathers the
@@ -403,6 +457,8 @@ def make_workload(name):
                              "launch per phase, peers pre-staged, 2 buffer sets (8 GiB) rotated")
     if name == "fused_resnet50_n8":
         return FusedResnet50()
+    if name == "fused_resnet50_n8_no_passes":
+        return FusedResnet50NoPasses()
     if name == "allgather_f32_n16":
         return AllgatherN16()
     raise SystemExit("unknown workload %r" % name)
@@ -410,7 +466,7 @@ def make_workload(name):
 
 WORKLOADS = ("allreduce_f32_64MiB_n8", "allreduce_i32_10000019_n6", "allreduce_i64_10000019_n6",
              "fused_resnet50_n8", "allgather_f32_n16", "allreduce_f32_1GiB_n64", "allreduce_f32_64MiB_n8_per_step",
-             "allreduce_f32_64MiB_n8_direct")
+             "allreduce_f32_64MiB_n8_direct", "fused_resnet50_n8_no_passes")
 
 
 def cpu_baseline(w):

@@ -161,6 +161,20 @@ int mpic_ring_allreduce_prestaged(int n, int r, int dtype, const void* input, vo
 int mpic_ring_allreduce_direct_prestaged(int n, int r, int dtype, const void* input, void* output,
                                          size_t count, const void* const* peer_segments,
                                          const void* const* ag_segments, void* stream, int flags);
+/* A fused (tensor-fusion) allreduce for rank r without pack and unpack passes.
+ * `plan` is a ring_fusion_plan (ring_abi.h) over the rank's tensors; the packed
+ * buffer exists only as `wire` (plan-elements long, device memory), where the
+ * sums a ring sends on are left. rs_segments / ag_segments as for
+ * mpic_ring_allreduce_prestaged, on the packed layout. Two launches: the
+ * reduce-scatter's accumulates read their local operand straight from the
+ * tensors (the segment that is only sent is packed alongside), and every
+ * finished segment goes straight into the tensors, divided when bits 8-30 of
+ * `flags` hold a divisor. Each tensor ends up exactly as pack, ring, unpack
+ * (and tf.div) would leave it. No counterpart in the reference. */
+struct ring_fusion_plan;
+int mpic_ring_allreduce_fused_prestaged(const struct ring_fusion_plan* plan, int n, int r, void* wire,
+                                        const void* const* rs_segments, const void* const* ag_segments,
+                                        void* stream, int flags);
 /* RingAllgather (ring.h:236-301) for rank r: rows[k] = rank k's first
  * dimension, segments[i] = what arrives at step i. */
 int mpic_ring_allgather_prestaged(int n, int r, int dtype, const void* input, const size_t* rows,

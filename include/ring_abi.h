@@ -255,6 +255,8 @@ typedef struct ring_fusion_plan ring_fusion_plan;
 int ring_fusion_plan_create(const void* const* tensors, const size_t* counts,
                             int k, int dtype, ring_fusion_plan** plan);
 int ring_fusion_plan_destroy(ring_fusion_plan* plan);
+/* The plan's ring_dtype (-1 for a null plan). */
+int ring_fusion_plan_dtype(const ring_fusion_plan* plan);
 /* Total elements of the fused buffer (sum of counts). */
 size_t ring_fusion_plan_elements(const ring_fusion_plan* plan);
 /* fused[offset_j + i] = tensors[j][i] for all j. `fused` must be 16-byte

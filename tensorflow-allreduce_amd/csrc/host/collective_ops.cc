@@ -1061,6 +1061,14 @@ int mpic_ring_allreduce_direct_prestaged(int n, int r, int dtype, const void* in
   return s.ok() ? MPIC_OK : mpic::Fail(s);
 }
 
+int mpic_ring_allreduce_fused_prestaged(const struct ring_fusion_plan* plan, int n, int r, void* wire,
+                                        const void* const* rs_segments, const void* const* ag_segments, void* stream,
+                                        int flags) {
+  mpic::Status s = mpic::RingAllreduceFusedPrestaged(plan, n, r, wire, rs_segments, ag_segments, stream,
+                                                     mpic::RingOptions::FromFlags(flags));
+  return s.ok() ? MPIC_OK : mpic::Fail(s);
+}
+
 int mpic_ring_allgather_prestaged(int n, int r, int dtype, const void* input, const size_t* rows,
                                   size_t elems_per_row, void* output, const void* const* segments, void* stream,
                                   int flags) {

@@ -180,6 +180,44 @@ Status RingAllreduceDirectPrestaged(int n, int r, DataType dt, const void* input
   return Status::OK();
 }
 
+Status RingAllreduceFusedPrestaged(const ring_fusion_plan* plan, int n, int r, void* wire,
+                                   const void* const* rs_recv, const void* const* ag_recv, void* stream,
+                                   const RingOptions& opts) {
+  if (!plan) return errors::InvalidArgument("no fusion plan");
+  const int code = ring_fusion_plan_dtype(plan);
+  if (n < 1 || r < 0 || r >= n) return errors::InvalidArgument("rank out of range for the ring");
+  if (opts.divisor < 0) return errors::InvalidArgument("negative divisor");
+  const size_t count = ring_fusion_plan_elements(plan);
+  if (count == 0) return Status::OK();
+  if (!wire) return errors::InvalidArgument("no wire buffer");
+  if (n > 1 && (!rs_recv || !ag_recv)) return errors::InvalidArgument("no staged peer segments");
+  const size_t esz = ring_dtype_size(code);
+  std::vector<size_t> sizes(static_cast<size_t>(n)), starts(static_cast<size_t>(n));
+  RING_RETURN_IF_ERROR(ring_segment_table(count, n, sizes.data(), starts.data()), "ring_segment_table");
+
+  // what arrives for each segment in either phase (ring.h:183-205, :211-225)
+  std::vector<const void*> rs_of(static_cast<size_t>(n), nullptr), ag_of(static_cast<size_t>(n), nullptr);
+  for (int i = 0; i < n - 1; i++) {
+    rs_of[static_cast<size_t>(Seg(RING_PHASE_REDUCE_SCATTER, n, r, i, true))] = rs_recv[i];
+    ag_of[static_cast<size_t>(Seg(RING_PHASE_ALLGATHER, n, r, i, true))] = ag_recv[i];
+  }
+  const size_t own = static_cast<size_t>((r + 1) % n);
+  std::vector<ring_fusion_span> gather, scatter;
+  for (size_t seg = 0; seg < static_cast<size_t>(n); seg++) {
+    // segment r has no arrival in the reduce-scatter: packed, as the first send needs it
+    gather.push_back(ring_fusion_span{starts[seg], sizes[seg], rs_of[seg], at(wire, starts[seg], esz)});
+    const void* finished = (seg == own || n == 1) ? at(static_cast<const void*>(wire), starts[seg], esz) : ag_of[seg];
+    if (sizes[seg] && !finished) return errors::InvalidArgument("null staged peer segment");
+    scatter.push_back(ring_fusion_span{starts[seg], sizes[seg], finished, nullptr});
+  }
+  for (size_t seg = 0; seg < static_cast<size_t>(n); seg++)
+    if (sizes[seg] && n > 1 && seg != static_cast<size_t>(r) && !rs_of[seg])
+      return errors::InvalidArgument("null staged peer segment");
+  RING_RETURN_IF_ERROR(ring_fusion_gather(plan, gather.data(), n, stream), "ring_fusion_gather");
+  RING_RETURN_IF_ERROR(ring_fusion_scatter(plan, scatter.data(), n, opts.divisor, stream), "ring_fusion_scatter");
+  return Status::OK();
+}
+
 Status RingAllgatherPrestaged(int n, int r, DataType dt, const void* input, const std::vector<size_t>& rows,
                               size_t elems_per_row, void* output, const void* const* recv, void* stream,
                               const RingOptions& opts) {

@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "framework.h"
+#include "ring_abi.h"
 
 namespace mpic {
 
@@ -69,6 +70,19 @@ Status RingAllreducePrestaged(int n, int r, DataType dt, const void* input, void
 Status RingAllreduceDirectPrestaged(int n, int r, DataType dt, const void* input, void* output, size_t count,
                                     const void* const* peers, const void* const* ag_recv, void* stream,
                                     const RingOptions& opts);
+
+// A fused allreduce for rank r of n without pack and unpack passes. `plan`
+// (ring_fusion_plan_create) lists the rank's tensors; the packed buffer exists
+// only as `wire`, plan-elements long, where the sums a ring sends on are left.
+// Reduce-scatter: wire[seg] = tensors[seg] + rs_recv[i] for the n-1 received
+// segments, and segment r, which is only sent, is packed (one launch, the local
+// operand read straight from the tensors). Allgather: every finished segment,
+// ag_recv[i] or the rank's own in `wire`, goes straight into the tensors,
+// divided when opts.divisor > 0 (one launch). Each tensor ends up as the
+// reference ring applied to the packed buffer would leave it.
+Status RingAllreduceFusedPrestaged(const ring_fusion_plan* plan, int n, int r, void* wire,
+                                   const void* const* rs_recv, const void* const* ag_recv, void* stream,
+                                   const RingOptions& opts);
 
 // ring.h:236-301 for rank r of n. recv[i]: the segment received at step i
 // (segment (r-i-1) mod n).

@@ -1316,6 +1316,8 @@ int ring_fusion_plan_create(const void* const* tensors, const size_t* counts, in
   return RING_OK;
 }
 
+int ring_fusion_plan_dtype(const ring_fusion_plan* plan) { return plan ? plan->dtype : -1; }
+
 int ring_fusion_plan_destroy(ring_fusion_plan* plan) {
   if (!plan) return RING_OK;
   hipError_t e = plan->d_table ? hipFree(plan->d_table) : hipSuccess;
@@ -1345,10 +1347,10 @@ namespace {
 
 template <typename T, bool GATHER, bool DIV>
 int launch_fusion_spans(const ring_fusion_plan* p, const FusionSpanTable& tab, uint32_t tile_lo, uint32_t tile_hi,
-                        hipStream_t stream) {
+                        hipStream_t stream, Role role) {
   uint32_t grid = tile_hi - tile_lo;
-  int nt = g_tuning.nt[GATHER ? kRolePack : kRoleUnpack];
-  if (nt < 0) nt = GATHER ? 2 : 3;
+  int nt = g_tuning.nt[role];
+  if (nt < 0) nt = 3;
 #define RING_SPANS(N)                                                                                        \
   launch(fusion_span_kernel<T, GATHER, N, DIV>, dim3(grid), dim3(kBlock), stream,                            \
          static_cast<const uint64_t*>(p->d_offsets), reinterpret_cast<T* const*>(p->d_ptrs),                 \
@@ -1396,17 +1398,20 @@ int fusion_spans_run(const ring_fusion_plan* p, const ring_fusion_span* spans, i
     const uint32_t tile_hi = static_cast<uint32_t>((tab.span[tab.n - 1].end + tile_elems - 1) / tile_elems);
     int rc;
     if (gather) {
-      // adds wrap on the unsigned carriers; a table without arrivals is a plain pack
-      if (p->dtype == RING_F32 && any_in) rc = launch_fusion_spans<float, true, false>(p, tab, tile_lo, tile_hi, s);
-      else if (p->esz == 8) rc = launch_fusion_spans<uint64_t, true, false>(p, tab, tile_lo, tile_hi, s);
-      else rc = launch_fusion_spans<uint32_t, true, false>(p, tab, tile_lo, tile_hi, s);
+      // Adds wrap on the unsigned carriers. A table with arrivals is an accumulate
+      // (every byte touched once); one without is a plain pack, whose output the
+      // next kernel reads.
+      const Role role = any_in ? kRoleAccumulate : kRolePack;
+      if (p->dtype == RING_F32 && any_in) rc = launch_fusion_spans<float, true, false>(p, tab, tile_lo, tile_hi, s, role);
+      else if (p->esz == 8) rc = launch_fusion_spans<uint64_t, true, false>(p, tab, tile_lo, tile_hi, s, role);
+      else rc = launch_fusion_spans<uint32_t, true, false>(p, tab, tile_lo, tile_hi, s, role);
     } else if (divisor > 0) {
-      if (p->dtype == RING_F32) rc = launch_fusion_spans<float, false, true>(p, tab, tile_lo, tile_hi, s);
-      else if (p->dtype == RING_I32) rc = launch_fusion_spans<int32_t, false, true>(p, tab, tile_lo, tile_hi, s);
-      else rc = launch_fusion_spans<int64_t, false, true>(p, tab, tile_lo, tile_hi, s);
+      if (p->dtype == RING_F32) rc = launch_fusion_spans<float, false, true>(p, tab, tile_lo, tile_hi, s, kRoleUnpack);
+      else if (p->dtype == RING_I32) rc = launch_fusion_spans<int32_t, false, true>(p, tab, tile_lo, tile_hi, s, kRoleUnpack);
+      else rc = launch_fusion_spans<int64_t, false, true>(p, tab, tile_lo, tile_hi, s, kRoleUnpack);
     } else {
-      if (p->esz == 8) rc = launch_fusion_spans<uint64_t, false, false>(p, tab, tile_lo, tile_hi, s);
-      else rc = launch_fusion_spans<uint32_t, false, false>(p, tab, tile_lo, tile_hi, s);
+      if (p->esz == 8) rc = launch_fusion_spans<uint64_t, false, false>(p, tab, tile_lo, tile_hi, s, kRoleUnpack);
+      else rc = launch_fusion_spans<uint32_t, false, false>(p, tab, tile_lo, tile_hi, s, kRoleUnpack);
     }
     if (rc != RING_OK) return rc;
   }

@@ -30,7 +30,8 @@ EXPORTS = (
     "mpic_world_flush", "mpic_stage_peers",
     "mpic_context_create", "mpic_context_add_input", "mpic_context_set_divisor", "mpic_context_compute", "mpic_context_wait",
     "mpic_context_message", "mpic_context_num_outputs", "mpic_context_output", "mpic_context_destroy",
-    "mpic_ring_allreduce_prestaged", "mpic_ring_allreduce_direct_prestaged", "mpic_ring_allgather_prestaged", "mpic_ring_allreduce_all_ranks",
+    "mpic_ring_allreduce_prestaged", "mpic_ring_allreduce_direct_prestaged", "mpic_ring_allreduce_fused_prestaged",
+    "mpic_ring_allgather_prestaged", "mpic_ring_allreduce_all_ranks",
     "mpic_ring_allgather_all_ranks", "mpic_ring_allreduce_transport", "mpic_ring_allgather_transport",
     "mpic_loopback_create", "mpic_loopback_destroy", "mpic_loopback_endpoint", "mpic_last_error",
 )
@@ -137,6 +138,7 @@ def load_library(name="libmpi_collectives.so", op_list=None):
             "mpic_context_destroy": (ci, [vp]),
             "mpic_ring_allreduce_prestaged": (ci, [ci, ci, ci, vp, vp, sz, pvp, pvp, vp, ci]),
             "mpic_ring_allreduce_direct_prestaged": (ci, [ci, ci, ci, vp, vp, sz, pvp, pvp, vp, ci]),
+            "mpic_ring_allreduce_fused_prestaged": (ci, [vp, ci, ci, vp, pvp, pvp, vp, ci]),
             "mpic_ring_allgather_prestaged": (ci, [ci, ci, ci, vp, psz, sz, vp, pvp, vp, ci]),
             "mpic_ring_allreduce_all_ranks": (ci, [ci, ci, pvp, pvp, sz, vp, ci]),
             "mpic_ring_allgather_all_ranks": (ci, [ci, ci, pvp, psz, sz, pvp, vp, ci]),

@@ -23,7 +23,7 @@ EXPORTS = (
     "ring_copy_bytes", "ring_accumulate_f32", "ring_accumulate_i32", "ring_accumulate_i64",
     "ring_accumulate", "ring_reduce_scatter_steps", "ring_reduce_scatter_steps_from",
     "ring_allgather_steps", "ring_apply_rows", "ring_apply_rows_avg", "ring_fold_rows", "ring_fold_and_copy_rows",
-    "ring_fusion_plan_create", "ring_fusion_plan_destroy", "ring_fusion_plan_elements",
+    "ring_fusion_plan_create", "ring_fusion_plan_destroy", "ring_fusion_plan_elements", "ring_fusion_plan_dtype",
     "ring_fusion_pack", "ring_fusion_unpack", "ring_fusion_unpack_scaled", "ring_fusion_gather",
     "ring_fusion_scatter", "ring_scale",
 )
@@ -119,6 +119,7 @@ def lib():
             "ring_fusion_plan_create": (ci, [ctypes.POINTER(vp), psz, ci, ci, ctypes.POINTER(vp)]),
             "ring_fusion_plan_destroy": (ci, [vp]),
             "ring_fusion_plan_elements": (sz, [vp]),
+            "ring_fusion_plan_dtype": (ci, [vp]),
             "ring_fusion_pack": (ci, [vp, vp, vp]),
             "ring_fusion_unpack": (ci, [vp, vp, vp]),
             "ring_fusion_unpack_scaled": (ci, [vp, vp, ci, vp]),

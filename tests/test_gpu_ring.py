@@ -470,6 +470,54 @@ def test_fused_resnet50_allreduce_matches_ring_on_the_packed_buffer(oracle):
             at += c
 
 
+@pytest.mark.parametrize("dtype", G.DTYPES)
+def test_fused_allreduce_without_pack_and_unpack_passes(oracle, dtype):
+    """mpic_ring_allreduce_fused_prestaged: the accumulates gather their local
+    operand from the tensors, the finished segments scatter into them. Every
+    tensor equals the oracle's ring on the packed buffer (then tf.div), and the
+    wire buffer holds what the ring would send on."""
+    L = _plugin.load_library()
+    rng = np.random.default_rng(8)
+    cases = [(8, [int(np.prod(s)) for s in G.resnet50_shapes()][:60], 8), (3, [5, 0, 4096, 1, 3, 8191, 2, 70_001], 0),
+             (6, [int(c) for c in rng.integers(0, 50, 400)], 6), (1, [10, 20], 4), (4, [2], 0)]
+    for n, counts, divisor in cases:
+        total = sum(counts)
+        grads = [[G.random_array(np.random.default_rng(100 * r + j), c, dtype) for j, c in enumerate(counts)]
+                 for r in range(n)]
+        packed = [np.concatenate(g) for g in grads]
+        outs, rs, ag = oracle.ring_allreduce(packed, tap=True)
+        want = _tf_div(outs[0], divisor) if divisor else outs[0]
+        sizes, starts = ring_abi.segment_table(total, n)
+        for r in sorted({0, n // 2, n - 1}):
+            dts = [G.dev(t, (j + r) % 4) for j, t in enumerate(grads[r])]
+            plan = ring_abi.FusionPlan([d[0].data_ptr() if c else None for d, c in zip(dts, counts)], counts,
+                                       G.NP2ABI[np.dtype(dtype)])
+            wire = torch.zeros(total + 4, dtype=G.NP2TORCH[np.dtype(dtype)], device="cuda")[1:total + 1]   # element-aligned only
+            rs_seg = [ring_abi.schedule(ring_abi.PHASE_REDUCE_SCATTER, n, r, i)[1] for i in range(n - 1)]
+            ag_seg = [ring_abi.schedule(ring_abi.PHASE_ALLGATHER, n, r, i)[1] for i in range(n - 1)]
+            rs_t = [cuda(rs[r][i][:sizes[g]]) for i, g in enumerate(rs_seg)]
+            ag_t = [cuda(ag[r][i][:sizes[g]]) for i, g in enumerate(ag_seg)]
+            rs_p = (ctypes.c_void_p * max(n - 1, 1))(*[t.data_ptr() if t.numel() else None for t in rs_t])
+            ag_p = (ctypes.c_void_p * max(n - 1, 1))(*[t.data_ptr() if t.numel() else None for t in ag_t])
+            rc = L.mpic_ring_allreduce_fused_prestaged(plan._h, n, r, wire.data_ptr(), rs_p, ag_p,
+                                                       torch.cuda.current_stream().cuda_stream, divisor << 8)
+            assert rc == 0, L.mpic_last_error()
+            torch.cuda.synchronize()
+            at = 0
+            for j, c in enumerate(counts):
+                G.assert_same_bits(G.host(dts[j][0]), want[at:at + c], "n=%d rank %d tensor %d /%d" % (n, r, j, divisor))
+                at += c
+            got_wire = G.host(wire)
+            for i, g in enumerate(rs_seg):                      # partial sums, as sent on at the next step
+                a, b = starts[g], starts[g] + sizes[g]
+                with np.errstate(all="ignore"):
+                    G.assert_same_bits(got_wire[a:b], (packed[r][a:b] + rs[r][i][:sizes[g]]).astype(dtype),
+                                       "wire segment %d" % g)
+            a, b = starts[r], starts[r] + sizes[r]
+            G.assert_same_bits(got_wire[a:b], packed[r][a:b], "wire segment r (packed only)")
+            plan.close()
+
+
 def test_distributed_optimizer_fused_and_unfused(oracle):
     """DistributedOptimizer.compute_gradients averages every gradient across
     ranks (__init__.py:195-205); with fusion=True through one fused buffer."""
