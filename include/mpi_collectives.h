@@ -170,7 +170,11 @@ int mpic_ring_allreduce_direct_prestaged(int n, int r, int dtype, const void* in
  * tensors (the segment that is only sent is packed alongside), and every
  * finished segment goes straight into the tensors, divided when bits 8-30 of
  * `flags` hold a divisor. Each tensor ends up exactly as pack, ring, unpack
- * (and tf.div) would leave it. No counterpart in the reference. */
+ * (and tf.div) would leave it. With bit 2 of `flags` (the direct form)
+ * rs_segments[k] is rank (r+1+k) mod n's raw copy of the segment this rank
+ * owns, in the packed layout: the rank packs its own copy of that segment into
+ * `wire`, folds the n copies there in ring order and scatters the finished
+ * segments (3 launches). No counterpart in the reference. */
 struct ring_fusion_plan;
 int mpic_ring_allreduce_fused_prestaged(const struct ring_fusion_plan* plan, int n, int r, void* wire,
                                         const void* const* rs_segments, const void* const* ag_segments,

@@ -195,13 +195,42 @@ Status RingAllreduceFusedPrestaged(const ring_fusion_plan* plan, int n, int r, v
   std::vector<size_t> sizes(static_cast<size_t>(n)), starts(static_cast<size_t>(n));
   RING_RETURN_IF_ERROR(ring_segment_table(count, n, sizes.data(), starts.data()), "ring_segment_table");
 
+  const size_t own = static_cast<size_t>((r + 1) % n);
+  if (opts.direct && n > 1) {
+    // Direct form: rs_recv[k] is rank (own+k)'s raw copy of the owned segment
+    // (packed layout). The rank packs its own copy of that segment into the
+    // wire buffer, folds the n copies there in ring order, and scatters the
+    // finished segments into the tensors.
+    std::vector<const void*> ag_direct(static_cast<size_t>(n), nullptr);
+    for (int i = 0; i < n - 1; i++)
+      ag_direct[static_cast<size_t>(Seg(RING_PHASE_ALLGATHER, n, r, i, true))] = ag_recv[i];
+    char* mine = at(wire, starts[own], esz);
+    ring_fusion_span pack{starts[own], sizes[own], nullptr, mine};
+    RING_RETURN_IF_ERROR(ring_fusion_gather(plan, &pack, 1, stream), "ring_fusion_gather");
+    std::vector<const void*> srcs;
+    for (int k = 0; k < n - 1; k++) {
+      if (sizes[own] && !rs_recv[k]) return errors::InvalidArgument("null staged peer segment");
+      srcs.push_back(rs_recv[k]);
+    }
+    srcs.push_back(mine);
+    ring_fold_row fold{mine, srcs.data(), sizes[own]};
+    RING_RETURN_IF_ERROR(ring_fold_rows(&fold, 1, n, 0, code, stream), "ring_fold_rows");
+    std::vector<ring_fusion_span> finished;
+    for (size_t seg = 0; seg < static_cast<size_t>(n); seg++) {
+      const void* from = seg == own ? static_cast<const void*>(mine) : ag_direct[seg];
+      if (sizes[seg] && !from) return errors::InvalidArgument("null staged peer segment");
+      finished.push_back(ring_fusion_span{starts[seg], sizes[seg], from, nullptr});
+    }
+    RING_RETURN_IF_ERROR(ring_fusion_scatter(plan, finished.data(), n, opts.divisor, stream), "ring_fusion_scatter");
+    return Status::OK();
+  }
+
   // what arrives for each segment in either phase (ring.h:183-205, :211-225)
   std::vector<const void*> rs_of(static_cast<size_t>(n), nullptr), ag_of(static_cast<size_t>(n), nullptr);
   for (int i = 0; i < n - 1; i++) {
     rs_of[static_cast<size_t>(Seg(RING_PHASE_REDUCE_SCATTER, n, r, i, true))] = rs_recv[i];
     ag_of[static_cast<size_t>(Seg(RING_PHASE_ALLGATHER, n, r, i, true))] = ag_recv[i];
   }
-  const size_t own = static_cast<size_t>((r + 1) % n);
   std::vector<ring_fusion_span> gather, scatter;
   for (size_t seg = 0; seg < static_cast<size_t>(n); seg++) {
     // segment r has no arrival in the reduce-scatter: packed, as the first send needs it

@@ -515,6 +515,24 @@ def test_fused_allreduce_without_pack_and_unpack_passes(oracle, dtype):
                                        "wire segment %d" % g)
             a, b = starts[r], starts[r] + sizes[r]
             G.assert_same_bits(got_wire[a:b], packed[r][a:b], "wire segment r (packed only)")
+            # the direct form: raw copies of the owned segment from every peer, folded in ring order
+            if n > 1:
+                for t, g in zip(dts, grads[r]):
+                    t[0].copy_(torch.from_numpy(g))
+                own = (r + 1) % n
+                raw_t = [cuda(packed[(own + k) % n][starts[own]:starts[own] + sizes[own]]) for k in range(n - 1)]
+                fin_t = [cuda(outs[0][starts[g]:starts[g] + sizes[g]]) for g in ag_seg]
+                raw_p = (ctypes.c_void_p * (n - 1))(*[t.data_ptr() if t.numel() else None for t in raw_t])
+                fin_p = (ctypes.c_void_p * (n - 1))(*[t.data_ptr() if t.numel() else None for t in fin_t])
+                rc = L.mpic_ring_allreduce_fused_prestaged(plan._h, n, r, wire.data_ptr(), raw_p, fin_p,
+                                                           torch.cuda.current_stream().cuda_stream, 4 | (divisor << 8))
+                assert rc == 0, L.mpic_last_error()
+                torch.cuda.synchronize()
+                at = 0
+                for j, c in enumerate(counts):
+                    G.assert_same_bits(G.host(dts[j][0]), want[at:at + c],
+                                       "direct fused n=%d rank %d tensor %d /%d" % (n, r, j, divisor))
+                    at += c
             plan.close()
 
 
