@@ -408,3 +408,17 @@ def test_without_a_gpu_every_device_call_fails_and_nothing_is_computed_on_the_ho
     # a GPU session cannot even initialise: its dedicated stream cannot be created
     with pytest.raises(mpi.UnknownError, match="Could not create the MPI stream"):
         mpi.Session(size=2, device="GPU")
+
+
+def test_bench_refuses_more_than_one_gpu_and_needs_a_gpu():
+    """bench.py's contract on this tier: one GPU only, said in a message; and no
+    number without the device (the benchmark never falls back to the host)."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    two = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert two.returncode != 0 and "ONE GPU" in two.stderr and not two.stdout.strip()
+    if not torch.cuda.is_available():
+        one = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--no-cpu-baseline"], capture_output=True,
+                             text=True)
+        assert one.returncode != 0 and "no GPU is visible" in one.stderr and not one.stdout.strip()
