@@ -736,6 +736,30 @@ def main():
                 "note": "same allreduce with the in->out copy folded into the accumulate (out = in + received; the "
                         "segment that is only sent is written by the first allgather step and never copied)",
             }
+        if args.variant == "all" and w.name == WORKLOADS[0]:
+            # the same allreduce in the direct form (one fold pass over pushed copies + copies, one launch)
+            d = make_workload("allreduce_f32_64MiB_n8_direct")
+            for k in range(50):
+                d.launch_step(k, stream)
+            ring_abi.stream_synchronize(stream)
+            t0 = time.perf_counter()
+            for k in range(steps):
+                d.launch_step(k, stream)
+            ring_abi.stream_synchronize(stream)
+            direct_elapsed = time.perf_counter() - t0
+            if not d.check(steps - 1):
+                sys.exit("bench.py: the output of the direct form is wrong; refusing to report a number")
+            result["direct_form"] = {
+                "ms_per_step": round(direct_elapsed / steps * 1e3, 5),
+                "bytes_per_step": d.bytes_per_step,
+                "GBps": round(d.bytes_per_step * steps / direct_elapsed / 1e9, 1),
+                "launches_per_step": 1,
+                "note": "same tensor and ranks, peers push raw copies of the owned segment instead of passing partial "
+                        "sums round: the owner folds the 8 copies in ring order in one pass and copies the 7 finished "
+                        "segments in, one launch; output bit-identical to the ring's (--workload "
+                        "allreduce_f32_64MiB_n8_direct)",
+            }
+            del d
         if not args.no_cpu_baseline:
             try:
                 result["cpu_baseline"] = cpu_baseline(w)
