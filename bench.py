@@ -621,7 +621,8 @@ def main():
     nph = len(w.phases)
     # events are created before the timed region: creating them inside it would
     # let the queue drain and the sampled launches start on an idle GPU
-    event_pool = [[ring_abi.event_create() for _ in range(2 * nph)] for _ in range(steps // SAMPLE_EVERY + 1)]
+    sample_every = max(1, min(SAMPLE_EVERY, steps))      # a short run still times at least one step's launches
+    event_pool = [[ring_abi.event_create() for _ in range(2 * nph)] for _ in range(steps // sample_every + 1)]
 
     def timed(nsteps, nwarm, fused=False, with_samples=False, hot=False):
         # hot: the same buffer set every step (what fits stays in the last-level
@@ -638,7 +639,7 @@ def main():
         samples = []
         t0 = time.perf_counter()
         for k in range(nsteps):
-            if with_samples and k % SAMPLE_EVERY == SAMPLE_EVERY // 2:
+            if with_samples and k % sample_every == sample_every // 2:
                 # the same launches, one ABI call each, every one carrying its own
                 # pair of HIP events in the dispatch (on the stream the kernels run on)
                 e = event_pool.pop()
@@ -711,7 +712,7 @@ def main():
                           "bytes": p[1]}
                    for i, (p, t) in enumerate(zip(w.phases, phase_us))},
         "phases_note": "HIP events carried by each launch of every %dth step of the timed region; us = mean"
-                       % SAMPLE_EVERY,
+                       % sample_every,
     }
     # the same steps on ONE buffer set: at the headline size the working set fits the
     # last-level cache, so this is the cache-resident rate, not the HBM one
