@@ -132,8 +132,10 @@ Status RingAllreducePrestaged(int n, int r, DataType dt, const void* input, void
   } else {
     for (int i = 0; i < n - 1; i++) {
       const size_t seg = static_cast<size_t>(Seg(RING_PHASE_ALLGATHER, n, r, i, true));
-      RING_RETURN_IF_ERROR(ring_copy_bytes(at(output, starts[seg], esz), ag_recv[i], sizes[seg] * esz, stream),
-                           "ring_copy_bytes");
+      // a one-row step table rather than ring_copy_bytes: a received segment is
+      // touched once, while the in->out copy's output is read again at once
+      const ring_step step{starts[seg], ag_recv[i], sizes[seg]};
+      RING_RETURN_IF_ERROR(ring_allgather_steps(output, &step, 1, code, stream), "ring_allgather_steps");
     }
   }
   return Status::OK();
@@ -291,14 +293,14 @@ Status RingAllgatherPrestaged(int n, int r, DataType dt, const void* input, cons
     if (opts.divisor > 0) {
       ring_row row{own ? at(output, starts[static_cast<size_t>(r)], esz) : nullptr, input, nullptr, own};
       RING_RETURN_IF_ERROR(ring_apply_rows_avg(&row, 1, nullptr, opts.divisor, code, stream), "ring_apply_rows_avg");
-    } else
-    RING_RETURN_IF_ERROR(ring_copy_bytes(at(output, starts[static_cast<size_t>(r)], esz), input, own * esz, stream),
-                         "ring_copy_bytes");
+    } else {
+      const ring_step mine{starts[static_cast<size_t>(r)], input, own};
+      RING_RETURN_IF_ERROR(ring_allgather_steps(output, &mine, 1, code, stream), "ring_allgather_steps");
+    }
     for (int i = 0; i < n - 1; i++) {
       const size_t seg = static_cast<size_t>(Seg(RING_PHASE_GATHER, n, r, i, true));
-      RING_RETURN_IF_ERROR(
-          ring_copy_bytes(at(output, starts[seg], esz), recv[i], elems_per_row * rows[seg] * esz, stream),
-          "ring_copy_bytes");
+      const ring_step step{starts[seg], recv[i], elems_per_row * rows[seg]};
+      RING_RETURN_IF_ERROR(ring_allgather_steps(output, &step, 1, code, stream), "ring_allgather_steps");
     }
   }
   return Status::OK();
