@@ -290,6 +290,38 @@ def test_fold_rows_is_the_sequential_fold(dtype):
         ring_abi.fold_rows([(x.data_ptr(), [x.data_ptr()], 8)], 1, -1, code, None)
 
 
+def test_fold_and_average_on_special_float_values():
+    """Denormals, signed zeros, infinities, NaN, the largest finite value: the
+    fold, the add-and-divide row and the divided scatter give numpy's bits
+    (denormal results of the division included; NaNs only have to be NaNs)."""
+    sp = special_f32()
+    pairs = np.array([(a, b) for a in sp for b in sp], dtype=np.float32)          # every pair of specials
+    a, b = pairs[:, 0].copy(), pairs[:, 1].copy()
+    c = np.resize(np.array([1e-38, -1e-38, 3e-39, 1.0, -0.0, 7e37], dtype=np.float32), a.size)
+    for divisor in (0, 3, 8):
+        da, db, dc = G.dev(a, 1), G.dev(b, 2), G.dev(c, 3)
+        out, _ = G.dev(np.zeros(a.size, dtype=np.float32), 1)
+        ring_abi.fold_rows([(out.data_ptr(), [da[0].data_ptr(), db[0].data_ptr(), dc[0].data_ptr()], a.size)], 3,
+                           divisor, ring_abi.F32, None)
+        G.sync()
+        G.assert_same_bits(G.host(out), _fold_reference([a, b, c], divisor, np.float32), "fold of specials /%d" % divisor)
+        if divisor:
+            out2, _ = G.dev(np.zeros(a.size, dtype=np.float32), 2)
+            ring_abi.apply_rows_avg([(out2.data_ptr(), da[0].data_ptr(), db[0].data_ptr(), a.size)], None, divisor,
+                                    ring_abi.F32, None)
+            G.sync()
+            with np.errstate(all="ignore"):
+                want = ((b + a).astype(np.float32) / np.float32(divisor)).astype(np.float32)
+            G.assert_same_bits(G.host(out2), want, "add-and-divide of specials /%d" % divisor)
+            t, _ = G.dev(np.zeros(a.size, dtype=np.float32), 3)
+            plan = ring_abi.FusionPlan([t.data_ptr()], [a.size], ring_abi.F32)
+            plan.scatter(ring_abi.make_spans([(0, a.size, da[0].data_ptr(), None)]), divisor, None)
+            G.sync()
+            with np.errstate(all="ignore"):
+                G.assert_same_bits(G.host(t), (a / np.float32(divisor)).astype(np.float32), "scatter of specials /%d" % divisor)
+            plan.close()
+
+
 @pytest.mark.parametrize("dtype", G.DTYPES)
 def test_fold_and_copy_rows_in_one_call(dtype):
     """Fold rows (divided) and plain copy rows (never divided) of one call; more
