@@ -42,7 +42,12 @@ for p in (ROOT, os.path.join(ROOT, "tensorflow-allreduce_amd")):
 HBM_PEAK_GBS = 8000.0
 SAMPLE_EVERY = 16                   # steps between launches that carry timing events
 METRIC = "per-rank ring allreduce GB/s & % of HBM peak, 64 MiB fp32, N=8 virtual ranks"
-TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "rows_kernel_f32_accumulate_64MiB_n8_pmc.txt")
+# committed rocprofv3 counter summaries holding a `traffic_bytes_per_launch:` line for a workload's dominant kernel
+TRAFFIC_PROFILES = {
+    "allreduce_f32_64MiB_n8": "rows_kernel_f32_accumulate_64MiB_n8_pmc.txt",
+    "allreduce_f32_64MiB_n8_direct": "fold_kernel_f32_64MiB_n8_direct.txt",
+    "fused_resnet50_n8_no_passes": "fusion_span_kernel_resnet50_161_tensors_n8_no_passes.txt",
+}
 
 
 def resnet50_counts():
@@ -567,12 +572,15 @@ def cpu_baseline(w):
     return out
 
 
-def measured_traffic():
-    """HBM bytes per launch of the headline's dominant kernel from the committed
+def measured_traffic(workload):
+    """HBM bytes per launch of the workload's dominant kernel from the committed
     rocprofv3 counter summary (FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel
     of known size), or None when no such summary exists."""
+    name = TRAFFIC_PROFILES.get(workload)
+    if name is None:
+        return None
     try:
-        text = open(TRAFFIC_PROFILE).read()
+        text = open(os.path.join(ROOT, "profiles", name)).read()
     except OSError:
         return None
     m = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", text, re.M)
@@ -699,7 +707,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": measured_traffic() if args.workload == WORKLOADS[0] else None,
+            "traffic": measured_traffic(args.workload),
             "algorithmic_bytes_per_launch": dom[1],
             "avg_launch_us": round(phase_us[w.dominant], 3),
             "launches_timed": len(samples),
