@@ -137,3 +137,50 @@ def test_fusion_pack_unpack_roundtrip(sizes, dtype, seed, divisor):
         G.assert_same_bits(G.host(d[0]), scaled[at:at + c].astype(dtype), "unpack_scaled")
         at += c
     plan.close()
+
+
+@settings(max_examples=25, **COMMON)
+@given(counts=st.lists(st.one_of(st.integers(0, 6), st.sampled_from([1023, 4095, 4096, 4097, 8192, 12_289]),
+                                 st.integers(0, 20_000)), min_size=1, max_size=30),
+       dtype=st.sampled_from(G.DTYPES), seed=st.integers(0, 2**31), divisor=st.sampled_from([0, 5]),
+       n_spans=st.integers(1, 6))
+def test_fusion_spans_with_boundaries_on_tiles_and_tensors(counts, dtype, seed, divisor, n_spans):
+    """Gather and scatter over spans whose ends fall on tensor boundaries, on
+    multiples of the kernel's tile, one element either side of them, or
+    anywhere; against numpy on the concatenation."""
+    rng = np.random.default_rng(seed)
+    total = sum(counts)
+    hosts = [G.random_array(rng, c, dtype) for c in counts]
+    devs = [G.dev(h, int(rng.integers(0, 4))) for h in hosts]
+    plan = ring_abi.FusionPlan([d[0].data_ptr() if c else None for d, c in zip(devs, counts)], counts,
+                               G.NP2ABI[np.dtype(dtype)])
+    flat = np.concatenate(hosts) if hosts else np.empty(0, dtype=dtype)
+    tile = 4096 if np.dtype(dtype).itemsize == 4 else 2048
+    marks = sorted({0, total} | {int(x) for x in np.cumsum(counts)} | set(range(0, total + 1, tile)))
+    marks = sorted({min(max(m + d, 0), total) for m in marks for d in (-1, 0, 1)})
+    cuts = sorted(int(rng.choice(marks)) if rng.random() < 0.7 else int(rng.integers(0, total + 1))
+                  for _ in range(2 * n_spans))
+    spans = [(cuts[2 * k], cuts[2 * k + 1] - cuts[2 * k]) for k in range(n_spans)]
+    incoming = [G.random_array(rng, c, dtype) for _, c in spans]
+    d_in = [G.dev(x, k % 4) for k, x in enumerate(incoming)]
+    d_out = [G.dev(np.zeros(c, dtype=dtype), (k + 2) % 4) for k, (_, c) in enumerate(spans)]
+    plan.gather(ring_abi.make_spans([(b, c, d_in[k][0].data_ptr() if c and k % 2 == 0 else None,
+                                      d_out[k][0].data_ptr() if c else None) for k, (b, c) in enumerate(spans)]), None)
+    torch.cuda.synchronize()
+    for k, (b, c) in enumerate(spans):
+        with np.errstate(all="ignore"):
+            want = (flat[b:b + c] + incoming[k]).astype(dtype) if k % 2 == 0 else flat[b:b + c]
+        G.assert_same_bits(G.host(d_out[k][0]), want, "gather span %d [%d,+%d) of %d" % (k, b, c, total))
+    plan.scatter(ring_abi.make_spans([(b, c, d_in[k][0].data_ptr() if c else None, None)
+                                      for k, (b, c) in enumerate(spans)]), divisor, None)
+    torch.cuda.synchronize()
+    want = flat.copy()
+    for k, (b, c) in enumerate(spans):
+        x = incoming[k]
+        if divisor:
+            with np.errstate(all="ignore"):
+                x = (x / np.float32(divisor) if dtype == np.float32 else x // dtype(divisor)).astype(dtype)
+        want[b:b + c] = x
+    got = np.concatenate([G.host(d[0]) for d in devs]) if devs else np.empty(0, dtype=dtype)
+    G.assert_same_bits(got, want, "scatter /%d spans %r" % (divisor, spans))
+    plan.close()
