@@ -184,3 +184,39 @@ def test_fusion_spans_with_boundaries_on_tiles_and_tensors(counts, dtype, seed, 
     got = np.concatenate([G.host(d[0]) for d in devs]) if devs else np.empty(0, dtype=dtype)
     G.assert_same_bits(got, want, "scatter /%d spans %r" % (divisor, spans))
     plan.close()
+
+
+@settings(max_examples=30, **COMMON)
+@given(m=st.integers(1, 12), count=counts, dtype=st.sampled_from(G.DTYPES), seed=st.integers(0, 2**31),
+       divisor=st.sampled_from([0, 0, 2, 7]), in_place=st.integers(-1, 11), n_copies=st.integers(0, 3))
+def test_fold_rows_any_source_may_be_the_destination(m, count, dtype, seed, divisor, in_place, n_copies):
+    """One fold row whose destination is a fresh buffer or any one of its own
+    sources, with copy rows in the same launch; against a numpy fold in the
+    same order."""
+    rng = np.random.default_rng(seed)
+    hs = [G.random_array(rng, count, dtype, wide=True) for _ in range(m)]
+    ds = [G.dev(h, int(rng.integers(0, 4))) for h in hs]
+    acc = hs[0].copy()
+    with np.errstate(all="ignore"):
+        for h in hs[1:]:
+            acc = (h + acc).astype(dtype)
+        if divisor:
+            acc = (acc / np.float32(divisor) if dtype == np.float32 else acc // dtype(divisor)).astype(dtype)
+    if 0 <= in_place < m:
+        dst = ds[in_place][0]
+    else:
+        dst = G.dev(np.zeros(count, dtype=dtype), int(rng.integers(0, 4)))[0]
+    copies_h = [G.random_array(rng, int(rng.integers(0, 5000)), dtype) for _ in range(n_copies)]
+    copies_s = [G.dev(h, k % 4) for k, h in enumerate(copies_h)]
+    copies_d = [G.dev(np.zeros(h.size, dtype=dtype), (k + 1) % 4) for k, h in enumerate(copies_h)]
+    ring_abi.fold_and_copy_rows(
+        [(dst.data_ptr() if count else None, [d[0].data_ptr() if count else None for d in ds], count)], m, divisor,
+        [(d[0].data_ptr() if h.size else None, s[0].data_ptr() if h.size else None, h.size)
+         for d, s, h in zip(copies_d, copies_s, copies_h)], G.NP2ABI[np.dtype(dtype)], None)
+    torch.cuda.synchronize()
+    G.assert_same_bits(G.host(dst), acc, "fold m=%d count=%d /%d in place %d" % (m, count, divisor, in_place))
+    for k, h in enumerate(copies_h):
+        G.assert_same_bits(G.host(copies_d[k][0]), h, "copy row %d" % k)
+    for k, h in enumerate(hs):                       # the other sources are never written
+        if k != in_place:
+            G.assert_same_bits(G.host(ds[k][0]), h, "source %d untouched" % k)
