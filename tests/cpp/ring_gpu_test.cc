@@ -98,7 +98,8 @@ static void ring_case(int n, size_t count, void* stream) {
     CHECK(std::memcmp(to_host(d_out, count).data(), want[r].data(), count * sizeof(T)) == 0);
     // the same through the ring driver, copy folded into the accumulate
     std::vector<const void*> rs_p(d_rs.begin(), d_rs.end()), ag_p(d_ag.begin(), d_ag.end());
-    HIP_OK(hipMemset(d_out, 0, count * sizeof(T)));
+    // on the ring's own stream: a memset on the null stream is not ordered with a non-blocking stream
+    HIP_OK(hipMemsetAsync(d_out, 0, count * sizeof(T), static_cast<hipStream_t>(stream)));
     CHECK(mpic_ring_allreduce_prestaged(n, r, Code<T>::mpic, d_in, d_out, count, rs_p.data(), ag_p.data(), stream, 3) == MPIC_OK);
     CHECK(ring_stream_synchronize(stream) == RING_OK);
     CHECK(std::memcmp(to_host(d_out, count).data(), want[r].data(), count * sizeof(T)) == 0);
@@ -109,7 +110,8 @@ static void ring_case(int n, size_t count, void* stream) {
       const std::vector<T>& peer = in[(own + k) % n];
       raw.push_back(to_device(std::vector<T>(peer.begin() + starts[own], peer.begin() + starts[own] + sizes[own]), k % 4));
     }
-    HIP_OK(hipMemset(d_out, 0, count * sizeof(T)));
+    // on the ring's own stream: a memset on the null stream is not ordered with a non-blocking stream
+    HIP_OK(hipMemsetAsync(d_out, 0, count * sizeof(T), static_cast<hipStream_t>(stream)));
     CHECK(mpic_ring_allreduce_direct_prestaged(n, r, Code<T>::mpic, d_in, d_out, count, raw.data(), ag_p.data(), stream,
                                                r % 2) == MPIC_OK);
     CHECK(ring_stream_synchronize(stream) == RING_OK);
