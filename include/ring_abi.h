@@ -127,7 +127,10 @@ int ring_schedule(int phase, int n, int r, int step, int* send_seg, int* recv_se
 
 /* ---- the dedicated stream — CudaStreamForMPI(), mpi_ops.cc:213-230, 582-583,
  * 872-876: one non-default stream for all ring copies and accumulates, so a
- * wait on it never waits for unrelated compute. Default priority. ---------- */
+ * wait on it never waits for unrelated compute. Default priority. The stream
+ * is non-blocking: work on the null stream (a plain hipMemset, say) is NOT
+ * ordered with it, so whatever prepares a buffer for these calls runs on the
+ * same stream or is synchronised first. ---------------------------------------- */
 int ring_stream_create(void** stream);
 int ring_stream_destroy(void* stream);
 int ring_stream_synchronize(void* stream);
