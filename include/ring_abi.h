@@ -54,7 +54,8 @@ enum ring_status {
   RING_ERR_DTYPE = 1,    /* not one of ring_dtype ("Invalid tensor type", mpi_ops.cc:844) */
   RING_ERR_ARGUMENT = 2, /* null pointer with a non-zero size, n < 1, rank out of range ... */
   RING_ERR_HIP = 3,      /* a HIP runtime call failed */
-  RING_ERR_NO_DEVICE = 4 /* no usable GPU */
+  RING_ERR_NO_DEVICE = 4, /* no usable GPU */
+  RING_ERR_LIMIT = 5      /* beyond a stated fixed capacity (ring_fusion_run_static) */
 };
 
 int ring_abi_version(void);
@@ -271,6 +272,25 @@ int ring_fusion_unpack(const ring_fusion_plan* plan, const void* fused, void* st
  * (the average of a fused allreduce folded into the unpack). divisor >= 1. */
 int ring_fusion_unpack_scaled(const ring_fusion_plan* plan, const void* fused, int divisor,
                               void* stream);
+
+/* Pack / unpack WITHOUT a plan and without any allocation. No counterpart in
+ * the reference; for callers that cannot allocate device memory: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * unpack == 0: fused[offset_j + i] = tensors[j][i] (divisor must be 0), as
+ * ring_fusion_pack; unpack != 0: tensors[j][i] = fused[offset_j + i], divided
+ * by divisor when divisor >= 1, as ring_fusion_unpack[_scaled]. `tensors` and
+ * `counts` are HOST arrays of k entries, read before the call returns. The
+ * offset table a plan keeps in an allocation of its own is built, by small
+ * kernels on `stream` ahead of the pack / unpack kernel, in a static device
+ * array of 540,680 bytes that every GPU the library runs on holds until the
+ * process ends. Limits: 1024 non-empty tensors and 268,435,456 four-byte
+ * (134,217,728 eight-byte) elements per call, beyond which the call returns
+ * RING_ERR_LIMIT and launches nothing. All calls on one GPU share that GPU's
+ * array: calls on the same stream are ordered, calls that overlap on
+ * different streams of one GPU race. Calls no hipMalloc / hipFree / hipMemcpy
+ * (the first call on a device looks up the array's address). */
+int ring_fusion_run_static(int unpack, const void* const* tensors, const size_t* counts, int k, int dtype,
+                           void* fused, int divisor, void* stream);
 
 /* Fusion without passes of its own. A span is `count` elements of the plan's
  * fused element space starting at `begin` (a ring segment of the packed

@@ -37,6 +37,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -817,9 +818,27 @@ struct ring_fusion_plan {
 
 namespace {
 
+// What the pack / unpack kernel reads besides the tensors: the offset table
+// of the fused buffer, wherever it lives (a plan's own allocation, or the
+// static array of the allocation-free entry point).
+struct FusionView {
+  int dtype;
+  size_t esz;
+  uint32_t ntiles;
+  uint64_t total;  // elements
+  const uint64_t* offsets;
+  void* const* ptrs;
+  const uint32_t* tile_first;
+  const uint32_t* tile_last;
+};
+
+inline FusionView view_of(const ring_fusion_plan* p) {
+  return FusionView{p->dtype, p->esz, p->ntiles, p->total, p->d_offsets, p->d_ptrs, p->d_tile_first, p->d_tile_last};
+}
+
 template <typename T, bool PACK, bool DIV>
-int launch_fusion(const ring_fusion_plan* p, void* fused, hipStream_t stream, int divisor) {
-  uint32_t grid = p->ntiles;
+int launch_fusion(const FusionView& p, void* fused, hipStream_t stream, int divisor) {
+  uint32_t grid = p.ntiles;
   if (g_tuning.blocks_per_cu > 0) {
     DeviceInfo info;
     int rc = device_info(&info);
@@ -829,9 +848,8 @@ int launch_fusion(const ring_fusion_plan* p, void* fused, hipStream_t stream, in
   }
 #define RING_FUSION(N)                                                                                   \
   launch(fusion_kernel<T, PACK, N, DIV>, dim3(grid), dim3(kBlock), stream, static_cast<T*>(fused),       \
-         static_cast<const uint64_t*>(p->d_offsets), reinterpret_cast<T* const*>(p->d_ptrs),             \
-         static_cast<const uint32_t*>(p->d_tile_first), static_cast<const uint32_t*>(p->d_tile_last),    \
-         p->ntiles, p->total, divisor)
+         p.offsets, reinterpret_cast<T* const*>(p.ptrs), p.tile_first, p.tile_last, p.ntiles, p.total,   \
+         divisor)
   int nt = g_tuning.nt[PACK ? kRolePack : kRoleUnpack];
   if (nt < 0) nt = 2;
   switch (nt & 3) {
@@ -846,19 +864,103 @@ int launch_fusion(const ring_fusion_plan* p, void* fused, hipStream_t stream, in
 }
 
 // divisor 0: plain pack / unpack. divisor >= 1: unpack and divide.
-int fusion_run(const ring_fusion_plan* p, void* fused, void* stream, bool pack, int divisor) {
-  if (!p) return RING_ERR_ARGUMENT;
-  if (p->total == 0) return RING_OK;
+int fusion_run(const FusionView& p, void* fused, void* stream, bool pack, int divisor) {
+  if (p.total == 0) return RING_OK;
   if (!fused || (reinterpret_cast<uintptr_t>(fused) & 15u)) return RING_ERR_ARGUMENT;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (divisor > 0) {
-    if (p->dtype == RING_F32) return launch_fusion<float, false, true>(p, fused, s, divisor);
-    if (p->dtype == RING_I32) return launch_fusion<int32_t, false, true>(p, fused, s, divisor);
+    if (p.dtype == RING_F32) return launch_fusion<float, false, true>(p, fused, s, divisor);
+    if (p.dtype == RING_I32) return launch_fusion<int32_t, false, true>(p, fused, s, divisor);
     return launch_fusion<int64_t, false, true>(p, fused, s, divisor);
   }
-  if (p->esz == 8)
+  if (p.esz == 8)
     return pack ? launch_fusion<uint64_t, true, false>(p, fused, s, 0) : launch_fusion<uint64_t, false, false>(p, fused, s, 0);
   return pack ? launch_fusion<uint32_t, true, false>(p, fused, s, 0) : launch_fusion<uint32_t, false, false>(p, fused, s, 0);
+}
+
+int fusion_run(const ring_fusion_plan* p, void* fused, void* stream, bool pack, int divisor) {
+  if (!p) return RING_ERR_ARGUMENT;
+  return fusion_run(view_of(p), fused, stream, pack, divisor);
+}
+
+// ---- the offset table in a static device array --------------------------------------
+// For callers that may not allocate device memory (code under HIP graph
+// capture, tight serving loops, harnesses that forbid hipMalloc): the table a
+// plan keeps in an allocation of its own is built in a file-scope device array
+// instead, by two small kernels, from values that travel in kernel arguments.
+// Every call on a GPU shares that GPU's copy of the array.
+
+constexpr uint32_t kStaticMaxTensors = 1024;  // non-empty tensors per call
+constexpr uint32_t kStaticMaxTiles = 65536;   // 16 KiB tiles of the fused buffer: 1 GiB
+struct StaticFusionTable {
+  uint64_t offsets[kStaticMaxTensors + 1];
+  void* ptrs[kStaticMaxTensors];
+  uint32_t tile_first[kStaticMaxTiles];
+  uint32_t tile_last[kStaticMaxTiles];
+};
+// 540,680 bytes per GPU the library runs on, held until the process ends.
+static __device__ __align__(256) unsigned char scratch[sizeof(StaticFusionTable)];
+
+// `scratch` is a host-side stand-in in host code: the array's device address is
+// looked up once per device and only that pointer is ever handed to a kernel.
+std::mutex g_scratch_mutex;
+StaticFusionTable* g_scratch_ptr[64] = {};
+
+int scratch_of_current_device(StaticFusionTable** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) { hip_fail(e); return RING_ERR_NO_DEVICE; }
+  if (dev < 0 || dev >= 64) return RING_ERR_NO_DEVICE;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    RING_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return RING_ERR_HIP;
+    g_scratch_ptr[dev] = static_cast<StaticFusionTable*>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return RING_OK;
+}
+
+// A piece of the offset / pointer table, by value in the kernel arguments.
+constexpr uint32_t kTableChunk = 128;
+struct TableChunk {
+  uint32_t base, n;  // entries [base, base + n) of the table
+  uint64_t end;      // written to offsets[base + n]: where the next tensor starts (the total after the last chunk)
+  uint64_t off[kTableChunk];
+  void* ptr[kTableChunk];
+};
+
+__global__ void __launch_bounds__(kBlock) table_chunk_kernel(StaticFusionTable* tab, const TableChunk c) {
+  const uint32_t i = threadIdx.x;
+  if (i < c.n) {
+    tab->offsets[c.base + i] = c.off[i];
+    tab->ptrs[c.base + i] = c.ptr[i];
+  }
+  if (i == 0) tab->offsets[c.base + c.n] = c.end;
+}
+
+// tile_first / tile_last of every tile, as ring_fusion_plan_create computes them
+// on the host: the first and the last tensor that overlap the tile.
+__global__ void __launch_bounds__(kBlock)
+table_tiles_kernel(StaticFusionTable* tab, uint32_t m, uint32_t ntiles, uint64_t tile_elems, uint64_t total) {
+  const uint32_t tile = blockIdx.x * kBlock + threadIdx.x;
+  if (tile >= ntiles) return;
+  const uint64_t e0 = static_cast<uint64_t>(tile) * tile_elems;
+  const uint64_t e1 = (e0 + tile_elems < total) ? e0 + tile_elems : total;
+  // offsets[0..m] is strictly increasing, offsets[0] = 0, offsets[m] = total
+  uint32_t lo = 0, hi = m;  // offsets[lo] <= e0 < offsets[hi]
+  while (hi - lo > 1) {
+    const uint32_t mid = (lo + hi) >> 1;
+    if (tab->offsets[mid] <= e0) lo = mid; else hi = mid;
+  }
+  tab->tile_first[tile] = lo;
+  hi = m;  // offsets[lo] < e1 <= offsets[hi]
+  while (hi - lo > 1) {
+    const uint32_t mid = (lo + hi) >> 1;
+    if (tab->offsets[mid] < e1) lo = mid; else hi = mid;
+  }
+  tab->tile_last[tile] = lo;
 }
 
 }  // namespace
@@ -877,6 +979,7 @@ const char* ring_status_string(int status) {
     case RING_ERR_ARGUMENT: return "invalid argument";
     case RING_ERR_HIP: return "HIP runtime call failed";
     case RING_ERR_NO_DEVICE: return "no usable GPU";
+    case RING_ERR_LIMIT: return "beyond the capacity of the static device table (1024 tensors, 65536 tiles of 16 KiB)";
     default: return "unknown status";
   }
 }
@@ -1339,6 +1442,59 @@ int ring_fusion_unpack(const ring_fusion_plan* plan, const void* fused, void* st
 int ring_fusion_unpack_scaled(const ring_fusion_plan* plan, const void* fused, int divisor, void* stream) {
   if (divisor < 1) return RING_ERR_ARGUMENT;
   return fusion_run(plan, const_cast<void*>(fused), stream, false, divisor);
+}
+
+int ring_fusion_run_static(int unpack, const void* const* tensors, const size_t* counts, int k, int dtype, void* fused,
+                           int divisor, void* stream) {
+  if (!dtype_ok(dtype)) return RING_ERR_DTYPE;
+  if (k < 0 || (k > 0 && (!tensors || !counts)) || divisor < 0 || (!unpack && divisor != 0)) return RING_ERR_ARGUMENT;
+  const size_t esz = dtype_size(dtype);
+  const uint64_t tile_elems = static_cast<uint64_t>(kFusionTileVecs) * (16 / esz);
+  // first pass over the host arrays: sizes only, so that nothing is launched for a call that is refused
+  uint64_t total = 0;
+  uint32_t m = 0;
+  for (int j = 0; j < k; j++) {
+    if (counts[j] == 0) continue;
+    if (!tensors[j] || (reinterpret_cast<uintptr_t>(tensors[j]) & (esz - 1))) return RING_ERR_ARGUMENT;
+    if (m == kStaticMaxTensors) return RING_ERR_LIMIT;
+    m++;
+    total += counts[j];
+    if (total > static_cast<uint64_t>(kStaticMaxTiles) * tile_elems) return RING_ERR_LIMIT;
+  }
+  if (total == 0) return RING_OK;
+  if (!fused || (reinterpret_cast<uintptr_t>(fused) & 15u)) return RING_ERR_ARGUMENT;
+  const uint32_t ntiles = static_cast<uint32_t>((total + tile_elems - 1) / tile_elems);
+
+  StaticFusionTable* tab = nullptr;
+  int rc = scratch_of_current_device(&tab);
+  if (rc != RING_OK) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+
+  // the table, kTableChunk tensors per launch; the fused-buffer offsets are the running sum of the counts
+  TableChunk chunk;
+  chunk.base = 0;
+  chunk.n = 0;
+  uint64_t at = 0;
+  for (int j = 0; j < k; j++) {
+    if (counts[j] == 0) continue;
+    chunk.off[chunk.n] = at;
+    chunk.ptr[chunk.n] = const_cast<void*>(tensors[j]);
+    chunk.n++;
+    at += counts[j];
+    if (chunk.n == kTableChunk || at == total) {
+      chunk.end = at;
+      hipLaunchKernelGGL(table_chunk_kernel, dim3(1), dim3(kBlock), 0, s, tab, chunk);
+      RING_HIP(hipGetLastError());
+      chunk.base += chunk.n;
+      chunk.n = 0;
+      if (at == total) break;  // only empty tensors can follow
+    }
+  }
+  hipLaunchKernelGGL(table_tiles_kernel, dim3((ntiles + kBlock - 1) / kBlock), dim3(kBlock), 0, s, tab, m, ntiles,
+                     tile_elems, total);
+  RING_HIP(hipGetLastError());
+  const FusionView view{dtype, esz, ntiles, total, tab->offsets, tab->ptrs, tab->tile_first, tab->tile_last};
+  return fusion_run(view, fused, stream, !unpack, divisor);
 }
 
 }  // extern "C"

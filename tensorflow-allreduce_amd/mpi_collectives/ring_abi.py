@@ -25,7 +25,7 @@ EXPORTS = (
     "ring_allgather_steps", "ring_apply_rows", "ring_apply_rows_avg", "ring_fold_rows", "ring_fold_and_copy_rows",
     "ring_fusion_plan_create", "ring_fusion_plan_destroy", "ring_fusion_plan_elements", "ring_fusion_plan_dtype",
     "ring_fusion_pack", "ring_fusion_unpack", "ring_fusion_unpack_scaled", "ring_fusion_gather",
-    "ring_fusion_scatter", "ring_scale",
+    "ring_fusion_scatter", "ring_scale", "ring_fusion_run_static",
 )
 
 
@@ -126,6 +126,7 @@ def lib():
             "ring_fusion_gather": (ci, [vp, ctypes.POINTER(FusionSpan), ci, vp]),
             "ring_fusion_scatter": (ci, [vp, ctypes.POINTER(FusionSpan), ci, ci, vp]),
             "ring_scale": (ci, [ci, vp, sz, ci, vp]),
+            "ring_fusion_run_static": (ci, [ci, ctypes.POINTER(vp), psz, ci, ci, vp, ci, vp]),
         }
         for name in EXPORTS:
             fn = getattr(L, name)          # AttributeError if the symbol is missing
@@ -299,6 +300,17 @@ def fold_and_copy_rows(fold, m, divisor, copies, dtype, stream):
 
 def scale(dtype, data, count, divisor, stream):
     check(lib().ring_scale(dtype, data, count, divisor, stream), "ring_scale")
+
+
+def fusion_run_static(unpack, ptrs, counts, dtype, fused, divisor, stream):
+    """Pack (unpack false) or unpack (optionally divided) without a plan and
+    without any allocation: the offset table is built in the library's static
+    device array. Limits: 1024 non-empty tensors, 65536 tiles of 16 KiB."""
+    k = len(ptrs)
+    p = (ctypes.c_void_p * max(k, 1))(*ptrs)
+    c = (ctypes.c_size_t * max(k, 1))(*counts)
+    check(lib().ring_fusion_run_static(1 if unpack else 0, p, c, k, dtype, fused, divisor, stream),
+          "ring_fusion_run_static")
 
 
 class FusionPlan:
