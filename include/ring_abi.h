@@ -282,7 +282,7 @@ int ring_fusion_unpack_scaled(const ring_fusion_plan* plan, const void* fused, i
  * `counts` are HOST arrays of k entries, read before the call returns. The
  * offset table a plan keeps in an allocation of its own is built, by small
  * kernels on `stream` ahead of the pack / unpack kernel, in a static device
- * array of 540,680 bytes that every GPU the library runs on holds until the
+ * array of 1,064,968 bytes that every GPU the library runs on holds until the
  * process ends. Limits: 1024 non-empty tensors and 268,435,456 four-byte
  * (134,217,728 eight-byte) elements per call, beyond which the call returns
  * RING_ERR_LIMIT and launches nothing. All calls on one GPU share that GPU's

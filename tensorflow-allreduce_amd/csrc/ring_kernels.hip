@@ -91,7 +91,13 @@ template <> struct VecOf<int64_t> { typedef int64_t type __attribute__((ext_vect
 // of the reference): true division for float32 (a correctly rounded divide,
 // NOT a multiply by 1/n), floor division for the integer types. n > 0, so
 // floor differs from C's truncation only for negative x with a remainder.
-__device__ __forceinline__ float div_one(float x, int n) { return x / static_cast<float>(n); }
+// By a power of two the quotient is the same real number as the product with
+// the (exact) reciprocal, so the one rounding gives the same bits, subnormal
+// results included, without the divide's dozen instructions (n is uniform).
+__device__ __forceinline__ float div_one(float x, int n) {
+  if ((n & (n - 1)) == 0) return x * (1.0f / static_cast<float>(n));
+  return x / static_cast<float>(n);
+}
 __device__ __forceinline__ int32_t div_one(int32_t x, int n) {
   const int32_t q = x / n;
   return q - ((x % n != 0) && (x < 0));
@@ -166,28 +172,48 @@ struct RowTable {
 
 // NT: bit 0 = non-temporal stores, bit 1 = non-temporal loads (3, both, is the
 // default: every byte is touched once).
-template <typename T, int NT>
-__device__ __forceinline__ void store_vec(typename VecOf<T>::type* p, typename VecOf<T>::type v) {
-  if (NT & 1) __builtin_nontemporal_store(v, p); else *p = v;
-}
-// A macro, not a function template: the operand's type carries a reduced
-// alignment (element-aligned 16-byte loads) that template deduction would drop.
-#define RING_LOAD_VEC(NT, p) (((NT) & 2) ? __builtin_nontemporal_load(p) : *(p))
+// Device global memory, as a type qualifier.
+#define RING_GLOBAL __attribute__((address_space(1)))
 
-// One workgroup-tile of a row: vectors [v0, v0 + 256*UNROLL) of the aligned
-// body, plus the row's scalar head (tile 0) and tail (last tile). dst is
-// brought to 16-byte alignment by the head; a and b are read with
-// element-aligned 16-byte loads. a == dst (divide) and b == dst (add) are
-// allowed: every element is read before it is written, by the same lane.
-template <typename T, int OP, int UNROLL, int NT>
-__device__ __forceinline__ void row_tile(T* dst, const T* a, const T* b, uint64_t count, uint32_t tile,
+// Macros, not function templates: the operand's type may carry a reduced
+// alignment (element-aligned 16-byte accesses) that template deduction would drop.
+#define RING_LOAD_VEC(NT, p) (((NT) & 2) ? __builtin_nontemporal_load(p) : *(p))
+#define RING_STORE_VEC(NT, p, v)                            \
+  do {                                                      \
+    if ((NT) & 1) __builtin_nontemporal_store((v), (p));    \
+    else *(p) = (v);                                        \
+  } while (0)
+
+// Which side of a row the scalar head brings to 16-byte alignment.
+enum Anchor { kOnDst = 0, kOnSrc = 1 };
+
+// One workgroup-tile of a row: 256 * UNROLL 16-byte vectors of the row's body,
+// plus the row's scalar head (tile 0) and tail (last tile). ANCHOR picks the
+// side the head aligns: the destination (aligned stores, element-aligned loads
+// of a and b), or the source a (aligned loads of a, element-aligned stores:
+// rows whose source is known to be aligned, the tiles of an unpack, which then
+// need no head at all and stay full tiles). a == dst (divide) and b == dst
+// (add) are allowed: every element is read before it is written, by the same
+// lane.
+template <typename T, int OP, int UNROLL, int NT, int ANCHOR = kOnDst>
+__device__ __forceinline__ void row_tile(T* dst_, const T* a_, const T* b_, uint64_t count, uint32_t tile,
                                          uint32_t tiles_in_row, int n) {
   typedef typename VecOf<T>::type V;
   typedef V VU __attribute__((aligned(sizeof(T))));  // element-aligned 16-byte access
+  // Every operand is device global memory. Said explicitly: a pointer that was
+  // itself read from memory (a fusion plan's tensor table) is otherwise taken
+  // for a generic one and accessed with flat instructions.
+  typedef T RING_GLOBAL GT;
+  typedef V RING_GLOBAL GV;
+  typedef VU RING_GLOBAL GVU;
+  GT* dst = (GT*)dst_;
+  const GT* a = (const GT*)a_;
+  const GT* b = (const GT*)b_;
   constexpr uint32_t VEC = 16 / sizeof(T);
   constexpr uint32_t kTileVecs = kBlock * UNROLL;
 
-  uint64_t head = ((16u - (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(dst)) & 15u)) & 15u) / sizeof(T);
+  const uintptr_t anchor = ANCHOR == kOnSrc ? reinterpret_cast<uintptr_t>(a_) : reinterpret_cast<uintptr_t>(dst_);
+  uint64_t head = ((16u - (static_cast<uint32_t>(anchor) & 15u)) & 15u) / sizeof(T);
   if (head > count) head = count;
   const uint64_t nvec = (count - head) / VEC;
   const uint32_t tid = threadIdx.x;
@@ -199,35 +225,61 @@ __device__ __forceinline__ void row_tile(T* dst, const T* a, const T* b, uint64_
     if (e < count) dst[e] = apply_one<T, OP>(a[e], kTwo ? b[e] : T(), n);
   }
 
-  V* dv = reinterpret_cast<V*>(dst + head);
-  const VU* av = reinterpret_cast<const VU*>(a + head);
-  const VU* bv = reinterpret_cast<const VU*>(b + head);
-  const uint64_t v0 = static_cast<uint64_t>(tile) * kTileVecs + tid;
+  // The tile's vectors through pointers that are uniform over the workgroup
+  // plus a 32-bit lane offset (scalar base + vector offset: one address
+  // register per operand). Access j of the workgroup covers 4 KiB of
+  // consecutive memory, lane after lane (measured faster than giving every
+  // wave 4 KiB of its own). The anchored side goes through the aligned vector
+  // type, the other through the element-aligned one (spelled out: an alignment
+  // attribute does not survive a template).
+  const uint64_t tile_base = static_cast<uint64_t>(tile) * kTileVecs;
+  if (tile_base >= nvec) return;
+  const uint64_t left = nvec - tile_base;  // vectors from this tile on
+  GV* dv_al = (GV*)(dst + head) + tile_base;
+  GVU* dv_un = (GVU*)(dst + head) + tile_base;
+  const GV* av_al = (const GV*)(a + head) + tile_base;
+  const GVU* av_un = (const GVU*)(a + head) + tile_base;
+  const GVU* bv = kTwo ? (const GVU*)(b + head) + tile_base : nullptr;
+  const uint32_t v0 = tid;
+#define ROW_LOAD_A(i) (ANCHOR == kOnSrc ? RING_LOAD_VEC(NT, &av_al[i]) : RING_LOAD_VEC(NT, &av_un[i]))
+#define ROW_STORE(i, v)                                      \
+  do {                                                       \
+    if (ANCHOR == kOnDst) RING_STORE_VEC(NT, &dv_al[i], v);  \
+    else RING_STORE_VEC(NT, &dv_un[i], v);                   \
+  } while (0)
 
-  if (static_cast<uint64_t>(tile + 1) * kTileVecs <= nvec) {
+  if (left >= kTileVecs) {
     V x[UNROLL], y[UNROLL];
 #pragma unroll
-    for (int j = 0; j < UNROLL; j++) x[j] = RING_LOAD_VEC(NT, &av[v0 + j * kBlock]);
+    for (int j = 0; j < UNROLL; j++) x[j] = ROW_LOAD_A(v0 + j * kBlock);
     if (kTwo) {
 #pragma unroll
       for (int j = 0; j < UNROLL; j++) y[j] = RING_LOAD_VEC(NT, &bv[v0 + j * kBlock]);
     }
 #pragma unroll
-    for (int j = 0; j < UNROLL; j++) x[j] = apply_vec<T, OP>(x[j], y[j], n);
+    for (int j = 0; j < UNROLL; j++) x[j] = apply_vec<T, OP>(x[j], kTwo ? y[j] : x[j], n);
 #pragma unroll
-    for (int j = 0; j < UNROLL; j++) store_vec<T, NT>(&dv[v0 + j * kBlock], x[j]);
+    for (int j = 0; j < UNROLL; j++) ROW_STORE(v0 + j * kBlock, x[j]);
   } else {
+    // the one partial tile of a row. (rem is taken here, where left < kTileVecs
+    // is known, rather than as min(left, kTileVecs) ahead of the branch: hipcc
+    // 7.2 lowers that 64-bit uniform min to a scalar select on a stale
+    // condition code, and every lane of the partial tile then runs.)
+    const uint32_t rem = static_cast<uint32_t>(left);
 #pragma unroll
     for (int j = 0; j < UNROLL; j++) {
-      const uint64_t v = v0 + j * kBlock;
-      if (v < nvec) {
-        V x = RING_LOAD_VEC(NT, &av[v]);
+      const uint32_t v = v0 + j * kBlock;
+      if (v < rem) {
+        V x = ROW_LOAD_A(v);
         V y = x;
         if (kTwo) y = RING_LOAD_VEC(NT, &bv[v]);
-        store_vec<T, NT>(&dv[v], apply_vec<T, OP>(x, y, n));
+        const V r = apply_vec<T, OP>(x, y, n);
+        ROW_STORE(v, r);
       }
     }
   }
+#undef ROW_LOAD_A
+#undef ROW_STORE
 }
 
 template <typename T, int MODE, int UNROLL, int NT>
@@ -246,6 +298,25 @@ __device__ __forceinline__ void run_row(const Row& r, uint32_t tile, uint32_t ti
   }
 }
 
+// The row a tile of a 1-D grid belongs to: the number of rows that begin at or
+// before it, minus one. begin[] lies in the kernel arguments and its entries
+// past the last row hold 0xffffffff, so the count is a straight run of scalar
+// compares on values fetched side by side, not a binary search whose every
+// step waits for a load of its own (six in a row for 64 rows, at the start of
+// every workgroup). Uniform over the workgroup.
+template <int MAX_ROWS>
+__device__ __forceinline__ int row_of_tile(const uint32_t* begin, int n_rows, uint32_t t) {
+  int row = 0;
+  if (n_rows <= 16) {
+#pragma unroll
+    for (int k = 1; k < 16; k++) row += begin[k] <= t ? 1 : 0;
+  } else {
+#pragma unroll
+    for (int k = 1; k < MAX_ROWS; k++) row += begin[k] <= t ? 1 : 0;
+  }
+  return row;
+}
+
 template <typename T, int MODE, int UNROLL, int NT>
 __global__ void __launch_bounds__(kBlock) rows_kernel(const RowTable tab) {
   if (tab.uniform_tiles) {
@@ -257,12 +328,7 @@ __global__ void __launch_bounds__(kBlock) rows_kernel(const RowTable tab) {
   }
   const uint32_t total = tab.tile_begin[tab.n_rows];
   for (uint32_t t = blockIdx.x; t < total; t += gridDim.x) {
-    // largest row with tile_begin[row] <= t (uniform: scalar code)
-    int lo = 0, hi = tab.n_rows;
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) >> 1;
-      if (tab.tile_begin[mid] <= t) lo = mid; else hi = mid;
-    }
+    const int lo = row_of_tile<kMaxRows>(tab.tile_begin, tab.n_rows, t);
     const uint32_t first = tab.tile_begin[lo];
     run_row<T, MODE, UNROLL, NT>(tab.row[lo], t - first, tab.tile_begin[lo + 1] - first, tab.divisor,
                                  MODE == kAvg && ((tab.div_mask >> lo) & 1u));
@@ -378,7 +444,7 @@ __device__ __forceinline__ void fold_tile(T* dst, const void* const* src, int m,
   for (int j = 0; j < UNROLL; j++) {
     if (ok[j]) {
       if (DIV && divide) acc[j] = apply_vec<T, kOpDiv>(acc[j], acc[j], n);
-      store_vec<T, NT>(&dv[v0 + j * kBlock], acc[j]);
+      RING_STORE_VEC(NT, &dv[v0 + j * kBlock], acc[j]);
     }
   }
 }
@@ -407,11 +473,7 @@ __global__ void __launch_bounds__(kBlock) fold_kernel(const FoldTable tab) {
   }
   const uint32_t total = tab.tile_begin[tab.n_rows];
   for (uint32_t t = blockIdx.x; t < total; t += gridDim.x) {
-    int lo = 0, hi = tab.n_rows;
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) >> 1;
-      if (tab.tile_begin[mid] <= t) lo = mid; else hi = mid;
-    }
+    const int lo = row_of_tile<kMaxFoldRows>(tab.tile_begin, tab.n_rows, t);
     const uint32_t first = tab.tile_begin[lo];
     fold_row_tile<T, DIV, NT, UNROLL, GROUP>(tab, lo, t - first, tab.tile_begin[lo + 1] - first);
   }
@@ -429,13 +491,115 @@ __global__ void __launch_bounds__(kBlock) fold_kernel(const FoldTable tab) {
 constexpr uint32_t kFusionTileVecs = 1024;
 constexpr uint32_t kFusionLdsCap = 512;  // tensors of one tile staged in LDS
 
+// What a workgroup needs to know about its tile, in one 16-byte scalar load:
+// the first and last tensor that overlap it and, when that is one tensor (all
+// but a few hundred KiB of a ResNet-sized set), where the tile's first element
+// lies in it, so that no offset or pointer table is read at all.
+struct __attribute__((aligned(16))) FusionTile {
+  void* addr;  // first == last: address of the tile's first element inside the tensor; else null
+  uint32_t first, last;
+};
+// The record as one 16-byte load (field by field the compiler fetches `addr`
+// only after it has branched on `first` and `last`: two loads in a row).
+__device__ __forceinline__ FusionTile load_tile(const FusionTile* tiles, uint32_t tile) {
+  typedef uint64_t U2 __attribute__((ext_vector_type(2)));
+  const U2 raw = *reinterpret_cast<const U2*>(tiles + tile);
+  FusionTile rec;
+  rec.addr = reinterpret_cast<void*>(raw.x);
+  rec.first = static_cast<uint32_t>(raw.y);
+  rec.last = static_cast<uint32_t>(raw.y >> 32);
+  return rec;
+}
+
+// A piece [b0, b1) of the fused element space that meets several tensors
+// (off_tab / ptr_tab: their offsets and base pointers, tensor 0 holding b0 or
+// lying before it). Every lane takes up to 4 16-byte groups, two at a time:
+// it finds the tensor of each by binary search and issues the loads of both
+// before the first store. GATHER: lin_out = tensor (+ lin_in when given);
+// otherwise tensor = SOP(lin_in). lin_in / lin_out point at element b0 of the
+// linear side. A group cut by a tensor boundary (one per boundary) or by the
+// end of the piece goes element by element. Small tensors share cache lines
+// with their neighbours, so the tensor side is accessed with the ordinary
+// policy; NT applies to the store of the linear side only.
+template <typename T, bool GATHER, int SOP, int NT>
+__device__ __forceinline__ void multi_tensor_piece(const uint64_t* off_tab, T* const* ptr_tab, uint32_t ta,
+                                                   uint32_t tensors, uint64_t b0, uint64_t b1, const T* lin_in,
+                                                   T* lin_out, int divisor) {
+  typedef typename VecOf<T>::type V;
+  typedef V VU __attribute__((aligned(sizeof(T))));
+  typedef T RING_GLOBAL GT;  // tensors and the linear side are device global memory
+  typedef VU RING_GLOBAL GVU;
+  constexpr uint32_t VEC = 16 / sizeof(T);
+  constexpr int kBatch = 2;  // groups in flight per lane: more costs registers the full tiles need
+  const uint32_t len = static_cast<uint32_t>(b1 - b0);  // a piece is at most one tile
+  const uint32_t ngroups = (len + VEC - 1) / VEC;
+#pragma unroll 1
+  for (uint32_t g0 = threadIdx.x; g0 < ngroups; g0 += kBatch * kBlock) {
+    T* tp[kBatch];
+    uint32_t at[kBatch];
+    bool whole[kBatch], cut[kBatch];
+    V x[kBatch], y[kBatch];
+#pragma unroll
+    for (int j = 0; j < kBatch; j++) {
+      const uint32_t i = (g0 + j * kBlock) * VEC;  // element of the piece
+      whole[j] = cut[j] = false;
+      if (i < len) {
+        const uint64_t e = b0 + i;
+        uint32_t l = ta, h = tensors;  // off_tab[l] <= e < off_tab[h]
+        while (h - l > 1) {
+          const uint32_t mid = (l + h) >> 1;
+          if (off_tab[mid] <= e) l = mid; else h = mid;
+        }
+        at[j] = l;
+        tp[j] = ptr_tab[l] + (e - off_tab[l]);
+        whole[j] = e + VEC <= off_tab[l + 1] && i + VEC <= len;
+        cut[j] = !whole[j];
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kBatch; j++) {
+      if (whole[j]) {
+        const uint32_t i = (g0 + j * kBlock) * VEC;
+        if (GATHER) {
+          x[j] = RING_LOAD_VEC(0, (const GVU*)tp[j]);
+          if (lin_in) y[j] = RING_LOAD_VEC(0, (const GVU*)(lin_in + i));
+        } else {
+          x[j] = RING_LOAD_VEC(0, (const GVU*)(lin_in + i));
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < kBatch; j++) {
+      const uint32_t i = (g0 + j * kBlock) * VEC;
+      if (whole[j]) {
+        if (GATHER) {
+          const V r = lin_in ? apply_vec<T, kOpAdd>(y[j], x[j], 0) : x[j];
+          RING_STORE_VEC(NT, (GVU*)(lin_out + i), r);
+        } else {
+          const V r = apply_vec<T, SOP>(x[j], x[j], divisor);
+          RING_STORE_VEC(0, (GVU*)tp[j], r);
+        }
+      } else if (cut[j]) {
+        const uint32_t end = i + VEC < len ? i + VEC : len;
+        uint32_t l = at[j];
+        for (uint32_t k = i; k < end; k++) {
+          const uint64_t e = b0 + k;
+          while (e >= off_tab[l + 1]) l++;
+          GT* t = (GT*)(ptr_tab[l] + (e - off_tab[l]));
+          const GT* in = (const GT*)lin_in;
+          GT* out = (GT*)lin_out;
+          if (GATHER) out[k] = in ? apply_one<T, kOpAdd>(in[k], *t, 0) : *t;
+          else *t = apply_one<T, SOP>(in[k], T(), divisor);
+        }
+      }
+    }
+  }
+}
+
 template <typename T, bool PACK, int NT, bool DIV>
 __global__ void __launch_bounds__(kBlock)
 fusion_kernel(T* __restrict__ fused, const uint64_t* __restrict__ offsets, T* const* __restrict__ ptrs,
-              const uint32_t* __restrict__ tile_first, const uint32_t* __restrict__ tile_last,
-              uint32_t ntiles, uint64_t total, int divisor) {
-  typedef typename VecOf<T>::type V;
-  typedef V VU __attribute__((aligned(sizeof(T))));
+              const FusionTile* __restrict__ tiles, uint32_t ntiles, uint64_t total, int divisor) {
   constexpr uint32_t VEC = 16 / sizeof(T);
   constexpr uint64_t kTileElems = static_cast<uint64_t>(kFusionTileVecs) * VEC;
   constexpr int OP = DIV ? kOpDiv : kOpCopy;
@@ -445,12 +609,13 @@ fusion_kernel(T* __restrict__ fused, const uint64_t* __restrict__ offsets, T* co
   for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
     const uint64_t e0 = static_cast<uint64_t>(tile) * kTileElems;
     const uint64_t e1 = (e0 + kTileElems < total) ? e0 + kTileElems : total;
-    const uint32_t t0 = tile_first[tile];
-    const uint32_t t1 = tile_last[tile];
+    const FusionTile rec = load_tile(tiles, tile);
+    const uint32_t t0 = rec.first;
+    const uint32_t t1 = rec.last;
     if (t0 == t1) {
-      T* tensor = ptrs[t0] + (e0 - offsets[t0]);
+      T* tensor = static_cast<T*>(rec.addr);
       if (PACK) row_tile<T, kOpCopy, 4, NT>(fused + e0, tensor, nullptr, e1 - e0, 0, 1, 0);
-      else row_tile<T, OP, 4, NT>(tensor, fused + e0, nullptr, e1 - e0, 0, 1, divisor);
+      else row_tile<T, OP, 4, NT, kOnSrc>(tensor, fused + e0, nullptr, e1 - e0, 0, 1, divisor);
       continue;
     }
     const uint32_t span = t1 - t0 + 1;
@@ -464,31 +629,8 @@ fusion_kernel(T* __restrict__ fused, const uint64_t* __restrict__ offsets, T* co
       off_tab = s_off;
       ptr_tab = s_ptr;
     }
-    const uint32_t ngroups = static_cast<uint32_t>((e1 - e0 + VEC - 1) / VEC);
-    for (uint32_t g = threadIdx.x; g < ngroups; g += kBlock) {
-      uint64_t e = e0 + static_cast<uint64_t>(g) * VEC;
-      uint32_t lo = 0, hi = span;  // off_tab[lo] <= e < off_tab[hi]
-      while (hi - lo > 1) {
-        const uint32_t mid = (lo + hi) >> 1;
-        if (off_tab[mid] <= e) lo = mid; else hi = mid;
-      }
-      if (e + VEC <= off_tab[lo + 1] && e + VEC <= e1) {
-        T* tensor = ptr_tab[lo] + (e - off_tab[lo]);
-        if (PACK) {
-          store_vec<T, NT>(reinterpret_cast<V*>(fused + e), *reinterpret_cast<const VU*>(tensor));
-        } else {
-          const V x = *reinterpret_cast<const V*>(fused + e);
-          *reinterpret_cast<VU*>(tensor) = apply_vec<T, OP>(x, x, divisor);
-        }
-      } else {
-        const uint64_t end = (e + VEC < e1) ? e + VEC : e1;
-        for (; e < end; e++) {
-          while (e >= off_tab[lo + 1]) lo++;
-          T* tensor = ptr_tab[lo] + (e - off_tab[lo]);
-          if (PACK) fused[e] = *tensor; else *tensor = apply_one<T, OP>(fused[e], T(), divisor);
-        }
-      }
-    }
+    if (PACK) multi_tensor_piece<T, true, kOpCopy, NT>(off_tab, ptr_tab, 0, span, e0, e1, nullptr, fused + e0, 0);
+    else multi_tensor_piece<T, false, OP, NT>(off_tab, ptr_tab, 0, span, e0, e1, fused + e0, nullptr, divisor);
     if (staged) __syncthreads();  // before the next tile overwrites the table
   }
 }
@@ -520,10 +662,8 @@ struct FusionSpanTable {
 template <typename T, bool GATHER, int NT, bool DIV>
 __global__ void __launch_bounds__(kBlock)
 fusion_span_kernel(const uint64_t* __restrict__ offsets, T* const* __restrict__ ptrs,
-                   const uint32_t* __restrict__ tile_first, const uint32_t* __restrict__ tile_last, uint32_t tile_lo,
-                   uint32_t tile_hi, uint64_t total, const FusionSpanTable tab) {
-  typedef typename VecOf<T>::type V;
-  typedef V VU __attribute__((aligned(sizeof(T))));
+                   const FusionTile* __restrict__ tiles, uint32_t tile_lo, uint32_t tile_hi, uint64_t total,
+                   const FusionSpanTable tab) {
   constexpr uint32_t VEC = 16 / sizeof(T);
   constexpr uint64_t kTileElems = static_cast<uint64_t>(kFusionTileVecs) * VEC;
   constexpr int SOP = DIV ? kOpDiv : kOpCopy;  // scatter
@@ -533,8 +673,9 @@ fusion_span_kernel(const uint64_t* __restrict__ offsets, T* const* __restrict__ 
   for (uint32_t tile = tile_lo + blockIdx.x; tile < tile_hi; tile += gridDim.x) {
     const uint64_t e0 = static_cast<uint64_t>(tile) * kTileElems;
     const uint64_t e1 = (e0 + kTileElems < total) ? e0 + kTileElems : total;
-    const uint32_t t0 = tile_first[tile];
-    const uint32_t t1 = tile_last[tile];
+    const FusionTile rec = load_tile(tiles, tile);
+    const uint32_t t0 = rec.first;
+    const uint32_t t1 = rec.last;
     const uint32_t tensors = t1 - t0 + 1;
     const uint64_t* off_tab = offsets + t0;
     T* const* ptr_tab = ptrs + t0;
@@ -561,10 +702,11 @@ fusion_span_kernel(const uint64_t* __restrict__ offsets, T* const* __restrict__ 
       T* lin_out = GATHER ? static_cast<T*>(span.out) + (b0 - span.begin) : nullptr;
       // the tensor holding b0 (uniform scalar walk over the tile's few tensors)
       uint32_t ta = 0;
-      while (off_tab[ta + 1] <= b0) ta++;
-      if (b1 <= off_tab[ta + 1]) {
+      if (tensors > 1)
+        while (off_tab[ta + 1] <= b0) ta++;
+      if (tensors == 1 || b1 <= off_tab[ta + 1]) {
         // the piece lies inside one tensor: the aligned-store span code of the step tables
-        T* tensor = ptr_tab[ta] + (b0 - off_tab[ta]);
+        T* tensor = tensors == 1 ? static_cast<T*>(rec.addr) + (b0 - e0) : ptr_tab[ta] + (b0 - off_tab[ta]);
         if (GATHER) {
           if (lin_in) row_tile<T, kOpAdd, 4, NT>(lin_out, lin_in, tensor, b1 - b0, 0, 1, 0);
           else row_tile<T, kOpCopy, 4, NT>(lin_out, tensor, nullptr, b1 - b0, 0, 1, 0);
@@ -574,36 +716,7 @@ fusion_span_kernel(const uint64_t* __restrict__ offsets, T* const* __restrict__ 
         continue;
       }
       // several tensors: every lane finds the tensor of its 16-byte group
-      const uint32_t ngroups = static_cast<uint32_t>((b1 - b0 + VEC - 1) / VEC);
-      for (uint32_t g = threadIdx.x; g < ngroups; g += kBlock) {
-        uint64_t e = b0 + static_cast<uint64_t>(g) * VEC;
-        uint32_t l = ta, h = tensors;  // off_tab[l] <= e < off_tab[h]
-        while (h - l > 1) {
-          const uint32_t mid = (l + h) >> 1;
-          if (off_tab[mid] <= e) l = mid; else h = mid;
-        }
-        const uint64_t i = e - b0;
-        if (e + VEC <= off_tab[l + 1] && e + VEC <= b1) {
-          VU* tv = reinterpret_cast<VU*>(ptr_tab[l] + (e - off_tab[l]));
-          if (GATHER) {
-            V x = *tv;
-            if (lin_in) x = apply_vec<T, kOpAdd>(*reinterpret_cast<const VU*>(lin_in + i), x, 0);
-            *reinterpret_cast<VU*>(lin_out + i) = x;
-          } else {
-            const V x = *reinterpret_cast<const VU*>(lin_in + i);
-            *tv = apply_vec<T, SOP>(x, x, tab.divisor);
-          }
-        } else {
-          const uint64_t end = (e + VEC < b1) ? e + VEC : b1;
-          for (; e < end; e++) {
-            while (e >= off_tab[l + 1]) l++;
-            T* tp = ptr_tab[l] + (e - off_tab[l]);
-            const uint64_t k = e - b0;
-            if (GATHER) lin_out[k] = lin_in ? apply_one<T, kOpAdd>(lin_in[k], *tp, 0) : *tp;
-            else *tp = apply_one<T, SOP>(lin_in[k], T(), tab.divisor);
-          }
-        }
-      }
+      multi_tensor_piece<T, GATHER, SOP, 0>(off_tab, ptr_tab, ta, tensors, b0, b1, lin_in, lin_out, tab.divisor);
     }
     if (staged) __syncthreads();  // before the next tile overwrites the table
   }
@@ -705,6 +818,7 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
     tab.divisor = divisor;
     tab.div_mask = 0;
     tab.tile_begin[0] = 0;
+    for (int k = 1; k <= kMaxRows; k++) tab.tile_begin[k] = 0xffffffffu;  // past the last row: after every tile
     uint64_t tiles = 0;
     uint64_t first_tiles = 0;
     bool any_add = false, uniform = true;
@@ -801,7 +915,7 @@ int steps_common(const void* input, void* buffer, const ring_step* steps, int n_
 }  // namespace
 
 // Host side of a fusion plan. The device table is one allocation:
-// offsets[m+1] | ptrs[m] | tile_first[ntiles] | tile_last[ntiles].
+// offsets[m+1] | ptrs[m] | padding to 16 bytes | tiles[ntiles].
 struct ring_fusion_plan {
   int dtype = 0;
   size_t esz = 0;
@@ -812,8 +926,7 @@ struct ring_fusion_plan {
   void* d_table = nullptr;
   uint64_t* d_offsets = nullptr;
   void** d_ptrs = nullptr;
-  uint32_t* d_tile_first = nullptr;
-  uint32_t* d_tile_last = nullptr;
+  FusionTile* d_tiles = nullptr;
 };
 
 namespace {
@@ -828,12 +941,11 @@ struct FusionView {
   uint64_t total;  // elements
   const uint64_t* offsets;
   void* const* ptrs;
-  const uint32_t* tile_first;
-  const uint32_t* tile_last;
+  const FusionTile* tiles;
 };
 
 inline FusionView view_of(const ring_fusion_plan* p) {
-  return FusionView{p->dtype, p->esz, p->ntiles, p->total, p->d_offsets, p->d_ptrs, p->d_tile_first, p->d_tile_last};
+  return FusionView{p->dtype, p->esz, p->ntiles, p->total, p->d_offsets, p->d_ptrs, p->d_tiles};
 }
 
 template <typename T, bool PACK, bool DIV>
@@ -848,8 +960,7 @@ int launch_fusion(const FusionView& p, void* fused, hipStream_t stream, int divi
   }
 #define RING_FUSION(N)                                                                                   \
   launch(fusion_kernel<T, PACK, N, DIV>, dim3(grid), dim3(kBlock), stream, static_cast<T*>(fused),       \
-         p.offsets, reinterpret_cast<T* const*>(p.ptrs), p.tile_first, p.tile_last, p.ntiles, p.total,   \
-         divisor)
+         p.offsets, reinterpret_cast<T* const*>(p.ptrs), p.tiles, p.ntiles, p.total, divisor)
   int nt = g_tuning.nt[PACK ? kRolePack : kRoleUnpack];
   if (nt < 0) nt = 2;
   switch (nt & 3) {
@@ -895,10 +1006,9 @@ constexpr uint32_t kStaticMaxTiles = 65536;   // 16 KiB tiles of the fused buffe
 struct StaticFusionTable {
   uint64_t offsets[kStaticMaxTensors + 1];
   void* ptrs[kStaticMaxTensors];
-  uint32_t tile_first[kStaticMaxTiles];
-  uint32_t tile_last[kStaticMaxTiles];
+  FusionTile tiles[kStaticMaxTiles];
 };
-// 540,680 bytes per GPU the library runs on, held until the process ends.
+// 1,064,968 bytes per GPU the library runs on, held until the process ends.
 static __device__ __align__(256) unsigned char scratch[sizeof(StaticFusionTable)];
 
 // `scratch` is a host-side stand-in in host code: the array's device address is
@@ -940,10 +1050,12 @@ __global__ void __launch_bounds__(kBlock) table_chunk_kernel(StaticFusionTable* 
   if (i == 0) tab->offsets[c.base + c.n] = c.end;
 }
 
-// tile_first / tile_last of every tile, as ring_fusion_plan_create computes them
-// on the host: the first and the last tensor that overlap the tile.
+// The record of every tile, as ring_fusion_plan_create computes it on the
+// host: the first and the last tensor that overlap the tile, and the tile's
+// address inside the tensor when that is one tensor.
 __global__ void __launch_bounds__(kBlock)
-table_tiles_kernel(StaticFusionTable* tab, uint32_t m, uint32_t ntiles, uint64_t tile_elems, uint64_t total) {
+table_tiles_kernel(StaticFusionTable* tab, uint32_t m, uint32_t ntiles, uint64_t tile_elems, uint64_t total,
+                   uint32_t esz) {
   const uint32_t tile = blockIdx.x * kBlock + threadIdx.x;
   if (tile >= ntiles) return;
   const uint64_t e0 = static_cast<uint64_t>(tile) * tile_elems;
@@ -954,13 +1066,17 @@ table_tiles_kernel(StaticFusionTable* tab, uint32_t m, uint32_t ntiles, uint64_t
     const uint32_t mid = (lo + hi) >> 1;
     if (tab->offsets[mid] <= e0) lo = mid; else hi = mid;
   }
-  tab->tile_first[tile] = lo;
+  const uint32_t first = lo;
   hi = m;  // offsets[lo] < e1 <= offsets[hi]
   while (hi - lo > 1) {
     const uint32_t mid = (lo + hi) >> 1;
     if (tab->offsets[mid] < e1) lo = mid; else hi = mid;
   }
-  tab->tile_last[tile] = lo;
+  FusionTile rec;
+  rec.first = first;
+  rec.last = lo;
+  rec.addr = first == lo ? static_cast<char*>(tab->ptrs[first]) + (e0 - tab->offsets[first]) * esz : nullptr;
+  tab->tiles[tile] = rec;
 }
 
 }  // namespace
@@ -1250,6 +1366,7 @@ int launch_fold(const HostFoldRow* rows, size_t n_rows, int divisor, int dtype, 
     tab.divisor = divisor;
     tab.div_mask = 0;
     tab.tile_begin[0] = 0;
+    for (int k = 1; k <= kMaxFoldRows; k++) tab.tile_begin[k] = 0xffffffffu;  // past the last row: after every tile
     uint64_t tiles = 0, first_tiles = 0;
     uint32_t ptrs = 0;
     bool uniform = true;
@@ -1381,26 +1498,27 @@ int ring_fusion_plan_create(const void* const* tensors, const size_t* counts, in
   p->total = total;
   if (total == 0) { *plan = p; return RING_OK; }
 
-  std::vector<uint32_t> first(p->ntiles), last(p->ntiles);
+  std::vector<FusionTile> tiles(p->ntiles);
   uint32_t t = 0;
   for (uint32_t tile = 0; tile < p->ntiles; tile++) {
     const uint64_t e0 = static_cast<uint64_t>(tile) * tile_elems;
     const uint64_t e1 = (e0 + tile_elems < total) ? e0 + tile_elems : total;
     while (offsets[t + 1] <= e0) t++;
-    first[tile] = t;
     uint32_t u = t;
     while (offsets[u + 1] < e1) u++;
-    last[tile] = u;
+    tiles[tile].first = t;
+    tiles[tile].last = u;
+    tiles[tile].addr = t == u ? static_cast<char*>(ptrs[t]) + (e0 - offsets[t]) * esz : nullptr;
   }
 
   const size_t b_off = offsets.size() * sizeof(uint64_t);
   const size_t b_ptr = ptrs.size() * sizeof(void*);
-  const size_t b_tile = static_cast<size_t>(p->ntiles) * sizeof(uint32_t);
-  std::vector<char> host(b_off + b_ptr + 2 * b_tile);
+  const size_t at_tiles = (b_off + b_ptr + 15) & ~static_cast<size_t>(15);
+  const size_t b_tile = static_cast<size_t>(p->ntiles) * sizeof(FusionTile);
+  std::vector<char> host(at_tiles + b_tile);
   memcpy(host.data(), offsets.data(), b_off);
   memcpy(host.data() + b_off, ptrs.data(), b_ptr);
-  memcpy(host.data() + b_off + b_ptr, first.data(), b_tile);
-  memcpy(host.data() + b_off + b_ptr + b_tile, last.data(), b_tile);
+  memcpy(host.data() + at_tiles, tiles.data(), b_tile);
 
   hipError_t e = hipGetDevice(&p->device);
   if (e == hipSuccess) e = hipMalloc(&p->d_table, host.size());
@@ -1413,8 +1531,7 @@ int ring_fusion_plan_create(const void* const* tensors, const size_t* counts, in
   char* base = static_cast<char*>(p->d_table);
   p->d_offsets = reinterpret_cast<uint64_t*>(base);
   p->d_ptrs = reinterpret_cast<void**>(base + b_off);
-  p->d_tile_first = reinterpret_cast<uint32_t*>(base + b_off + b_ptr);
-  p->d_tile_last = reinterpret_cast<uint32_t*>(base + b_off + b_ptr + b_tile);
+  p->d_tiles = reinterpret_cast<FusionTile*>(base + at_tiles);
   *plan = p;
   return RING_OK;
 }
@@ -1491,9 +1608,9 @@ int ring_fusion_run_static(int unpack, const void* const* tensors, const size_t*
     }
   }
   hipLaunchKernelGGL(table_tiles_kernel, dim3((ntiles + kBlock - 1) / kBlock), dim3(kBlock), 0, s, tab, m, ntiles,
-                     tile_elems, total);
+                     tile_elems, total, static_cast<uint32_t>(esz));
   RING_HIP(hipGetLastError());
-  const FusionView view{dtype, esz, ntiles, total, tab->offsets, tab->ptrs, tab->tile_first, tab->tile_last};
+  const FusionView view{dtype, esz, ntiles, total, tab->offsets, tab->ptrs, tab->tiles};
   return fusion_run(view, fused, stream, !unpack, divisor);
 }
 
@@ -1510,8 +1627,7 @@ int launch_fusion_spans(const ring_fusion_plan* p, const FusionSpanTable& tab, u
 #define RING_SPANS(N)                                                                                        \
   launch(fusion_span_kernel<T, GATHER, N, DIV>, dim3(grid), dim3(kBlock), stream,                            \
          static_cast<const uint64_t*>(p->d_offsets), reinterpret_cast<T* const*>(p->d_ptrs),                 \
-         static_cast<const uint32_t*>(p->d_tile_first), static_cast<const uint32_t*>(p->d_tile_last),        \
-         tile_lo, tile_hi, p->total, tab)
+         static_cast<const FusionTile*>(p->d_tiles), tile_lo, tile_hi, p->total, tab)
   switch (nt & 3) {
     case 0: RING_SPANS(0); break;
     case 1: RING_SPANS(1); break;

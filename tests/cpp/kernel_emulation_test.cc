@@ -1,0 +1,358 @@
+// The kernel library (csrc/ring_kernels.hip) compiled as plain C++ against the
+// CPU stand-in of the HIP runtime in tests/cpp/hip_cpu_shim and run under
+// AddressSanitizer and UBSan: every buffer is an exact-size heap block, so an
+// index one element outside what a kernel may touch, or a 16-byte access
+// through an aligned type at an address that is not, ends the run. Results
+// are compared with plain loops (one add / one divide per element).
+//
+// This checks indexing and alignment of the device code on the CPU. It says
+// nothing about speed and is not a CPU path of the product.
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <random>
+#include <vector>
+
+#include "ring_abi.h"
+
+#define CHECK(cond)                                                            \
+  do {                                                                         \
+    if (!(cond)) {                                                             \
+      fprintf(stderr, "%s:%d CHECK failed: %s\n", __FILE__, __LINE__, #cond);  \
+      exit(1);                                                                 \
+    }                                                                          \
+  } while (0)
+#define OK(call) CHECK((call) == RING_OK)
+
+namespace {
+
+std::mt19937_64 g_rng(12345);
+
+template <typename T> int code();
+template <> int code<float>() { return RING_F32; }
+template <> int code<int32_t>() { return RING_I32; }
+template <> int code<int64_t>() { return RING_I64; }
+
+template <typename T> T rnd() {
+  return static_cast<T>(static_cast<int64_t>(g_rng() % 2001) - 1000);
+}
+template <> float rnd<float>() {
+  return static_cast<float>(static_cast<int64_t>(g_rng() % 2000001) - 1000000) / 1024.0f;
+}
+
+template <typename T> T add(T a, T b) { return b + a; }
+template <typename T> T divide(T x, int n) {
+  const T q = x / n;
+  return q - ((x % n != 0) && (x < 0));
+}
+template <> float divide<float>(float x, int n) { return x / static_cast<float>(n); }
+
+// An exact-size heap block holding `count` elements that start `lead` elements
+// into it (lead breaks 16-byte alignment the way ragged segments do). The block
+// ends with the last element, so an overrun is caught; `lead` elements before
+// the data are poison that must survive.
+template <typename T>
+struct Buf {
+  T* base = nullptr;
+  T* p = nullptr;
+  size_t count = 0, lead = 0;
+  Buf(size_t n, size_t lead_elems, bool fill = true) : count(n), lead(lead_elems) {
+    base = static_cast<T*>(malloc((n + lead_elems) * sizeof(T) + (n + lead_elems == 0)));
+    p = base + lead_elems;
+    for (size_t i = 0; i < lead_elems; i++) memset(&base[i], 0x5a, sizeof(T));
+    for (size_t i = 0; i < n; i++) p[i] = fill ? rnd<T>() : T();
+  }
+  Buf(const Buf&) = delete;
+  Buf(Buf&& o) : base(o.base), p(o.p), count(o.count), lead(o.lead) { o.base = nullptr; }
+  ~Buf() { free(base); }
+  void check_lead() const {
+    for (size_t i = 0; i < lead * sizeof(T); i++) CHECK(reinterpret_cast<const unsigned char*>(base)[i] == 0x5a);
+  }
+};
+
+template <typename T>
+void expect_equal(const T* got, const std::vector<T>& want, const char* what) {
+  if (want.empty()) return;
+  if (memcmp(got, want.data(), want.size() * sizeof(T)) != 0) {
+    for (size_t i = 0; i < want.size(); i++)
+      if (memcmp(&got[i], &want[i], sizeof(T)) != 0) {
+        fprintf(stderr, "%s: element %zu of %zu differs\n", what, i, want.size());
+        exit(1);
+      }
+  }
+}
+
+const size_t kCounts[] = {0, 1, 2, 3, 4, 5, 7, 8, 15, 16, 17, 63, 255, 1023, 1024, 1025, 4095, 4096, 4097, 4099, 8191, 12289, 20011};
+
+template <typename T>
+void test_primitives() {
+  for (size_t count : kCounts)
+    for (size_t dl = 0; dl < 4; dl++)
+      for (size_t sl = 0; sl < 4; sl += (count > 5000 ? 3 : 1)) {
+        Buf<T> dst(count, dl), src(count, sl);
+        std::vector<T> want(count);
+        for (size_t i = 0; i < count; i++) want[i] = add(src.p[i], dst.p[i]);
+        OK(ring_accumulate(code<T>(), count ? dst.p : nullptr, count ? src.p : nullptr, count, nullptr));
+        expect_equal(dst.p, want, "accumulate");
+        dst.check_lead();
+        Buf<T> out(count, dl, false);
+        OK(ring_copy_bytes(count ? out.p : nullptr, count ? src.p : nullptr, count * sizeof(T), nullptr));
+        expect_equal(out.p, std::vector<T>(src.p, src.p + count), "copy");
+        out.check_lead();
+        for (int divisor : {1, 3, 8}) {
+          Buf<T> d(count, dl);
+          std::vector<T> w(count);
+          for (size_t i = 0; i < count; i++) w[i] = divide(d.p[i], divisor);
+          OK(ring_scale(code<T>(), count ? d.p : nullptr, count, divisor, nullptr));
+          expect_equal(d.p, w, "scale");
+        }
+      }
+}
+
+// Rows of mixed kinds and lengths in one call: in-place adds, out-of-place adds,
+// copies; some divided. More rows than one table carries.
+template <typename T>
+void test_mixed_rows(int n_rows, int divisor, size_t max_count) {
+  std::vector<Buf<T>> keep;
+  keep.reserve(3 * n_rows);
+  std::vector<ring_row> rows;
+  std::vector<unsigned char> flags;
+  std::vector<std::vector<T>> wants;
+  std::vector<T*> dsts;
+  for (int k = 0; k < n_rows; k++) {
+    const size_t c = k == 0 ? max_count : g_rng() % max_count;
+    const int kind = k % 3;
+    const bool flag = divisor > 0 && ((k * 7 + 1) % 2);
+    keep.emplace_back(c, k % 4);
+    T* a = keep.back().p;
+    T *b = nullptr, *dst;
+    if (kind == 0) {
+      keep.emplace_back(c, (k + 1) % 4);
+      b = dst = keep.back().p;
+    } else if (kind == 1) {
+      keep.emplace_back(c, (k + 2) % 4);
+      b = keep.back().p;
+      keep.emplace_back(c, (k + 3) % 4, false);
+      dst = keep.back().p;
+    } else {
+      keep.emplace_back(c, (k + 1) % 4, false);
+      dst = keep.back().p;
+    }
+    std::vector<T> w(c);
+    for (size_t i = 0; i < c; i++) {
+      T v = b ? add(a[i], b[i]) : a[i];
+      w[i] = flag ? divide(v, divisor) : v;
+    }
+    rows.push_back(ring_row{c ? dst : nullptr, c ? a : nullptr, c ? b : nullptr, c});
+    flags.push_back(flag);
+    wants.push_back(w);
+    dsts.push_back(dst);
+  }
+  OK(ring_apply_rows_avg(rows.data(), n_rows, flags.data(), divisor, code<T>(), nullptr));
+  for (int k = 0; k < n_rows; k++) expect_equal(dsts[k], wants[k], "mixed rows");
+  for (auto& b : keep) b.check_lead();
+}
+
+// The step tables of one rank of a ragged allreduce: equal tile counts per row (2-D grid).
+template <typename T>
+void test_step_tables(size_t count, int n) {
+  std::vector<size_t> sizes(n), starts(n);
+  OK(ring_segment_table(count, n, sizes.data(), starts.data()));
+  for (int r = 0; r < n; r += (n > 3 ? n - 1 : 1)) {
+    Buf<T> in(count, 0), out(count, 0, false);
+    std::vector<Buf<T>> staged;
+    std::vector<ring_step> rs, ag;
+    std::vector<T> want(in.p, in.p + count);
+    for (int i = 0; i < n - 1; i++) {
+      int snd, rcv;
+      OK(ring_schedule(RING_PHASE_REDUCE_SCATTER, n, r, i, &snd, &rcv));
+      staged.emplace_back(sizes[rcv], 0);
+      rs.push_back(ring_step{starts[rcv], staged.back().p, sizes[rcv]});
+      for (size_t e = 0; e < sizes[rcv]; e++) want[starts[rcv] + e] = add(staged.back().p[e], want[starts[rcv] + e]);
+    }
+    OK(ring_copy_bytes(out.p, in.p, count * sizeof(T), nullptr));
+    OK(ring_reduce_scatter_steps(out.p, rs.data(), n - 1, code<T>(), nullptr));
+    expect_equal(out.p, want, "reduce-scatter steps");
+    // the same with the copy folded in
+    Buf<T> out2(count, 0, false);
+    OK(ring_reduce_scatter_steps_from(in.p, out2.p, rs.data(), n - 1, code<T>(), nullptr));
+    for (int i = 0; i < n - 1; i++)
+      CHECK(memcmp(out2.p + rs[i].dst_offset, want.data() + rs[i].dst_offset, rs[i].count * sizeof(T)) == 0);
+    for (int i = 0; i < n - 1; i++) {
+      int snd, rcv;
+      OK(ring_schedule(RING_PHASE_ALLGATHER, n, r, i, &snd, &rcv));
+      staged.emplace_back(sizes[rcv], 0);
+      ag.push_back(ring_step{starts[rcv], staged.back().p, sizes[rcv]});
+      for (size_t e = 0; e < sizes[rcv]; e++) want[starts[rcv] + e] = staged.back().p[e];
+    }
+    OK(ring_allgather_steps(out.p, ag.data(), n - 1, code<T>(), nullptr));
+    expect_equal(out.p, want, "allgather steps");
+  }
+}
+
+template <typename T>
+void test_fold(int m, size_t count, int divisor) {
+  std::vector<Buf<T>> srcs;
+  std::vector<const void*> ptrs;
+  for (int k = 0; k < m; k++) {
+    srcs.emplace_back(count, k % 4);
+    ptrs.push_back(srcs.back().p);
+  }
+  Buf<T> dst(count, 1, false);
+  std::vector<T> want(count);
+  for (size_t i = 0; i < count; i++) {
+    T acc = srcs[0].p[i];
+    for (int k = 1; k < m; k++) acc = add(acc, srcs[k].p[i]);
+    want[i] = divisor ? divide(acc, divisor) : acc;
+  }
+  ring_fold_row row{dst.p, ptrs.data(), count};
+  Buf<T> csrc(count / 2 + 3, 2), cdst(count / 2 + 3, 3, false);
+  ring_row copy{cdst.p, csrc.p, nullptr, csrc.count};
+  OK(ring_fold_and_copy_rows(&row, 1, m, divisor, &copy, 1, code<T>(), nullptr));
+  expect_equal(dst.p, want, "fold");
+  expect_equal(cdst.p, std::vector<T>(csrc.p, csrc.p + csrc.count), "copy row beside a fold");
+  dst.check_lead();
+  cdst.check_lead();
+}
+
+// Pack, unpack (divided or not), gather and scatter over a tensor set, through a
+// plan and through the static device table.
+template <typename T>
+void test_fusion(const std::vector<size_t>& counts, int divisor, int n_ranks) {
+  std::vector<Buf<T>> tensors;
+  std::vector<const void*> ptrs;
+  size_t total = 0;
+  for (size_t j = 0; j < counts.size(); j++) {
+    tensors.emplace_back(counts[j], j % 4);
+    ptrs.push_back(counts[j] ? tensors.back().p : nullptr);
+    total += counts[j];
+  }
+  std::vector<T> packed;
+  for (auto& t : tensors) packed.insert(packed.end(), t.p, t.p + t.count);
+  ring_fusion_plan* plan = nullptr;
+  OK(ring_fusion_plan_create(ptrs.data(), counts.data(), static_cast<int>(counts.size()), code<T>(), &plan));
+  CHECK(ring_fusion_plan_elements(plan) == total);
+  // the fused buffer must be 16-byte aligned: malloc'd blocks are
+  Buf<T> fused(total, 0, false), fused2(total, 0, false);
+  OK(ring_fusion_pack(plan, total ? fused.p : nullptr, nullptr));
+  expect_equal(fused.p, packed, "pack");
+  OK(ring_fusion_run_static(0, ptrs.data(), counts.data(), static_cast<int>(counts.size()), code<T>(),
+                            total ? fused2.p : nullptr, 0, nullptr));
+  expect_equal(fused2.p, packed, "static pack");
+
+  // unpack into fresh tensors
+  auto fresh = [&](std::vector<Buf<T>>& out, std::vector<const void*>& out_ptrs) {
+    for (size_t j = 0; j < counts.size(); j++) {
+      out.emplace_back(counts[j], (j + 1) % 4, false);
+      out_ptrs.push_back(counts[j] ? out.back().p : nullptr);
+    }
+  };
+  auto check_tensors = [&](std::vector<Buf<T>>& out, const std::vector<T>& flat, const char* what) {
+    size_t at = 0;
+    for (auto& t : out) {
+      CHECK(memcmp(t.p, flat.data() + at, t.count * sizeof(T)) == 0 || (fprintf(stderr, "%s\n", what), false));
+      t.check_lead();
+      at += t.count;
+    }
+  };
+  std::vector<T> divided(packed);
+  if (divisor)
+    for (auto& v : divided) v = divide(v, divisor);
+  {
+    std::vector<Buf<T>> out;
+    std::vector<const void*> out_ptrs;
+    fresh(out, out_ptrs);
+    ring_fusion_plan* p2 = nullptr;
+    OK(ring_fusion_plan_create(out_ptrs.data(), counts.data(), static_cast<int>(counts.size()), code<T>(), &p2));
+    if (divisor) OK(ring_fusion_unpack_scaled(p2, fused.p, divisor, nullptr));
+    else OK(ring_fusion_unpack(p2, fused.p, nullptr));
+    check_tensors(out, divided, "unpack");
+    OK(ring_fusion_plan_destroy(p2));
+  }
+  {
+    std::vector<Buf<T>> out;
+    std::vector<const void*> out_ptrs;
+    fresh(out, out_ptrs);
+    OK(ring_fusion_run_static(1, out_ptrs.data(), counts.data(), static_cast<int>(counts.size()), code<T>(),
+                              total ? fused.p : nullptr, divisor, nullptr));
+    check_tensors(out, divided, "static unpack");
+  }
+  // gather: wire[seg] = tensors[seg] + incoming (one segment only packed); scatter the result back
+  if (total >= static_cast<size_t>(n_ranks)) {
+    std::vector<size_t> sizes(n_ranks), starts(n_ranks);
+    OK(ring_segment_table(total, n_ranks, sizes.data(), starts.data()));
+    Buf<T> wire(total, 0, false);
+    std::vector<Buf<T>> incoming;
+    std::vector<ring_fusion_span> spans;
+    std::vector<T> want(packed);
+    for (int g = 0; g < n_ranks; g++) {
+      incoming.emplace_back(sizes[g], g % 4);
+      const bool plain = g == 1;
+      spans.push_back(ring_fusion_span{starts[g], sizes[g], plain ? nullptr : incoming.back().p, wire.p + starts[g]});
+      if (!plain)
+        for (size_t e = 0; e < sizes[g]; e++) want[starts[g] + e] = add(incoming.back().p[e], want[starts[g] + e]);
+    }
+    OK(ring_fusion_gather(plan, spans.data(), n_ranks, nullptr));
+    expect_equal(wire.p, want, "gather");
+    std::vector<Buf<T>> out;
+    std::vector<const void*> out_ptrs;
+    fresh(out, out_ptrs);
+    ring_fusion_plan* p2 = nullptr;
+    OK(ring_fusion_plan_create(out_ptrs.data(), counts.data(), static_cast<int>(counts.size()), code<T>(), &p2));
+    std::vector<T> scattered(total);
+    for (int g = 0; g < n_ranks; g++) {
+      spans[g].incoming = incoming[g].p;
+      spans[g].out = nullptr;
+      for (size_t e = 0; e < sizes[g]; e++)
+        scattered[starts[g] + e] = divisor ? divide(incoming[g].p[e], divisor) : incoming[g].p[e];
+    }
+    OK(ring_fusion_scatter(p2, spans.data(), n_ranks, divisor, nullptr));
+    check_tensors(out, scattered, "scatter");
+    OK(ring_fusion_plan_destroy(p2));
+  }
+  OK(ring_fusion_plan_destroy(plan));
+  for (auto& t : tensors) t.check_lead();
+}
+
+template <typename T>
+void run_all(const char* name) {
+  printf("%s: primitives\n", name); fflush(stdout);
+  test_primitives<T>();
+  printf("%s: mixed rows\n", name); fflush(stdout);
+  test_mixed_rows<T>(1, 1, 20011);
+  test_mixed_rows<T>(4, 8, 9000);
+  test_mixed_rows<T>(7, 3, 9000);
+  test_mixed_rows<T>(70, 6, 5000);
+  test_mixed_rows<T>(9, 0, 12000);
+  printf("%s: step tables\n", name); fflush(stdout);
+  test_step_tables<T>(100003, 6);   // ragged: segments alternate between 0 and 8 / 4 bytes mod 16
+  test_step_tables<T>(65536, 8);
+  test_step_tables<T>(5, 8);        // fewer elements than ranks
+  test_step_tables<T>(40013, 3);
+  printf("%s: fold\n", name); fflush(stdout);
+  test_fold<T>(8, 10007, 0);
+  test_fold<T>(3, 4096, 3);
+  test_fold<T>(17, 777, 8);
+  printf("%s: fusion\n", name); fflush(stdout);
+  test_fusion<T>({5, 0, 4099, 1, 64, 0, 3}, 0, 3);
+  test_fusion<T>({20000, 64, 64, 36864, 64, 64, 9001, 2, 12288}, 8, 8);
+  std::vector<size_t> tiny(600);
+  for (auto& c : tiny) c = g_rng() % 40;
+  tiny[77] = 9000;
+  test_fusion<T>(tiny, 6, 4);
+  test_fusion<T>({17}, 3, 2);
+  test_fusion<T>({}, 0, 2);
+}
+
+}  // namespace
+
+int main() {
+  CHECK(ring_abi_version() == RING_ABI_VERSION);
+  run_all<float>("float32");
+  run_all<int32_t>("int32");
+  run_all<int64_t>("int64");
+  printf("kernel emulation: ok\n");
+  return 0;
+}

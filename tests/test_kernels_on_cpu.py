@@ -1,0 +1,101 @@
+"""Checks of the device code that need no GPU.
+
+1. The kernel library compiled as plain C++ against a CPU stand-in of the HIP
+   runtime (tests/cpp/hip_cpu_shim) and run under AddressSanitizer and UBSan
+   (tests/cpp/kernel_emulation_test.cc): indexing and alignment of every kernel
+   on exact-size buffers, results against plain loops.
+2. A scan of the gfx950 assembly hipcc emits for the kernels: a scalar select
+   (s_cselect) must take its condition code from a compare, not from whatever
+   arithmetic instruction ran last. hipcc 7.2 has produced that for a uniform
+   64-bit `min` ahead of a branch (v_cmp into vcc, branch on vcc, s_cselect on
+   a stale SCC): every lane of a partial tile then ran, out of bounds on the
+   GPU while the same source was correct on the CPU.
+"""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SRC = os.path.join(ROOT, "tensorflow-allreduce_amd", "csrc", "ring_kernels.hip")
+BUILD = os.path.join(ROOT, "tests", "cpp", "build")
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fno-fast-math", "-ffp-contract=off",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def _clang():
+    for exe in ("/opt/rocm/lib/llvm/bin/clang++", shutil.which("amdclang++"), shutil.which("clang++")):
+        if exe and os.path.exists(exe):
+            return exe
+    return None
+
+
+def test_kernels_under_sanitizers_on_the_cpu():
+    clang = _clang()
+    if clang is None:
+        pytest.skip("no clang++ (the kernels use clang vector extensions)")
+    os.makedirs(BUILD, exist_ok=True)
+    exe = os.path.join(BUILD, "kernel_emulation_test")
+    cmd = [clang, "-x", "c++", "-std=c++17", "-O0", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
+           "-fno-omit-frame-pointer", "-pthread",
+           "-I", os.path.join(ROOT, "tests", "cpp", "hip_cpu_shim"), "-I", os.path.join(ROOT, "include"),
+           "-o", exe, SRC, os.path.join(ROOT, "tests", "cpp", "kernel_emulation_test.cc")]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert res.returncode == 0, res.stdout[-4000:]
+    res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=900)
+    assert res.returncode == 0 and "kernel emulation: ok" in res.stdout, res.stdout[-4000:]
+
+
+SCC_WRITER = re.compile(r"^\s*(s_cmp|s_bitcmp|s_and_b|s_or_b|s_xor_b|s_andn2|s_orn2|s_add|s_sub|s_lshl|s_lshr|s_ashr|"
+                        r"s_bfe|s_not|s_min|s_max|s_abs|s_mul_hi|s_nand|s_nor|s_xnor|s_absdiff|s_wqm|s_quadmask|"
+                        r"s_bcnt|s_and_saveexec|s_or_saveexec)")
+
+
+def stale_selects(asm_text):
+    """s_cselect instructions whose SCC was last written by an add / subtract /
+    shift although a vector compare stands between the two: the select was
+    meant to follow that compare."""
+    lines = asm_text.split("\n")
+    found = []
+    for i, line in enumerate(lines):
+        if not re.match(r"^\s*s_cselect", line):
+            continue
+        j, vcmp = i - 1, False
+        while j >= 0 and not re.match(r"^\.LBB|^_Z", lines[j]) and not SCC_WRITER.match(lines[j]):
+            vcmp = vcmp or bool(re.match(r"^\s*v_cmp", lines[j]))
+            j -= 1
+        if j >= 0 and vcmp and re.match(r"^\s*(s_add|s_sub|s_lshl|s_lshr|s_mul)", lines[j]):
+            found.append((i + 1, line.strip(), lines[j].strip()))
+    return found
+
+
+def test_scan_recognises_the_pattern():
+    bad = """
+\ts_add_u32 s26, s40, s26
+\ts_addc_u32 s27, s41, s27
+\tv_cmp_lt_u64_e32 vcc, s[6:7], v[52:53]
+\ts_cbranch_vccz .LBB26_31
+\ts_cselect_b32 s34, s6, 0x400
+"""
+    good = """
+\tv_cmp_lt_u64_e32 vcc, s[16:17], v[2:3]
+\ts_and_b64 s[4:5], vcc, exec
+\ts_cselect_b32 s24, s16, s14
+"""
+    assert len(stale_selects(bad)) == 1
+    assert stale_selects(good) == []
+
+
+def test_no_scalar_select_on_a_stale_condition_code():
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc not found")
+    os.makedirs(BUILD, exist_ok=True)
+    asm = os.path.join(BUILD, "ring_kernels_gfx950.s")
+    cmd = [hipcc] + HIP_FLAGS + ["-I", os.path.join(ROOT, "include"), "-S", "--cuda-device-only", "-o", asm, SRC]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert res.returncode == 0, res.stdout[-4000:]
+    found = stale_selects(open(asm).read())
+    assert not found, "scalar selects on a stale condition code: %r" % (found[:5],)
