@@ -41,6 +41,8 @@ for p in (ROOT, os.path.join(ROOT, "tensorflow-allreduce_amd")):
 
 HBM_PEAK_GBS = 8000.0
 SAMPLE_EVERY = 16                   # steps between launches that carry timing events
+MIN_SAMPLES = 16                    # timed launches per phase, whatever --steps is
+COLD_SAMPLES = 32                   # timed launches of the cold-operand accumulate
 METRIC = "per-rank ring allreduce GB/s & % of HBM peak, 64 MiB fp32, N=8 virtual ranks"
 # committed rocprofv3 counter summaries holding a `traffic_bytes_per_launch:` line for a workload's dominant kernel
 TRAFFIC_PROFILES = {
@@ -161,6 +163,18 @@ class RingAllreduce(Workload):
         elif i == 1:
             A.check(R.ring_reduce_scatter_steps(s["out"].data_ptr(), s["rs_steps"][0], s["rs_steps"][1], self.code,
                                                 stream), "reduce-scatter")
+        else:
+            A.check(R.ring_allgather_steps(s["out"].data_ptr(), s["ag_steps"][0], s["ag_steps"][1], self.code,
+                                           stream), "allgather")
+
+    def launch_phase_fused(self, k, i, stream):
+        """The two launches of the step with the in->out copy folded in: the
+        accumulate out = in + received (every operand read for the first time),
+        then the allgather copies."""
+        s, A, R = self.sets[k % self.nsets], self.ring_abi, self.R
+        if i == 0:
+            A.check(R.ring_reduce_scatter_steps_from(s["inp"].data_ptr(), s["out"].data_ptr(), s["rs_steps"][0],
+                                                     s["rs_steps"][1], self.code, stream), "reduce-scatter from input")
         else:
             A.check(R.ring_allgather_steps(s["out"].data_ptr(), s["ag_steps"][0], s["ag_steps"][1], self.code,
                                            stream), "allgather")
@@ -306,9 +320,10 @@ class FusedResnet50(Workload):
             ag_seg = [ring_abi.schedule(1, 8, r, i)[1] for i in range(7)]
             rs = [torch.randn(sizes[g], device="cuda", generator=gen) * 1e-3 for g in rs_seg]
             ag = [torch.randn(sizes[g], device="cuda", generator=gen) * 1e-3 for g in ag_seg]
-            self.sets.append(dict(grads=grads, plan=plan, fused=fused, rs=rs, ag=ag,
+            self.sets.append(dict(grads=grads, plan=plan, fused=fused, rs=rs, ag=ag, r=r, rs_seg=rs_seg, ag_seg=ag_seg,
                                   rs_steps=ring_abi.make_steps([(starts[g], t.data_ptr(), sizes[g]) for g, t in zip(rs_seg, rs)]),
                                   ag_steps=ring_abi.make_steps([(starts[g], t.data_ptr(), sizes[g]) for g, t in zip(ag_seg, ag)])))
+        self.counts, self.sizes, self.starts = counts, sizes, starts
         seg = total // 8
         self.phases = (
             ("pack", total * 8, "fusion_kernel<unsigned int, pack> (161 tensors, 25,557,032 elements)"),
@@ -335,6 +350,45 @@ class FusedResnet50(Workload):
     def launch_step(self, k, stream, fused=False):
         for i in range(4):
             self.launch_phase(k, i, stream)
+
+    def owned_sum(self, s, packed):
+        """The finished owned segment: the rank's own values plus the partial sum
+        that arrives at the last reduce-scatter step."""
+        own = (s["r"] + 1) % 8
+        a, b = self.starts[own], self.starts[own] + self.sizes[own]
+        return packed[a:b] + s["rs"][6]
+
+    def check(self, k, stream=None):
+        """One more step of the timed path on set k from freshly drawn gradients
+        (a step overwrites its own inputs), compared tensor by tensor with what
+        the schedule says: the owned segment is the rank's values plus what it
+        received last (the fold of the staged copies in the direct form), every
+        other segment is the one received in the allgather phase, all divided
+        by 8 (one IEEE add and one IEEE divide per element, as torch computes
+        them)."""
+        s, torch = self.sets[k % self.nsets], self.torch
+        gen = torch.Generator(device="cuda").manual_seed(4242 + k)
+        for g in s["grads"]:
+            g.copy_(torch.randn(g.numel(), device="cuda", generator=gen) * 1e-3)
+        packed = torch.cat(s["grads"])
+        own = (s["r"] + 1) % 8
+        want = torch.empty_like(packed)
+        a, b = self.starts[own], self.starts[own] + self.sizes[own]
+        want[a:b] = self.owned_sum(s, packed)
+        for g, t in zip(s["ag_seg"], s["ag"]):
+            want[self.starts[g]:self.starts[g] + self.sizes[g]] = t
+        want = want / 8
+        torch.cuda.synchronize()
+        st = stream if stream is not None else self.ring_abi.stream_create()
+        self.launch_step(k, st)
+        self.ring_abi.stream_synchronize(st)
+        if stream is None:
+            self.ring_abi.stream_destroy(st)
+        at, ok = 0, True
+        for g in s["grads"]:
+            ok = ok and torch.equal(g, want[at:at + g.numel()])
+            at += g.numel()
+        return bool(ok)
 
 
 class FusedResnet50NoPasses(FusedResnet50):
@@ -422,6 +476,15 @@ class FusedResnet50NoPassesDirect(FusedResnet50NoPasses):
                             "3,194,629-element segment packed, folded in ring order with the 7 peers' staged raw "
                             "copies, and the 8 finished segments scattered into the tensors with the divide by 8; "
                             "3 launches per step")
+
+    def owned_sum(self, s, packed):
+        """The fold of the 7 staged raw copies and the rank's own copy, in ring order."""
+        own = s["own"]
+        a, b = self.starts[own], self.starts[own] + self.sizes[own]
+        acc = s["raw"][0].clone()
+        for t in s["raw"][1:]:
+            acc = t + acc
+        return packed[a:b] + acc
 
     def launch_phase(self, k, i, stream):
         s, A = self.sets[k % self.nsets], self.ring_abi
@@ -629,10 +692,11 @@ def main():
     nph = len(w.phases)
     # events are created before the timed region: creating them inside it would
     # let the queue drain and the sampled launches start on an idle GPU
-    sample_every = max(1, min(SAMPLE_EVERY, steps))      # a short run still times at least one step's launches
-    event_pool = [[ring_abi.event_create() for _ in range(2 * nph)] for _ in range(steps // sample_every + 1)]
+    sample_every = max(1, min(SAMPLE_EVERY, steps))
+    event_pool = [[ring_abi.event_create() for _ in range(2 * max(nph, 2))]
+                  for _ in range(steps // sample_every + 1 + MIN_SAMPLES + COLD_SAMPLES)]
 
-    def timed(nsteps, nwarm, fused=False, with_samples=False, hot=False):
+    def timed(nsteps, nwarm, fused=False, with_samples=False, hot=False, sample_every=sample_every):
         # hot: the same buffer set every step (what fits stays in the last-level
         # cache); otherwise the sets rotate and every step starts cold
         if hot:
@@ -675,6 +739,12 @@ def main():
                                      "launches_per_step": 2}}))
         return
     elapsed, samples = timed(steps, warmup, with_samples=True)
+    in_region = len(samples)
+    if in_region < MIN_SAMPLES:
+        # a short timed region carries too few timed launches: a sampling pass of its own, the same
+        # steps on the same rotating buffers, every 4th one timed; not part of the wall clock
+        _, more = timed((MIN_SAMPLES - in_region) * 4, 4, with_samples=True, sample_every=4)
+        samples += more
     if not w.check(steps - 1):
         sys.exit("bench.py: the output of the timed path is wrong; refusing to report a number")
     ms_per_step = elapsed / steps * 1e3
@@ -682,7 +752,32 @@ def main():
     phase_times = [[ring_abi.event_elapsed_us(e[2 * i], e[2 * i + 1]) for e in samples] for i in range(nph)]
     phase_us = [statistics.mean(t) for t in phase_times]
     dom = w.phases[w.dominant]
-    achieved = dom[1] / phase_us[w.dominant] / 1e3
+    dom_median = statistics.median(phase_times[w.dominant])
+    achieved = dom[1] / dom_median / 1e3
+
+    # the same accumulate on operands nothing has touched before it: the step with the in->out copy
+    # folded in (out = in + received), every 4th step timed
+    cold = None
+    if isinstance(w, RingAllreduce) and not isinstance(w, RingAllreducePerStep) and args.variant == "all":
+        for k in range(8):
+            w.launch_step(k, stream, True)
+        cold_events = []
+        for k in range(COLD_SAMPLES * 4):
+            if k % 4 == 2:
+                e = event_pool.pop()
+                for i in range(2):
+                    ring_abi.time_next_launch(e[2 * i], e[2 * i + 1])
+                    w.launch_phase_fused(k, i, stream)
+                cold_events.append(e)
+            else:
+                w.launch_step(k, stream, True)
+        ring_abi.stream_synchronize(stream)
+        cold_acc = [ring_abi.event_elapsed_us(e[0], e[1]) for e in cold_events]
+        cold_ag = [ring_abi.event_elapsed_us(e[2], e[3]) for e in cold_events]
+        cold = {"accumulate_median_us": round(statistics.median(cold_acc), 3),
+                "accumulate_mean_us": round(statistics.mean(cold_acc), 3),
+                "allgather_median_us": round(statistics.median(cold_ag), 3),
+                "launches_timed": len(cold_events)}
 
     result = {
         "metric": METRIC if args.workload == WORKLOADS[0] else "per-rank ring data path GB/s, " + w.name,
@@ -709,19 +804,28 @@ def main():
             "frac": round(achieved / HBM_PEAK_GBS, 4),
             "traffic": measured_traffic(args.workload),
             "algorithmic_bytes_per_launch": dom[1],
+            "median_launch_us": round(dom_median, 3),
             "avg_launch_us": round(phase_us[w.dominant], 3),
             "launches_timed": len(samples),
-            "note": "achieved = algorithmic bytes / launch duration; in an allreduce step the accumulate reads the "
-                    "buffer the in->out copy has just written, so part of its reads can come from the last-level "
-                    "cache instead of HBM",
+            "launches_timed_inside_the_wall_clock_region": in_region,
+            "note": "achieved = algorithmic bytes / median launch duration (HIP events carried in the dispatch). "
+                    "In the reference-shaped step the accumulate reads the buffer the in->out copy has just written "
+                    "with ordinary stores, so part of its reads are served by the last-level cache: `frac` is that "
+                    "LLC-assisted figure. `frac_cold` is the same kernel where no operand was touched before it (the "
+                    "step with the copy folded in, out = in + received): the HBM figure.",
         },
         "phases": {p[0]: {"us": round(t, 3), "median_us": round(statistics.median(phase_times[i]), 3),
                           "min_us": round(min(phase_times[i]), 3), "GBps": round(p[1] / t / 1e3, 1),
                           "bytes": p[1]}
                    for i, (p, t) in enumerate(zip(w.phases, phase_us))},
-        "phases_note": "HIP events carried by each launch of every %dth step of the timed region; us = mean"
-                       % sample_every,
+        "phases_note": "HIP events carried by each launch of every %dth step of the timed region%s; us = mean"
+                       % (sample_every, "" if in_region >= MIN_SAMPLES else
+                          " plus a sampling pass after it (every 4th step) to reach %d timed launches" % MIN_SAMPLES),
     }
+    if cold is not None:
+        result["roofline"]["frac_cold"] = round(dom[1] / cold["accumulate_median_us"] / 1e3 / HBM_PEAK_GBS, 4)
+        result["roofline"]["achieved_cold"] = round(dom[1] / cold["accumulate_median_us"] / 1e3, 1)
+        result["roofline"]["cold"] = cold
     # the same steps on ONE buffer set: at the headline size the working set fits the
     # last-level cache, so this is the cache-resident rate, not the HBM one
     if args.variant == "all":

@@ -100,6 +100,15 @@ int ring_time_next_launch(void* start_event, void* stop_event);
  * waits for that chunk only. */
 int ring_event_record(void* event, void* stream);
 int ring_event_synchronize(void* event);
+/* Ordering between two streams without the host: work enqueued on `stream`
+ * after this call starts only when the work `event` marked (ring_event_record
+ * on the producer's stream, or any hipEvent_t the embedding framework
+ * recorded there) has finished. This is how a producer hands a tensor to the
+ * ring's non-blocking stream: the reference defers its enqueue with a host
+ * callback on the producer's stream, stream->ThenDoHostCallback
+ * (mpi_ops.cc:1099-1105), so that the executor thread never blocks; here the
+ * dependency stays on the device and no thread blocks at all. */
+int ring_stream_wait_event(void* stream, void* event);
 
 /* ---- host-side tables (no GPU involved) ---------------------------------- */
 

@@ -1171,6 +1171,12 @@ int ring_event_synchronize(void* event) {
   return RING_OK;
 }
 
+int ring_stream_wait_event(void* stream, void* event) {
+  if (!event) return RING_ERR_ARGUMENT;
+  RING_HIP(hipStreamWaitEvent(static_cast<hipStream_t>(stream), static_cast<hipEvent_t>(event), 0));
+  return RING_OK;
+}
+
 int ring_time_next_launch(void* start_event, void* stop_event) {
   g_time_start = static_cast<hipEvent_t>(start_event);
   g_time_stop = static_cast<hipEvent_t>(stop_event);

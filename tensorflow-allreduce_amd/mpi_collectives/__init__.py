@@ -246,12 +246,20 @@ class Session:
         return base if k == 0 else "%s_%d" % (base, k)
 
     def _submit(self, r, op, node_name, inputs, device, divisor=0):
-        if any(t.is_cuda for t in inputs):
-            # the inputs' producers must have finished before the ring reads them (the
-            # reference defers the enqueue with a stream host callback, mpi_ops.cc:1099-1105)
+        if any(t.is_cuda for t in inputs) and not self.stream:
+            torch.cuda.current_stream(inputs[0].device).synchronize()      # before MPIInit there is no stream to order
+        elif any(t.is_cuda for t in inputs):
+            # The inputs' producers must have finished before the ring reads them. The
+            # reference defers the enqueue with a host callback on the producer's stream
+            # (mpi_ops.cc:1099-1105); here the world's stream waits, on the device, for an
+            # event recorded on the stream the inputs were produced on: torch's current
+            # stream (inputs produced on another stream must be ordered with it first).
+            # Nothing on the host blocks.
             producers = torch.cuda.current_stream(inputs[0].device)
             if not producers.query():
-                producers.synchronize()
+                ready = torch.cuda.Event()
+                ready.record(producers)
+                ring_abi.stream_wait_event(self.stream, ready.cuda_event)
         pending = _plugin.PendingOp(self._world, r, op, node_name, inputs, device, divisor)
         pending.rank = r
         pending.handle = pending.fail_handle = pending.on_done = pending.next_op = None

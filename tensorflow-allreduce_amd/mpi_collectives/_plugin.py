@@ -7,6 +7,7 @@ and `run_op` builds an op context, feeds torch tensors as inputs and lets the
 op allocate its outputs through a callback, as an OpKernelContext would.
 """
 import ctypes
+import itertools
 import os
 
 import torch
@@ -191,8 +192,10 @@ def infer_shape(op, shape):
 
 # One allocator callback serves every op: `user` carries the op's key. (Creating a
 # ctypes callback per op costs more than the rest of the submission.)
+# Ranks may be driven from one thread each: next() on an itertools.count is
+# atomic under the interpreter lock, a read-then-increment of a list cell is not.
 _live_ops = {}
-_next_key = [1]
+_next_key = itertools.count(1)
 _have_gpu = []      # torch.cuda.is_available(), asked once
 
 
@@ -234,8 +237,7 @@ class PendingOp:
         self._waited = False
         self._alloc_error = None
         self.op, self.node_name = op, node_name
-        self._key = _next_key[0]
-        _next_key[0] += 1
+        self._key = next(_next_key)
         _live_ops[self._key] = self
         h = ctypes.c_void_p()
         rc = L.mpic_context_create(world, rank, op.encode(), (node_name or "").encode(), device.encode(),

@@ -237,6 +237,22 @@ def test_prestaged_rank_matches_oracle_small(oracle, dtype):
                 G.assert_same_bits(G.host(got), outs[r], "prestaged n=%d r=%d flags=%d" % (n, r, flags))
 
 
+@pytest.mark.parametrize("dtype", [np.int32, np.int64])
+def test_prestaged_ragged_integers_n6_full_size(oracle, dtype):
+    """The ragged 10,000,019-element allreduce at N=6 through the per-rank
+    step-table path the benchmark times (mpic_ring_allreduce_prestaged,
+    batched, without and with the folded copy), peers' traffic from the
+    oracle's ring."""
+    n, count = 6, 10_000_019
+    ins = [np.random.default_rng(r).integers(-1000, 1001, count).astype(dtype) for r in range(n)]
+    outs, rs, ag = oracle.ring_allreduce(ins, tap=True)
+    assert np.array_equal(outs[0], sum(x.astype(np.int64) for x in ins).astype(dtype))
+    for r in (0, 3, 5):
+        for flags in (1, 3):
+            got = _prestaged(n, r, ins, rs, ag, flags, dtype)
+            G.assert_same_bits(G.host(got), outs[r], "prestaged ragged %s r=%d flags=%d" % (dtype.__name__, r, flags))
+
+
 def _tf_div(x, n):
     with np.errstate(all="ignore"):
         return (x / np.float32(n) if x.dtype == np.float32 else x // x.dtype.type(n)).astype(x.dtype)
@@ -480,6 +496,9 @@ def test_fused_allreduce_without_pack_and_unpack_passes(oracle, dtype):
     rng = np.random.default_rng(8)
     cases = [(8, [int(np.prod(s)) for s in G.resnet50_shapes()][:60], 8), (3, [5, 0, 4096, 1, 3, 8191, 2, 70_001], 0),
              (6, [int(c) for c in rng.integers(0, 50, 400)], 6), (1, [10, 20], 4), (4, [2], 0)]
+    if dtype == np.float32:
+        # the whole 161-tensor ResNet-50 set (25,557,032 elements) at N=8: the size the benchmark times
+        cases.append((8, [int(np.prod(s)) for s in G.resnet50_shapes()], 8))
     for n, counts, divisor in cases:
         total = sum(counts)
         grads = [[G.random_array(np.random.default_rng(100 * r + j), c, dtype) for j, c in enumerate(counts)]
@@ -863,3 +882,37 @@ def test_committed_known_answer_vectors_on_the_gpu(direct):
         for r in range(n):
             G.assert_same_bits(G.host(outs[r]), want,
                                "KAT %s n=%d count=%d rank %d direct=%d" % (case["dtype"], n, case["count"], r, direct))
+
+
+def test_inputs_still_being_produced_on_another_stream(oracle):
+    """The producer hands its tensor to the ring without the host waiting: the
+    inputs are written by a long chain of kernels on a side stream and the
+    allreduce is submitted while that chain is still running; the world's
+    stream waits for the producer on the device (ring_stream_wait_event), so
+    the ring reads the finished values."""
+    n, count, rounds = 4, 8 * 1024 * 1024, 60
+    base = make_inputs(n, count, np.float32, seed=5, wide=False)
+    side = torch.cuda.Stream()
+    dins = [cuda(x) for x in base]
+    torch.cuda.synchronize()
+    with mpi.Session(size=n) as session:
+        handles = []
+        with torch.cuda.stream(side):
+            for r in range(n):
+                for _ in range(rounds):
+                    dins[r].add_(1.0)                 # ~60 kernels per rank queued on the side stream
+                with session.as_rank(r):
+                    handles.append(mpi.allreduce(dins[r], average=False))
+            still_running = not side.query()
+        outs = session.run(handles)
+    torch.cuda.synchronize()
+    produced = [G.host(t) for t in dins]
+    for r in range(n):          # what the producers finally wrote, rounded as the GPU rounded it
+        acc = base[r].copy()
+        for _ in range(rounds):
+            acc = (acc + np.float32(1.0)).astype(np.float32)
+        G.assert_same_bits(produced[r], acc, "producer chain rank %d" % r)
+    want = oracle.ring_allreduce(produced)
+    for r in range(n):
+        G.assert_same_bits(G.host(outs[r]), want[r], "allreduce of inputs produced on a side stream, rank %d" % r)
+    assert still_running, "the producers had already finished at submission: the test did not exercise the hand-off"
