@@ -144,7 +144,18 @@ int mpic_context_destroy(mpic_context* ctx);
  * RingAllreduce (ring.h:136-228) for rank r of n whose incoming segments are
  * already in device memory. `flags`: bit 0 = batched, bit 1 = fuse the
  * in->out copy, bits 8-30 = divisor (0: none; see mpic_context_set_divisor).
- * Asynchronous on `stream`. `dtype` is an mpic_dtype. */
+ * Asynchronous on `stream`. `dtype` is an mpic_dtype.
+ *
+ * WHO DIVIDES, when a divisor is given, differs between the entry points, so
+ * the same staged traffic must not be fed to both kinds:
+ *   - mpic_ring_allreduce_prestaged and mpic_ring_allreduce_direct_prestaged:
+ *     THE OWNER DIVIDES. The rank divides only the segment it owns (in the
+ *     accumulate / fold that completes it) and copies ag_segments verbatim:
+ *     ag_segments must hold quotients, what peers that do the same send round.
+ *   - mpic_ring_allreduce_fused_prestaged: THE RECEIVER DIVIDES. Every finished
+ *     segment, ag_segments included, is divided on its way into the tensors:
+ *     ag_segments must hold undivided sums, and `wire` is left undivided (it is
+ *     what a ring of such ranks sends on). */
 int mpic_ring_allreduce_prestaged(int n, int r, int dtype, const void* input, void* output,
                                   size_t count, const void* const* rs_segments,
                                   const void* const* ag_segments, void* stream, int flags);
@@ -156,8 +167,9 @@ int mpic_ring_allreduce_prestaged(int n, int r, int dtype, const void* input, vo
  * (ring_fold_rows), into output[s]; ag_segments[i] is the finished segment
  * (r-i) mod n. The output is bit-identical to mpic_ring_allreduce_prestaged
  * fed with the ring's traffic. `flags`: bit 0 = fold and copies in one launch
- * (they write disjoint segments), bits 8-30 = divisor. No counterpart in the
- * reference. */
+ * (they write disjoint segments), bits 8-30 = divisor. At most 256 ranks (the
+ * copies one fold launch can address); more is refused with INVALID_ARGUMENT.
+ * No counterpart in the reference. */
 int mpic_ring_allreduce_direct_prestaged(int n, int r, int dtype, const void* input, void* output,
                                          size_t count, const void* const* peer_segments,
                                          const void* const* ag_segments, void* stream, int flags);
@@ -189,7 +201,8 @@ int mpic_ring_allgather_prestaged(int n, int r, int dtype, const void* input, co
  * the direct form (every segment folded by its owner in one launch, every
  * finished segment copied straight from its owner in a second; for the
  * allgather, every slice copied from its owner's input into every output in
- * one launch). */
+ * one launch). An allreduce of more than 256 ranks runs the lockstep ring
+ * whatever bit 2 says (a fold launch addresses at most 256 copies). */
 int mpic_ring_allreduce_all_ranks(int n, int dtype, const void* const* inputs,
                                   void* const* outputs, size_t count, void* stream, int flags);
 int mpic_ring_allgather_all_ranks(int n, int dtype, const void* const* inputs, const size_t* rows,

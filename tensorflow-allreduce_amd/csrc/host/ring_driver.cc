@@ -148,6 +148,9 @@ Status RingAllreduceDirectPrestaged(int n, int r, DataType dt, const void* input
   Status s = RingDataType(dt, &code);
   if (!s.ok()) return s;
   if (n < 1 || r < 0 || r >= n) return errors::InvalidArgument("rank out of range for the ring");
+  if (n > kMaxDirectRanks)
+    return errors::InvalidArgument("the direct form folds at most 256 copies of a segment; use the ring form for " +
+                                   std::to_string(n) + " ranks");
   if (opts.divisor < 0) return errors::InvalidArgument("negative divisor");
   const size_t esz = ring_dtype_size(code);
   if (count == 0) return Status::OK();
@@ -198,6 +201,9 @@ Status RingAllreduceFusedPrestaged(const ring_fusion_plan* plan, int n, int r, v
   RING_RETURN_IF_ERROR(ring_segment_table(count, n, sizes.data(), starts.data()), "ring_segment_table");
 
   const size_t own = static_cast<size_t>((r + 1) % n);
+  if (opts.direct && n > kMaxDirectRanks)
+    return errors::InvalidArgument("the direct form folds at most 256 copies of a segment; use the ring form for " +
+                                   std::to_string(n) + " ranks");
   if (opts.direct && n > 1) {
     // Direct form: rs_recv[k] is rank (own+k)'s raw copy of the owned segment
     // (packed layout). The rank packs its own copy of that segment into the
@@ -322,7 +328,9 @@ Status RingAllreduceAllRanks(int n, DataType dt, const void* const* inputs, void
   for (int r = 0; r < n; r++)
     if (!inputs[r] || !outputs[r]) return errors::InvalidArgument("null tensor with a non-zero element count");
 
-  if (opts.direct) {
+  // The fold kernel carries at most kMaxDirectRanks source pointers per launch; a
+  // larger ring runs the lockstep form below, which handles any n (ring.h:136-228).
+  if (opts.direct && n <= kMaxDirectRanks) {
     // One launch: the owner of every segment folds the n copies in ring order.
     std::vector<std::vector<const void*>> srcs(static_cast<size_t>(n));
     std::vector<ring_fold_row> folds;

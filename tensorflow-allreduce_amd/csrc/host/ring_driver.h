@@ -15,6 +15,10 @@
 
 namespace mpic {
 
+// Most copies of a segment one fold launch can address (ring_fold_rows): the
+// direct forms are limited to rings of this many ranks.
+constexpr int kMaxDirectRanks = 256;
+
 struct RingOptions {
   // One launch per ring phase (all n-1 steps of a rank) instead of one per
   // step. Steps of one rank write disjoint segments, so the order inside a

@@ -249,22 +249,24 @@ class PendingOp:
         if rc != OK:
             raise error_for(rc, "could not create a context for %s (rank %d)" % (op, rank))
         self._h = h.value
-        for t in inputs:
-            host = not t.is_cuda
-            if t.dtype not in TORCH2DT:
-                dt = 0                                  # DT_INVALID: rejected by the op
-            else:
-                dt = TORCH2DT[t.dtype]
-            dims = (ctypes.c_int64 * max(t.dim(), 1))(*t.shape)
-            rc = L.mpic_context_add_input(self._h, dt, t.dim(), dims, t.data_ptr() if t.numel() else None, int(host))
-            if rc != OK:
-                raise error_for(rc, "bad input for %s" % op)
-        if divisor:
-            rc = L.mpic_context_set_divisor(self._h, divisor)
-            if rc != OK:
-                raise error_for(rc, "bad divisor for %s" % op)
-        rc = L.mpic_context_compute(self._h)       # outputs are allocated during this call
-        _live_ops.pop(self._key, None)
+        try:
+            for t in inputs:
+                host = not t.is_cuda
+                if t.dtype not in TORCH2DT:
+                    dt = 0                                  # DT_INVALID: rejected by the op
+                else:
+                    dt = TORCH2DT[t.dtype]
+                dims = (ctypes.c_int64 * max(t.dim(), 1))(*t.shape)
+                rc = L.mpic_context_add_input(self._h, dt, t.dim(), dims, t.data_ptr() if t.numel() else None, int(host))
+                if rc != OK:
+                    raise error_for(rc, "bad input for %s" % op)
+            if divisor:
+                rc = L.mpic_context_set_divisor(self._h, divisor)
+                if rc != OK:
+                    raise error_for(rc, "bad divisor for %s" % op)
+            rc = L.mpic_context_compute(self._h)       # outputs are allocated during this call
+        finally:
+            _live_ops.pop(self._key, None)             # the allocator is only called from compute
         if rc != OK:
             raise error_for(rc, "could not start %s" % op)
 

@@ -916,3 +916,20 @@ def test_inputs_still_being_produced_on_another_stream(oracle):
     for r in range(n):
         G.assert_same_bits(G.host(outs[r]), want[r], "allreduce of inputs produced on a side stream, rank %d" % r)
     assert still_running, "the producers had already finished at submission: the test did not exercise the hand-off"
+
+
+def test_more_ranks_than_the_direct_form_addresses(oracle):
+    """A session of 257 virtual ranks with its default options: the direct form
+    folds at most 256 copies of a segment, so the allreduce runs as the
+    lockstep ring, which takes any number of ranks, with the same result."""
+    n, count = 257, 1000
+    ins = make_inputs(n, count, np.float32, seed=9, wide=False)
+    want = oracle.ring_allreduce_lockstep(ins)[0]
+    with mpi.Session(size=n) as session:
+        handles = []
+        for r in range(n):
+            with session.as_rank(r):
+                handles.append(mpi.allreduce(cuda(ins[r]), average=False))
+        outs = session.run(handles)
+    for r in (0, 1, 128, 256):
+        G.assert_same_bits(G.host(outs[r]), want, "257 ranks, rank %d" % r)

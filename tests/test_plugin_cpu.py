@@ -422,3 +422,45 @@ def test_bench_refuses_more_than_one_gpu_and_needs_a_gpu():
         one = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--no-cpu-baseline"], capture_output=True,
                              text=True)
         assert one.returncode != 0 and "no GPU is visible" in one.stderr and not one.stdout.strip()
+
+
+def test_ops_submitted_from_many_threads_keep_their_own_outputs():
+    """One thread per virtual rank, all submitting at once (the mode
+    Session.as_rank supports for ranks driven like separate processes): every op
+    instance must receive exactly the outputs its own allocator callback made.
+    The scalar ops run on the CPU device, so this needs no GPU."""
+    import threading
+    n, rounds = 16, 200
+    with mpi.Session(size=n, device="CPU") as session:
+        errors, start = [], threading.Barrier(n)
+
+        def drive(r):
+            try:
+                start.wait()
+                for _ in range(rounds):
+                    with session.as_rank(r):
+                        p = session._submit(r, 'MPIRank', session._node_name(r, 'MPIRank', None), [], "CPU")
+                        outs = p.wait()
+                        assert len(outs) == 1, "rank %d: %d outputs" % (r, len(outs))
+                        assert int(outs[0].item()) == r, "rank %d got the output of rank %d" % (r, int(outs[0].item()))
+            except Exception as e:                      # reported from the main thread
+                errors.append(e)
+
+        threads = [threading.Thread(target=drive, args=(r,)) for r in range(n)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        assert not errors, errors[:3]
+    assert not _plugin._live_ops
+
+
+def test_direct_form_refuses_more_ranks_than_a_fold_addresses():
+    """The direct pre-staged forms fold at most 256 copies of a segment: a larger
+    ring is refused with a message that says so, before anything is launched."""
+    L = _plugin.load_library()
+    n = 257
+    ptrs = (ctypes.c_void_p * n)(*([0x1000] * n))
+    rc = L.mpic_ring_allreduce_direct_prestaged(n, 0, _plugin.DT_FLOAT, 0x1000, 0x2000, 1000, ptrs, ptrs, None, 1)
+    assert rc == _plugin.INVALID_ARGUMENT
+    assert b"at most 256 copies" in L.mpic_last_error()
