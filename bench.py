@@ -567,6 +567,11 @@ def make_workload(name):
                              "%s ring allreduce of a ragged 10,000,019-element tensor, N=6 virtual ranks (segments "
                              "1,666,670 x5 + 1,666,669): copy + 5 accumulates + 5 copies per step, peers pre-staged, "
                              "12 buffer sets rotated" % {"i32": "int32", "i64": "int64"}[dt])
+    if name == "allreduce_f32_1MiB_n8":
+        return RingAllreduce(name, "f32", 262_144, 8, 8,
+                             "float32 ring allreduce of one 262,144-element (1 MiB) tensor, N=8 virtual ranks: a "
+                             "launch-bound step (copy + 7 accumulates + 7 copies on 128 KiB segments, 3 launches), "
+                             "peers pre-staged, buffers rotated over 8 virtual ranks")
     if name == "allreduce_f32_1GiB_n64":
         return RingAllreduce(name, "f32", 268_435_456, 64, 2,
                              "float32 ring allreduce of one 268,435,456-element (1 GiB) tensor, N=64 virtual ranks: "
@@ -585,6 +590,7 @@ def make_workload(name):
 
 WORKLOADS = ("allreduce_f32_64MiB_n8", "allreduce_i32_10000019_n6", "allreduce_i64_10000019_n6",
              "fused_resnet50_n8", "allgather_f32_n16", "allreduce_f32_1GiB_n64", "allreduce_f32_64MiB_n8_per_step",
+             "allreduce_f32_1MiB_n8",
              "allreduce_f32_64MiB_n8_direct", "fused_resnet50_n8_no_passes",
              "fused_resnet50_n8_no_passes_direct")
 
@@ -662,6 +668,9 @@ def main():
                          "the in->out copy folded into the accumulate, and the hot (one buffer set) rate. "
                          "reference / fused: that path alone, for kernel traces (kernel names do not tell the two "
                          "accumulates apart, and the extras would mix into the per-kernel averages)")
+    ap.add_argument("--recorded", type=int, default=0, metavar="STEPS",
+                    help="allreduce workloads: record this many consecutive steps as ONE HIP graph (ring_graph_*) and "
+                         "time its replays; for launch-bound sizes. --steps is rounded down to a multiple of it")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="launch option of the kernel library (unroll, blocks_per_cu, nontemporal[_copy|_accumulate|"
                          "_allgather|_pack|_unpack]), "
@@ -685,6 +694,11 @@ def main():
         ring_abi.set_option(name, int(value))
         options[name] = int(value)
     w = make_workload(args.workload)
+    if args.recorded and (not isinstance(w, RingAllreduce) or isinstance(w, RingAllreducePerStep)):
+        sys.exit("bench.py: --recorded applies to the allreduce workloads")
+    if options.get("dry_launch"):
+        # the kernels return at entry: what is timed is the launches themselves, and there is no output to check
+        w.check = lambda k: True
     torch.cuda.synchronize()
 
     # the dedicated stream every ring kernel is launched on (CudaStreamForMPI)
@@ -725,6 +739,41 @@ def main():
         torch.cuda.synchronize()
         return time.perf_counter() - t0, samples
 
+    if args.recorded:
+        # `recorded` consecutive steps (rotating over the buffer sets) as one HIP graph, replayed
+        fused = args.variant == "fused"
+        L = ring_abi.lib()
+        for k in range(8):
+            w.launch_step(k, stream, fused)
+        ring_abi.stream_synchronize(stream)
+        ring_abi.check(L.ring_graph_begin_capture(stream), "ring_graph_begin_capture")
+        for k in range(args.recorded):
+            w.launch_step(k, stream, fused)
+        graph = ctypes.c_void_p()
+        ring_abi.check(L.ring_graph_end_capture(stream, ctypes.byref(graph)), "ring_graph_end_capture")
+        replays = max(steps // args.recorded, 1)
+        for _ in range(max(warmup // args.recorded, 1)):
+            ring_abi.check(L.ring_graph_launch(graph, stream), "ring_graph_launch")
+        ring_abi.stream_synchronize(stream)
+        t0 = time.perf_counter()
+        for _ in range(replays):
+            ring_abi.check(L.ring_graph_launch(graph, stream), "ring_graph_launch")
+        ring_abi.stream_synchronize(stream)
+        elapsed = time.perf_counter() - t0
+        ok = all(w.check(k) for k in range(min(args.recorded, w.nsets)))
+        ring_abi.check(L.ring_graph_destroy(graph), "ring_graph_destroy")
+        if not ok:
+            sys.exit("bench.py: the output of the replayed graph is wrong; refusing to report a number")
+        nsteps = replays * args.recorded
+        nbytes = w.fused_bytes if fused else w.bytes_per_step
+        print(json.dumps({"metric": "per-rank ring data path GB/s, %s, %d steps per replayed HIP graph" % (w.name, args.recorded),
+                          "value": round(nbytes * nsteps / elapsed / 1e9, 1), "unit": "GB/s", "n_gpus": 1,
+                          "steps": nsteps, "warmup": warmup, "ms_per_step": round(elapsed / nsteps * 1e3, 5),
+                          "higher_is_better": True, "dtype": w.dtype, "data": "synthetic",
+                          "config": {"workload": w.description, "name": w.name, "bytes_per_step": nbytes,
+                                     "launches_per_step": 2 if fused else 3,
+                                     "steps_per_recorded_hip_graph": args.recorded}}))
+        return
     if args.variant == "fused":
         if not isinstance(w, RingAllreduce) or isinstance(w, RingAllreducePerStep):
             sys.exit("bench.py: --variant fused applies to the allreduce workloads")
@@ -793,7 +842,8 @@ def main():
         "dtype": w.dtype,
         "data": "synthetic",
         "config": {"workload": w.description, "name": w.name, "bytes_per_step": w.bytes_per_step,
-                   "launches_per_step": w.step_launches or nph, **({"launch_options": options} if options else {})},
+                   "launches_per_step": w.step_launches or nph, **({"launch_options": options} if options else {}),
+                   **({"steps_per_recorded_hip_graph": args.recorded} if args.recorded else {})},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "roofline": {
             "bound": "hbm",
@@ -849,7 +899,7 @@ def main():
                 "note": "same allreduce with the in->out copy folded into the accumulate (out = in + received; the "
                         "segment that is only sent is written by the first allgather step and never copied)",
             }
-        if args.variant == "all" and w.name == WORKLOADS[0]:
+        if args.variant == "all" and w.name == WORKLOADS[0] and not options.get("dry_launch"):
             # the same allreduce in the direct form (one fold pass over pushed copies + copies, one launch)
             d = make_workload("allreduce_f32_64MiB_n8_direct")
             for k in range(50):

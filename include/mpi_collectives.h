@@ -140,11 +140,39 @@ int mpic_context_output(const mpic_context* ctx, int index, int* dtype, int* ndi
                         int64_t* dims /* room for 8 */, void** data);
 int mpic_context_destroy(mpic_context* ctx);
 
+/* k MPIAllreduce nodes of one rank in one call: what k rounds of
+ * mpic_context_create / add_input / set_divisor / compute do, for callers that
+ * reduce a whole gradient set per step (the reference's DistributedOptimizer
+ * issues one MPIAllreduce per gradient, __init__.py:195-205, and so does this
+ * call: every tensor is its own node, negotiated and validated under its own
+ * node name, and the coordinator's tensor fusion groups them as it would
+ * group separately submitted ones). Tensor j has element type dtypes[j]
+ * (mpic_dtype) and ndims[j] dimensions, taken in order from `dims` (all
+ * tensors' dimensions back to back); inputs[j] is its device memory and
+ * outputs[j] device memory of the same size for the result (the caller
+ * supplies it where a single node asks its allocator). divisor as
+ * mpic_context_set_divisor, for every node. contexts[j] receives node j's
+ * context: wait / message / destroy as for any other. */
+int mpic_allreduce_batch(mpic_world* world, int rank, int k, const char* const* node_names, const int* dtypes,
+                         const int* ndims, const int64_t* dims, const void* const* inputs, void* const* outputs,
+                         int divisor, mpic_context** contexts);
+/* Waits for every context of the array (NULL entries are skipped); codes[j],
+ * when given, receives node j's status code. With destroy_ok, contexts that
+ * ended OK are destroyed and their entries set to NULL, so that what is left
+ * are the failed ones, whose message can still be read. Returns the first
+ * status that is not OK. */
+int mpic_context_wait_batch(mpic_context** contexts, int k, int destroy_ok, int* codes);
+
 /* ---- the ring driver, callable without the op layer ------------------------
  * RingAllreduce (ring.h:136-228) for rank r of n whose incoming segments are
  * already in device memory. `flags`: bit 0 = batched, bit 1 = fuse the
  * in->out copy, bits 8-30 = divisor (0: none; see mpic_context_set_divisor).
  * Asynchronous on `stream`. `dtype` is an mpic_dtype.
+ * The calls only enqueue kernels, so any number of them can be recorded
+ * between ring_graph_begin_capture and ring_graph_end_capture (ring_abi.h)
+ * and replayed with ring_graph_launch: for launch-bound tensors (up to a few
+ * MiB) a graph of 8 or more steps costs half of what the same steps cost
+ * launched one by one; a graph of a single step costs more than the step.
  *
  * WHO DIVIDES, when a divisor is given, differs between the entry points, so
  * the same staged traffic must not be fed to both kinds:

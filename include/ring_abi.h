@@ -21,7 +21,8 @@
  *   - a whole phase of the ring (all n-1 accumulates, all n-1 allgather
  *     copies) can be issued as ONE launch from a step table, because the
  *     steps of one rank write disjoint segments (ring.h:183-205, :211-225);
- *   - nothing allocates device memory unless its name says "create".
+ *   - nothing allocates device memory unless its name says "create" (host
+ *     memory: a table of more than 64 rows takes a heap buffer for the call).
  *
  * Conventions: `count` is in elements, `bytes` in bytes; a count of 0 with
  * null pointers is valid and does nothing (an empty tensor reaches the
@@ -77,8 +78,10 @@ size_t ring_dtype_size(int dtype);
  * bit 1 = non-temporal loads, -1 = the default: 3, except ordinary stores
  * where the next kernel reads the output (copy, pack, fold), ordinary loads
  * for a source several rows share (broadcast), and loads by size for the copy.
- * "nontemporal" sets all seven. No counterpart in the reference, whose
- * launch shape is the constant <<<32, 256>>> (ring.cu.cc:64). */
+ * "nontemporal" sets all seven. "dry_launch" = 1 makes the step-table / copy /
+ * accumulate kernels return at entry: what is then timed is what a launch of
+ * that grid costs by itself. No counterpart in the reference, whose launch
+ * shape is the constant <<<32, 256>>> (ring.cu.cc:64). */
 int ring_set_option(const char* name, int value);
 
 /* Timing of single launches, for benchmarks (no counterpart in the
@@ -109,6 +112,20 @@ int ring_event_synchronize(void* event);
  * (mpi_ops.cc:1099-1105), so that the executor thread never blocks; here the
  * dependency stays on the device and no thread blocks at all. */
 int ring_stream_wait_event(void* stream, void* event);
+
+/* HIP graphs, for steps that are bound by launches rather than bytes (a small
+ * tensor's allreduce is 2-3 launches of 4-5 us each whatever it moves): what
+ * is enqueued on `stream` between begin and end is recorded instead of run,
+ * end returns an executable graph, and launch replays it as one submission.
+ * A replay has a fixed cost of its own (about 12 us), so it pays from about
+ * four steps per graph: the allreduces of a whole gradient set, say. The
+ * recorded launches carry their kernel arguments, pointers included, so a
+ * graph is only good for the buffers it was recorded with. `stream` must not
+ * be the null stream. No counterpart in the reference. */
+int ring_graph_begin_capture(void* stream);
+int ring_graph_end_capture(void* stream, void** graph_exec);
+int ring_graph_launch(void* graph_exec, void* stream);
+int ring_graph_destroy(void* graph_exec);
 
 /* ---- host-side tables (no GPU involved) ---------------------------------- */
 

@@ -15,6 +15,10 @@
   tests/cpp/build/ring_gpu_test
                           a C++ test of the C ABI (test code, linked with the
                           oracle), run on the GPU by tests/test_gpu_cpp.py.
+  tests/cpp/build/binding_gpu_test
+                          integration/ring_hip_binding.cc (the file that takes
+                          the place of the reference's ring.cu.cc) with its
+                          test, run on the GPU by tests/test_gpu_cpp.py.
 
 hipcc cross-compiles for gfx950 without a GPU. Packed FP32 instructions are
 disabled for all device code.
@@ -105,12 +109,21 @@ def build_cpp_gpu_test(verbose=True):
          "-L", LIB_DIR, "-lmpi_collectives", "-lring_hip", "-L", os.path.join(rocm, "lib"), "-lamdhip64",
          "-Wl,-rpath," + LIB_DIR, "-Wl,-rpath," + os.path.join(rocm, "lib")],
     ]
+    # the reference-side binding (integration/ring_hip_binding.cc, the file that takes the place of
+    # the reference's ring.cu.cc) and its test: the seam called as ring.h calls it
+    binding_exe = os.path.join(out_dir, "binding_gpu_test")
+    cmds.append([cxx, "-O2", "-std=c++17", "-Wall", "-Wextra", "-pthread", "-D__HIP_PLATFORM_AMD__",
+                 "-I", os.path.join(rocm, "include"), "-I", os.path.join(ROOT, "include"), "-I", os.path.join(ROOT, "oracle"),
+                 "-o", binding_exe, os.path.join(ROOT, "tests", "cpp", "binding_gpu_test.cc"),
+                 os.path.join(HERE, "integration", "ring_hip_binding.cc"), obj,
+                 "-L", LIB_DIR, "-lring_hip", "-L", os.path.join(rocm, "lib"), "-lamdhip64",
+                 "-Wl,-rpath," + LIB_DIR, "-Wl,-rpath," + os.path.join(rocm, "lib")])
     for cmd in cmds:
         if verbose:
             print(" ".join(cmd), flush=True)
         res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
         if res.returncode != 0:
-            raise RuntimeError("building the C++ GPU test failed:\n" + res.stdout)
+            raise RuntimeError("building the C++ GPU tests failed:\n" + res.stdout)
     return exe
 
 

@@ -1042,6 +1042,57 @@ int mpic_context_destroy(mpic_context* c) {
   return MPIC_OK;
 }
 
+// ---- many MPIAllreduce nodes in one call ------------------------------------------------
+
+int mpic_allreduce_batch(mpic_world* world, int rank, int k, const char* const* node_names, const int* dtypes,
+                         const int* ndims, const int64_t* dims, const void* const* inputs, void* const* outputs,
+                         int divisor, mpic_context** contexts) {
+  if (!world || k < 0 || divisor < 0) return MPIC_INVALID_ARGUMENT;
+  if (k > 0 && (!node_names || !dtypes || !ndims || !inputs || !outputs || !contexts)) return MPIC_INVALID_ARGUMENT;
+  if (rank < 0 || rank >= world->size || (world->real_rank >= 0 && rank != world->real_rank))
+    return MPIC_INVALID_ARGUMENT;
+  const mpic::KernelDef* kdef = OpRegistry::Global()->FindKernel("MPIAllreduce", "GPU");
+  if (!kdef) return MPIC_NOT_FOUND;
+  size_t at = 0;
+  for (int j = 0; j < k; j++) {
+    if (ndims[j] < 0 || ndims[j] > 8 || (ndims[j] > 0 && !dims) || !node_names[j]) {
+      for (int i = 0; i < j; i++) { delete contexts[i]; contexts[i] = nullptr; }
+      return MPIC_INVALID_ARGUMENT;
+    }
+    mpic_context* c = new mpic_context();
+    mpic::OpKernelConstruction construction(*node_names[j] ? node_names[j] : "MPIAllreduce");
+    c->kernel.reset(kdef->factory(&construction));
+    void* out = outputs[j];
+    // the node's one output has the input's shape: the caller supplies its memory
+    mpic::OutputAllocator allocator = [out](mpic::DataType, const mpic::TensorShape&, bool) -> void* { return out; };
+    c->ctx.reset(new mpic::OpKernelContext(world, rank, true, allocator));
+    std::vector<int64_t> d(dims + at, dims + at + ndims[j]);
+    at += static_cast<size_t>(ndims[j]);
+    c->ctx->AddInput(mpic::Tensor(static_cast<mpic::DataType>(dtypes[j]), mpic::TensorShape(d),
+                                  const_cast<void*>(inputs[j]), false));
+    c->ctx->set_fused_divisor(divisor);
+    contexts[j] = c;
+  }
+  for (int j = 0; j < k; j++) mpic_context_compute(contexts[j]);
+  return MPIC_OK;
+}
+
+int mpic_context_wait_batch(mpic_context** contexts, int k, int destroy_ok, int* codes) {
+  if (k < 0 || (k > 0 && !contexts)) return MPIC_INVALID_ARGUMENT;
+  int first = MPIC_OK;
+  for (int j = 0; j < k; j++) {
+    if (!contexts[j]) continue;
+    const int code = mpic_context_wait(contexts[j]);
+    if (codes) codes[j] = code;
+    if (code != MPIC_OK && first == MPIC_OK) first = code;
+    if (code == MPIC_OK && destroy_ok) {
+      mpic_context_destroy(contexts[j]);
+      contexts[j] = nullptr;
+    }
+  }
+  return first;
+}
+
 // ---- the ring driver without the op layer --------------------------------------------
 
 int mpic_ring_allreduce_prestaged(int n, int r, int dtype, const void* input, void* output, size_t count,

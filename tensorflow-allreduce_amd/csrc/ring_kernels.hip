@@ -159,6 +159,7 @@ struct Row {
 };
 struct RowTable {
   int n_rows;
+  int dry;  // measurement only: every workgroup returns at once
   // > 0: every row has this many tiles and the grid is (tiles, rows), so a
   // workgroup reads its row straight from blockIdx.y (the n-1 near-equal
   // segments of an allreduce). 0: rows differ; the grid is 1-D over all tiles
@@ -319,6 +320,7 @@ __device__ __forceinline__ int row_of_tile(const uint32_t* begin, int n_rows, ui
 
 template <typename T, int MODE, int UNROLL, int NT>
 __global__ void __launch_bounds__(kBlock) rows_kernel(const RowTable tab) {
+  if (tab.dry) return;
   if (tab.uniform_tiles) {
     const Row r = tab.row[blockIdx.y];  // one scalar load, no search
     const bool divide = MODE == kAvg && ((tab.div_mask >> blockIdx.y) & 1u);
@@ -742,6 +744,7 @@ struct Tuning {
   // the ordinary policy so that it is fetched from HBM once
   int nt[kRoles] = {-1, 3, 3, 2, 3, 2, 1};
   int blocks_per_cu = 0;   // 0: one workgroup per tile; >0: persistent grid of CUs x this
+  int dry_launch = 0;      // measurement only: the step-table kernels return at entry (what a launch of that grid costs)
 };
 Tuning g_tuning;
 
@@ -787,6 +790,20 @@ int launch_rows_typed(const RowTable& tab, dim3 grid, hipStream_t stream, int nt
   return RING_OK;
 }
 
+// Room for n items: on the stack up to N of them (the rows of one launch), on the heap beyond.
+template <typename T, size_t N>
+struct RowBuffer {
+  T stack[N];
+  std::vector<T> heap;
+  T* data;
+  explicit RowBuffer(size_t n) : data(stack) {
+    if (n > N) {
+      heap.resize(n);
+      data = heap.data();
+    }
+  }
+};
+
 struct HostRow {
   void* dst;
   const void* a;
@@ -815,6 +832,7 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
   while (i < n_rows) {
     RowTable tab;
     tab.n_rows = 0;
+    tab.dry = g_tuning.dry_launch;
     tab.divisor = divisor;
     tab.div_mask = 0;
     tab.tile_begin[0] = 0;
@@ -896,8 +914,8 @@ int steps_common(const void* input, void* buffer, const ring_step* steps, int n_
   if (n_steps == 0) return RING_OK;
   if (!steps) return RING_ERR_ARGUMENT;
   const size_t esz = dtype_size(dtype);
-  std::vector<HostRow> rows;
-  rows.reserve(static_cast<size_t>(n_steps));
+  RowBuffer<HostRow, kMaxRows> rows(static_cast<size_t>(n_steps));
+  size_t n_rows = 0;
   for (int i = 0; i < n_steps; i++) {
     if (steps[i].count == 0) continue;
     if (!buffer || !steps[i].src || (kind == kStepAddFrom && !input)) return RING_ERR_ARGUMENT;
@@ -906,9 +924,9 @@ int steps_common(const void* input, void* buffer, const ring_step* steps, int n_
     if ((reinterpret_cast<uintptr_t>(d) | reinterpret_cast<uintptr_t>(steps[i].src) |
          reinterpret_cast<uintptr_t>(local)) & (esz - 1))
       return RING_ERR_ARGUMENT;
-    rows.push_back(HostRow{d, steps[i].src, kind == kStepCopy ? nullptr : local, steps[i].count, false});
+    rows.data[n_rows++] = HostRow{d, steps[i].src, kind == kStepCopy ? nullptr : local, steps[i].count, false};
   }
-  return launch_rows(rows.data(), rows.size(), esz, dtype == RING_F32, static_cast<hipStream_t>(stream),
+  return launch_rows(rows.data, n_rows, esz, dtype == RING_F32, static_cast<hipStream_t>(stream),
                      kind == kStepCopy ? kRoleAllgather : kRoleAccumulate);
 }
 
@@ -1129,6 +1147,8 @@ int ring_set_option(const char* name, int value) {
   } else if (!strcmp(name, "blocks_per_cu")) {
     if (value < 0 || value > 64) return RING_ERR_ARGUMENT;
     g_tuning.blocks_per_cu = value;
+  } else if (!strcmp(name, "dry_launch")) {
+    g_tuning.dry_launch = value != 0;
   } else {
     return RING_ERR_ARGUMENT;
   }
@@ -1168,6 +1188,37 @@ int ring_event_record(void* event, void* stream) {
 int ring_event_synchronize(void* event) {
   if (!event) return RING_ERR_ARGUMENT;
   RING_HIP(hipEventSynchronize(static_cast<hipEvent_t>(event)));
+  return RING_OK;
+}
+
+int ring_graph_begin_capture(void* stream) {
+  if (!stream) return RING_ERR_ARGUMENT;  // the null stream cannot be captured
+  RING_HIP(hipStreamBeginCapture(static_cast<hipStream_t>(stream), hipStreamCaptureModeThreadLocal));
+  return RING_OK;
+}
+
+int ring_graph_end_capture(void* stream, void** graph_exec) {
+  if (!stream || !graph_exec) return RING_ERR_ARGUMENT;
+  *graph_exec = nullptr;
+  hipGraph_t graph = nullptr;
+  RING_HIP(hipStreamEndCapture(static_cast<hipStream_t>(stream), &graph));
+  hipGraphExec_t exec = nullptr;
+  const hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(graph);
+  if (e != hipSuccess) return hip_fail(e);
+  *graph_exec = exec;
+  return RING_OK;
+}
+
+int ring_graph_launch(void* graph_exec, void* stream) {
+  if (!graph_exec) return RING_ERR_ARGUMENT;
+  RING_HIP(hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec), static_cast<hipStream_t>(stream)));
+  return RING_OK;
+}
+
+int ring_graph_destroy(void* graph_exec) {
+  if (!graph_exec) return RING_OK;
+  RING_HIP(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec)));
   return RING_OK;
 }
 
@@ -1314,33 +1365,28 @@ int ring_apply_rows_avg(const ring_row* rows, int n_rows, const unsigned char* d
   if (n_rows == 0) return RING_OK;
   if (!rows) return RING_ERR_ARGUMENT;
   const size_t esz = dtype_size(dtype);
-  std::vector<HostRow> host;
-  host.reserve(static_cast<size_t>(n_rows));
+  RowBuffer<HostRow, kMaxRows> host(static_cast<size_t>(n_rows));
+  size_t n_host = 0;
+  bool copies_only = true;
   for (int i = 0; i < n_rows; i++) {
     if (rows[i].count == 0) continue;
     if (!rows[i].dst || !rows[i].a) return RING_ERR_ARGUMENT;
     if ((reinterpret_cast<uintptr_t>(rows[i].dst) | reinterpret_cast<uintptr_t>(rows[i].a) |
          reinterpret_cast<uintptr_t>(rows[i].b)) & (esz - 1))
       return RING_ERR_ARGUMENT;
-    host.push_back(HostRow{rows[i].dst, rows[i].a, rows[i].b, rows[i].count,
-                           divisor > 0 && (!divide || divide[i] != 0)});
+    host.data[n_host++] = HostRow{rows[i].dst, rows[i].a, rows[i].b, rows[i].count,
+                                  divisor > 0 && (!divide || divide[i] != 0)};
+    copies_only = copies_only && rows[i].b == nullptr;
   }
   // copy rows that share a source: one buffer handed to several destinations
   Role role = kRoleAccumulate;
-  if (divisor == 0 && host.size() > 1) {
-    std::vector<const void*> sources;
-    bool copies_only = true;
-    for (const HostRow& r : host) {
-      copies_only = copies_only && r.b == nullptr;
-      sources.push_back(r.a);
-    }
-    if (copies_only) {
-      std::sort(sources.begin(), sources.end());
-      if (std::adjacent_find(sources.begin(), sources.end()) != sources.end()) role = kRoleBroadcast;
-    }
+  if (divisor == 0 && n_host > 1 && copies_only) {
+    RowBuffer<const void*, kMaxRows> sources(n_host);
+    for (size_t k = 0; k < n_host; k++) sources.data[k] = host.data[k].a;
+    std::sort(sources.data, sources.data + n_host);
+    if (std::adjacent_find(sources.data, sources.data + n_host) != sources.data + n_host) role = kRoleBroadcast;
   }
-  return launch_rows(host.data(), host.size(), esz, dtype == RING_F32, static_cast<hipStream_t>(stream), role,
-                     divisor);
+  return launch_rows(host.data, n_host, esz, dtype == RING_F32, static_cast<hipStream_t>(stream), role, divisor);
 }
 
 int ring_allgather_steps(void* buffer, const ring_step* steps, int n_steps, int dtype, void* stream) {
@@ -1449,15 +1495,15 @@ int ring_fold_and_copy_rows(const ring_fold_row* fold_rows, int n_fold, int m, i
   if (n_fold < 0 || n_copy < 0 || divisor < 0) return RING_ERR_ARGUMENT;
   if (n_fold > 0 && (m < 1 || m > kMaxFoldPtrs || !fold_rows)) return RING_ERR_ARGUMENT;
   if (n_copy > 0 && !copy_rows) return RING_ERR_ARGUMENT;
-  std::vector<HostFoldRow> host;
-  host.reserve(static_cast<size_t>(n_fold) + static_cast<size_t>(n_copy));
+  RowBuffer<HostFoldRow, kMaxRows> host(static_cast<size_t>(n_fold) + static_cast<size_t>(n_copy));
+  size_t n_host = 0;
   for (int i = 0; i < n_fold; i++)
-    host.push_back(HostFoldRow{fold_rows[i].dst, fold_rows[i].srcs, m, fold_rows[i].count, true});
+    host.data[n_host++] = HostFoldRow{fold_rows[i].dst, fold_rows[i].srcs, m, fold_rows[i].count, true};
   for (int i = 0; i < n_copy; i++) {
     if (copy_rows[i].b != nullptr) return RING_ERR_ARGUMENT;  // copy rows only
-    host.push_back(HostFoldRow{copy_rows[i].dst, &copy_rows[i].a, 1, copy_rows[i].count, false});
+    host.data[n_host++] = HostFoldRow{copy_rows[i].dst, &copy_rows[i].a, 1, copy_rows[i].count, false};
   }
-  return launch_fold(host.data(), host.size(), divisor, dtype, static_cast<hipStream_t>(stream));
+  return launch_fold(host.data, n_host, divisor, dtype, static_cast<hipStream_t>(stream));
 }
 
 int ring_scale(int dtype, void* data, size_t count, int divisor, void* stream) {

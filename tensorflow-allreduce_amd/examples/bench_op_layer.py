@@ -6,8 +6,10 @@ float32) with mpi.allreduce, as the reference's DistributedOptimizer does
 (tensorflow/contrib/mpi_collectives/__init__.py:195-205: one MPIAllreduce per
 gradient), and session.run() completes them. Compared: one ring per gradient
 (the reference's behaviour; there each op also waits for a coordinator tick of
-at least 1 ms, mpi_ops.cc:635), the coordinator's tensor fusion, and a single
-pre-packed tensor. All ranks live on one GPU, so a ring step is one launch for
+at least 1 ms, mpi_ops.cc:635), the coordinator's tensor fusion, each of them
+also with the gradients of a rank submitted by one call (mpi.allreduce_batch,
+what DistributedOptimizer.compute_gradients does), and a single pre-packed
+tensor. All ranks live on one GPU, so a ring step is one launch for
 all ranks.
 
     python tensorflow-allreduce_amd/examples/bench_op_layer.py [--ranks 8] [--steps 5]
@@ -37,13 +39,16 @@ def resnet50_counts():
     return counts + [2048 * 1000, 1000]
 
 
-def step(session, grads, average=True):
+def step(session, grads, average=True, batch=False):
     """One step: every rank submits all its gradients, then the session runs."""
     t0 = time.perf_counter()
     handles = []
     for r, gs in enumerate(grads):
         with session.as_rank(r):
-            handles.append([mpi.allreduce(g, average=average) for g in gs])
+            if batch:
+                handles.append(mpi.allreduce_batch(gs, average=average))
+            else:
+                handles.append([mpi.allreduce(g, average=average) for g in gs])
     t1 = time.perf_counter()
     session.run()
     torch.cuda.synchronize()
@@ -62,13 +67,15 @@ def main():
     grads = [[torch.randn(c, device="cuda", generator=gen) * 1e-3 for c in counts] for _ in range(args.ranks)]
     packed = [[torch.cat(gs)] for gs in grads]
     print("%d ranks x %d gradients, %d float32 (%.1f MB) per rank" % (args.ranks, len(counts), total, total * 4 / 1e6))
-    for label, kwargs, data in (
-            ("one ring per gradient", {}, grads),
-            ("coordinator fusion (128 MiB buffer per rank)", {"fusion_threshold": 128 << 20}, grads),
-            ("one pre-packed tensor", {}, packed)):
+    for label, kwargs, data, batch in (
+            ("one ring per gradient", {}, grads, False),
+            ("one ring per gradient, submitted as a batch", {}, grads, True),
+            ("coordinator fusion (128 MiB buffer per rank)", {"fusion_threshold": 128 << 20}, grads, False),
+            ("coordinator fusion, submitted as a batch", {"fusion_threshold": 128 << 20}, grads, True),
+            ("one pre-packed tensor", {}, packed, False)):
         with mpi.Session(size=args.ranks, **kwargs) as session:
-            step(session, data)                                  # warm-up (fusion plans, allocator)
-            submit, run = zip(*[step(session, data) for _ in range(args.steps)])
+            step(session, data, batch=batch)                     # warm-up (fusion plans, allocator)
+            submit, run = zip(*[step(session, data, batch=batch) for _ in range(args.steps)])
         print("%-46s submit %7.2f ms   run %7.2f ms   total %7.2f ms per step"
               % (label, 1e3 * min(submit), 1e3 * min(run), 1e3 * min(s + r for s, r in zip(submit, run))))
 

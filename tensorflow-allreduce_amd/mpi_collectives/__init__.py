@@ -29,6 +29,7 @@ collectives complete at once.
 @@Session
 @@DistributedOptimizer
 @@allreduce
+@@allreduce_batch
 @@allgather
 """
 import contextlib
@@ -245,23 +246,60 @@ class Session:
             self._counters[(r, base)] = k + 1
         return base if k == 0 else "%s_%d" % (base, k)
 
+    def _order_after_producers(self, inputs):
+        """The inputs' producers must have finished before the ring reads them. The
+        reference defers the enqueue with a host callback on the producer's stream
+        (mpi_ops.cc:1099-1105); here the world's stream waits, on the device, for an
+        event recorded on the stream the inputs were produced on: torch's current
+        stream (inputs produced on another stream must be ordered with it first).
+        Nothing on the host blocks."""
+        if not any(t.is_cuda for t in inputs):
+            return
+        producers = torch.cuda.current_stream(inputs[0].device)
+        if not self.stream:
+            producers.synchronize()      # before MPIInit there is no stream to order
+        elif not producers.query():
+            ready = torch.cuda.Event()
+            ready.record(producers)
+            ring_abi.stream_wait_event(self.stream, ready.cuda_event)
+
+    def _submit_batch(self, r, names, tensors, divisor=0):
+        """One MPIAllreduce node per tensor, all filed with one call into the plugin.
+        Returns one handle per tensor."""
+        inputs = [t.contiguous() for t in tensors]
+        self._order_after_producers(inputs)
+        node_names = [self._node_name(r, 'MPIAllreduce', name) for name in names]
+        # the outputs: one allocation per element type, cut into the tensors' shapes
+        outputs = [None] * len(inputs)
+        by_dtype = {}
+        for j, t in enumerate(inputs):
+            by_dtype.setdefault((t.dtype, t.device), []).append(j)
+        for (dtype, device), idx in by_dtype.items():
+            flat = torch.empty(sum(inputs[j].numel() for j in idx), dtype=dtype, device=device)
+            for j, piece in zip(idx, flat.split([inputs[j].numel() for j in idx])):
+                outputs[j] = piece.view(inputs[j].shape)
+        batch = _plugin.PendingBatch(self._world, r, node_names, inputs, outputs, divisor)
+        batch.rank = r
+        batch.next_op = batch.on_done = batch.handle = batch.fail_handle = None
+        batch.lock = threading.Lock()
+        batch.completed = False
+        batch.error = None
+        batch.handles = []
+        for _ in inputs:
+            h = PendingTensor(self)
+            h._first_op = batch
+            batch.handles.append(h)
+        with self._lock:
+            for name in node_names:
+                self._submitted.setdefault(name, set()).add(r)
+            self._pending.append(batch)
+        return batch.handles
+
     def _submit(self, r, op, node_name, inputs, device, divisor=0):
-        if any(t.is_cuda for t in inputs) and not self.stream:
-            torch.cuda.current_stream(inputs[0].device).synchronize()      # before MPIInit there is no stream to order
-        elif any(t.is_cuda for t in inputs):
-            # The inputs' producers must have finished before the ring reads them. The
-            # reference defers the enqueue with a host callback on the producer's stream
-            # (mpi_ops.cc:1099-1105); here the world's stream waits, on the device, for an
-            # event recorded on the stream the inputs were produced on: torch's current
-            # stream (inputs produced on another stream must be ordered with it first).
-            # Nothing on the host blocks.
-            producers = torch.cuda.current_stream(inputs[0].device)
-            if not producers.query():
-                ready = torch.cuda.Event()
-                ready.record(producers)
-                ring_abi.stream_wait_event(self.stream, ready.cuda_event)
+        self._order_after_producers(inputs)
         pending = _plugin.PendingOp(self._world, r, op, node_name, inputs, device, divisor)
         pending.rank = r
+        pending.node_names = [node_name]
         pending.handle = pending.fail_handle = pending.on_done = pending.next_op = None
         pending.lock = threading.Lock()
         pending.completed = False
@@ -321,26 +359,38 @@ class Session:
         with p.lock:
             if p.completed:
                 return p.error
-            try:
-                outputs = p.wait()
-                if p.on_done:
-                    p.on_done(outputs)
-                if p.handle is not None:
-                    p.handle._set(value=outputs[0])
-            except OpError as e:
-                p.error = e
-                for h in (p.handle, p.fail_handle):
-                    if h is not None:
+            if isinstance(p, _plugin.PendingBatch):
+                for h, out, e in zip(p.handles, p.outputs, p.wait()):
+                    if e is None:
+                        h._set(value=out)
+                    else:
                         h._set(error=e)
+                        p.error = p.error or e
+            else:
+                try:
+                    outputs = p.wait()
+                    if p.on_done:
+                        p.on_done(outputs)
+                    if p.handle is not None:
+                        p.handle._set(value=outputs[0])
+                except OpError as e:
+                    p.error = e
+                    for h in (p.handle, p.fail_handle):
+                        if h is not None:
+                            h._set(error=e)
             p.completed = True
+        return self._retire(p)
+
+    def _retire(self, p):
         with self._lock:
             if p in self._pending:
                 self._pending.remove(p)
-            ranks = self._submitted.get(p.node_name)
-            if ranks is not None:
-                ranks.discard(p.rank)
-                if not ranks:
-                    self._submitted.pop(p.node_name, None)
+            for name in p.node_names:
+                ranks = self._submitted.get(name)
+                if ranks is not None:
+                    ranks.discard(p.rank)
+                    if not ranks:
+                        self._submitted.pop(name, None)
         return p.error
 
     def _check_all_ranks_submitted(self, batch):
@@ -349,11 +399,12 @@ class Session:
         for p in batch:
             if p.completed:
                 continue
-            ranks = self._submitted.get(p.node_name, set())
-            if len(ranks) != self.size:
-                raise FailedPreconditionError(
-                    "collective %r was submitted by ranks %s of %d; every rank must submit it "
-                    "before the session runs" % (p.node_name, sorted(ranks), self.size))
+            for name in p.node_names:
+                ranks = self._submitted.get(name, set())
+                if len(ranks) != self.size:
+                    raise FailedPreconditionError(
+                        "collective %r was submitted by ranks %s of %d; every rank must submit it "
+                        "before the session runs" % (name, sorted(ranks), self.size))
 
     def _drain(self):
         first_error = None
@@ -439,6 +490,23 @@ def allreduce(tensor, average=True):
     return _div(session, summed_tensor) if average and not fold else summed_tensor
 
 
+def allreduce_batch(tensors, average=True):
+    """allreduce() of every dense tensor of a list; returns the list of results
+    (not in the reference, whose callers loop over allreduce).
+
+    Each tensor is its own MPIAllreduce node, named, negotiated, validated and
+    (with a fusion threshold) grouped exactly as the same calls made one by one
+    would be; what changes is the cost of making them: one call into the plugin
+    for all of them instead of several per tensor. This is what
+    DistributedOptimizer.compute_gradients uses for the gradient set of a step."""
+    session, r = mpi_ops._current()
+    tensors = list(tensors)
+    if session._immediate or not tensors:
+        return [allreduce(t, average=average) for t in tensors]      # pre-staged peers / one rank: nothing to batch
+    fold = session.size if average else 0
+    return session._submit_batch(r, [None] * len(tensors), tensors, fold)
+
+
 class DistributedOptimizer:
     """An optimizer that wraps a torch.optim.Optimizer, using an MPI allreduce
     to average gradient values before applying gradients to model weights
@@ -481,6 +549,10 @@ class DistributedOptimizer:
         params = [p for p in self._params(var_list) if p.grad is not None]
         if self._fusion:
             return self._compute_fused(params)
+        # one MPIAllreduce per gradient, as in the reference (__init__.py:195-205); the dense ones
+        # are submitted together
+        dense = [p for p in params if not p.grad.is_sparse]
+        reduced = dict(zip((id(p) for p in dense), allreduce_batch([p.grad for p in dense])))
         out = []
         for p in params:
             g = p.grad
@@ -489,7 +561,7 @@ class DistributedOptimizer:
                 slices = IndexedSlices(g.values().contiguous(), g.indices()[0].contiguous(), dense_shape=g.shape)
                 out.append((allreduce(slices), p))
             else:
-                out.append((allreduce(g.contiguous()), p))
+                out.append((reduced[id(p)], p))
         return out
 
     def _compute_fused(self, params):

@@ -31,6 +31,7 @@ EXPORTS = (
     "mpic_world_flush", "mpic_stage_peers",
     "mpic_context_create", "mpic_context_add_input", "mpic_context_set_divisor", "mpic_context_compute", "mpic_context_wait",
     "mpic_context_message", "mpic_context_num_outputs", "mpic_context_output", "mpic_context_destroy",
+    "mpic_allreduce_batch", "mpic_context_wait_batch",
     "mpic_ring_allreduce_prestaged", "mpic_ring_allreduce_direct_prestaged", "mpic_ring_allreduce_fused_prestaged",
     "mpic_ring_allgather_prestaged", "mpic_ring_allreduce_all_ranks",
     "mpic_ring_allgather_all_ranks", "mpic_ring_allreduce_transport", "mpic_ring_allgather_transport",
@@ -137,6 +138,8 @@ def load_library(name="libmpi_collectives.so", op_list=None):
             "mpic_context_num_outputs": (ci, [vp]),
             "mpic_context_output": (ci, [vp, ci, pint, pint, p64, pvp]),
             "mpic_context_destroy": (ci, [vp]),
+            "mpic_allreduce_batch": (ci, [vp, ci, ci, ctypes.POINTER(cp), pint, pint, p64, pvp, pvp, ci, pvp]),
+            "mpic_context_wait_batch": (ci, [pvp, ci, ci, pint]),
             "mpic_ring_allreduce_prestaged": (ci, [ci, ci, ci, vp, vp, sz, pvp, pvp, vp, ci]),
             "mpic_ring_allreduce_direct_prestaged": (ci, [ci, ci, ci, vp, vp, sz, pvp, pvp, vp, ci]),
             "mpic_ring_allreduce_fused_prestaged": (ci, [vp, ci, ci, vp, pvp, pvp, vp, ci]),
@@ -299,3 +302,50 @@ class PendingOp:
 
     # An op that was never waited for keeps its C context: the background
     # thread may still call back into it, so it is not destroyed from a finalizer.
+
+
+class PendingBatch:
+    """k MPIAllreduce nodes of one rank submitted with one call into the plugin
+    (mpic_allreduce_batch): one node per tensor, as a loop over single ops
+    would create, but one crossing of the language boundary for all of them
+    and one for waiting. Keeps inputs, outputs and the C contexts alive."""
+
+    def __init__(self, world, rank, node_names, inputs, outputs, divisor=0):
+        L = lib()
+        k = len(inputs)
+        self._inputs, self._outputs = inputs, outputs
+        self.node_names = node_names
+        self._k = k
+        self._errors = None
+        names = (ctypes.c_char_p * max(k, 1))(*[n.encode() for n in node_names])
+        dtypes = (ctypes.c_int * max(k, 1))(*[TORCH2DT.get(t.dtype, 0) for t in inputs])
+        ndims = (ctypes.c_int * max(k, 1))(*[t.dim() for t in inputs])
+        flat_dims = [d for t in inputs for d in t.shape]
+        dims = (ctypes.c_int64 * max(len(flat_dims), 1))(*flat_dims)
+        ins = (ctypes.c_void_p * max(k, 1))(*[t.data_ptr() if t.numel() else None for t in inputs])
+        outs = (ctypes.c_void_p * max(k, 1))(*[t.data_ptr() if t.numel() else None for t in outputs])
+        self._contexts = (ctypes.c_void_p * max(k, 1))()
+        rc = L.mpic_allreduce_batch(world, rank, k, names, dtypes, ndims, dims, ins, outs, divisor, self._contexts)
+        if rc != OK:
+            raise error_for(rc, "could not submit %d allreduces (rank %d)" % (k, rank))
+
+    def wait(self):
+        """Blocks until every node's done() has run. Returns a list with None
+        for a node that ended OK and its OpError otherwise."""
+        if self._errors is None:
+            L = lib()
+            codes = (ctypes.c_int * max(self._k, 1))()
+            first = L.mpic_context_wait_batch(self._contexts, self._k, 1, codes)
+            errors = [None] * self._k
+            if first != OK:
+                for j in range(self._k):
+                    if codes[j] != OK:
+                        errors[j] = error_for(codes[j], L.mpic_context_message(self._contexts[j]).decode())
+                        L.mpic_context_destroy(self._contexts[j])
+                        self._contexts[j] = None
+            self._errors = errors
+        return self._errors
+
+    @property
+    def outputs(self):
+        return self._outputs

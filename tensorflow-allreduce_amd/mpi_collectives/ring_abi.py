@@ -18,7 +18,7 @@ LIB_PATH = os.path.join(_PKG_ROOT, "lib", "libring_hip.so")
 EXPORTS = (
     "ring_abi_version", "ring_status_string", "ring_last_hip_error", "ring_dtype_size",
     "ring_set_option", "ring_event_create", "ring_event_destroy", "ring_event_elapsed_us",
-    "ring_time_next_launch", "ring_event_record", "ring_event_synchronize", "ring_stream_wait_event", "ring_segment_table", "ring_temp_elements", "ring_allgather_table",
+    "ring_time_next_launch", "ring_event_record", "ring_event_synchronize", "ring_stream_wait_event", "ring_graph_begin_capture", "ring_graph_end_capture", "ring_graph_launch", "ring_graph_destroy", "ring_segment_table", "ring_temp_elements", "ring_allgather_table",
     "ring_schedule", "ring_stream_create", "ring_stream_destroy", "ring_stream_synchronize",
     "ring_copy_bytes", "ring_accumulate_f32", "ring_accumulate_i32", "ring_accumulate_i64",
     "ring_accumulate", "ring_reduce_scatter_steps", "ring_reduce_scatter_steps_from",
@@ -98,6 +98,10 @@ def lib():
             "ring_event_record": (ci, [vp, vp]),
             "ring_event_synchronize": (ci, [vp]),
             "ring_stream_wait_event": (ci, [vp, vp]),
+            "ring_graph_begin_capture": (ci, [vp]),
+            "ring_graph_end_capture": (ci, [vp, ctypes.POINTER(vp)]),
+            "ring_graph_launch": (ci, [vp, vp]),
+            "ring_graph_destroy": (ci, [vp]),
             "ring_segment_table": (ci, [sz, ci, psz, psz]),
             "ring_temp_elements": (sz, [sz, ci]),
             "ring_allgather_table": (ci, [psz, ci, sz, psz]),

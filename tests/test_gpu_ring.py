@@ -933,3 +933,100 @@ def test_more_ranks_than_the_direct_form_addresses(oracle):
         outs = session.run(handles)
     for r in (0, 1, 128, 256):
         G.assert_same_bits(G.host(outs[r]), want, "257 ranks, rank %d" % r)
+
+
+@pytest.mark.parametrize("dtype", G.DTYPES)
+def test_recorded_steps_replay_with_the_eager_results(oracle, dtype):
+    """Several per-rank steps recorded as one HIP graph through the C ABI
+    (ring_graph_begin_capture ... ring_graph_end_capture) and replayed. Every
+    replay, with the program's own eager work and synchronisations between
+    them and new values in the same buffers, gives the oracle's result bit for
+    bit on every recorded step."""
+    L, R = _plugin.load_library(), ring_abi.lib()
+    cases = ((8, 262_144, 1), (6, 100_003, 3), (3, 17, 3), (1, 9, 1))
+    tdt = G.NP2TORCH[np.dtype(dtype)]
+    bufs = []
+    for n, count, flags in cases:
+        sizes, _ = ring_abi.segment_table(count, n)
+        r = n // 2
+        rs_seg = [ring_abi.schedule(ring_abi.PHASE_REDUCE_SCATTER, n, r, i)[1] for i in range(n - 1)]
+        ag_seg = [ring_abi.schedule(ring_abi.PHASE_ALLGATHER, n, r, i)[1] for i in range(n - 1)]
+        rs_t = [torch.zeros(sizes[g], dtype=tdt, device="cuda") for g in rs_seg]
+        ag_t = [torch.zeros(sizes[g], dtype=tdt, device="cuda") for g in ag_seg]
+        bufs.append(dict(n=n, r=r, count=count, flags=flags, sizes=sizes, rs_seg=rs_seg, ag_seg=ag_seg, rs_t=rs_t, ag_t=ag_t,
+                         din=torch.zeros(count, dtype=tdt, device="cuda"), dout=torch.zeros(count, dtype=tdt, device="cuda"),
+                         rs_p=(ctypes.c_void_p * max(n - 1, 1))(*[t.data_ptr() if t.numel() else None for t in rs_t]),
+                         ag_p=(ctypes.c_void_p * max(n - 1, 1))(*[t.data_ptr() if t.numel() else None for t in ag_t])))
+    stream = ring_abi.stream_create()
+    graph = ctypes.c_void_p()
+    try:
+        torch.cuda.synchronize()
+        ring_abi.check(R.ring_graph_begin_capture(stream), "begin capture")
+        for b in bufs:
+            rc = L.mpic_ring_allreduce_prestaged(b["n"], b["r"], DT[np.dtype(dtype)], b["din"].data_ptr(), b["dout"].data_ptr(),
+                                                 b["count"], b["rs_p"], b["ag_p"], stream, b["flags"])
+            assert rc == 0, L.mpic_last_error()
+        ring_abi.check(R.ring_graph_end_capture(stream, ctypes.byref(graph)), "end capture")
+        for replay in range(4):
+            wants = []
+            for b in bufs:      # eager work of the program itself between the replays
+                ins = make_inputs(b["n"], b["count"], dtype, seed=40 * replay + b["n"])
+                outs, rs, ag = oracle.ring_allreduce(ins, tap=True)
+                b["din"].copy_(torch.from_numpy(ins[b["r"]]))
+                for i in range(b["n"] - 1):
+                    b["rs_t"][i].copy_(torch.from_numpy(np.ascontiguousarray(rs[b["r"]][i][:b["sizes"][b["rs_seg"][i]]])))
+                    b["ag_t"][i].copy_(torch.from_numpy(np.ascontiguousarray(ag[b["r"]][i][:b["sizes"][b["ag_seg"][i]]])))
+                b["dout"].zero_()
+                wants.append((outs[b["r"]], ins[b["r"]]))
+            torch.cuda.synchronize()
+            ring_abi.check(R.ring_graph_launch(graph, stream), "graph launch")
+            ring_abi.stream_synchronize(stream)
+            for b, (want, inp) in zip(bufs, wants):
+                G.assert_same_bits(G.host(b["dout"]), want, "recorded step n=%d replay %d" % (b["n"], replay))
+                G.assert_same_bits(G.host(b["din"]), inp, "the input is never written")
+    finally:
+        if graph.value:
+            ring_abi.check(R.ring_graph_destroy(graph), "graph destroy")
+        ring_abi.stream_destroy(stream)
+    assert R.ring_graph_begin_capture(None) == 2        # the null stream cannot be recorded
+
+
+def test_allreduce_batch_is_one_node_per_tensor(oracle):
+    """mpi.allreduce_batch: every tensor is its own MPIAllreduce node (same
+    results as a loop over mpi.allreduce, bit for bit, sum and average, mixed
+    element types and shapes, an empty tensor among them), and a tensor whose
+    shape differs between ranks fails alone, with the reference's message,
+    while the others of the batch complete."""
+    n = 4
+    shapes = [(1000, 3), (0,), (70_001,), (5,), (128, 64)]
+    dtypes = [np.float32, np.float32, np.int32, np.int64, np.float32]
+    ins = [[G.random_array(np.random.default_rng(10 * r + j), int(np.prod(s)), dt).reshape(s)
+            for j, (s, dt) in enumerate(zip(shapes, dtypes))] for r in range(n)]
+    for average in (False, True):
+        with mpi.Session(size=n) as session:
+            handles = []
+            for r in range(n):
+                with session.as_rank(r):
+                    handles.append(mpi.allreduce_batch([cuda(x) for x in ins[r]], average=average))
+            outs = session.run(handles)
+        for j in range(len(shapes)):
+            want = oracle.ring_allreduce([ins[r][j].reshape(-1) for r in range(n)])
+            for r in range(n):
+                w = _tf_div(want[r], n) if average else want[r]
+                assert tuple(outs[r][j].shape) == shapes[j]
+                G.assert_same_bits(G.host(outs[r][j]).reshape(-1), w, "batch tensor %d rank %d average=%s" % (j, r, average))
+    # one tensor's shape differs on one rank: that node fails on every rank, the rest complete
+    with mpi.Session(size=n) as session:
+        handles = []
+        for r in range(n):
+            with session.as_rank(r):
+                xs = [cuda(ins[r][0]), cuda(ins[r][3] if r != 2 else np.zeros(6, np.int64)), cuda(ins[r][4])]
+                handles.append(mpi.allreduce_batch(xs, average=False))
+        with pytest.raises(mpi.FailedPreconditionError) as e:
+            session.run()
+        assert "Mismatched allreduce tensor shapes" in str(e.value)
+        for r in range(n):
+            G.assert_same_bits(G.host(handles[r][0].result()).reshape(-1),
+                               oracle.ring_allreduce([ins[q][0].reshape(-1) for q in range(n)])[r], "first of the batch")
+            with pytest.raises(mpi.FailedPreconditionError):
+                handles[r][1].result()
