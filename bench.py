@@ -46,9 +46,15 @@ COLD_SAMPLES = 32                   # timed launches of the cold-operand accumul
 METRIC = "per-rank ring allreduce GB/s & % of HBM peak, 64 MiB fp32, N=8 virtual ranks"
 # committed rocprofv3 counter summaries holding a `traffic_bytes_per_launch:` line for a workload's dominant kernel
 TRAFFIC_PROFILES = {
-    "allreduce_f32_64MiB_n8": "rows_kernel_f32_accumulate_64MiB_n8_pmc.txt",
-    "allreduce_f32_64MiB_n8_direct": "fold_kernel_f32_64MiB_n8_direct.txt",
+    "allreduce_f32_64MiB_n8": "rows_kernel_f32_64MiB_n8_headline.txt",
+    "allreduce_i32_10000019_n6": "rows_kernel_i32_10000019_n6.txt",
+    "allreduce_i64_10000019_n6": "rows_kernel_i64_10000019_n6.txt",
+    "allgather_f32_n16": "rows_kernel_allgather_f32_n16.txt",
+    "allreduce_f32_1GiB_n64": "rows_kernel_f32_1GiB_n64.txt",
+    "fused_resnet50_n8": "fusion_kernel_resnet50_161_tensors_n8.txt",
     "fused_resnet50_n8_no_passes": "fusion_span_kernel_resnet50_161_tensors_n8_no_passes.txt",
+    "fused_resnet50_n8_no_passes_direct": "fusion_span_kernel_resnet50_161_tensors_n8_direct.txt",
+    "allreduce_f32_64MiB_n8_direct": "fold_kernel_f32_64MiB_n8_direct.txt",
 }
 
 
@@ -163,18 +169,6 @@ class RingAllreduce(Workload):
         elif i == 1:
             A.check(R.ring_reduce_scatter_steps(s["out"].data_ptr(), s["rs_steps"][0], s["rs_steps"][1], self.code,
                                                 stream), "reduce-scatter")
-        else:
-            A.check(R.ring_allgather_steps(s["out"].data_ptr(), s["ag_steps"][0], s["ag_steps"][1], self.code,
-                                           stream), "allgather")
-
-    def launch_phase_fused(self, k, i, stream):
-        """The two launches of the step with the in->out copy folded in: the
-        accumulate out = in + received (every operand read for the first time),
-        then the allgather copies."""
-        s, A, R = self.sets[k % self.nsets], self.ring_abi, self.R
-        if i == 0:
-            A.check(R.ring_reduce_scatter_steps_from(s["inp"].data_ptr(), s["out"].data_ptr(), s["rs_steps"][0],
-                                                     s["rs_steps"][1], self.code, stream), "reduce-scatter from input")
         else:
             A.check(R.ring_allgather_steps(s["out"].data_ptr(), s["ag_steps"][0], s["ag_steps"][1], self.code,
                                            stream), "allgather")
@@ -813,19 +807,15 @@ def main():
         cold_events = []
         for k in range(COLD_SAMPLES * 4):
             if k % 4 == 2:
+                # the driver's own step; the events ride on its first launch, the accumulate
                 e = event_pool.pop()
-                for i in range(2):
-                    ring_abi.time_next_launch(e[2 * i], e[2 * i + 1])
-                    w.launch_phase_fused(k, i, stream)
+                ring_abi.time_next_launch(e[0], e[1])
                 cold_events.append(e)
-            else:
-                w.launch_step(k, stream, True)
+            w.launch_step(k, stream, True)
         ring_abi.stream_synchronize(stream)
         cold_acc = [ring_abi.event_elapsed_us(e[0], e[1]) for e in cold_events]
-        cold_ag = [ring_abi.event_elapsed_us(e[2], e[3]) for e in cold_events]
         cold = {"accumulate_median_us": round(statistics.median(cold_acc), 3),
                 "accumulate_mean_us": round(statistics.mean(cold_acc), 3),
-                "allgather_median_us": round(statistics.median(cold_ag), 3),
                 "launches_timed": len(cold_events)}
 
     result = {
