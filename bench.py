@@ -701,7 +701,9 @@ def main():
     # events are created before the timed region: creating them inside it would
     # let the queue drain and the sampled launches start on an idle GPU
     sample_every = max(1, min(SAMPLE_EVERY, steps))
-    event_pool = [[ring_abi.event_create() for _ in range(2 * max(nph, 2))]
+    # (a set = one pair per launch of the sampled step and one per launch of the step before it)
+    npairs = max(nph, 2)
+    event_pool = [[ring_abi.event_create() for _ in range(4 * npairs)]
                   for _ in range(steps // sample_every + 1 + MIN_SAMPLES + COLD_SAMPLES)]
 
     def timed(nsteps, nwarm, fused=False, with_samples=False, hot=False, sample_every=sample_every):
@@ -718,8 +720,18 @@ def main():
         torch.cuda.synchronize()
         samples = []
         t0 = time.perf_counter()
+        launches = 2 if fused else nph
         for k in range(nsteps):
-            if with_samples and k % sample_every == sample_every // 2:
+            if with_samples and sample_every > 1 and (k + 1) % sample_every == sample_every // 2:
+                # the step before a sampled one is timed as well (its figures are not used): a timed
+                # dispatch ends when its stores have drained, so the sampled step's first launch does
+                # not pay for its predecessor's, as under a profiler's kernel trace
+                spare = event_pool[-1]
+                for i in range(launches):
+                    ring_abi.time_next_launch(spare[2 * (npairs + i)], spare[2 * (npairs + i) + 1])
+                launch_step(k, stream, fused)
+                ring_abi.time_next_launch(None, None)       # a step of fewer launches leaves none armed
+            elif with_samples and k % sample_every == sample_every // 2:
                 # the same launches, one ABI call each, every one carrying its own
                 # pair of HIP events in the dispatch (on the stream the kernels run on)
                 e = event_pool.pop()
@@ -806,16 +818,25 @@ def main():
             w.launch_step(k, stream, True)
         cold_events = []
         for k in range(COLD_SAMPLES * 4):
+            if k % 4 == 1:
+                # the step before, timed too (see timed())
+                spare = event_pool[-1]
+                for i in range(2):
+                    ring_abi.time_next_launch(spare[2 * (npairs + i)], spare[2 * (npairs + i) + 1])
             if k % 4 == 2:
-                # the driver's own step; the events ride on its first launch, the accumulate
+                # the driver's own step; the events ride on its two launches, accumulate and allgather
                 e = event_pool.pop()
-                ring_abi.time_next_launch(e[0], e[1])
+                for i in range(2):
+                    ring_abi.time_next_launch(e[2 * i], e[2 * i + 1])
                 cold_events.append(e)
             w.launch_step(k, stream, True)
+            ring_abi.time_next_launch(None, None)
         ring_abi.stream_synchronize(stream)
         cold_acc = [ring_abi.event_elapsed_us(e[0], e[1]) for e in cold_events]
+        cold_ag = [ring_abi.event_elapsed_us(e[2], e[3]) for e in cold_events]
         cold = {"accumulate_median_us": round(statistics.median(cold_acc), 3),
                 "accumulate_mean_us": round(statistics.mean(cold_acc), 3),
+                "allgather_behind_it_median_us": round(statistics.median(cold_ag), 3),
                 "launches_timed": len(cold_events)}
 
     result = {

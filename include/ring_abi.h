@@ -89,8 +89,14 @@ int ring_set_option(const char* name, int value);
  * makes the NEXT step-table / copy / accumulate kernel this thread launches
  * record its own begin and end into them (the events travel in the dispatch,
  * so their difference is the kernel's execution time and nothing else). Read
- * with ring_event_elapsed_us after the stream has been synchronised. A call
- * that needs several launches times the first one only. */
+ * with ring_event_elapsed_us after the stream has been synchronised. Each
+ * call arms one more launch, in order, up to 8 ahead (RING_ERR_LIMIT beyond):
+ * a call that needs several launches is timed launch by launch by arming as
+ * many pairs before it. Two null events disarm whatever is still queued.
+ * A timed dispatch signals its own completion, so it ends only when its
+ * stores have drained, and one that follows an untimed dispatch also waits
+ * for that one's: durations agree with a profiler's kernel trace (where
+ * every dispatch is timed) when the launch before is timed as well. */
 int ring_event_create(void** event);
 int ring_event_destroy(void* event);
 int ring_event_elapsed_us(void* start, void* stop, double* us);

@@ -49,20 +49,27 @@ constexpr int kBlock = 256;   // threads per workgroup: 4 wave64
 constexpr int kMaxRows = 64;  // rows one launch carries in its kernel arguments
 
 thread_local int g_last_hip_error = 0;
-// Events the next kernel launch of this thread records its own begin and end
-// into (ring_time_next_launch); cleared by that launch.
-thread_local hipEvent_t g_time_start = nullptr;
-thread_local hipEvent_t g_time_stop = nullptr;
+// Events the next kernel launches of this thread record their own begin and
+// end into (ring_time_next_launch): a short queue, one pair per armed launch,
+// taken in order by the launches that follow.
+constexpr int kMaxArmedLaunches = 8;
+struct ArmedLaunch { hipEvent_t start, stop; };
+thread_local ArmedLaunch g_armed[kMaxArmedLaunches];
+thread_local int g_armed_head = 0, g_armed_count = 0;
 
 // Every kernel launch of the library goes through here. A launch armed by
 // ring_time_next_launch carries its events in the dispatch itself, so they
 // bracket the kernel's execution and nothing else.
 template <typename... Params, typename... Args>
 inline void launch(void (*kernel)(Params...), dim3 grid, dim3 block, hipStream_t stream, Args... args) {
-  hipEvent_t t0 = g_time_start, t1 = g_time_stop;
-  g_time_start = g_time_stop = nullptr;
-  if (t0 || t1) hipExtLaunchKernelGGL(kernel, grid, block, 0, stream, t0, t1, 0, args...);
-  else hipLaunchKernelGGL(kernel, grid, block, 0, stream, args...);
+  if (g_armed_count > 0) {
+    const ArmedLaunch a = g_armed[g_armed_head];
+    g_armed_head = (g_armed_head + 1) % kMaxArmedLaunches;
+    --g_armed_count;
+    hipExtLaunchKernelGGL(kernel, grid, block, 0, stream, a.start, a.stop, 0, args...);
+  } else {
+    hipLaunchKernelGGL(kernel, grid, block, 0, stream, args...);
+  }
 }
 
 inline int hip_fail(hipError_t e) {
@@ -1229,8 +1236,14 @@ int ring_stream_wait_event(void* stream, void* event) {
 }
 
 int ring_time_next_launch(void* start_event, void* stop_event) {
-  g_time_start = static_cast<hipEvent_t>(start_event);
-  g_time_stop = static_cast<hipEvent_t>(stop_event);
+  if (!start_event && !stop_event) {
+    g_armed_head = g_armed_count = 0;
+    return RING_OK;
+  }
+  if (g_armed_count == kMaxArmedLaunches) return RING_ERR_LIMIT;
+  g_armed[(g_armed_head + g_armed_count) % kMaxArmedLaunches] =
+      ArmedLaunch{static_cast<hipEvent_t>(start_event), static_cast<hipEvent_t>(stop_event)};
+  ++g_armed_count;
   return RING_OK;
 }
 
