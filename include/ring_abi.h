@@ -78,7 +78,11 @@ size_t ring_dtype_size(int dtype);
  * bit 1 = non-temporal loads, -1 = the default: 3, except ordinary stores
  * where the next kernel reads the output (copy, pack, fold), ordinary loads
  * for a source several rows share (broadcast), and loads by size for the copy.
- * "nontemporal" sets all seven. "dry_launch" = 1 makes the step-table / copy /
+ * "nontemporal" sets all seven. "paced_copy": the copies of an allgather
+ * phase as one read phase and one write phase (every workgroup waits for all
+ * its loads, then keeps one store in flight per wave): 1 always, 0 never,
+ * -1 (default) when every tile of the launch is on the chip at the same time
+ * (between 2 and 7 tiles of 32 KiB per CU). "dry_launch" = 1 makes the step-table / copy /
  * accumulate kernels return at entry: what is then timed is what a launch of
  * that grid costs by itself. No counterpart in the reference, whose launch
  * shape is the constant <<<32, 256>>> (ring.cu.cc:64). */

@@ -114,6 +114,9 @@ static void reference_loop(int n, size_t count) {
       const int send = mod(r - i), to = mod(r + 1);
       HIP_OK(hipMemcpy(temp[to], buffer[r] + starts[send], sizes[send] * sizeof(T), hipMemcpyDeviceToDevice));
     }
+    // a device-to-device hipMemcpy may return before the copy has run, and the binding's stream does
+    // not wait for the null stream: the "receive" is complete (MPI_Wait, ring.h:200) only after this
+    HIP_OK(hipDeviceSynchronize());
     for (int r = 0; r < n; r++) {
       const int recv = mod(r - i - 1);
       AccumulateTensorData<GPUDevice, T>(buffer[r] + starts[recv], temp[r], sizes[recv]);

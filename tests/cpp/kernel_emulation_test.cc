@@ -331,6 +331,10 @@ void run_all(const char* name) {
   test_step_tables<T>(65536, 8);
   test_step_tables<T>(5, 8);        // fewer elements than ranks
   test_step_tables<T>(40013, 3);
+  CHECK(ring_set_option("paced_copy", 1) == RING_OK);   // the allgather copies in their paced form
+  test_step_tables<T>(100003, 6);
+  test_step_tables<T>(70001, 3);
+  CHECK(ring_set_option("paced_copy", -1) == RING_OK);
   printf("%s: fold\n", name); fflush(stdout);
   test_fold<T>(8, 10007, 0);
   test_fold<T>(3, 4096, 3);

@@ -19,7 +19,7 @@ COUNTS = [0, 1, 2, 3, 4, 5, 7, 8, 1023, 1024, 1025, 4096, 4097, 3 * 4096 + 7, 26
 def _gpu():
     G.require_gpu()
     yield
-    for k, v in (("unroll", 4), ("nontemporal", -1), ("blocks_per_cu", 0)):
+    for k, v in (("unroll", 4), ("nontemporal", -1), ("blocks_per_cu", 0), ("paced_copy", -1)):
         ring_abi.set_option(k, v)
 
 
@@ -153,6 +153,37 @@ def test_step_tables_match_oracle(oracle, dtype, n_rows):
         fn(dbuf.data_ptr(), steps, n, code, None)
         G.sync()
         G.assert_same_bits(G.host(dbuf), want, "table rows=%d acc=%s" % (n_rows, accumulate))
+
+
+@pytest.mark.parametrize("dtype", G.DTYPES)
+@pytest.mark.parametrize("paced", [1, 0])
+def test_paced_allgather_copies_match(dtype, paced):
+    """The allgather copies as one read phase and one write phase (32 KiB tiles that wait
+    for all their loads and keep one store in flight), forced on for launches of any size
+    and forced off: the same bytes either way, ragged rows at any alignment, rows shorter
+    than a tile, a row of many tiles with a partial last one."""
+    rng = np.random.default_rng(41 + paced)
+    code = G.NP2ABI[np.dtype(dtype)]
+    ring_abi.set_option("paced_copy", paced)
+    try:
+        for n_rows, max_count in ((1, 300_000), (7, 70_000), (16, 9_000), (64, 3_000)):
+            table, total = _random_table(rng, n_rows, dtype, max_count)
+            buf = G.random_array(rng, total + 5, dtype)
+            dbuf, _ = G.dev(buf, int(rng.integers(0, 4)))
+            want = buf.copy()
+            rows, keep = [], []
+            for off, cnt in table:
+                src = G.random_array(rng, cnt, dtype)
+                ds, base = G.dev(src, int(rng.integers(0, 4)))
+                keep.append(base)
+                rows.append((off, ds.data_ptr() if cnt else None, cnt))
+                want[off:off + cnt] = src
+            steps, n = ring_abi.make_steps(rows)
+            ring_abi.allgather_steps(dbuf.data_ptr(), steps, n, code, None)
+            G.sync()
+            G.assert_same_bits(G.host(dbuf), want, "paced=%d rows=%d" % (paced, n_rows))
+    finally:
+        ring_abi.set_option("paced_copy", -1)
 
 
 @pytest.mark.parametrize("opt", [("unroll", 2), ("unroll", 8), ("nontemporal", 0),

@@ -894,10 +894,15 @@ def test_inputs_still_being_produced_on_another_stream(oracle):
     base = make_inputs(n, count, np.float32, seed=5, wide=False)
     side = torch.cuda.Stream()
     dins = [cuda(x) for x in base]
+    ballast = torch.zeros(256 * 1024 * 1024, dtype=torch.float32, device="cuda")     # 1 GiB per pass
     torch.cuda.synchronize()
     with mpi.Session(size=n) as session:
         handles = []
         with torch.cuda.stream(side):
+            # several milliseconds of work ahead of the producers on the same stream, so that
+            # they are certainly still queued when the host reaches the submissions
+            for _ in range(24):
+                ballast.add_(1.0)
             for r in range(n):
                 for _ in range(rounds):
                     dins[r].add_(1.0)                 # ~60 kernels per rank queued on the side stream
