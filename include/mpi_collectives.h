@@ -163,6 +163,27 @@ int mpic_allreduce_batch(mpic_world* world, int rank, int k, const char* const* 
  * status that is not OK. */
 int mpic_context_wait_batch(mpic_context** contexts, int k, int destroy_ok, int* codes);
 
+/* The same k nodes built ONCE and run every step, the way a TensorFlow graph's
+ * nodes are constructed once and executed by every session.run() (the
+ * reference's MPIAllreduceOp objects live as long as the graph; only its
+ * OpKernelContext is per step, mpi_ops.cc:1039-1117). Arguments as
+ * mpic_allreduce_batch; the tensors' memory must stay where it is for the life
+ * of the batch. mpic_batch_submit files one MPIAllreduce request per node, as
+ * k executions of the kernels would (FAILED_PRECONDITION while the previous
+ * submission is still running); mpic_batch_wait blocks until all of them have
+ * finished, returns the first status that is not OK and fills codes[j] (when
+ * given) with node j's; mpic_batch_message(batch, j) is node j's message
+ * until the next submit. mpic_batch_destroy waits for a running submission. */
+typedef struct mpic_batch mpic_batch;
+int mpic_batch_create(mpic_world* world, int rank, int k, const char* const* node_names, const int* dtypes,
+                      const int* ndims, const int64_t* dims, const void* const* inputs, void* const* outputs,
+                      int divisor, mpic_batch** batch);
+int mpic_batch_size(const mpic_batch* batch);
+int mpic_batch_submit(mpic_batch* batch);
+int mpic_batch_wait(mpic_batch* batch, int* codes);
+const char* mpic_batch_message(const mpic_batch* batch, int index);
+int mpic_batch_destroy(mpic_batch* batch);
+
 /* ---- the ring driver, callable without the op layer ------------------------
  * RingAllreduce (ring.h:136-228) for rank r of n whose incoming segments are
  * already in device memory. `flags`: bit 0 = batched, bit 1 = fuse the

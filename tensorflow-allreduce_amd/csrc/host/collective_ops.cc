@@ -117,7 +117,7 @@ TensorShape ShapeOf(const MPIRequest& r) { return TensorShape(r.tensor_shape); }
 // mpi_ops.cc:277-432: all the cross-rank checks, with the reference's messages.
 MPIResponse ConstructMPIResponse(MessageTable* table, const std::string& name) {
   bool error = false;
-  std::vector<MPIRequest> requests = (*table)[name];
+  const std::vector<MPIRequest>& requests = (*table)[name];
   std::ostringstream err;
 
   const MPIDataType data_type = requests[0].tensor_type;
@@ -140,14 +140,12 @@ MPIResponse ConstructMPIResponse(MessageTable* table, const std::string& name) {
   }
 
   if (message_type == MPIRequest::ALLREDUCE) {
-    const TensorShape tensor_shape = ShapeOf(requests[0]);
     for (size_t i = 1; i < requests.size() && !error; i++) {
-      const TensorShape request_shape = ShapeOf(requests[i]);
-      if (tensor_shape != request_shape) {
+      if (requests[0].tensor_shape != requests[i].tensor_shape) {
         error = true;
         err << "Mismatched allreduce tensor shapes: One rank reduced a tensor of shape "
-            << tensor_shape.DebugString() << ", but another rank sent a tensor of shape "
-            << request_shape.DebugString() << ".";
+            << ShapeOf(requests[0]).DebugString() << ", but another rank sent a tensor of shape "
+            << ShapeOf(requests[i]).DebugString() << ".";
       }
     }
   }
@@ -212,6 +210,20 @@ WorldOptions SnapshotOptions(mpic_world* w) {
 
 // mpi_ops.cc:435-515: run the collective for every rank that lives here, then
 // resume their ops.
+// The end of a collective: its records are released BEFORE the waiting ops are
+// told. A thread that is told starts its next step at once, and what this
+// thread still had to free (several allocations per record, made by those
+// threads) would then compete with it for the allocator: measured on 8 x 161
+// gradients, the next step's submission took 1.6 ms instead of 0.4.
+template <typename Records>
+void FinishRecords(Records* records, std::vector<CommunicationDoneCallback>* callbacks, const Status& status) {
+  records->clear();
+  for (auto& done : *callbacks) {
+    done(status);
+    done = nullptr;  // and its captured state, while the waiters still wait for the last ones
+  }
+}
+
 void PerformCollectiveOp(mpic_world* w, const MPIResponse& response) {
   const WorldOptions opt = SnapshotOptions(w);
   std::map<int, CollectiveOpRecord> records;
@@ -306,7 +318,9 @@ void PerformCollectiveOp(mpic_world* w, const MPIResponse& response) {
     const int rc = ring_stream_synchronize(w->stream);
     if (rc != RING_OK) status = errors::Unknown("MPI operation failed unexpectedly.");  // ring.h:36-39
   }
-  for (auto& kv : records) kv.second.callback(status);
+  std::vector<CommunicationDoneCallback> callbacks;
+  for (auto& kv : records) callbacks.push_back(std::move(kv.second.callback));
+  FinishRecords(&records, &callbacks, status);
 }
 
 // A fusion plan for these tensors, created on first use. Training loops reduce
@@ -402,8 +416,10 @@ void PerformFusedAllreduce(mpic_world* w, const std::vector<std::string>& names,
   }
   if (status.ok() && opt.sync_on_done && ring_stream_synchronize(w->stream) != RING_OK)
     status = errors::Unknown("MPI operation failed unexpectedly.");
+  std::vector<CommunicationDoneCallback> callbacks;
   for (auto& rec : records)
-    for (auto& kv : rec) kv.second.callback(status);
+    for (auto& kv : rec) callbacks.push_back(std::move(kv.second.callback));
+  FinishRecords(&records, &callbacks, status);
 }
 
 // One tick's ready collectives, in the order they became ready. With fusion on,
@@ -547,19 +563,26 @@ Status DataTypeToMPIType(DataType tf_dtype, MPIDataType* mpi_dtype) {
 }
 
 // mpi_ops.cc:853-868
-void EnqueueTensorCollective(mpic_world* w, const CollectiveOpRecord& record, MPIRequest::RequestType rtype) {
+void EnqueueTensorCollective(mpic_world* w, CollectiveOpRecord record, MPIRequest::RequestType rtype) {
   MPIRequest message;
   message.request_rank = record.rank;
   message.tensor_name = record.name;
   message.tensor_type = record.dtype;
   message.request_type = rtype;
   message.tensor_shape = record.in_t->shape().dim_sizes();
+  std::string wire = message.SerializeAsString();
+  bool wake;
   {
     std::lock_guard<std::mutex> guard(w->mu);
-    w->tensor_table[record.name][record.rank] = record;
-    w->message_queue.push(message.SerializeAsString());
+    std::map<int, CollectiveOpRecord>& by_rank = w->tensor_table[record.name];
+    const int rank = record.rank;
+    by_rank[rank] = std::move(record);
+    w->message_queue.push(std::move(wire));
+    // with fusion on, requests wait for a flush: waking the thread for each
+    // would only have it look at the queue and go back to sleep
+    wake = !(w->fusion_bytes > 0 && !w->flush_requested);
   }
-  w->work_cv.notify_one();
+  if (wake) w->work_cv.notify_one();
 }
 
 mpic_world* WorldOf(OpKernelContext* context) { return static_cast<mpic_world*>(context->world()); }
@@ -699,7 +722,7 @@ class MPIAllreduceOp : public AsyncOpKernel {
     // The caller's producer work is ordered before the collective by the
     // embedding framework (the reference defers this call with a stream host
     // callback, mpi_ops.cc:1099-1105).
-    EnqueueTensorCollective(world, record, MPIRequest::ALLREDUCE);
+    EnqueueTensorCollective(world, std::move(record), MPIRequest::ALLREDUCE);
   }
 };
 REGISTER_KERNEL_BUILDER(Name("MPIAllreduce").Device(DEVICE_GPU), MPIAllreduceOp<GPUDevice>);
@@ -783,7 +806,7 @@ class MPIAllgatherOp : public AsyncOpKernel {
       context->SetStatus(status);
       done();
     };
-    EnqueueTensorCollective(world, record, MPIRequest::ALLGATHER);
+    EnqueueTensorCollective(world, std::move(record), MPIRequest::ALLGATHER);
   }
 };
 REGISTER_OP("MPIAllgather")
@@ -1091,6 +1114,104 @@ int mpic_context_wait_batch(mpic_context** contexts, int k, int destroy_ok, int*
     }
   }
   return first;
+}
+
+// ---- a rank's MPIAllreduce nodes, built once and run every step ---------------------------
+
+struct mpic_batch {
+  mpic_world* world = nullptr;
+  int rank = 0;
+  // the graph's nodes: kernels are constructed once, as a TensorFlow graph's are,
+  // and every submission is one execution of each
+  std::vector<std::unique_ptr<mpic::OpKernel>> kernels;
+  std::vector<std::unique_ptr<mpic::OpKernelContext>> contexts;
+  std::mutex mu;
+  std::condition_variable cv;
+  int outstanding = 0;  // nodes of the current submission that have not called done()
+};
+
+int mpic_batch_create(mpic_world* world, int rank, int k, const char* const* node_names, const int* dtypes,
+                      const int* ndims, const int64_t* dims, const void* const* inputs, void* const* outputs,
+                      int divisor, mpic_batch** batch) {
+  if (!world || !batch || k < 0 || divisor < 0) return MPIC_INVALID_ARGUMENT;
+  if (k > 0 && (!node_names || !dtypes || !ndims || !inputs || !outputs)) return MPIC_INVALID_ARGUMENT;
+  if (rank < 0 || rank >= world->size || (world->real_rank >= 0 && rank != world->real_rank))
+    return MPIC_INVALID_ARGUMENT;
+  const mpic::KernelDef* kdef = OpRegistry::Global()->FindKernel("MPIAllreduce", "GPU");
+  if (!kdef) return MPIC_NOT_FOUND;
+  std::unique_ptr<mpic_batch> b(new mpic_batch());
+  b->world = world;
+  b->rank = rank;
+  size_t at = 0;
+  for (int j = 0; j < k; j++) {
+    if (ndims[j] < 0 || ndims[j] > 8 || (ndims[j] > 0 && !dims) || !node_names[j]) return MPIC_INVALID_ARGUMENT;
+    mpic::OpKernelConstruction construction(*node_names[j] ? node_names[j] : "MPIAllreduce");
+    b->kernels.emplace_back(kdef->factory(&construction));
+    void* out = outputs[j];
+    mpic::OutputAllocator allocator = [out](mpic::DataType, const mpic::TensorShape&, bool) -> void* { return out; };
+    b->contexts.emplace_back(new mpic::OpKernelContext(world, rank, true, allocator));
+    std::vector<int64_t> d(dims + at, dims + at + ndims[j]);
+    at += static_cast<size_t>(ndims[j]);
+    b->contexts.back()->AddInput(mpic::Tensor(static_cast<mpic::DataType>(dtypes[j]), mpic::TensorShape(d),
+                                              const_cast<void*>(inputs[j]), false));
+    b->contexts.back()->set_fused_divisor(divisor);
+  }
+  *batch = b.release();
+  return MPIC_OK;
+}
+
+int mpic_batch_size(const mpic_batch* b) { return b ? static_cast<int>(b->kernels.size()) : 0; }
+
+int mpic_batch_submit(mpic_batch* b) {
+  if (!b) return MPIC_INVALID_ARGUMENT;
+  {
+    std::lock_guard<std::mutex> guard(b->mu);
+    if (b->outstanding != 0) {
+      mpic::g_last_error = "the batch's previous submission has not finished";
+      return MPIC_FAILED_PRECONDITION;
+    }
+    b->outstanding = static_cast<int>(b->kernels.size());
+  }
+  auto done = [b] {
+    // notify under the lock: the waiter may destroy the batch as soon as it sees zero
+    std::lock_guard<std::mutex> guard(b->mu);
+    if (--b->outstanding == 0) b->cv.notify_all();
+  };
+  for (size_t j = 0; j < b->kernels.size(); j++) {
+    b->contexts[j]->Reset();
+    static_cast<mpic::AsyncOpKernel*>(b->kernels[j].get())->ComputeAsync(b->contexts[j].get(), done);
+  }
+  return MPIC_OK;
+}
+
+int mpic_batch_wait(mpic_batch* b, int* codes) {
+  if (!b) return MPIC_INVALID_ARGUMENT;
+  {
+    std::unique_lock<std::mutex> lock(b->mu);
+    b->cv.wait(lock, [b] { return b->outstanding == 0; });
+  }
+  int first = MPIC_OK;
+  for (size_t j = 0; j < b->contexts.size(); j++) {
+    const int code = static_cast<int>(b->contexts[j]->status().code());
+    if (codes) codes[j] = code;
+    if (code != MPIC_OK && first == MPIC_OK) first = code;
+  }
+  return first;
+}
+
+const char* mpic_batch_message(const mpic_batch* b, int index) {
+  if (!b || index < 0 || static_cast<size_t>(index) >= b->contexts.size()) return "";
+  return b->contexts[static_cast<size_t>(index)]->status().error_message().c_str();
+}
+
+int mpic_batch_destroy(mpic_batch* b) {
+  if (!b) return MPIC_OK;
+  {  // never free nodes the background thread may still call back into
+    std::unique_lock<std::mutex> lock(b->mu);
+    b->cv.wait(lock, [b] { return b->outstanding == 0; });
+  }
+  delete b;
+  return MPIC_OK;
 }
 
 // ---- the ring driver without the op layer --------------------------------------------

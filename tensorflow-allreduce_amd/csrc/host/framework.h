@@ -208,6 +208,13 @@ class OpKernelContext {
   int num_outputs() const { return static_cast<int>(outputs_.size()); }
   const Tensor* output(int i) const { return outputs_[static_cast<size_t>(i)].get(); }
 
+  // For a node that runs again with the same inputs (a step of a training
+  // loop): forgets the last run's outputs and status.
+  void Reset() {
+    outputs_.clear();
+    status_ = Status();
+  }
+
   void SetStatus(const Status& s) { if (status_.ok()) status_ = s; }
   const Status& status() const { return status_; }
 

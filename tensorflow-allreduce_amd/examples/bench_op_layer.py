@@ -7,7 +7,8 @@ float32) with mpi.allreduce, as the reference's DistributedOptimizer does
 gradient), and session.run() completes them. Compared: one ring per gradient
 (the reference's behaviour; there each op also waits for a coordinator tick of
 at least 1 ms, mpi_ops.cc:635), the coordinator's tensor fusion, each of them
-also with the gradients of a rank submitted by one call (mpi.allreduce_batch,
+also with the gradients of a rank submitted by one call (mpi.allreduce_batch)
+and with the nodes built once and run every step (mpi.prepare_allreduce_batch,
 what DistributedOptimizer.compute_gradients does), and a single pre-packed
 tensor. All ranks live on one GPU, so a ring step is one launch for
 all ranks.
@@ -39,11 +40,14 @@ def resnet50_counts():
     return counts + [2048 * 1000, 1000]
 
 
-def step(session, grads, average=True, batch=False):
+def step(session, grads, average=True, batch=False, prepared=None):
     """One step: every rank submits all its gradients, then the session runs."""
     t0 = time.perf_counter()
     handles = []
-    for r, gs in enumerate(grads):
+    if prepared is not None:
+        for b in prepared:
+            handles.append(b.submit())
+    for r, gs in enumerate(grads if prepared is None else []):
         with session.as_rank(r):
             if batch:
                 handles.append(mpi.allreduce_batch(gs, average=average))
@@ -70,12 +74,20 @@ def main():
     for label, kwargs, data, batch in (
             ("one ring per gradient", {}, grads, False),
             ("one ring per gradient, submitted as a batch", {}, grads, True),
+            ("one ring per gradient, nodes built once", {}, grads, "prepared"),
             ("coordinator fusion (128 MiB buffer per rank)", {"fusion_threshold": 128 << 20}, grads, False),
             ("coordinator fusion, submitted as a batch", {"fusion_threshold": 128 << 20}, grads, True),
+            ("coordinator fusion, nodes built once", {"fusion_threshold": 128 << 20}, grads, "prepared"),
             ("one pre-packed tensor", {}, packed, False)):
         with mpi.Session(size=args.ranks, **kwargs) as session:
-            step(session, data, batch=batch)                     # warm-up (fusion plans, allocator)
-            submit, run = zip(*[step(session, data, batch=batch) for _ in range(args.steps)])
+            prepared = None
+            if batch == "prepared":
+                prepared = []
+                for r, gs in enumerate(data):
+                    with session.as_rank(r):
+                        prepared.append(mpi.prepare_allreduce_batch(gs))
+            step(session, data, batch=batch, prepared=prepared)  # warm-up (fusion plans, allocator)
+            submit, run = zip(*[step(session, data, batch=batch, prepared=prepared) for _ in range(args.steps)])
         print("%-46s submit %7.2f ms   run %7.2f ms   total %7.2f ms per step"
               % (label, 1e3 * min(submit), 1e3 * min(run), 1e3 * min(s + r for s, r in zip(submit, run))))
 

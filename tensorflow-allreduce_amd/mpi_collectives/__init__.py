@@ -148,6 +148,7 @@ class Session:
         self._lock = threading.RLock()   # ranks may be driven from separate threads
         self._pending = []          # ops submitted and not yet waited for
         self._submitted = {}        # node name -> set of ranks, for the run() guard
+        self._batches = []          # AllreduceBatch objects built on this session
         self._counters = {}         # (rank, op) -> next auto-name index
         self._keep = []             # staged buffers kept alive until consumed
         self._prev = None
@@ -193,8 +194,10 @@ class Session:
 
     def close(self):
         if self._world is not None:
-            _plugin.lib().mpic_world_destroy(self._world)
+            _plugin.lib().mpic_world_destroy(self._world)      # fails whatever is still running
             self._world = None
+            for b in list(self._batches):
+                b.close()
             if mpi_ops._scope.session is self and self._prev is not None:
                 mpi_ops._scope.session, mpi_ops._scope.rank = self._prev
             self._pending, self._keep = [], []
@@ -359,7 +362,11 @@ class Session:
         with p.lock:
             if p.completed:
                 return p.error
-            if isinstance(p, _plugin.PendingBatch):
+            if isinstance(p, AllreduceBatch):
+                errors = p._c.wait()
+                p.errors = errors
+                p.error = next((e for e in errors if e is not None), None) if errors else None
+            elif isinstance(p, _plugin.PendingBatch):
                 for h, out, e in zip(p.handles, p.outputs, p.wait()):
                     if e is None:
                         h._set(value=out)
@@ -385,6 +392,13 @@ class Session:
         with self._lock:
             if p in self._pending:
                 self._pending.remove(p)
+            if isinstance(p, AllreduceBatch):
+                ranks = self._submitted.get(p.names_key)
+                if ranks is not None:
+                    ranks.discard(p.rank)
+                    if not ranks:
+                        self._submitted.pop(p.names_key, None)
+                return p.error
             for name in p.node_names:
                 ranks = self._submitted.get(name)
                 if ranks is not None:
@@ -396,11 +410,15 @@ class Session:
     def _check_all_ranks_submitted(self, batch):
         if self.real_rank is not None:
             return
+        prepared = [p for p in batch if isinstance(p, AllreduceBatch) and not p.completed]
         for p in batch:
             if p.completed:
                 continue
+            if isinstance(p, AllreduceBatch) and len(self._submitted.get(p.names_key, ())) == self.size:
+                continue            # every rank submitted this same set of nodes as one batch
             for name in p.node_names:
-                ranks = self._submitted.get(name, set())
+                ranks = set(self._submitted.get(name, ()))
+                ranks.update(q.rank for q in prepared if name in q.name_set)
                 if len(ranks) != self.size:
                     raise FailedPreconditionError(
                         "collective %r was submitted by ranks %s of %d; every rank must submit it "
@@ -434,6 +452,8 @@ class Session:
 def _resolve(x):
     if isinstance(x, PendingTensor):
         return x.result()
+    if isinstance(x, AllreduceBatch):
+        return x.results()
     if isinstance(x, IndexedSlices):
         return IndexedSlices(_resolve(x.values), _resolve(x.indices), x.dense_shape)
     if isinstance(x, (list, tuple)):
@@ -507,6 +527,131 @@ def allreduce_batch(tensors, average=True):
     return session._submit_batch(r, [None] * len(tensors), tensors, fold)
 
 
+class _BatchResult(PendingTensor):
+    """Result j of an AllreduceBatch: a handle like any other, whose tensor is
+    the batch's output j after the latest submission."""
+
+    def __init__(self, batch, index):
+        self._batch, self._index = batch, index
+
+    def _tensor(self):
+        errors = self._batch.errors
+        if errors and errors[self._index] is not None:
+            raise errors[self._index]
+        return self._batch.outputs[self._index]
+
+    def result(self):
+        if not self._batch.completed:
+            self._batch.session.run()
+        return self._tensor()
+
+    def wait(self):
+        self._batch.wait()
+        return self._tensor()
+
+
+class AllreduceBatch:
+    """The allreduces of a list of dense tensors, built once and run every step.
+
+    In the reference the graph is built once (one MPIAllreduce node per
+    gradient, each with its name, __init__.py:195-205) and every session.run()
+    executes the same nodes again. This is that graph fragment for one rank:
+    construction names the nodes and creates their kernels; submit() runs each
+    of them once more on the same tensors (new values, same memory), one call
+    into the plugin for all of them; results are valid until the next submit().
+    Every rank builds its batch in the same order, so the k-th node of each
+    rank carries the same name.
+
+      tensors: contiguous CUDA tensors; their memory is read at every submit.
+      average: divide by the number of ranks (fused into the collective).
+      inplace: the results replace the inputs' values instead of going to
+               memory of their own (one allocation per element type, made once).
+    """
+
+    def __init__(self, tensors, average=True, inplace=False):
+        session, r = mpi_ops._current()
+        tensors = list(tensors)
+        if session._immediate:
+            raise InvalidArgumentError("a prepared batch needs a session that holds every rank")
+        for t in tensors:
+            if not (isinstance(t, torch.Tensor) and t.is_cuda and t.is_contiguous()):
+                raise InvalidArgumentError("a prepared batch takes contiguous CUDA tensors")
+        self.session, self.rank, self.inputs = session, r, tensors
+        self.node_names = [session._node_name(r, 'MPIAllreduce', None) for _ in tensors]
+        self.names_key = tuple(self.node_names)
+        self.name_set = frozenset(self.node_names)
+        if inplace:
+            self.outputs = tensors
+        else:
+            self.outputs = [None] * len(tensors)
+            by_dtype = {}
+            for j, t in enumerate(tensors):
+                by_dtype.setdefault((t.dtype, t.device), []).append(j)
+            for (dtype, device), idx in by_dtype.items():
+                flat = torch.empty(sum(tensors[j].numel() for j in idx), dtype=dtype, device=device)
+                for j, piece in zip(idx, flat.split([tensors[j].numel() for j in idx])):
+                    self.outputs[j] = piece.view(tensors[j].shape)
+        self._c = _plugin.Batch(session._world, r, self.node_names, tensors, self.outputs,
+                                session.size if average else 0)
+        self.handles = [_BatchResult(self, j) for j in range(len(tensors))]
+        self.lock = threading.Lock()
+        self.completed = True          # nothing submitted yet
+        self.error = None
+        self.errors = None
+        self.next_op = self.on_done = self.handle = self.fail_handle = None
+        session._batches.append(self)
+
+    def submit(self):
+        """Runs the nodes once more. Returns the handles of the results (the
+        same objects every time)."""
+        session = self.session
+        if session._world is None:
+            raise FailedPreconditionError("the session of this batch is closed")
+        if not self.completed:
+            raise FailedPreconditionError("the batch's previous submission has not been completed; "
+                                          "run the session first")
+        session._order_after_producers(self.inputs[:1])
+        self.error = self.errors = None
+        self.completed = False
+        try:
+            self._c.submit()
+        except OpError:
+            self.completed = True
+            raise
+        with session._lock:
+            session._submitted.setdefault(self.names_key, set()).add(self.rank)
+            session._pending.append(self)
+        return self.handles
+
+    def wait(self):
+        """Blocks until the submission has run (ranks driven from separate threads)."""
+        self.session._flush()
+        error = self.session._complete(self)
+        if self.session.stream:
+            ring_abi.stream_synchronize(self.session.stream)
+        if error is not None:
+            raise error
+
+    def results(self):
+        """The output tensors, running the session if the submission is still pending."""
+        if not self.completed:
+            self.session.run()
+        if self.error is not None:
+            raise self.error
+        return self.outputs
+
+    def close(self):
+        self._c.close()
+        if self in self.session._batches:
+            self.session._batches.remove(self)
+
+
+def prepare_allreduce_batch(tensors, average=True, inplace=False):
+    """An AllreduceBatch for the current rank (not in the reference, where
+    building the graph once is what a TensorFlow program does anyway)."""
+    return AllreduceBatch(tensors, average=average, inplace=inplace)
+
+
 class DistributedOptimizer:
     """An optimizer that wraps a torch.optim.Optimizer, using an MPI allreduce
     to average gradient values before applying gradients to model weights
@@ -530,6 +675,8 @@ class DistributedOptimizer:
         self._use_locking = use_locking
         self._fusion = fusion
         self._fused = None      # (FusionPlan, fused buffer, grads) while a fused allreduce is in flight
+        self._batch = None      # the dense gradients' allreduces, built once (AllreduceBatch)
+        self._batch_key = None
 
     @property
     def param_groups(self):
@@ -552,7 +699,7 @@ class DistributedOptimizer:
         # one MPIAllreduce per gradient, as in the reference (__init__.py:195-205); the dense ones
         # are submitted together
         dense = [p for p in params if not p.grad.is_sparse]
-        reduced = dict(zip((id(p) for p in dense), allreduce_batch([p.grad for p in dense])))
+        reduced = dict(zip((id(p) for p in dense), self._reduce_dense([p.grad for p in dense])))
         out = []
         for p in params:
             g = p.grad
@@ -563,6 +710,23 @@ class DistributedOptimizer:
             else:
                 out.append((reduced[id(p)], p))
         return out
+
+    def _reduce_dense(self, grads):
+        """Handles of the averaged dense gradients. A training loop presents the
+        same gradient tensors every step, so their MPIAllreduce nodes are built
+        once (the reference's graph) and run again while the tensors stay where
+        they are; anything else goes through allreduce_batch."""
+        session, _ = mpi_ops._current()
+        if session._immediate or not grads or not all(g.is_cuda and g.is_contiguous() for g in grads):
+            return allreduce_batch(grads)
+        key = (id(session),) + tuple(g.data_ptr() for g in grads) + tuple(g.shape for g in grads)
+        if self._batch is None or self._batch_key != key:
+            if self._batch is not None and self._batch.completed:
+                self._batch.close()
+            # in place: the averaged gradient takes the gradient's memory, so tensors that stay
+            # where they are between steps (zero_grad(set_to_none=False)) keep the batch valid
+            self._batch, self._batch_key = AllreduceBatch(grads, inplace=True), key
+        return self._batch.submit()
 
     def _compute_fused(self, params):
         session, _ = mpi_ops._current()

@@ -32,6 +32,8 @@ EXPORTS = (
     "mpic_context_create", "mpic_context_add_input", "mpic_context_set_divisor", "mpic_context_compute", "mpic_context_wait",
     "mpic_context_message", "mpic_context_num_outputs", "mpic_context_output", "mpic_context_destroy",
     "mpic_allreduce_batch", "mpic_context_wait_batch",
+    "mpic_batch_create", "mpic_batch_size", "mpic_batch_submit", "mpic_batch_wait", "mpic_batch_message",
+    "mpic_batch_destroy",
     "mpic_ring_allreduce_prestaged", "mpic_ring_allreduce_direct_prestaged", "mpic_ring_allreduce_fused_prestaged",
     "mpic_ring_allgather_prestaged", "mpic_ring_allreduce_all_ranks",
     "mpic_ring_allgather_all_ranks", "mpic_ring_allreduce_transport", "mpic_ring_allgather_transport",
@@ -140,6 +142,12 @@ def load_library(name="libmpi_collectives.so", op_list=None):
             "mpic_context_destroy": (ci, [vp]),
             "mpic_allreduce_batch": (ci, [vp, ci, ci, ctypes.POINTER(cp), pint, pint, p64, pvp, pvp, ci, pvp]),
             "mpic_context_wait_batch": (ci, [pvp, ci, ci, pint]),
+            "mpic_batch_create": (ci, [vp, ci, ci, ctypes.POINTER(cp), pint, pint, p64, pvp, pvp, ci, pvp]),
+            "mpic_batch_size": (ci, [vp]),
+            "mpic_batch_submit": (ci, [vp]),
+            "mpic_batch_wait": (ci, [vp, pint]),
+            "mpic_batch_message": (cp, [vp, ci]),
+            "mpic_batch_destroy": (ci, [vp]),
             "mpic_ring_allreduce_prestaged": (ci, [ci, ci, ci, vp, vp, sz, pvp, pvp, vp, ci]),
             "mpic_ring_allreduce_direct_prestaged": (ci, [ci, ci, ci, vp, vp, sz, pvp, pvp, vp, ci]),
             "mpic_ring_allreduce_fused_prestaged": (ci, [vp, ci, ci, vp, pvp, pvp, vp, ci]),
@@ -349,3 +357,54 @@ class PendingBatch:
     @property
     def outputs(self):
         return self._outputs
+
+
+class Batch:
+    """k MPIAllreduce nodes of one rank built once and run every step
+    (mpic_batch_*): the kernels live as long as this object, as a TensorFlow
+    graph's nodes live as long as the graph; submit() runs each of them once
+    more on the same tensors. Keeps the tensors alive."""
+
+    def __init__(self, world, rank, node_names, inputs, outputs, divisor=0):
+        L = lib()
+        k = len(inputs)
+        self._inputs, self._outputs = inputs, outputs
+        self.node_names = node_names
+        self._k = k
+        names = (ctypes.c_char_p * max(k, 1))(*[n.encode() for n in node_names])
+        dtypes = (ctypes.c_int * max(k, 1))(*[TORCH2DT.get(t.dtype, 0) for t in inputs])
+        ndims = (ctypes.c_int * max(k, 1))(*[t.dim() for t in inputs])
+        flat_dims = [d for t in inputs for d in t.shape]
+        dims = (ctypes.c_int64 * max(len(flat_dims), 1))(*flat_dims)
+        ins = (ctypes.c_void_p * max(k, 1))(*[t.data_ptr() if t.numel() else None for t in inputs])
+        outs = (ctypes.c_void_p * max(k, 1))(*[t.data_ptr() if t.numel() else None for t in outputs])
+        self._handle = ctypes.c_void_p()
+        rc = L.mpic_batch_create(world, rank, k, names, dtypes, ndims, dims, ins, outs, divisor,
+                                 ctypes.byref(self._handle))
+        if rc != OK:
+            raise error_for(rc, "could not build a batch of %d allreduces (rank %d)" % (k, rank))
+        self._codes = (ctypes.c_int * max(k, 1))()
+
+    def submit(self):
+        rc = lib().mpic_batch_submit(self._handle)
+        if rc != OK:
+            raise error_for(rc, lib().mpic_last_error().decode() or "could not submit the batch")
+
+    def wait(self):
+        """Blocks until every node's done() has run. Returns None when all of
+        them ended OK, else a list with None or the OpError of each node."""
+        L = lib()
+        if L.mpic_batch_wait(self._handle, self._codes) == OK:
+            return None
+        return [None if self._codes[j] == OK
+                else error_for(self._codes[j], L.mpic_batch_message(self._handle, j).decode())
+                for j in range(self._k)]
+
+    @property
+    def outputs(self):
+        return self._outputs
+
+    def close(self):
+        if self._handle:
+            lib().mpic_batch_destroy(self._handle)      # waits for a submission that is still running
+            self._handle = ctypes.c_void_p()

@@ -121,6 +121,44 @@ int main() {
   }
   CHECK(mpic_world_destroy(w) == MPIC_OK);
 
+  // a rank's nodes built once and run again and again (mpic_batch_*): two ranks on two threads, shapes
+  // that differ in the second node, so each run ends with one OK-less node and its message; the
+  // nodes' done() calls race with the waiters
+  CHECK(mpic_world_create(2, &w) == MPIC_OK);
+  run_scalar(w, 0, "MPIInit");
+  {
+    mpic_batch* bs[2] = {nullptr, nullptr};
+    const char* names[3] = {"g0", "g1", "g2"};
+    const int dts[3] = {MPIC_DT_FLOAT, MPIC_DT_FLOAT, MPIC_DT_FLOAT}, nd[3] = {1, 1, 0};
+    for (int r = 0; r < 2; r++) {
+      const int64_t d[2] = {0, 3 + r};        // g0: empty on both ranks; g1: 3 against 4 elements; g2: a scalar
+      const void* ins[3] = {nullptr, buf, buf};
+      void* outs[3] = {nullptr, buf, buf};
+      CHECK(mpic_batch_create(w, r, 3, names, dts, nd, d, ins, outs, 0, &bs[r]) == MPIC_OK);
+      CHECK(mpic_batch_size(bs[r]) == 3);
+    }
+    CHECK(mpic_batch_create(w, 2, 3, names, dts, nd, nullptr, nullptr, nullptr, 0, &bs[0]) == MPIC_INVALID_ARGUMENT);
+    for (int round = 0; round < 50; round++) {
+      std::vector<std::thread> ts;
+      for (int r = 0; r < 2; r++) {
+        ts.emplace_back([&bs, r] {
+          CHECK(mpic_batch_submit(bs[r]) == MPIC_OK);
+          int codes[3] = {-1, -1, -1};
+          CHECK(mpic_batch_wait(bs[r], codes) != MPIC_OK);      // (without a GPU the valid nodes fail too, in their own way)
+          CHECK(codes[0] != -1 && codes[2] != -1 && codes[1] == MPIC_FAILED_PRECONDITION);
+          CHECK(std::strstr(mpic_batch_message(bs[r], 1), "Mismatched allreduce tensor shapes") != nullptr);
+        });
+      }
+      for (auto& t : ts) t.join();
+    }
+    // a submission nobody answers: the second submit is refused, destroying the world ends the first
+    CHECK(mpic_batch_submit(bs[0]) == MPIC_OK);
+    CHECK(mpic_batch_submit(bs[0]) == MPIC_FAILED_PRECONDITION);
+    CHECK(mpic_world_destroy(w) == MPIC_OK);
+    CHECK(mpic_batch_wait(bs[0], nullptr) == MPIC_UNKNOWN);
+    for (int r = 0; r < 2; r++) CHECK(mpic_batch_destroy(bs[r]) == MPIC_OK);
+  }
+
   // the in-process transport under concurrent ranks: every rank posts its
   // receives, sends to the right and waits, as the ring's steps do (zero-byte
   // messages: no device is touched)

@@ -1035,3 +1035,134 @@ def test_allreduce_batch_is_one_node_per_tensor(oracle):
                                oracle.ring_allreduce([ins[q][0].reshape(-1) for q in range(n)])[r], "first of the batch")
             with pytest.raises(mpi.FailedPreconditionError):
                 handles[r][1].result()
+
+
+def test_prepared_batch_runs_the_same_nodes_every_step(oracle):
+    """mpi.prepare_allreduce_batch: a rank's MPIAllreduce nodes built once (the
+    reference builds its graph once) and run on new values every step, in memory
+    of their own or in place; each step's results equal a loop over
+    mpi.allreduce, bit for bit, with and without the coordinator's fusion."""
+    n, steps = 4, 3
+    shapes = [(1000, 3), (0,), (70_001,), (5,), (128, 64)]
+    dtypes = [np.float32, np.float32, np.int32, np.int64, np.float32]
+
+    def values(step, r):
+        return [G.random_array(np.random.default_rng(1000 * step + 10 * r + j), int(np.prod(s)), dt).reshape(s)
+                for j, (s, dt) in enumerate(zip(shapes, dtypes))]
+
+    for inplace, fusion in ((False, 0), (True, 0), (False, 1 << 22), (True, 1 << 22)):
+        with mpi.Session(size=n, fusion_threshold=fusion) as session:
+            tensors = [[cuda(x) for x in values(0, r)] for r in range(n)]
+            batches = []
+            for r in range(n):
+                with session.as_rank(r):
+                    batches.append(mpi.prepare_allreduce_batch(tensors[r], average=True, inplace=inplace))
+            assert batches[0].node_names == batches[n - 1].node_names
+            for step in range(steps):
+                ins = [values(step, r) for r in range(n)]
+                for r in range(n):
+                    for t, x in zip(tensors[r], ins[r]):
+                        t.copy_(torch.from_numpy(x))
+                handles = [b.submit() for b in batches]
+                with pytest.raises(mpi.FailedPreconditionError):
+                    batches[0].submit()                     # still pending
+                outs = session.run(handles)
+                for j in range(len(shapes)):
+                    if fusion and dtypes[j] == np.float32:
+                        continue        # fused float32 sums round as the ring over the packed buffer does (checked below)
+                    want = oracle.ring_allreduce([ins[r][j].reshape(-1) for r in range(n)])
+                    for r in range(n):
+                        got = G.host(outs[r][j])
+                        assert tuple(got.shape) == shapes[j]
+                        G.assert_same_bits(got.reshape(-1), _tf_div(want[r], n),
+                                           "step %d tensor %d rank %d inplace=%s fusion=%d" % (step, j, r, inplace, fusion))
+                        if inplace:
+                            assert outs[r][j].data_ptr() == tensors[r][j].data_ptr()
+                if fusion:
+                    f32 = [j for j in range(len(shapes)) if dtypes[j] == np.float32]
+                    # consecutive ready allreduces of one type fuse: tensors 0 and 1; tensor 4 comes after the integers
+                    want = _expected_with_fusion(oracle, [[ins[r][j].reshape(-1) for j in f32] for r in range(n)],
+                                                 [[0, 1], [2]])
+                    for r in range(n):
+                        for k, j in enumerate(f32):
+                            G.assert_same_bits(G.host(outs[r][j]).reshape(-1), want[k] / np.float32(n),
+                                               "fused step %d tensor %d rank %d" % (step, j, r))
+
+
+def test_prepared_batch_mixes_with_single_ops_and_reports_one_bad_node(oracle):
+    """A prepared batch on some ranks and the same nodes submitted one by one on
+    the others meet under their node names; a node whose shape differs on one
+    rank fails alone, every step, with the reference's message."""
+    n = 3
+    xs = [[G.random_array(np.random.default_rng(7 * r + j), 5000 + j, np.float32) for j in range(3)] for r in range(n)]
+    with mpi.Session(size=n) as session:
+        handles = []
+        with session.as_rank(0):
+            batch = mpi.prepare_allreduce_batch([cuda(x) for x in xs[0]], average=False)
+            handles.append(batch.submit())
+        for r in (1, 2):
+            with session.as_rank(r):
+                handles.append([mpi.allreduce(cuda(x), average=False) for x in xs[r]])
+        outs = session.run(handles)
+        for j in range(3):
+            want = oracle.ring_allreduce([xs[r][j] for r in range(n)])
+            for r in range(n):
+                G.assert_same_bits(G.host(outs[r][j]), want[r], "mixed submission tensor %d rank %d" % (j, r))
+    with mpi.Session(size=n) as session:
+        batches = []
+        for r in range(n):
+            with session.as_rank(r):
+                ts = [cuda(xs[r][0]), cuda(xs[r][1] if r != 1 else xs[r][1][:17]), cuda(xs[r][2])]
+                batches.append(mpi.prepare_allreduce_batch(ts, average=False))
+        for step in range(2):
+            handles = [b.submit() for b in batches]
+            with pytest.raises(mpi.FailedPreconditionError) as e:
+                session.run()
+            assert "Mismatched allreduce tensor shapes" in str(e.value)
+            for r in range(n):
+                G.assert_same_bits(G.host(handles[r][0].result()), oracle.ring_allreduce([xs[q][0] for q in range(n)])[r],
+                                   "good node of a batch with a bad one")
+                with pytest.raises(mpi.FailedPreconditionError):
+                    handles[r][1].result()
+    with pytest.raises(mpi.FailedPreconditionError):
+        batches[0].submit()                                 # its session is closed
+
+
+def test_distributed_optimizer_builds_its_nodes_once(oracle):
+    """DistributedOptimizer over gradients that stay where they are
+    (zero_grad(set_to_none=False)): the allreduce nodes are built at the first
+    step and run again at the next ones, in place; every step's gradients are
+    the ring's averages and all replicas stay equal."""
+    n, steps = 3, 3
+    torch.manual_seed(3)
+    base = torch.nn.Sequential(torch.nn.Linear(29, 17), torch.nn.Tanh(), torch.nn.Linear(17, 4)).cuda()
+    replicas, opts = [], []
+    for r in range(n):
+        m = torch.nn.Sequential(torch.nn.Linear(29, 17), torch.nn.Tanh(), torch.nn.Linear(17, 4)).cuda()
+        m.load_state_dict(base.state_dict())
+        replicas.append(m)
+        opts.append(mpi.DistributedOptimizer(torch.optim.SGD(m.parameters(), lr=0.1)))
+    with mpi.Session(size=n) as session:
+        built = []
+        for step in range(steps):
+            local, gvs = [], []
+            for r in range(n):
+                with session.as_rank(r):
+                    opts[r].zero_grad(set_to_none=False)
+                    x = torch.randn(13, 29, generator=torch.Generator().manual_seed(100 * step + r)).cuda()
+                    replicas[r](x).square().mean().backward()
+                    local.append([G.host(p.grad).reshape(-1).copy() for p in replicas[r].parameters()])
+                    gvs.append(opts[r].compute_gradients())
+            session.run()
+            for r in range(n):
+                with session.as_rank(r):
+                    opts[r].apply_gradients(gvs[r])
+            built.append([id(o._batch) for o in opts])
+            for j in range(len(local[0])):
+                want = oracle.ring_allreduce([local[r][j] for r in range(n)])[0] / np.float32(n)
+                for r in range(n):
+                    G.assert_same_bits(G.host(list(replicas[r].parameters())[j].grad).reshape(-1), want,
+                                       "step %d rank %d gradient %d" % (step, r, j))
+            for p0, p1 in zip(replicas[0].parameters(), replicas[n - 1].parameters()):
+                assert torch.equal(p0, p1)
+        assert built[1] == built[2], "the nodes were rebuilt although the gradients stayed in place"
