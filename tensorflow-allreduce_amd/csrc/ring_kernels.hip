@@ -47,6 +47,11 @@ namespace {
 
 constexpr int kBlock = 256;   // threads per workgroup: 4 wave64
 constexpr int kMaxRows = 64;  // rows one launch carries in its kernel arguments
+// The scalar head of a step-table row brings its destination to a whole
+// 128-byte line, so that the 1 KiB a wave stores per access covers whole lines
+// (a 16-byte-aligned start would split a 32-byte sector at both ends of every
+// access: 3 % more sectors written, and partial ones).
+constexpr int kRowHeadAlign = 128;
 constexpr int kPacedUnroll = 8;  // vectors per lane per tile of the paced copy (32 KiB tiles)
 
 thread_local int g_last_hip_error = 0;
@@ -216,7 +221,7 @@ enum Anchor { kOnDst = 0, kOnSrc = 1 };
 // same time the chip then reads first and writes after, which HBM serves
 // faster than the two interleaved; the launcher picks it for those launches
 // only (a tile that has to wait for a free slot would pay for the short store queue).
-template <typename T, int OP, int UNROLL, int NT, int ANCHOR = kOnDst, int PACE = 0>
+template <typename T, int OP, int UNROLL, int NT, int ANCHOR = kOnDst, int PACE = 0, int HEAD_ALIGN = 16>
 __device__ __forceinline__ void row_tile(T* dst_, const T* a_, const T* b_, uint64_t count, uint32_t tile,
                                          uint32_t tiles_in_row, int n) {
   typedef typename VecOf<T>::type V;
@@ -234,7 +239,8 @@ __device__ __forceinline__ void row_tile(T* dst_, const T* a_, const T* b_, uint
   constexpr uint32_t kTileVecs = kBlock * UNROLL;
 
   const uintptr_t anchor = ANCHOR == kOnSrc ? reinterpret_cast<uintptr_t>(a_) : reinterpret_cast<uintptr_t>(dst_);
-  uint64_t head = ((16u - (static_cast<uint32_t>(anchor) & 15u)) & 15u) / sizeof(T);
+  constexpr uint32_t kAlign = HEAD_ALIGN;  // 16, or a whole 128-byte line (at most 31 scalar elements, fewer than a workgroup has lanes)
+  uint64_t head = ((kAlign - (static_cast<uint32_t>(anchor) & (kAlign - 1))) & (kAlign - 1)) / sizeof(T);
   if (head > count) head = count;
   const uint64_t nvec = (count - head) / VEC;
   const uint32_t tid = threadIdx.x;
@@ -318,12 +324,12 @@ __device__ __forceinline__ void run_row(const Row& r, uint32_t tile, uint32_t ti
   const T* b = static_cast<const T*>(r.b);
   // every condition is uniform over the workgroup (kernel arguments only)
   if (MODE == kAvg && divide) {
-    if (b != nullptr) row_tile<T, kOpAddDiv, UNROLL, NT>(dst, a, b, r.count, tile, tiles, divisor);
-    else row_tile<T, kOpDiv, UNROLL, NT>(dst, a, nullptr, r.count, tile, tiles, divisor);
+    if (b != nullptr) row_tile<T, kOpAddDiv, UNROLL, NT, kOnDst, 0, kRowHeadAlign>(dst, a, b, r.count, tile, tiles, divisor);
+    else row_tile<T, kOpDiv, UNROLL, NT, kOnDst, 0, kRowHeadAlign>(dst, a, nullptr, r.count, tile, tiles, divisor);
   } else if (MODE != kCopy && b != nullptr) {
-    row_tile<T, kOpAdd, UNROLL, NT>(dst, a, b, r.count, tile, tiles, 0);
+    row_tile<T, kOpAdd, UNROLL, NT, kOnDst, 0, kRowHeadAlign>(dst, a, b, r.count, tile, tiles, 0);
   } else {
-    row_tile<T, kOpCopy, UNROLL, NT, kOnDst, PACE>(dst, a, nullptr, r.count, tile, tiles, 0);
+    row_tile<T, kOpCopy, UNROLL, NT, kOnDst, PACE, kRowHeadAlign>(dst, a, nullptr, r.count, tile, tiles, 0);
   }
 }
 
@@ -911,7 +917,7 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
       const HostRow& r = rows[i];
       if (r.count == 0) { i++; continue; }
       const uintptr_t d = reinterpret_cast<uintptr_t>(r.dst);
-      uint64_t head = ((16u - (d & 15u)) & 15u) / esz;
+      uint64_t head = ((kRowHeadAlign - (d & (kRowHeadAlign - 1))) & (kRowHeadAlign - 1)) / esz;
       if (head > r.count) head = r.count;
       const uint64_t nvec = (r.count - head) / vec;
       uint64_t t = (nvec + tile_vecs - 1) / tile_vecs;
