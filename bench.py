@@ -26,6 +26,7 @@ The other workloads (--workload) time the remaining benchmark configurations
 the same way; they exist so that their profiles can be reproduced.
 """
 import argparse
+import gc
 import ctypes
 import json
 import os
@@ -719,6 +720,11 @@ def main():
         ring_abi.stream_synchronize(stream)
         torch.cuda.synchronize()
         samples = []
+        # a collection of the interpreter's garbage in the middle of the region stalls the
+        # launching thread for tens of milliseconds; workloads whose step is one short launch
+        # have no queue of launches ahead of the GPU to hide that behind
+        gc.collect()
+        gc.disable()
         t0 = time.perf_counter()
         launches = 2 if fused else nph
         for k in range(nsteps):
@@ -743,7 +749,9 @@ def main():
                 launch_step(k, stream, fused)
         ring_abi.stream_synchronize(stream)
         torch.cuda.synchronize()
-        return time.perf_counter() - t0, samples
+        elapsed = time.perf_counter() - t0
+        gc.enable()
+        return elapsed, samples
 
     if args.recorded:
         # `recorded` consecutive steps (rotating over the buffer sets) as one HIP graph, replayed
