@@ -247,11 +247,14 @@ int mpic_ring_allgather_prestaged(int n, int r, int dtype, const void* input, co
                                   const void* const* segments, void* stream, int flags);
 /* All n ranks resident on this GPU: inputs[k] / outputs[k] are rank k's
  * tensors; a neighbour's buffer is read in place of a transfer. `flags` bit 2:
- * the direct form (every segment folded by its owner in one launch, every
- * finished segment copied straight from its owner in a second; for the
- * allgather, every slice copied from its owner's input into every output in
- * one launch). An allreduce of more than 256 ranks runs the lockstep ring
- * whatever bit 2 says (a fold launch addresses at most 256 copies). */
+ * the direct form: every segment folded by its owner in ring order and the
+ * result stored into every rank's output by the same pass, ONE launch for the
+ * whole allreduce (up to 128 ranks; from 129 to 256 the fold and the copies of
+ * the finished segments are two launches); for the allgather, every slice
+ * copied from its owner's input into every output in one launch. inputs[k] may
+ * be outputs[k] (an allreduce in place). An allreduce of more than 256 ranks
+ * runs the lockstep ring whatever bit 2 says (a fold launch addresses at most
+ * 256 pointers). */
 int mpic_ring_allreduce_all_ranks(int n, int dtype, const void* const* inputs,
                                   void* const* outputs, size_t count, void* stream, int flags);
 int mpic_ring_allgather_all_ranks(int n, int dtype, const void* const* inputs, const size_t* rows,

@@ -73,12 +73,13 @@ size_t ring_dtype_size(int dtype);
  * launch: "nontemporal_copy" (ring_copy_bytes), "nontemporal_accumulate"
  * (accumulates, reduce-scatter tables, row tables, scale),
  * "nontemporal_allgather" (copy tables), "nontemporal_pack",
- * "nontemporal_unpack", "nontemporal_fold", "nontemporal_broadcast" (copy
+ * "nontemporal_unpack", "nontemporal_fold", "nontemporal_fold_all" (a fold
+ * stored to every rank), "nontemporal_broadcast" (copy
  * rows of one call that share a source); value bit 0 = non-temporal stores,
  * bit 1 = non-temporal loads, -1 = the default: 3, except ordinary stores
  * where the next kernel reads the output (copy, pack, fold), ordinary loads
  * for a source several rows share (broadcast), and loads by size for the copy.
- * "nontemporal" sets all seven. "paced_copy": the copies of an allgather
+ * "nontemporal" sets all eight. "paced_copy": the copies of an allgather
  * phase as one read phase and one write phase (every workgroup waits for all
  * its loads, then keeps one store in flight per wave): 1 always, 0 never,
  * -1 (default) when every tile of the launch is on the chip at the same time
@@ -280,6 +281,24 @@ int ring_fold_rows(const ring_fold_row* rows, int n_rows, int m, int divisor, in
  * drain of a second. */
 int ring_fold_and_copy_rows(const ring_fold_row* fold_rows, int n_fold, int m, int divisor,
                             const ring_row* copy_rows, int n_copy, int dtype, void* stream);
+/* The fold of a row stored to n_dst destinations at once: where the ranks of a
+ * ring share a GPU (or an owner can write into its peers' memory), the owner
+ * of a segment hands the finished segment to every rank in the pass that
+ * reduces it, instead of each rank copying it from the owner afterwards
+ * (ring.h:211-225 moves the same values round the ring in n-1 steps). n reads
+ * and n_dst writes per element, one launch for a whole allreduce of all
+ * ranks. dsts[0] is the destination whose alignment the vector stores follow;
+ * the others need only be element-aligned. Any destination may be one of the
+ * row's own sources (an allreduce in place): a lane reads every source of its
+ * elements before it stores them. m + n_dst - 1 <= 256. `rows`, `dsts` and
+ * `srcs` are HOST arrays. No counterpart in the reference. */
+typedef struct ring_fold_to_all_row {
+  void* const* dsts;       /* n_dst device pointers */
+  const void* const* srcs; /* m device pointers, in fold order */
+  uint64_t count;          /* elements */
+} ring_fold_to_all_row;
+int ring_fold_to_all_rows(const ring_fold_to_all_row* rows, int n_rows, int m, int n_dst, int divisor, int dtype,
+                          void* stream);
 
 /* ---- tensor fusion (no counterpart in the reference, which issues one
  * MPIAllreduce per gradient, __init__.py:195-205): k tensors are packed back

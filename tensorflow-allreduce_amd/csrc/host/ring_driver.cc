@@ -330,8 +330,30 @@ Status RingAllreduceAllRanks(int n, DataType dt, const void* const* inputs, void
 
   // The fold kernel carries at most kMaxDirectRanks source pointers per launch; a
   // larger ring runs the lockstep form below, which handles any n (ring.h:136-228).
+  if (opts.direct && 2 * n - 1 <= kMaxDirectRanks) {
+    // One launch for the whole allreduce: the owner of every segment folds the n
+    // copies in ring order and stores the result into every rank's output. Rank
+    // (seg-1) owns segment seg; its own output leads the destinations.
+    std::vector<std::vector<const void*>> srcs(static_cast<size_t>(n));
+    std::vector<std::vector<void*>> dsts(static_cast<size_t>(n));
+    std::vector<ring_fold_to_all_row> folds;
+    for (int j = 0; j < n; j++) {
+      const size_t seg = static_cast<size_t>((j + 1) % n);
+      for (int k = 0; k < n; k++) {
+        srcs[static_cast<size_t>(j)].push_back(at(inputs[(static_cast<int>(seg) + k) % n], starts[seg], esz));
+        dsts[static_cast<size_t>(j)].push_back(at(outputs[(j + k) % n], starts[seg], esz));
+      }
+      folds.push_back(ring_fold_to_all_row{dsts[static_cast<size_t>(j)].data(), srcs[static_cast<size_t>(j)].data(),
+                                           sizes[seg]});
+    }
+    if (!(n == 1 && inputs[0] == outputs[0] && opts.divisor == 0))
+      RING_RETURN_IF_ERROR(ring_fold_to_all_rows(folds.data(), n, n, n, opts.divisor, code, stream),
+                           "ring_fold_to_all_rows");
+    return Status::OK();
+  }
   if (opts.direct && n <= kMaxDirectRanks) {
-    // One launch: the owner of every segment folds the n copies in ring order.
+    // More ranks than one row's pointers hold twice over: the owner of every
+    // segment folds the n copies in ring order (one launch) ...
     std::vector<std::vector<const void*>> srcs(static_cast<size_t>(n));
     std::vector<ring_fold_row> folds;
     for (int j = 0; j < n; j++) {
@@ -340,9 +362,8 @@ Status RingAllreduceAllRanks(int n, DataType dt, const void* const* inputs, void
         srcs[static_cast<size_t>(j)].push_back(at(inputs[(static_cast<int>(seg) + k) % n], starts[seg], esz));
       folds.push_back(ring_fold_row{at(outputs[j], starts[seg], esz), srcs[static_cast<size_t>(j)].data(), sizes[seg]});
     }
-    if (!(n == 1 && inputs[0] == outputs[0] && opts.divisor == 0))
-      RING_RETURN_IF_ERROR(ring_fold_rows(folds.data(), n, n, opts.divisor, code, stream), "ring_fold_rows");
-    // One more: every rank copies each finished segment from its owner.
+    RING_RETURN_IF_ERROR(ring_fold_rows(folds.data(), n, n, opts.divisor, code, stream), "ring_fold_rows");
+    // ... and every rank copies each finished segment from its owner (one more).
     std::vector<ring_row> copies;
     for (int r = 0; r < n; r++) {
       for (int seg = 0; seg < n; seg++) {

@@ -36,10 +36,12 @@ struct RingOptions {
   // segments are therefore expected divided, as a peer would send them.
   int divisor = 0;
   // Where every rank's copy of a segment is addressable at once: its owner
-  // folds the n copies in ring order in one pass (ring_fold_rows) instead of
-  // n-1 accumulate steps, and every rank copies each finished segment straight
-  // from its owner instead of passing it round. Same additions in the same
-  // order, so the same bits; 2 launches instead of 2(n-1)+1.
+  // folds the n copies in ring order in one pass instead of n-1 accumulate
+  // steps. A rank with pre-staged peers then copies each finished segment
+  // straight from where it was pushed; ranks that share the GPU get the result
+  // stored into all their outputs by the fold itself (ring_fold_to_all_rows).
+  // Same additions in the same order, so the same bits; 1 launch (2 beyond 128
+  // ranks) instead of 2(n-1)+1.
   bool direct = false;
   // Transport-driven rings only: pieces a segment travels in (1..16).
   int chunks = 1;

@@ -396,12 +396,17 @@ constexpr int kMaxFoldPtrs = 256;
 // per lane (half as many workgroups) 17.3-18.0.
 constexpr int kFoldUnroll = 2;
 constexpr int kFoldGroup = 8;
+// A fold that stores its result to every rank (8 sources, 8 destinations of
+// 64 MiB): 1 vector per lane 194 us, 2 vectors 199 us, 4 vectors 213 us.
+constexpr int kFoldToAllUnroll = 1;
 
 struct FoldRow {
   void* dst;
   uint64_t count;      // elements
   uint32_t first_ptr;  // index of the row's first source in FoldTable::src
   uint32_t m;          // sources, folded in the order they are listed; 1 = a copy row
+  uint32_t first_dst;  // index in FoldTable::src of the row's further destinations
+  uint32_t n_more;     // how many: the result is stored to dst and to each of them
 };
 struct FoldTable {
   int n_rows;
@@ -410,15 +415,20 @@ struct FoldTable {
   uint32_t uniform_tiles;  // as RowTable
   uint32_t tile_begin[kMaxFoldRows + 1];
   FoldRow row[kMaxFoldRows];
-  const void* src[kMaxFoldPtrs];
+  const void* src[kMaxFoldPtrs];  // the rows' sources, and their further destinations
 };
 
 // One tile of a fold row. dst may be one of the row's own sources: a lane reads
 // every source of its elements before it stores them. DIV && divide: the fold
 // is divided by n before it is stored (divide is uniform over the workgroup).
+// more[0..n_more): further destinations of the same result (every rank's copy
+// of a finished segment, written by the owner's fold instead of being copied
+// from it afterwards); they may be sources of the row too, and need only be
+// element-aligned.
 template <typename T, int UNROLL, int GROUP, bool DIV, int NT>
 __device__ __forceinline__ void fold_tile(T* dst, const void* const* src, int m, uint64_t count, uint32_t tile,
-                                          uint32_t tiles_in_row, int n, bool divide) {
+                                          uint32_t tiles_in_row, int n, bool divide,
+                                          const void* const* more = nullptr, int n_more = 0) {
   typedef typename VecOf<T>::type V;
   typedef V VU __attribute__((aligned(sizeof(T))));
   constexpr uint32_t VEC = 16 / sizeof(T);
@@ -434,7 +444,9 @@ __device__ __forceinline__ void fold_tile(T* dst, const void* const* src, int m,
   auto scalar = [&](uint64_t e) {
     T acc = static_cast<const T*>(src[0])[e];
     for (int k = 1; k < m; k++) acc = add_one(acc, static_cast<const T*>(src[k])[e]);
-    dst[e] = (DIV && divide) ? div_one(acc, n) : acc;
+    const T r = (DIV && divide) ? div_one(acc, n) : acc;
+    dst[e] = r;
+    for (int d = 0; d < n_more; d++) static_cast<T*>(const_cast<void*>(more[d]))[e] = r;
   };
   if (tile == 0 && tid < head) scalar(tid);
   if (tile + 1 == tiles_in_row) {
@@ -483,6 +495,12 @@ __device__ __forceinline__ void fold_tile(T* dst, const void* const* src, int m,
       RING_STORE_VEC(NT, &dv[v0 + j * kBlock], acc[j]);
     }
   }
+  for (int d = 0; d < n_more; d++) {  // uniform
+    VU* ov = reinterpret_cast<VU*>(static_cast<T*>(const_cast<void*>(more[d])) + head);
+#pragma unroll
+    for (int j = 0; j < UNROLL; j++)
+      if (ok[j]) RING_STORE_VEC(NT, &ov[v0 + j * kBlock], acc[j]);
+  }
 }
 
 // A row with one source and no divide is a plain copy (the finished segments a
@@ -497,7 +515,8 @@ __device__ __forceinline__ void fold_row_tile(const FoldTable& tab, int row, uin
                                           0, false);
   else
     fold_tile<T, UNROLL, GROUP, DIV, NT>(static_cast<T*>(r.dst), tab.src + r.first_ptr, static_cast<int>(r.m), r.count,
-                                         tile, tiles_in_row, tab.divisor, divide);
+                                         tile, tiles_in_row, tab.divisor, divide, tab.src + r.first_dst,
+                                         static_cast<int>(r.n_more));
 }
 
 template <typename T, bool DIV, int NT, int UNROLL, int GROUP>
@@ -762,7 +781,9 @@ fusion_span_kernel(const uint64_t* __restrict__ offsets, T* const* __restrict__ 
 
 constexpr uint64_t kCacheResidentBytes = 128ull << 20;
 
-enum Role { kRoleCopy, kRoleAccumulate, kRoleAllgather, kRolePack, kRoleUnpack, kRoleFold, kRoleBroadcast, kRoles };
+enum Role {
+  kRoleCopy, kRoleAccumulate, kRoleAllgather, kRolePack, kRoleUnpack, kRoleFold, kRoleBroadcast, kRoleFoldAll, kRoles
+};
 
 struct Tuning {
   int unroll = 4;          // 16-byte vectors per lane per tile: 2, 4 or 8
@@ -776,7 +797,8 @@ struct Tuning {
   // the fold's result is what the allgather reads next; a source that several
   // rows copy (a finished segment fetched by every other rank) is loaded with
   // the ordinary policy so that it is fetched from HBM once
-  int nt[kRoles] = {-1, 3, 3, 2, 3, 2, 1};
+  // (a fold that stores its result to every rank writes final outputs: touched once)
+  int nt[kRoles] = {-1, 3, 3, 2, 3, 2, 1, 3};
   // Allgather copies whose tiles all fit on the chip at once run as one read
   // phase and one write phase (rows_kernel's PACE): -1 chosen by the size of
   // the launch, 0 never, 1 always.
@@ -1209,7 +1231,7 @@ int ring_set_option(const char* name, int value) {
     g_tuning.paced_copy = value;
   } else if (!strncmp(name, "nontemporal", 11)) {
     static const char* const kSuffix[kRoles] = {"_copy", "_accumulate", "_allgather", "_pack", "_unpack",
-                                                "_fold", "_broadcast"};
+                                                "_fold", "_broadcast", "_fold_all"};
     if (value < -1 || value > 3) return RING_ERR_ARGUMENT;
     const Tuning defaults;
     bool known = name[11] == 0;
@@ -1483,16 +1505,20 @@ struct HostFoldRow {
   int m;
   uint64_t count;
   bool divide;
+  void* const* more = nullptr;  // further destinations of the result
+  int n_more = 0;
 };
 
 // Launches fold rows (any number, any mix of source counts) in tables of at most
 // kMaxFoldRows rows and kMaxFoldPtrs source pointers.
 int launch_fold(const HostFoldRow* rows, size_t n_rows, int divisor, int dtype, hipStream_t s) {
   const size_t esz = dtype_size(dtype);
-  constexpr uint64_t kTileVecs = static_cast<uint64_t>(kBlock) * kFoldUnroll;
   const uint64_t vec = 16 / esz;
-  int nt = g_tuning.nt[kRoleFold];
-  if (nt < 0) nt = 2;
+  bool to_all = false;
+  for (size_t k = 0; k < n_rows; k++) to_all = to_all || rows[k].n_more > 0;
+  const uint64_t kTileVecs = static_cast<uint64_t>(kBlock) * (to_all ? kFoldToAllUnroll : kFoldUnroll);
+  int nt = g_tuning.nt[to_all ? kRoleFoldAll : kRoleFold];
+  if (nt < 0) nt = to_all ? 3 : 2;
   size_t i = 0;
   while (i < n_rows) {
     FoldTable tab;
@@ -1507,8 +1533,8 @@ int launch_fold(const HostFoldRow* rows, size_t n_rows, int divisor, int dtype, 
     while (i < n_rows && tab.n_rows < kMaxFoldRows) {
       const HostFoldRow& r = rows[i];
       if (r.count == 0) { i++; continue; }
-      if (r.m < 1 || r.m > kMaxFoldPtrs) return RING_ERR_ARGUMENT;
-      if (ptrs + static_cast<uint32_t>(r.m) > static_cast<uint32_t>(kMaxFoldPtrs)) break;  // next table
+      if (r.m < 1 || r.n_more < 0 || r.m + r.n_more > kMaxFoldPtrs) return RING_ERR_ARGUMENT;
+      if (ptrs + static_cast<uint32_t>(r.m + r.n_more) > static_cast<uint32_t>(kMaxFoldPtrs)) break;  // next table
       if (!r.dst || !r.srcs || (reinterpret_cast<uintptr_t>(r.dst) & (esz - 1))) return RING_ERR_ARGUMENT;
       const uintptr_t d = reinterpret_cast<uintptr_t>(r.dst);
       uint64_t head = ((16u - (d & 15u)) & 15u) / esz;
@@ -1520,10 +1546,15 @@ int launch_fold(const HostFoldRow* rows, size_t n_rows, int divisor, int dtype, 
         break;
       }
       const int k = tab.n_rows++;
-      tab.row[k] = FoldRow{r.dst, r.count, ptrs, static_cast<uint32_t>(r.m)};
+      tab.row[k] = FoldRow{r.dst, r.count, ptrs, static_cast<uint32_t>(r.m),
+                           ptrs + static_cast<uint32_t>(r.m), static_cast<uint32_t>(r.n_more)};
       for (int j = 0; j < r.m; j++) {
         if (!r.srcs[j] || (reinterpret_cast<uintptr_t>(r.srcs[j]) & (esz - 1))) return RING_ERR_ARGUMENT;
         tab.src[ptrs++] = r.srcs[j];
+      }
+      for (int j = 0; j < r.n_more; j++) {
+        if (!r.more[j] || (reinterpret_cast<uintptr_t>(r.more[j]) & (esz - 1))) return RING_ERR_ARGUMENT;
+        tab.src[ptrs++] = r.more[j];
       }
       if (divisor > 0 && r.divide) tab.div_mask |= 1u << k;
       if (k == 0) first_tiles = t;
@@ -1541,7 +1572,9 @@ int launch_fold(const HostFoldRow* rows, size_t n_rows, int divisor, int dtype, 
       tab.uniform_tiles = 0;
       grid = dim3(static_cast<uint32_t>(tiles));
     }
-#define RING_FOLD_UG(T, D, N) launch(fold_kernel<T, D, N, kFoldUnroll, kFoldGroup>, grid, dim3(kBlock), s, tab);
+#define RING_FOLD_UG(T, D, N)                                                                      \
+  if (to_all) launch(fold_kernel<T, D, N, kFoldToAllUnroll, kFoldGroup>, grid, dim3(kBlock), s, tab); \
+  else launch(fold_kernel<T, D, N, kFoldUnroll, kFoldGroup>, grid, dim3(kBlock), s, tab);
 #define RING_FOLD(T, D)                          \
   switch (nt & 3) {                              \
     case 0: RING_FOLD_UG(T, D, 0) break;         \
@@ -1586,6 +1619,22 @@ int ring_fold_and_copy_rows(const ring_fold_row* fold_rows, int n_fold, int m, i
     host.data[n_host++] = HostFoldRow{copy_rows[i].dst, &copy_rows[i].a, 1, copy_rows[i].count, false};
   }
   return launch_fold(host.data, n_host, divisor, dtype, static_cast<hipStream_t>(stream));
+}
+
+int ring_fold_to_all_rows(const ring_fold_to_all_row* rows, int n_rows, int m, int n_dst, int divisor, int dtype,
+                          void* stream) {
+  if (!dtype_ok(dtype)) return RING_ERR_DTYPE;
+  if (n_rows < 0 || divisor < 0 || (n_rows > 0 && !rows)) return RING_ERR_ARGUMENT;
+  if (n_rows > 0 && (m < 1 || n_dst < 1 || m + n_dst - 1 > kMaxFoldPtrs)) return RING_ERR_ARGUMENT;
+  RowBuffer<HostFoldRow, kMaxRows> host(static_cast<size_t>(n_rows));
+  for (int i = 0; i < n_rows; i++) {
+    if (rows[i].count > 0 && (!rows[i].dsts || !rows[i].srcs)) return RING_ERR_ARGUMENT;
+    HostFoldRow r{rows[i].count > 0 ? rows[i].dsts[0] : nullptr, rows[i].srcs, m, rows[i].count, true};
+    r.more = rows[i].count > 0 ? rows[i].dsts + 1 : nullptr;
+    r.n_more = n_dst - 1;
+    host.data[i] = r;
+  }
+  return launch_fold(host.data, static_cast<size_t>(n_rows), divisor, dtype, static_cast<hipStream_t>(stream));
 }
 
 int ring_scale(int dtype, void* data, size_t count, int divisor, void* stream) {

@@ -22,7 +22,7 @@ EXPORTS = (
     "ring_schedule", "ring_stream_create", "ring_stream_destroy", "ring_stream_synchronize",
     "ring_copy_bytes", "ring_accumulate_f32", "ring_accumulate_i32", "ring_accumulate_i64",
     "ring_accumulate", "ring_reduce_scatter_steps", "ring_reduce_scatter_steps_from",
-    "ring_allgather_steps", "ring_apply_rows", "ring_apply_rows_avg", "ring_fold_rows", "ring_fold_and_copy_rows",
+    "ring_allgather_steps", "ring_apply_rows", "ring_apply_rows_avg", "ring_fold_rows", "ring_fold_and_copy_rows", "ring_fold_to_all_rows",
     "ring_fusion_plan_create", "ring_fusion_plan_destroy", "ring_fusion_plan_elements", "ring_fusion_plan_dtype",
     "ring_fusion_pack", "ring_fusion_unpack", "ring_fusion_unpack_scaled", "ring_fusion_gather",
     "ring_fusion_scatter", "ring_scale", "ring_fusion_run_static",
@@ -56,6 +56,12 @@ _lib = None
 class FoldRow(ctypes.Structure):
     """ring_fold_row: dst = srcs[m-1] + (... + (srcs[1] + srcs[0]))."""
     _fields_ = [("dst", ctypes.c_void_p), ("srcs", ctypes.POINTER(ctypes.c_void_p)), ("count", ctypes.c_uint64)]
+
+
+class FoldToAllRow(ctypes.Structure):
+    """ring_fold_to_all_row: the fold of srcs stored to every pointer of dsts."""
+    _fields_ = [("dsts", ctypes.POINTER(ctypes.c_void_p)), ("srcs", ctypes.POINTER(ctypes.c_void_p)),
+                ("count", ctypes.c_uint64)]
 
 
 class FusionSpan(ctypes.Structure):
@@ -121,6 +127,7 @@ def lib():
             "ring_apply_rows_avg": (ci, [ctypes.POINTER(Row), ci, ctypes.POINTER(ctypes.c_ubyte), ci, ci, vp]),
             "ring_fold_rows": (ci, [ctypes.POINTER(FoldRow), ci, ci, ci, ci, vp]),
             "ring_fold_and_copy_rows": (ci, [ctypes.POINTER(FoldRow), ci, ci, ci, ctypes.POINTER(Row), ci, ci, vp]),
+            "ring_fold_to_all_rows": (ci, [ctypes.POINTER(FoldToAllRow), ci, ci, ci, ci, ci, vp]),
             "ring_fusion_plan_create": (ci, [ctypes.POINTER(vp), psz, ci, ci, ctypes.POINTER(vp)]),
             "ring_fusion_plan_destroy": (ci, [vp]),
             "ring_fusion_plan_elements": (sz, [vp]),
@@ -307,6 +314,21 @@ def fold_and_copy_rows(fold, m, divisor, copies, dtype, stream):
         carr[i].dst, carr[i].a, carr[i].b, carr[i].count = d, a, None, cnt
     check(lib().ring_fold_and_copy_rows(arr, n, m, divisor, carr, len(copies), dtype, stream),
           "ring_fold_and_copy_rows")
+
+
+def fold_to_all_rows(rows, m, n_dst, divisor, dtype, stream):
+    """rows: iterable of ([n_dst destination pointers], [m source pointers in fold order], count)."""
+    rows = list(rows)
+    arr = (FoldToAllRow * max(len(rows), 1))()
+    keep = []
+    for i, (dsts, srcs, cnt) in enumerate(rows):
+        d = (ctypes.c_void_p * n_dst)(*dsts)
+        p = (ctypes.c_void_p * m)(*srcs)
+        keep += [d, p]
+        arr[i].dsts = ctypes.cast(d, ctypes.POINTER(ctypes.c_void_p))
+        arr[i].srcs = ctypes.cast(p, ctypes.POINTER(ctypes.c_void_p))
+        arr[i].count = cnt
+    check(lib().ring_fold_to_all_rows(arr, len(rows), m, n_dst, divisor, dtype, stream), "ring_fold_to_all_rows")
 
 
 def scale(dtype, data, count, divisor, stream):

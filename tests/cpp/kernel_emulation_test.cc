@@ -217,6 +217,57 @@ void test_fold(int m, size_t count, int divisor) {
   cdst.check_lead();
 }
 
+// The fold of m sources stored to n_dst destinations of any element alignment, two rows of
+// different lengths in one call; then the same in place (every destination is a source).
+template <typename T>
+void test_fold_to_all(int m, int n_dst, size_t count, int divisor) {
+  std::vector<Buf<T>> keep;
+  keep.reserve(2 * (m + n_dst) + 4 * m);
+  std::vector<std::vector<const void*>> srcs(2);
+  std::vector<std::vector<void*>> dsts(2);
+  std::vector<std::vector<T>> wants(2);
+  const size_t counts[2] = {count, count / 3 + 1};
+  std::vector<ring_fold_to_all_row> rows;
+  for (int q = 0; q < 2; q++) {
+    for (int k = 0; k < m; k++) {
+      keep.emplace_back(counts[q], (k + q) % 4);
+      srcs[q].push_back(keep.back().p);
+    }
+    for (int d = 0; d < n_dst; d++) {
+      keep.emplace_back(counts[q], (d + 2 * q + 1) % 4, false);
+      dsts[q].push_back(keep.back().p);
+    }
+    wants[q].resize(counts[q]);
+    for (size_t i = 0; i < counts[q]; i++) {
+      T acc = static_cast<const T*>(srcs[q][0])[i];
+      for (int k = 1; k < m; k++) acc = add(acc, static_cast<const T*>(srcs[q][k])[i]);
+      wants[q][i] = divisor ? divide(acc, divisor) : acc;
+    }
+    rows.push_back(ring_fold_to_all_row{dsts[q].data(), srcs[q].data(), counts[q]});
+  }
+  OK(ring_fold_to_all_rows(rows.data(), 2, m, n_dst, divisor, code<T>(), nullptr));
+  for (int q = 0; q < 2; q++)
+    for (int d = 0; d < n_dst; d++) expect_equal(static_cast<T*>(dsts[q][d]), wants[q], "fold stored to every destination");
+  for (auto& b : keep) b.check_lead();
+  // in place: an allreduce of m ranks whose outputs are their inputs
+  std::vector<const void*> in_place_src;
+  std::vector<void*> in_place_dst;
+  for (int k = 0; k < m; k++) {
+    keep.emplace_back(count, k % 4);
+    in_place_src.push_back(keep.back().p);
+    in_place_dst.push_back(keep.back().p);
+  }
+  std::vector<T> want(count);
+  for (size_t i = 0; i < count; i++) {
+    T acc = static_cast<const T*>(in_place_src[0])[i];
+    for (int k = 1; k < m; k++) acc = add(acc, static_cast<const T*>(in_place_src[k])[i]);
+    want[i] = divisor ? divide(acc, divisor) : acc;
+  }
+  ring_fold_to_all_row row{in_place_dst.data(), in_place_src.data(), count};
+  OK(ring_fold_to_all_rows(&row, 1, m, m, divisor, code<T>(), nullptr));
+  for (int k = 0; k < m; k++) expect_equal(static_cast<T*>(in_place_dst[k]), want, "fold to all, in place");
+}
+
 // Pack, unpack (divided or not), gather and scatter over a tensor set, through a
 // plan and through the static device table.
 template <typename T>
@@ -339,6 +390,9 @@ void run_all(const char* name) {
   test_fold<T>(8, 10007, 0);
   test_fold<T>(3, 4096, 3);
   test_fold<T>(17, 777, 8);
+  test_fold_to_all<T>(8, 8, 10007, 8);
+  test_fold_to_all<T>(3, 5, 4099, 0);
+  test_fold_to_all<T>(1, 2, 700, 3);
   printf("%s: fusion\n", name); fflush(stdout);
   test_fusion<T>({5, 0, 4099, 1, 64, 0, 3}, 0, 3);
   test_fusion<T>({20000, 64, 64, 36864, 64, 64, 9001, 2, 12288}, 8, 8);

@@ -321,6 +321,50 @@ def test_fold_rows_is_the_sequential_fold(dtype):
         ring_abi.fold_rows([(x.data_ptr(), [x.data_ptr()], 8)], 1, -1, code, None)
 
 
+@pytest.mark.parametrize("dtype", G.DTYPES)
+def test_fold_stored_to_every_rank(dtype):
+    """ring_fold_to_all_rows: the numpy fold in the same order, stored to n_dst
+    destinations of differing alignment; rows of unequal length, the divide, an
+    allreduce in place (every destination is a source), more pointers than one
+    launch's table holds."""
+    rng = np.random.default_rng(7)
+    code = G.NP2ABI[np.dtype(dtype)]
+    for m, n_dst, counts in ((1, 1, [33]), (2, 3, [4099, 0, 12]), (8, 8, [30_011] * 8), (5, 7, [9000, 5, 2049]),
+                             (40, 40, [1500] * 6), (128, 129, [777])):
+        for divisor in (0, 6):
+            rows, checks, keep = [], [], []
+            for k, c in enumerate(counts):
+                hs = [G.random_array(rng, c, dtype, wide=dtype == np.float32) for _ in range(m)]
+                if dtype != np.float32 and c:
+                    hs[0][: c // 2] = -np.abs(hs[0][: c // 2]) - 7
+                ds = [G.dev(h, (k + j) % 4) for j, h in enumerate(hs)]
+                outs = [G.dev(np.zeros(c, dtype=dtype), (k + 3 * j + 1) % 4) for j in range(n_dst)]
+                keep += [ds, outs]
+                rows.append(([o[0].data_ptr() if c else None for o in outs], [d[0].data_ptr() if c else None for d in ds], c))
+                want = _fold_reference(hs, divisor, dtype)
+                checks += [(o[0], want, "row %d destination %d" % (k, j)) for j, o in enumerate(outs)]
+            ring_abi.fold_to_all_rows(rows, m, n_dst, divisor, code, None)
+            G.sync()
+            for t, want, what in checks:
+                G.assert_same_bits(G.host(t), want, "fold to all m=%d n_dst=%d /%d %s" % (m, n_dst, divisor, what))
+    # in place: 6 ranks whose outputs are their inputs, two segments
+    for divisor in (0, 6):
+        hs = [[G.random_array(rng, c, dtype) for _ in range(6)] for c in (20_011, 4097)]
+        ds = [[G.dev(h, j % 4) for j, h in enumerate(seg)] for seg in hs]
+        rows = [([d[0].data_ptr() for d in seg], [d[0].data_ptr() for d in seg], seg[0][0].numel()) for seg in ds]
+        ring_abi.fold_to_all_rows(rows, 6, 6, divisor, code, None)
+        G.sync()
+        for seg_h, seg_d in zip(hs, ds):
+            want = _fold_reference(seg_h, divisor, dtype)
+            for j, d in enumerate(seg_d):
+                G.assert_same_bits(G.host(d[0]), want, "in place, rank %d /%d" % (j, divisor))
+    x, _ = G.dev(np.ones(8, dtype=dtype), 0)
+    with pytest.raises(ring_abi.RingError):
+        ring_abi.fold_to_all_rows([([x.data_ptr()] * 129, [x.data_ptr()] * 129, 8)], 129, 129, 0, code, None)
+    with pytest.raises(ring_abi.RingError):
+        ring_abi.fold_to_all_rows([([None], [x.data_ptr()], 8)], 1, 1, 0, code, None)
+
+
 def test_fold_and_average_on_special_float_values():
     """Denormals, signed zeros, infinities, NaN, the largest finite value: the
     fold, the add-and-divide row and the divided scatter give numpy's bits
