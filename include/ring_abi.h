@@ -368,6 +368,22 @@ int ring_fusion_gather(const ring_fusion_plan* plan, const ring_fusion_span* spa
 int ring_fusion_scatter(const ring_fusion_plan* plan, const ring_fusion_span* spans, int n_spans, int divisor,
                         void* stream);
 
+/* The fused allreduce of n ranks that share the GPU, without a fused buffer:
+ * in_plans[k] / out_plans[k] are plans over rank k's input and output tensors
+ * (the same plan for an allreduce in place), all with the same element type
+ * and the same tensor sizes in the same order, i.e. one fused element space.
+ * One launch computes what pack, the ring over the packed buffers and unpack
+ * compute: element e of the space lies in ring segment s of the packed layout
+ * (ring_segment_table of the total), every rank's tensor receives the ring's
+ * fold of the n values in the order s, s+1, ..., s+n-1 (mod n), divided by
+ * `divisor` when it is > 0 (tf.div, as ring_fusion_unpack_scaled). Each
+ * tensor's result is bit-identical to the reference ring applied to the packed
+ * buffer; the tensors are read once and written once. 1 <= n <= 16
+ * (RING_ERR_LIMIT beyond). `in_plans` and `out_plans` are HOST arrays. No
+ * counterpart in the reference. */
+int ring_fusion_allreduce_all(const ring_fusion_plan* const* in_plans, const ring_fusion_plan* const* out_plans, int n,
+                              int divisor, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -323,6 +323,13 @@ void PerformCollectiveOp(mpic_world* w, const MPIResponse& response) {
   FinishRecords(&records, &callbacks, status);
 }
 
+constexpr size_t kMaxCachedFusionPlans = 256;
+void DropFusionPlans(mpic_world* w) {
+  ring_stream_synchronize(w->stream);  // launches in flight still read the plans' device tables
+  for (auto& kv : w->fusion_plans) ring_fusion_plan_destroy(kv.second);
+  w->fusion_plans.clear();
+}
+
 // A fusion plan for these tensors, created on first use. Training loops reduce
 // the same gradient buffers every step, so plans are found again by the
 // tensors' addresses and sizes; the table is dropped when it grows large.
@@ -333,17 +340,16 @@ ring_fusion_plan* FusionPlanFor(mpic_world* w, const std::vector<const void*>& p
   key.push_back(static_cast<char>(ring_dtype));
   auto it = w->fusion_plans.find(key);
   if (it != w->fusion_plans.end()) return it->second;
-  if (w->fusion_plans.size() >= 256) {
-    ring_stream_synchronize(w->stream);  // launches in flight still read the plans' device tables
-    for (auto& kv : w->fusion_plans) ring_fusion_plan_destroy(kv.second);
-    w->fusion_plans.clear();
-  }
+  if (w->fusion_plans.size() >= kMaxCachedFusionPlans) DropFusionPlans(w);
   ring_fusion_plan* plan = nullptr;
   if (ring_fusion_plan_create(ptrs.data(), counts.data(), static_cast<int>(ptrs.size()), ring_dtype, &plan) != RING_OK)
     return nullptr;
   w->fusion_plans[key] = plan;
   return plan;
 }
+
+// ring_fusion_allreduce_all addresses this many ranks' tensor tables in one launch
+constexpr int kMaxFusedDirectRanks = 16;
 
 // Tensor fusion (no counterpart in the reference, where every gradient is its
 // own collective and its own negotiation round, __init__.py:195-205): the
@@ -372,15 +378,6 @@ void PerformFusedAllreduce(mpic_world* w, const std::vector<std::string>& names,
     counts.push_back(static_cast<size_t>(rec.begin()->second.in_t->NumElements()));
     total += counts.back();
   }
-  std::vector<void*> bufs(static_cast<size_t>(n));
-  for (int r = 0; r < n && status.ok(); r++) {
-    bufs[static_cast<size_t>(r)] = static_cast<char*>(opt.fusion_buffer) + static_cast<size_t>(r) * opt.fusion_bytes;
-    std::vector<const void*> ins;
-    for (auto& rec : records) ins.push_back(rec.at(r).in_t->data());
-    ring_fusion_plan* plan = FusionPlanFor(w, ins, counts, code);
-    if (!plan || ring_fusion_pack(plan, bufs[static_cast<size_t>(r)], w->stream) != RING_OK)
-      status = errors::Unknown("MPI operation failed unexpectedly.");
-  }
   // fused tf.div consumers: when the whole group asks for the same division it
   // rides on the unpack, otherwise each tensor that asks for one is divided
   // after the unpack
@@ -395,6 +392,46 @@ void PerformFusedAllreduce(mpic_world* w, const std::vector<std::string>& names,
     uniform = uniform && rec.begin()->second.divisor == divisor;
   }
   if (!uniform) divisor = 0;
+
+  // Direct form: the ranks share the GPU, so the ring over the packed buffers is
+  // computed on the tensors themselves, one launch, no fusion buffer (each
+  // tensor still equals the reference ring applied to the packed buffer).
+  if (status.ok() && opt.ring.direct && uniform && n <= kMaxFusedDirectRanks) {
+    // all the plans of this launch must be alive together: make room first, so
+    // that looking one up cannot drop the table under the ones already taken
+    if (w->fusion_plans.size() + 2 * static_cast<size_t>(n) > kMaxCachedFusionPlans) DropFusionPlans(w);
+    std::vector<const ring_fusion_plan*> in_plans, out_plans;
+    for (int r = 0; r < n; r++) {
+      std::vector<const void*> ins, outs;
+      for (auto& rec : records) {
+        ins.push_back(rec.at(r).in_t->data());
+        outs.push_back(rec.at(r).out_t->data());
+      }
+      in_plans.push_back(FusionPlanFor(w, ins, counts, code));
+      out_plans.push_back(ins == outs ? in_plans.back() : FusionPlanFor(w, outs, counts, code));
+      if (!in_plans.back() || !out_plans.back()) status = errors::Unknown("MPI operation failed unexpectedly.");
+    }
+    if (status.ok() &&
+        ring_fusion_allreduce_all(in_plans.data(), out_plans.data(), n, divisor, w->stream) != RING_OK)
+      status = errors::Unknown("MPI operation failed unexpectedly.");
+    if (status.ok() && opt.sync_on_done && ring_stream_synchronize(w->stream) != RING_OK)
+      status = errors::Unknown("MPI operation failed unexpectedly.");
+    std::vector<CommunicationDoneCallback> callbacks;
+    for (auto& rec : records)
+      for (auto& kv : rec) callbacks.push_back(std::move(kv.second.callback));
+    FinishRecords(&records, &callbacks, status);
+    return;
+  }
+
+  std::vector<void*> bufs(static_cast<size_t>(n));
+  for (int r = 0; r < n && status.ok(); r++) {
+    bufs[static_cast<size_t>(r)] = static_cast<char*>(opt.fusion_buffer) + static_cast<size_t>(r) * opt.fusion_bytes;
+    std::vector<const void*> ins;
+    for (auto& rec : records) ins.push_back(rec.at(r).in_t->data());
+    ring_fusion_plan* plan = FusionPlanFor(w, ins, counts, code);
+    if (!plan || ring_fusion_pack(plan, bufs[static_cast<size_t>(r)], w->stream) != RING_OK)
+      status = errors::Unknown("MPI operation failed unexpectedly.");
+  }
   if (status.ok()) {
     std::vector<const void*> ins(bufs.begin(), bufs.end());
     status = RingAllreduceAllRanks(n, dtype, ins.data(), bufs.data(), total, w->stream, opt.ring);

@@ -777,6 +777,80 @@ fusion_span_kernel(const uint64_t* __restrict__ offsets, T* const* __restrict__ 
   }
 }
 
+// ---- a fused allreduce of ranks that share the GPU, without a fused buffer -----------
+// What pack, ring and unpack compute for n resident ranks, in one pass over the
+// fused element space: element e lies in ring segment s(e) of the packed
+// layout, the ring leaves there the fold of the ranks' values in the order
+// s, s+1, ..., s+n-1 (mod n), and every rank's tensor receives it (divided,
+// for an average). A tile of the space is cut where a segment or a tensor
+// ends; each piece is then one fold row with n sources and n destinations
+// whose pointers the first lanes look up in the ranks' tensor tables.
+
+constexpr int kMaxFusedRanks = 16;
+struct FusedRanks {
+  int n;
+  int divisor;
+  uint64_t total;   // elements of the fused space
+  uint64_t seg;     // total / n
+  uint64_t rem;     // total % n: the first rem segments hold one more
+  const void* const* in[kMaxFusedRanks];   // rank k's input tensor table
+  void* const* out[kMaxFusedRanks];        // rank k's output tensor table
+};
+
+template <typename T, bool DIV, int NT>
+__global__ void __launch_bounds__(kBlock)
+fusion_allreduce_kernel(const uint64_t* __restrict__ offsets, const FusionTile* __restrict__ tiles, uint32_t ntiles,
+                        const FusedRanks ranks) {
+  constexpr uint32_t VEC = 16 / sizeof(T);
+  constexpr uint64_t kTileElems = static_cast<uint64_t>(kFusionTileVecs) * VEC;
+  __shared__ const void* s_src[kMaxFusedRanks];
+  __shared__ const void* s_dst[kMaxFusedRanks];
+  const int n = ranks.n;
+  auto seg_start = [&](uint64_t s) { return s * ranks.seg + (s < ranks.rem ? s : ranks.rem); };
+
+  for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+    const uint64_t e0 = static_cast<uint64_t>(tile) * kTileElems;
+    const uint64_t e1 = (e0 + kTileElems < ranks.total) ? e0 + kTileElems : ranks.total;
+    const FusionTile rec = load_tile(tiles, tile);
+    uint32_t t = rec.first;  // the tensor holding the current position (all uniform over the workgroup)
+    // the segment holding e0: segments 0..rem-1 have seg+1 elements
+    uint64_t s;
+    {
+      const uint64_t big = ranks.rem * (ranks.seg + 1);
+      s = e0 < big ? e0 / (ranks.seg + 1) : ranks.rem + (ranks.seg ? (e0 - big) / ranks.seg : 0);
+    }
+    uint64_t b0 = e0;
+    while (b0 < e1) {
+      while (offsets[t + 1] <= b0) t++;
+      while (seg_start(s + 1) <= b0) s++;
+      uint64_t b1 = e1;
+      if (offsets[t + 1] < b1) b1 = offsets[t + 1];
+      if (seg_start(s + 1) < b1) b1 = seg_start(s + 1);
+      const uint64_t within = b0 - offsets[t];
+      // rank (s + k) mod n is source k (the ring's order for segment s); rank k is destination k
+      if (threadIdx.x < static_cast<uint32_t>(n)) {
+        const int k = static_cast<int>(threadIdx.x);
+        const int r = static_cast<int>((s + static_cast<uint64_t>(k)) % static_cast<uint64_t>(n));
+        s_src[k] = static_cast<const T*>(ranks.in[r][t]) + within;
+        s_dst[k] = static_cast<T*>(ranks.out[k][t]) + within;
+      }
+      __syncthreads();
+      T* dst = static_cast<T*>(const_cast<void*>(s_dst[0]));
+      const uint64_t count = b1 - b0;
+      uint64_t head = ((16u - (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(dst)) & 15u)) & 15u) / sizeof(T);
+      if (head > count) head = count;
+      const uint64_t nvec = (count - head) / VEC;
+      uint32_t sub_tiles = static_cast<uint32_t>((nvec + kBlock * kFoldToAllUnroll - 1) / (kBlock * kFoldToAllUnroll));
+      if (sub_tiles == 0) sub_tiles = 1;
+      for (uint32_t sub = 0; sub < sub_tiles; sub++)
+        fold_tile<T, kFoldToAllUnroll, kFoldGroup, DIV, NT>(dst, s_src, n, count, sub, sub_tiles, ranks.divisor, DIV,
+                                                            s_dst + 1, n - 1);
+      __syncthreads();  // before the next piece overwrites the pointers
+      b0 = b1;
+    }
+  }
+}
+
 // ---- launch configuration -----------------------------------------------------
 
 constexpr uint64_t kCacheResidentBytes = 128ull << 20;
@@ -1040,6 +1114,7 @@ struct ring_fusion_plan {
   uint64_t* d_offsets = nullptr;
   void** d_ptrs = nullptr;
   FusionTile* d_tiles = nullptr;
+  std::vector<uint64_t> h_offsets;  // host copy of the offsets: what two plans must share to describe one fused space
 };
 
 namespace {
@@ -1679,6 +1754,7 @@ int ring_fusion_plan_create(const void* const* tensors, const size_t* counts, in
   p->m = static_cast<uint32_t>(ptrs.size());
   p->ntiles = static_cast<uint32_t>(ntiles64);
   p->total = total;
+  p->h_offsets = offsets;
   if (total == 0) { *plan = p; return RING_OK; }
 
   std::vector<FusionTile> tiles(p->ntiles);
@@ -1876,6 +1952,58 @@ int fusion_spans_run(const ring_fusion_plan* p, const ring_fusion_span* spans, i
 }  // namespace
 
 extern "C" {
+
+int ring_fusion_allreduce_all(const ring_fusion_plan* const* in_plans, const ring_fusion_plan* const* out_plans, int n,
+                              int divisor, void* stream) {
+  if (n < 1 || !in_plans || !out_plans || divisor < 0) return RING_ERR_ARGUMENT;
+  if (n > kMaxFusedRanks) return RING_ERR_LIMIT;
+  const ring_fusion_plan* first = in_plans[0];
+  if (!first) return RING_ERR_ARGUMENT;
+  for (int k = 0; k < n; k++) {
+    for (const ring_fusion_plan* p : {in_plans[k], out_plans[k]}) {
+      // one fused space: the same element type and the same tensor sizes in the same order
+      if (!p || p->dtype != first->dtype || p->h_offsets != first->h_offsets) return RING_ERR_ARGUMENT;
+    }
+  }
+  if (first->total == 0) return RING_OK;
+  FusedRanks ranks;
+  ranks.n = n;
+  ranks.divisor = divisor;
+  ranks.total = first->total;
+  ranks.seg = first->total / static_cast<uint64_t>(n);
+  ranks.rem = first->total % static_cast<uint64_t>(n);
+  for (int k = 0; k < kMaxFusedRanks; k++) {
+    ranks.in[k] = k < n ? in_plans[k]->d_ptrs : nullptr;
+    ranks.out[k] = k < n ? out_plans[k]->d_ptrs : nullptr;
+  }
+  int nt = g_tuning.nt[kRoleFoldAll];
+  if (nt < 0) nt = 3;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(first->ntiles);
+#define RING_FUSED_ALL(T, D, N)                                                                              \
+  launch(fusion_allreduce_kernel<T, D, N>, grid, dim3(kBlock), s, static_cast<const uint64_t*>(first->d_offsets), \
+         static_cast<const FusionTile*>(first->d_tiles), first->ntiles, ranks)
+#define RING_FUSED_ALL_NT(T, D)                 \
+  switch (nt & 3) {                             \
+    case 0: RING_FUSED_ALL(T, D, 0); break;     \
+    case 1: RING_FUSED_ALL(T, D, 1); break;     \
+    case 2: RING_FUSED_ALL(T, D, 2); break;     \
+    default: RING_FUSED_ALL(T, D, 3); break;    \
+  }
+  if (divisor > 0) {
+    if (first->dtype == RING_F32) { RING_FUSED_ALL_NT(float, true) }
+    else if (first->dtype == RING_I32) { RING_FUSED_ALL_NT(int32_t, true) }
+    else { RING_FUSED_ALL_NT(int64_t, true) }
+  } else {
+    if (first->dtype == RING_F32) { RING_FUSED_ALL_NT(float, false) }
+    else if (first->dtype == RING_I32) { RING_FUSED_ALL_NT(int32_t, false) }
+    else { RING_FUSED_ALL_NT(int64_t, false) }
+  }
+#undef RING_FUSED_ALL_NT
+#undef RING_FUSED_ALL
+  RING_HIP(hipGetLastError());
+  return RING_OK;
+}
 
 int ring_fusion_gather(const ring_fusion_plan* plan, const ring_fusion_span* spans, int n_spans, void* stream) {
   return fusion_spans_run(plan, spans, n_spans, true, 0, stream);

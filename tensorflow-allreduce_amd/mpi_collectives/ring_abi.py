@@ -22,7 +22,7 @@ EXPORTS = (
     "ring_schedule", "ring_stream_create", "ring_stream_destroy", "ring_stream_synchronize",
     "ring_copy_bytes", "ring_accumulate_f32", "ring_accumulate_i32", "ring_accumulate_i64",
     "ring_accumulate", "ring_reduce_scatter_steps", "ring_reduce_scatter_steps_from",
-    "ring_allgather_steps", "ring_apply_rows", "ring_apply_rows_avg", "ring_fold_rows", "ring_fold_and_copy_rows", "ring_fold_to_all_rows",
+    "ring_allgather_steps", "ring_apply_rows", "ring_apply_rows_avg", "ring_fold_rows", "ring_fold_and_copy_rows", "ring_fold_to_all_rows", "ring_fusion_allreduce_all",
     "ring_fusion_plan_create", "ring_fusion_plan_destroy", "ring_fusion_plan_elements", "ring_fusion_plan_dtype",
     "ring_fusion_pack", "ring_fusion_unpack", "ring_fusion_unpack_scaled", "ring_fusion_gather",
     "ring_fusion_scatter", "ring_scale", "ring_fusion_run_static",
@@ -128,6 +128,7 @@ def lib():
             "ring_fold_rows": (ci, [ctypes.POINTER(FoldRow), ci, ci, ci, ci, vp]),
             "ring_fold_and_copy_rows": (ci, [ctypes.POINTER(FoldRow), ci, ci, ci, ctypes.POINTER(Row), ci, ci, vp]),
             "ring_fold_to_all_rows": (ci, [ctypes.POINTER(FoldToAllRow), ci, ci, ci, ci, ci, vp]),
+            "ring_fusion_allreduce_all": (ci, [ctypes.POINTER(vp), ctypes.POINTER(vp), ci, ci, vp]),
             "ring_fusion_plan_create": (ci, [ctypes.POINTER(vp), psz, ci, ci, ctypes.POINTER(vp)]),
             "ring_fusion_plan_destroy": (ci, [vp]),
             "ring_fusion_plan_elements": (sz, [vp]),
@@ -344,6 +345,15 @@ def fusion_run_static(unpack, ptrs, counts, dtype, fused, divisor, stream):
     c = (ctypes.c_size_t * max(k, 1))(*counts)
     check(lib().ring_fusion_run_static(1 if unpack else 0, p, c, k, dtype, fused, divisor, stream),
           "ring_fusion_run_static")
+
+
+def fusion_allreduce_all(in_plans, out_plans, divisor, stream):
+    """The fused allreduce of ranks that share the GPU, without a fused buffer:
+    in_plans[k] / out_plans[k] are FusionPlans over rank k's input and output tensors."""
+    n = len(in_plans)
+    a = (ctypes.c_void_p * n)(*[p._h for p in in_plans])
+    b = (ctypes.c_void_p * n)(*[p._h for p in out_plans])
+    check(lib().ring_fusion_allreduce_all(a, b, n, divisor, stream), "ring_fusion_allreduce_all")
 
 
 class FusionPlan:

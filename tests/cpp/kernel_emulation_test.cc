@@ -268,6 +268,72 @@ void test_fold_to_all(int m, int n_dst, size_t count, int divisor) {
   for (int k = 0; k < m; k++) expect_equal(static_cast<T*>(in_place_dst[k]), want, "fold to all, in place");
 }
 
+// The fused allreduce of n resident ranks without a fused buffer, into fresh tensors and in
+// place: every tensor element equals the ring's fold of the packed layout's segment it lies in.
+template <typename T>
+void test_fused_allreduce_of_all_ranks(const std::vector<size_t>& counts, int divisor, int n) {
+  size_t total = 0;
+  for (size_t c : counts) total += c;
+  std::vector<std::vector<Buf<T>>> in(n), out(n);
+  std::vector<std::vector<const void*>> in_ptrs(n), out_ptrs(n);
+  std::vector<std::vector<T>> packed(n);
+  std::vector<ring_fusion_plan*> in_plans(n), out_plans(n);
+  for (int r = 0; r < n; r++) {
+    in[r].reserve(counts.size());
+    out[r].reserve(counts.size());
+    for (size_t j = 0; j < counts.size(); j++) {
+      in[r].emplace_back(counts[j], (j + r) % 4);
+      out[r].emplace_back(counts[j], (j + 2 * r + 1) % 4, false);
+      in_ptrs[r].push_back(counts[j] ? in[r].back().p : nullptr);
+      out_ptrs[r].push_back(counts[j] ? out[r].back().p : nullptr);
+      packed[r].insert(packed[r].end(), in[r].back().p, in[r].back().p + counts[j]);
+    }
+    OK(ring_fusion_plan_create(in_ptrs[r].data(), counts.data(), static_cast<int>(counts.size()), code<T>(), &in_plans[r]));
+    OK(ring_fusion_plan_create(out_ptrs[r].data(), counts.data(), static_cast<int>(counts.size()), code<T>(), &out_plans[r]));
+  }
+  std::vector<size_t> sizes(n), starts(n);
+  OK(ring_segment_table(total, n, sizes.data(), starts.data()));
+  std::vector<T> want(total);
+  for (int sg = 0; sg < n; sg++)
+    for (size_t e = starts[sg]; e < starts[sg] + sizes[sg]; e++) {
+      T acc = packed[sg][e];
+      for (int k = 1; k < n; k++) acc = add(acc, packed[(sg + k) % n][e]);
+      want[e] = divisor ? divide(acc, divisor) : acc;
+    }
+  auto check = [&](std::vector<std::vector<Buf<T>>>& got, const char* what) {
+    for (int r = 0; r < n; r++) {
+      size_t at = 0;
+      for (auto& t : got[r]) {
+        CHECK(memcmp(t.p, want.data() + at, t.count * sizeof(T)) == 0 || (fprintf(stderr, "%s, rank %d\n", what, r), false));
+        t.check_lead();
+        at += t.count;
+      }
+    }
+  };
+  OK(ring_fusion_allreduce_all(in_plans.data(), out_plans.data(), n, divisor, nullptr));
+  check(out, "fused allreduce of all ranks");
+  OK(ring_fusion_allreduce_all(in_plans.data(), in_plans.data(), n, divisor, nullptr));
+  check(in, "fused allreduce of all ranks, in place");
+  // plans over different tensor sizes do not describe one fused space
+  if (counts.size() >= 2 && counts[0] != counts[1] && counts[0] && counts[1] && n >= 2) {
+    std::vector<size_t> swapped(counts);
+    std::swap(swapped[0], swapped[1]);
+    std::vector<const void*> p(in_ptrs[1]);
+    std::swap(p[0], p[1]);
+    ring_fusion_plan* other = nullptr;
+    OK(ring_fusion_plan_create(p.data(), swapped.data(), static_cast<int>(swapped.size()), code<T>(), &other));
+    std::vector<ring_fusion_plan*> mixed(in_plans);
+    mixed[1] = other;
+    CHECK(ring_fusion_allreduce_all(mixed.data(), out_plans.data(), n, divisor, nullptr) == RING_ERR_ARGUMENT);
+    OK(ring_fusion_plan_destroy(other));
+  }
+  CHECK(ring_fusion_allreduce_all(in_plans.data(), out_plans.data(), 17, divisor, nullptr) == RING_ERR_LIMIT);
+  for (int r = 0; r < n; r++) {
+    OK(ring_fusion_plan_destroy(in_plans[r]));
+    OK(ring_fusion_plan_destroy(out_plans[r]));
+  }
+}
+
 // Pack, unpack (divided or not), gather and scatter over a tensor set, through a
 // plan and through the static device table.
 template <typename T>
@@ -365,6 +431,7 @@ void test_fusion(const std::vector<size_t>& counts, int divisor, int n_ranks) {
   }
   OK(ring_fusion_plan_destroy(plan));
   for (auto& t : tensors) t.check_lead();
+  test_fused_allreduce_of_all_ranks<T>(counts, divisor, n_ranks);
 }
 
 template <typename T>

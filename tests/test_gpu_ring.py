@@ -1166,3 +1166,50 @@ def test_distributed_optimizer_builds_its_nodes_once(oracle):
             for p0, p1 in zip(replicas[0].parameters(), replicas[n - 1].parameters()):
                 assert torch.equal(p0, p1)
         assert built[1] == built[2], "the nodes were rebuilt although the gradients stayed in place"
+
+
+@pytest.mark.parametrize("dtype", G.DTYPES)
+def test_fused_allreduce_of_resident_ranks_without_a_fused_buffer(oracle, dtype):
+    """ring_fusion_allreduce_all: one launch over the tensors of all ranks gives
+    every tensor what pack, the reference ring on the packed buffer and unpack
+    give (tf.div included), into tensors of their own and in place; tensor sets
+    with tiny, empty and misaligned tensors, ring segments that cut through
+    tensors, and the full 161-tensor ResNet-50 set at N=8 for float32."""
+    rng = np.random.default_rng(17)
+    code = G.NP2ABI[np.dtype(dtype)]
+    cases = [(3, [5, 0, 4099, 1, 64, 0, 3]), (8, [20_000, 64, 64, 36_864, 64, 64, 9_001, 2, 12_288]),
+             (5, [int(c) for c in rng.integers(0, 40, 500)] + [9_000]), (16, [70_001]), (1, [100, 7])]
+    if dtype == np.float32:
+        cases.append((8, [int(np.prod(s)) for s in G.resnet50_shapes()]))
+    for n, counts in cases:
+        total = sum(counts)
+        for divisor in (0, n):
+            hosts = [[G.random_array(rng, c, dtype) for c in counts] for _ in range(n)]
+            if dtype != np.float32:
+                for r in range(n):
+                    for h in hosts[r]:
+                        h[: h.size // 2] = -np.abs(h[: h.size // 2])          # negative sums for the floor division
+            ins = [[G.dev(h, (j + r) % 4) for j, h in enumerate(hosts[r])] for r in range(n)]
+            outs = [[G.dev(np.zeros(c, dtype=dtype), (j + 2 * r + 1) % 4) for j, c in enumerate(counts)] for r in range(n)]
+            in_plans = [ring_abi.FusionPlan([t[0].data_ptr() if c else None for t, c in zip(ins[r], counts)], counts, code)
+                        for r in range(n)]
+            out_plans = [ring_abi.FusionPlan([t[0].data_ptr() if c else None for t, c in zip(outs[r], counts)], counts, code)
+                         for r in range(n)]
+            packed = [np.concatenate(hosts[r]) if total else np.zeros(0, dtype=dtype) for r in range(n)]
+            want = oracle.ring_allreduce(packed)[0] if total else packed[0]
+            if divisor:
+                want = _tf_div(want, divisor)
+            ring_abi.fusion_allreduce_all(in_plans, out_plans, divisor, None)
+            G.sync()
+            for where, plans_in, tensors in (("fresh tensors", None, outs), ("in place", in_plans, ins)):
+                if plans_in is not None:
+                    ring_abi.fusion_allreduce_all(plans_in, plans_in, divisor, None)
+                    G.sync()
+                for r in range(n):
+                    at = 0
+                    for j, c in enumerate(counts):
+                        G.assert_same_bits(G.host(tensors[r][j][0]), want[at:at + c],
+                                           "n=%d /%d %s rank %d tensor %d of %d" % (n, divisor, where, r, j, len(counts)))
+                        at += c
+            for p in in_plans + out_plans:
+                p.close()
