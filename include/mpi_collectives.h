@@ -93,7 +93,11 @@ int mpic_world_set_option(mpic_world* world, const char* name, int value);
  * tensor's result is then the reference ring applied to the packed buffer,
  * which for float32 rounds differently from a ring per tensor (an element
  * lands in another segment); grouping depends only on submission order and
- * flush points, not on timing. Worlds with pre-staged peers never fuse. */
+ * flush points, not on timing. Worlds with pre-staged peers never fuse. In
+ * the direct form (option "direct", the default) a group of up to 16 ranks
+ * whose tensors ask for the same divisor is reduced on the tensors themselves
+ * by one launch (ring_fusion_allreduce_all), with the same results, and the
+ * buffer only bounds the size of a group. */
 int mpic_world_set_fusion_buffer(mpic_world* world, void* buffer, size_t bytes_per_rank);
 /* Start a tick now: everything submitted so far is negotiated and run. */
 int mpic_world_flush(mpic_world* world);
