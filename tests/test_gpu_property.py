@@ -220,3 +220,35 @@ def test_fold_rows_any_source_may_be_the_destination(m, count, dtype, seed, divi
     for k, h in enumerate(hs):                       # the other sources are never written
         if k != in_place:
             G.assert_same_bits(G.host(ds[k][0]), h, "source %d untouched" % k)
+
+
+@settings(max_examples=30, **COMMON)
+@given(n=st.integers(1, 16), sizes=st.lists(st.one_of(st.integers(0, 40), st.integers(0, 9000)), min_size=1, max_size=40),
+       dtype=st.sampled_from(G.DTYPES), seed=st.integers(0, 2**31), divisor=st.sampled_from([0, 0, 1, 3, 8]),
+       in_place=st.booleans())
+def test_fused_allreduce_of_all_ranks_is_the_ring_on_the_packed_buffer(oracle, n, sizes, dtype, seed, divisor, in_place):
+    """ring_fusion_allreduce_all on random tensor sets: every tensor of every rank equals
+    the oracle's ring over the concatenations, divided as tf.div divides."""
+    rng = np.random.default_rng(seed)
+    code = G.NP2ABI[np.dtype(dtype)]
+    hosts = [[G.random_array(rng, c, dtype) for c in sizes] for _ in range(n)]
+    ins = [[G.dev(h, int(rng.integers(0, 4))) for h in hosts[r]] for r in range(n)]
+    outs = ins if in_place else [[G.dev(np.zeros(c, dtype=dtype), int(rng.integers(0, 4))) for c in sizes] for _ in range(n)]
+    in_plans = [ring_abi.FusionPlan([t[0].data_ptr() if c else None for t, c in zip(ins[r], sizes)], sizes, code) for r in range(n)]
+    out_plans = in_plans if in_place else [
+        ring_abi.FusionPlan([t[0].data_ptr() if c else None for t, c in zip(outs[r], sizes)], sizes, code) for r in range(n)]
+    total = sum(sizes)
+    want = oracle.ring_allreduce([np.concatenate(h) for h in hosts])[0] if total else np.empty(0, dtype=dtype)
+    if divisor and total:
+        with np.errstate(all="ignore"):
+            want = (want / np.float32(divisor)).astype(np.float32) if dtype == np.float32 else want // dtype(divisor)
+    ring_abi.fusion_allreduce_all(in_plans, out_plans, divisor, None)
+    torch.cuda.synchronize()
+    for r in range(n):
+        at = 0
+        for j, c in enumerate(sizes):
+            G.assert_same_bits(G.host(outs[r][j][0]), want[at:at + c].astype(dtype),
+                               "n=%d sizes=%r /%d in_place=%s rank %d tensor %d" % (n, sizes, divisor, in_place, r, j))
+            at += c
+    for p in set(in_plans + out_plans):
+        p.close()
