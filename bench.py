@@ -56,6 +56,8 @@ TRAFFIC_PROFILES = {
     "fused_resnet50_n8_no_passes": "fusion_span_kernel_resnet50_161_tensors_n8_no_passes.txt",
     "fused_resnet50_n8_no_passes_direct": "fusion_span_kernel_resnet50_161_tensors_n8_direct.txt",
     "allreduce_f32_64MiB_n8_direct": "fold_kernel_f32_64MiB_n8_direct.txt",
+    "allreduce_f32_64MiB_all_ranks_n8": "fold_kernel_f32_64MiB_all_ranks_n8.txt",
+    "fused_resnet50_all_ranks_n8": "fusion_allreduce_kernel_resnet50_161_tensors_all_ranks_n8.txt",
 }
 
 
@@ -539,7 +541,83 @@ class AllgatherN16(Workload):
         return bool(self.torch.equal(s["out"], self.torch.cat(s["parts"])))
 
 
+class AllRanksAllreduce(Workload):
+    """All n ranks of the ring resident on the GPU (a world of virtual ranks): a
+    step is the whole allreduce of all ranks, in the direct form one launch in
+    which the owner of every segment folds the n copies in ring order and
+    stores the result into every rank's output. With `counts` the ranks hold
+    tensor sets and the same launch works on the tensors themselves (what pack,
+    ring and unpack of a fused allreduce compute). Averaged (divided by n)."""
+
+    def __init__(self, name, counts, n, nsets, what):
+        import torch
+        from mpi_collectives import _plugin, ring_abi
+        self.torch, self.ring_abi = torch, ring_abi
+        self.L = _plugin.load_library('libmpi_collectives.so', ['MPIAllreduce', 'MPIAllgather'])
+        self.pdt = _plugin.DT_FLOAT
+        self.name, self.dtype, self.n, self.nsets, self.counts = name, "f32", n, nsets, counts
+        self.count = total = sum(counts)
+        self.fused = len(counts) > 1
+        self.sizes, self.starts = ring_abi.segment_table(total, n)
+        self.sets = []
+        for s in range(nsets):
+            gen = torch.Generator(device="cuda").manual_seed(s)
+            ins = [torch.randn(total, device="cuda", generator=gen) for _ in range(n)]
+            outs = [torch.empty(total, device="cuda") for _ in range(n)]
+            d = dict(ins=ins, outs=outs,
+                     ip=(ctypes.c_void_p * n)(*[t.data_ptr() for t in ins]),
+                     op=(ctypes.c_void_p * n)(*[t.data_ptr() for t in outs]))
+            if self.fused:
+                # every tensor its own allocation, as gradients are
+                d["tin"] = [[t.clone() for t in x.split(counts)] for x in ins]
+                d["tout"] = [[torch.empty(c, device="cuda") for c in counts] for _ in range(n)]
+                d["in_plans"] = [ring_abi.FusionPlan([t.data_ptr() for t in ts], counts, ring_abi.F32) for ts in d["tin"]]
+                d["out_plans"] = [ring_abi.FusionPlan([t.data_ptr() for t in ts], counts, ring_abi.F32) for ts in d["tout"]]
+            self.sets.append(d)
+        kernel = ("fusion_allreduce_kernel<float> (%d tensors per rank)" % len(counts) if self.fused
+                  else "fold_kernel<float> (%d rows of %d sources and %d destinations)" % (n, n, n))
+        self.phases = (("fold_to_all", 2 * n * total * 4, kernel),)
+        self.dominant = 0
+        self.description = what
+
+    def launch_step(self, k, stream, fused=False):
+        s = self.sets[k % self.nsets]
+        if self.fused:
+            self.ring_abi.fusion_allreduce_all(s["in_plans"], s["out_plans"], self.n, stream)
+            return
+        rc = self.L.mpic_ring_allreduce_all_ranks(self.n, self.pdt, s["ip"], s["op"], self.count, stream,
+                                                  7 | (self.n << 8))
+        if rc != 0:
+            raise RuntimeError("mpic_ring_allreduce_all_ranks failed: %s" % self.L.mpic_last_error().decode())
+
+    def launch_phase(self, k, i, stream):
+        self.launch_step(k, stream)
+
+    def check(self, k):
+        s, torch, n = self.sets[k % self.nsets], self.torch, self.n
+        want = torch.empty(self.count, device="cuda")
+        for seg in range(n):
+            a, b = self.starts[seg], self.starts[seg] + self.sizes[seg]
+            acc = s["ins"][seg][a:b].clone()
+            for j in range(1, n):
+                acc = s["ins"][(seg + j) % n][a:b] + acc
+            want[a:b] = acc / n
+        if self.fused:
+            return all(torch.equal(torch.cat(ts), want) for ts in s["tout"])
+        return all(torch.equal(o, want) for o in s["outs"])
+
+
 def make_workload(name):
+    if name == "allreduce_f32_64MiB_all_ranks_n8":
+        return AllRanksAllreduce(name, [16 * 1024 * 1024], 8, 3,
+                                 "float32 averaged allreduce of a 64 MiB tensor per rank, all 8 virtual ranks resident: "
+                                 "ONE launch, the owner of every segment folds the 8 copies in ring order and stores "
+                                 "the result into all 8 outputs (8 reads + 8 writes per element); 3 buffer sets rotated")
+    if name == "fused_resnet50_all_ranks_n8":
+        return AllRanksAllreduce(name, resnet50_counts(), 8, 2,
+                                 "float32 averaged allreduce of the 161 ResNet-50 gradients (25,557,032 elements) of all "
+                                 "8 resident virtual ranks: ONE launch on the tensors themselves, every tensor equal to "
+                                 "the ring on the packed buffer; 2 buffer sets rotated")
     if name == "allreduce_f32_64MiB_n8":
         return RingAllreduce(name, "f32", 16 * 1024 * 1024, 8, 8,
                              "float32 ring allreduce of one 16,777,216-element (64 MiB) tensor, N=8 virtual ranks: "
@@ -587,7 +665,8 @@ WORKLOADS = ("allreduce_f32_64MiB_n8", "allreduce_i32_10000019_n6", "allreduce_i
              "fused_resnet50_n8", "allgather_f32_n16", "allreduce_f32_1GiB_n64", "allreduce_f32_64MiB_n8_per_step",
              "allreduce_f32_1MiB_n8",
              "allreduce_f32_64MiB_n8_direct", "fused_resnet50_n8_no_passes",
-             "fused_resnet50_n8_no_passes_direct")
+             "fused_resnet50_n8_no_passes_direct", "allreduce_f32_64MiB_all_ranks_n8",
+             "fused_resnet50_all_ranks_n8")
 
 
 def cpu_baseline(w):
@@ -877,11 +956,14 @@ def main():
             "avg_launch_us": round(phase_us[w.dominant], 3),
             "launches_timed": len(samples),
             "launches_timed_inside_the_wall_clock_region": in_region,
-            "note": "achieved = algorithmic bytes / median launch duration (HIP events carried in the dispatch). "
-                    "In the reference-shaped step the accumulate reads the buffer the in->out copy has just written "
-                    "with ordinary stores, so part of its reads are served by the last-level cache: `frac` is that "
-                    "LLC-assisted figure. `frac_cold` is the same kernel where no operand was touched before it (the "
-                    "step with the copy folded in, out = in + received): the HBM figure.",
+            "note": "achieved = algorithmic bytes / median launch duration (HIP events carried in the dispatch)."
+                    + (" In the reference-shaped step the accumulate reads the buffer the in->out copy has just "
+                       "written with ordinary stores, so part of its reads are served by the last-level cache: `frac` "
+                       "is that LLC-assisted figure. `frac_cold` is the same kernel where no operand was touched "
+                       "before it (the step with the copy folded in, out = in + received): the HBM figure."
+                       if cold is not None else
+                       " Buffer sets are rotated, so no operand of a launch was left in the last-level cache by the "
+                       "launch before it."),
         },
         "phases": {p[0]: {"us": round(t, 3), "median_us": round(statistics.median(phase_times[i]), 3),
                           "min_us": round(min(phase_times[i]), 3), "GBps": round(p[1] / t / 1e3, 1),
@@ -950,8 +1032,9 @@ def main():
                                           "sample": "failed: %s" % e}
     elif not args.no_cpu_baseline:
         result["cpu_baseline"] = {"value": None, "unit": "GB/s", "cores": 0, "kind": "port",
-                                  "sample": "not run for this workload: the reference has no fusion buffer, and its "
-                                            "allgather moves bytes only"}
+                                  "sample": "not run for this workload (the reference has no fusion buffer, no "
+                                            "direct form and no ranks that share a device, and its allgather moves "
+                                            "bytes only): the default workload carries the CPU baseline"}
     ring_abi.stream_destroy(stream)
     print(json.dumps(result))
 
