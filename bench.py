@@ -629,6 +629,11 @@ def make_workload(name):
                                    "2,097,152-element segment folded in ring order from the 7 peers' staged raw copies "
                                    "and its own (8 reads, 1 write per element) + 7 copies of finished segments, all in "
                                    "one launch; buffers rotated over 8 virtual ranks")
+    if name == "allreduce_f32_1MiB_n8_direct":
+        return RingAllreduceDirect(name, 262_144, 8, 8,
+                                   "float32 allreduce of one 1 MiB tensor, N=8 virtual ranks, DIRECT form: the launch-bound "
+                                   "size in ONE launch per allreduce (fold of the 8 copies of the rank's 128 KiB segment "
+                                   "+ 7 copies of finished segments); buffers rotated over 8 virtual ranks")
     if name == "allreduce_f32_64MiB_n8_per_step":
         return RingAllreducePerStep(name, "f32", 16 * 1024 * 1024, 8, 8,
                                     "float32 ring allreduce of one 64 MiB tensor, N=8 virtual ranks, ONE LAUNCH PER RING "
@@ -663,7 +668,7 @@ def make_workload(name):
 
 WORKLOADS = ("allreduce_f32_64MiB_n8", "allreduce_i32_10000019_n6", "allreduce_i64_10000019_n6",
              "fused_resnet50_n8", "allgather_f32_n16", "allreduce_f32_1GiB_n64", "allreduce_f32_64MiB_n8_per_step",
-             "allreduce_f32_1MiB_n8",
+             "allreduce_f32_1MiB_n8", "allreduce_f32_1MiB_n8_direct",
              "allreduce_f32_64MiB_n8_direct", "fused_resnet50_n8_no_passes",
              "fused_resnet50_n8_no_passes_direct", "allreduce_f32_64MiB_all_ranks_n8",
              "fused_resnet50_all_ranks_n8")

@@ -170,7 +170,8 @@ struct Row {
   const void* b;   // local operand of an add row, null for a copy row
   uint64_t count;  // elements
 };
-struct RowTable {
+template <int MAXROWS>
+struct RowTableT {
   int n_rows;
   int dry;  // measurement only: every workgroup returns at once
   // > 0: every row has this many tiles and the grid is (tiles, rows), so a
@@ -180,9 +181,20 @@ struct RowTable {
   uint32_t uniform_tiles;
   int divisor;                        // kAvg only
   uint64_t div_mask;                  // kAvg only: bit k set = row k divides
-  uint32_t tile_begin[kMaxRows + 1];  // prefix sum of tiles per row
-  Row row[kMaxRows];
+  uint32_t tile_begin[MAXROWS + 1];  // prefix sum of tiles per row
+  Row row[MAXROWS];
 };
+typedef RowTableT<kMaxRows> RowTable;
+// The same table with room for 8 rows (the 7 segments of an 8-rank phase): 320
+// bytes of kernel arguments instead of 2.3 KB. What a launch costs the host
+// grows with the size of its arguments (a stream of empty kernels: 2.4 us per
+// launch at 24 bytes, 2.5 at 264, 3.0 at 648, 4.5 from 1.3 KB on), and a step on
+// a small tensor costs what its launches cost the host: the three launches of a
+// 1 MiB, 8-rank step driven from C++ take 8.2 us instead of 8.8 (12.0 instead
+// of 13.4 on a slower host). The fold kernel gained nothing from a small table
+// (its one launch per step is bound by the GPU's side of a dispatch, 3.9 us).
+constexpr int kSmallRows = 8;
+typedef RowTableT<kSmallRows> SmallRowTable;
 
 // NT: bit 0 = non-temporal stores, bit 1 = non-temporal loads (3, both, is the
 // default: every byte is touched once).
@@ -342,9 +354,10 @@ __device__ __forceinline__ void run_row(const Row& r, uint32_t tile, uint32_t ti
 template <int MAX_ROWS>
 __device__ __forceinline__ int row_of_tile(const uint32_t* begin, int n_rows, uint32_t t) {
   int row = 0;
-  if (n_rows <= 16) {
+  constexpr int kShort = MAX_ROWS < 16 ? MAX_ROWS : 16;
+  if (n_rows <= kShort) {
 #pragma unroll
-    for (int k = 1; k < 16; k++) row += begin[k] <= t ? 1 : 0;
+    for (int k = 1; k < kShort; k++) row += begin[k] <= t ? 1 : 0;
   } else {
 #pragma unroll
     for (int k = 1; k < MAX_ROWS; k++) row += begin[k] <= t ? 1 : 0;
@@ -352,24 +365,37 @@ __device__ __forceinline__ int row_of_tile(const uint32_t* begin, int n_rows, ui
   return row;
 }
 
+// The kernel's body, textually in each of the two kernels below (as a function
+// that takes the table by reference the paced copy compiled to per-lane 64-bit
+// addresses and ran 12 % slower).
+#define RING_ROWS_KERNEL_BODY(MAXROWS, UNROLL, PACE)                                                              \
+  if (tab.dry) return;                                                                                            \
+  if (tab.uniform_tiles) {                                                                                        \
+    const Row r = tab.row[blockIdx.y]; /* one scalar load, no search */                                           \
+    const bool divide = MODE == kAvg && ((tab.div_mask >> blockIdx.y) & 1u);                                      \
+    for (uint32_t t = blockIdx.x; t < tab.uniform_tiles; t += gridDim.x)                                          \
+      run_row<T, MODE, UNROLL, NT, PACE>(r, t, tab.uniform_tiles, tab.divisor, divide);                           \
+    return;                                                                                                       \
+  }                                                                                                               \
+  const uint32_t total = tab.tile_begin[tab.n_rows];                                                              \
+  for (uint32_t t = blockIdx.x; t < total; t += gridDim.x) {                                                      \
+    const int lo = row_of_tile<MAXROWS>(tab.tile_begin, tab.n_rows, t);                                           \
+    const uint32_t first = tab.tile_begin[lo];                                                                    \
+    run_row<T, MODE, UNROLL, NT, PACE>(tab.row[lo], t - first, tab.tile_begin[lo + 1] - first, tab.divisor,       \
+                                       MODE == kAvg && ((tab.div_mask >> lo) & 1u));                              \
+  }
+
 template <typename T, int MODE, int UNROLL, int NT, int PACE = 0>
 __global__ void __launch_bounds__(kBlock) rows_kernel(const RowTable tab) {
-  if (tab.dry) return;
-  if (tab.uniform_tiles) {
-    const Row r = tab.row[blockIdx.y];  // one scalar load, no search
-    const bool divide = MODE == kAvg && ((tab.div_mask >> blockIdx.y) & 1u);
-    for (uint32_t t = blockIdx.x; t < tab.uniform_tiles; t += gridDim.x)
-      run_row<T, MODE, UNROLL, NT, PACE>(r, t, tab.uniform_tiles, tab.divisor, divide);
-    return;
-  }
-  const uint32_t total = tab.tile_begin[tab.n_rows];
-  for (uint32_t t = blockIdx.x; t < total; t += gridDim.x) {
-    const int lo = row_of_tile<kMaxRows>(tab.tile_begin, tab.n_rows, t);
-    const uint32_t first = tab.tile_begin[lo];
-    run_row<T, MODE, UNROLL, NT, PACE>(tab.row[lo], t - first, tab.tile_begin[lo + 1] - first, tab.divisor,
-                                 MODE == kAvg && ((tab.div_mask >> lo) & 1u));
-  }
+  RING_ROWS_KERNEL_BODY(kMaxRows, UNROLL, PACE)
 }
+
+// The same kernel (4 vectors per lane, plain tiles) on the 8-row table.
+template <typename T, int MODE, int NT>
+__global__ void __launch_bounds__(kBlock) rows_kernel_small(const SmallRowTable tab) {
+  RING_ROWS_KERNEL_BODY(kSmallRows, 4, 0)
+}
+#undef RING_ROWS_KERNEL_BODY
 
 // Byte copy for operands that are not 4-byte compatible (never produced by the
 // three element types; kept so ring_copy_bytes is total).
@@ -913,7 +939,23 @@ int launch_rows_typed(const RowTable& tab, dim3 grid, hipStream_t stream, int nt
     case 2: RING_LAUNCH(U, 2); break;           \
     default: RING_LAUNCH(U, 3); break;          \
   }
-  if (MODE == kCopy && paced) {
+  if (!paced && unroll == 4 && tab.n_rows <= kSmallRows) {
+    SmallRowTable small;
+    small.n_rows = tab.n_rows;
+    small.dry = tab.dry;
+    small.uniform_tiles = tab.uniform_tiles;
+    small.divisor = tab.divisor;
+    small.div_mask = tab.div_mask;
+    for (int k = 0; k <= kSmallRows; k++) small.tile_begin[k] = tab.tile_begin[k];
+    for (int k = 0; k < tab.n_rows; k++) small.row[k] = tab.row[k];
+    for (int k = tab.n_rows; k < kSmallRows; k++) small.row[k] = Row{nullptr, nullptr, nullptr, 0};
+    switch (nt & 3) {
+      case 0: launch(rows_kernel_small<T, MODE, 0>, grid, dim3(kBlock), stream, small); break;
+      case 1: launch(rows_kernel_small<T, MODE, 1>, grid, dim3(kBlock), stream, small); break;
+      case 2: launch(rows_kernel_small<T, MODE, 2>, grid, dim3(kBlock), stream, small); break;
+      default: launch(rows_kernel_small<T, MODE, 3>, grid, dim3(kBlock), stream, small); break;
+    }
+  } else if (MODE == kCopy && paced) {
     if constexpr (MODE == kCopy) {
       switch (nt & 3) {
         case 0: launch(rows_kernel<T, kCopy, kPacedUnroll, 0, 1>, grid, dim3(kBlock), stream, tab); break;
