@@ -444,9 +444,11 @@ class FusedResnet50NoPasses(FusedResnet50):
 
 class FusedResnet50NoPassesDirect(FusedResnet50NoPasses):
     """The same without passes in the direct form: the 7 peers' raw copies of the
-    owned segment (packed layout) lie in staging slots; the rank packs its own
-    copy of that one segment, folds the 8 copies in ring order, and scatters the
-    8 finished segments into the tensors with the divide. Three launches."""
+    owned segment (packed layout) lie in staging slots; ONE launch folds them
+    with the rank's own copy, read from the tensors, in ring order, leaves the
+    sum in the wire buffer (what the rank sends on) and the quotient in the
+    tensors, and scatters the 7 other finished segments into the tensors with
+    the divide."""
 
     def __init__(self, nsets=4):
         super().__init__(nsets)
@@ -458,21 +460,20 @@ class FusedResnet50NoPassesDirect(FusedResnet50NoPasses):
             gen = torch.Generator(device="cuda").manual_seed(77 + st["r"])
             st["raw"] = [torch.randn(sizes[own], device="cuda", generator=gen) * 1e-3 for _ in range(7)]
             st["raw_ptrs"] = (ctypes.c_void_p * 7)(*[t.data_ptr() for t in st["raw"]])
-            mine = st["fused"].data_ptr() + starts[own] * 4
-            st["own"], st["mine"] = own, mine
-            st["pack_own"] = A.make_spans([(starts[own], sizes[own], None, mine)])
-            st["fold_srcs"] = [t.data_ptr() for t in st["raw"]] + [mine]
+            st["own"], st["mine"] = own, st["fused"].data_ptr() + starts[own] * 4
+            ag_of = {g: t for g, t in zip(st["ag_seg"], st["ag"])}
+            st["others"] = A.make_spans([(starts[g], sizes[g], ag_of[g].data_ptr(), None) for g in range(8) if g != own])
         seg = self.total // 8
         self.phases = (
-            ("pack_own_segment", seg * 8, "fusion_span_kernel<unsigned int, gather> (the owned segment packed)"),
-            ("fold", seg * 4 * 9, "fold_kernel<float> (8 copies of the owned segment -> 1)"),
-            ("scatter_scaled", 8 * seg * 8, "fusion_span_kernel<float, scatter, divide> (8 finished segments -> 161 tensors, /8)"))
-        self.dominant = 2
+            ("fold_and_scatter", seg * 4 * 10 + 7 * seg * 8,
+             "fusion_direct_kernel<float, divide> (owned segment: 7 staged copies + tensors -> wire and tensors/8; "
+             "7 finished segments -> tensors/8)"),)
+        self.dominant = 0
         self.description = ("tensor-fusion allreduce of a ResNet-50 v1 gradient set (161 float32 tensors, 25,557,032 "
-                            "elements) at N=8 virtual ranks, DIRECT form without pack and unpack passes: the owned "
-                            "3,194,629-element segment packed, folded in ring order with the 7 peers' staged raw "
-                            "copies, and the 8 finished segments scattered into the tensors with the divide by 8; "
-                            "3 launches per step")
+                            "elements) at N=8 virtual ranks, DIRECT form in ONE launch: the owned 3,194,629-element "
+                            "segment folded in ring order from the 7 peers' staged raw copies and the tensors (sum to "
+                            "the wire buffer, sum/8 into the tensors), the 7 other finished segments scattered into "
+                            "the tensors with the divide by 8")
 
     def owned_sum(self, s, packed):
         """The fold of the 7 staged raw copies and the rank's own copy, in ring order."""
@@ -484,13 +485,9 @@ class FusedResnet50NoPassesDirect(FusedResnet50NoPasses):
         return packed[a:b] + acc
 
     def launch_phase(self, k, i, stream):
-        s, A = self.sets[k % self.nsets], self.ring_abi
-        if i == 0:
-            s["plan"].gather(s["pack_own"], stream)
-        elif i == 1:
-            A.fold_rows([(s["mine"], s["fold_srcs"], self.total // 8)], 8, 0, A.F32, stream)
-        else:
-            s["plan"].scatter(s["scatter"], 8, stream)
+        s = self.sets[k % self.nsets]
+        s["plan"].fold_scatter(self.starts[s["own"]], self.sizes[s["own"]], [t.data_ptr() for t in s["raw"]], s["mine"],
+                               s["others"], 8, stream)
 
     def launch_step(self, k, stream, fused=False):
         s = self.sets[k % self.nsets]
@@ -498,6 +495,16 @@ class FusedResnet50NoPassesDirect(FusedResnet50NoPasses):
                                                         s["ag_ptrs"], stream, 4 | (8 << 8))
         if rc != 0:
             raise RuntimeError("mpic_ring_allreduce_fused_prestaged failed: %s" % self.L.mpic_last_error().decode())
+
+    def check(self, k, stream=None):
+        """The tensors as the parent checks them, and the wire buffer: the owned
+        segment's sum, undivided."""
+        if not super().check(k, stream):
+            return False
+        s, torch = self.sets[k % self.nsets], self.torch
+        a, b = self.starts[s["own"]], self.starts[s["own"]] + self.sizes[s["own"]]
+        # the tensors now hold sum / 8 and the wire the sum: dividing the wire must give the tensors bit for bit
+        return bool(torch.equal(s["fused"][a:b] / 8, torch.cat(s["grads"])[a:b]))
 
 
 class AllgatherN16(Workload):

@@ -368,6 +368,26 @@ int ring_fusion_gather(const ring_fusion_plan* plan, const ring_fusion_span* spa
 int ring_fusion_scatter(const ring_fusion_plan* plan, const ring_fusion_span* spans, int n_spans, int divisor,
                         void* stream);
 
+/* The direct form of a fused allreduce for one rank, in one launch. The
+ * rank's own ring segment is the `fold_count` elements of the fused space from
+ * `fold_begin`: `staged[0..m)` are the peers' raw copies of it (packed layout,
+ * element 0 = element fold_begin), listed in the ring's order for that
+ * segment, and the rank's own copy, which comes last in that order, is read
+ * from the plan's tensors. The fold `staged[0], staged[1] + ., ..., tensors + .`
+ * is stored to `wire` (element 0 = element fold_begin: what the rank sends to
+ * its peers, a sum) and, divided by `divisor` when that is > 0 (tf.div), into
+ * the tensors. `finished` are the other segments, as ring_fusion_scatter takes
+ * them (sorted, disjoint, none meeting the fold span; sums, divided on the way
+ * into the tensors). Bit-identical to ring_fusion_gather of the owned segment,
+ * ring_fold_rows over the m + 1 copies and ring_fusion_scatter of all
+ * segments, which read and write the owned segment three times where this
+ * reads and writes it once. m and n_finished at most 32 (RING_ERR_LIMIT
+ * beyond). No counterpart in the reference (its ring passes partial sums
+ * round, ring.h:183-205). */
+int ring_fusion_fold_scatter(const ring_fusion_plan* plan, uint64_t fold_begin, uint64_t fold_count,
+                             const void* const* staged, int m, void* wire, const ring_fusion_span* finished,
+                             int n_finished, int divisor, void* stream);
+
 /* The fused allreduce of n ranks that share the GPU, without a fused buffer:
  * in_plans[k] / out_plans[k] are plans over rank k's input and output tensors
  * (the same plan for an allreduce in place), all with the same element type

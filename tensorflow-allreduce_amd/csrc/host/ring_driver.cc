@@ -213,6 +213,25 @@ Status RingAllreduceFusedPrestaged(const ring_fusion_plan* plan, int n, int r, v
     for (int i = 0; i < n - 1; i++)
       ag_direct[static_cast<size_t>(Seg(RING_PHASE_ALLGATHER, n, r, i, true))] = ag_recv[i];
     char* mine = at(wire, starts[own], esz);
+    if (n - 1 <= kMaxOneLaunchDirectRanks) {
+      // one launch: the owned segment folded from the staged copies and the
+      // tensors, its sum left in the wire buffer, everything scattered
+      std::vector<const void*> staged;
+      for (int k = 0; k < n - 1; k++) {
+        if (sizes[own] && !rs_recv[k]) return errors::InvalidArgument("null staged peer segment");
+        staged.push_back(rs_recv[k]);
+      }
+      std::vector<ring_fusion_span> others;
+      for (size_t seg = 0; seg < static_cast<size_t>(n); seg++) {
+        if (seg == own) continue;
+        if (sizes[seg] && !ag_direct[seg]) return errors::InvalidArgument("null staged peer segment");
+        others.push_back(ring_fusion_span{starts[seg], sizes[seg], ag_direct[seg], nullptr});
+      }
+      RING_RETURN_IF_ERROR(ring_fusion_fold_scatter(plan, starts[own], sizes[own], staged.data(), n - 1, mine,
+                                                    others.data(), n - 1, opts.divisor, stream),
+                           "ring_fusion_fold_scatter");
+      return Status::OK();
+    }
     ring_fusion_span pack{starts[own], sizes[own], nullptr, mine};
     RING_RETURN_IF_ERROR(ring_fusion_gather(plan, &pack, 1, stream), "ring_fusion_gather");
     std::vector<const void*> srcs;

@@ -18,6 +18,9 @@ namespace mpic {
 // Most copies of a segment one fold launch can address (ring_fold_rows): the
 // direct forms are limited to rings of this many ranks.
 constexpr int kMaxDirectRanks = 256;
+// Most peers whose staged copies the one-launch direct form of a fused
+// allreduce takes (ring_fusion_fold_scatter); larger rings run it as three launches.
+constexpr int kMaxOneLaunchDirectRanks = 32;
 
 struct RingOptions {
   // One launch per ring phase (all n-1 steps of a rank) instead of one per

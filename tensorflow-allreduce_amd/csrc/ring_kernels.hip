@@ -450,8 +450,10 @@ struct FoldTable {
 // more[0..n_more): further destinations of the same result (every rank's copy
 // of a finished segment, written by the owner's fold instead of being copied
 // from it afterwards); they may be sources of the row too, and need only be
-// element-aligned.
-template <typename T, int UNROLL, int GROUP, bool DIV, int NT>
+// element-aligned. MORE_UNDIVIDED: they take the fold as it is and only dst the
+// quotient (a rank's finished segment: the sum goes on the wire, the average
+// into the rank's own tensors).
+template <typename T, int UNROLL, int GROUP, bool DIV, int NT, bool MORE_UNDIVIDED = false>
 __device__ __forceinline__ void fold_tile(T* dst, const void* const* src, int m, uint64_t count, uint32_t tile,
                                           uint32_t tiles_in_row, int n, bool divide,
                                           const void* const* more = nullptr, int n_more = 0) {
@@ -472,7 +474,7 @@ __device__ __forceinline__ void fold_tile(T* dst, const void* const* src, int m,
     for (int k = 1; k < m; k++) acc = add_one(acc, static_cast<const T*>(src[k])[e]);
     const T r = (DIV && divide) ? div_one(acc, n) : acc;
     dst[e] = r;
-    for (int d = 0; d < n_more; d++) static_cast<T*>(const_cast<void*>(more[d]))[e] = r;
+    for (int d = 0; d < n_more; d++) static_cast<T*>(const_cast<void*>(more[d]))[e] = MORE_UNDIVIDED ? acc : r;
   };
   if (tile == 0 && tid < head) scalar(tid);
   if (tile + 1 == tiles_in_row) {
@@ -513,6 +515,16 @@ __device__ __forceinline__ void fold_tile(T* dst, const void* const* src, int m,
           if (ok[j]) acc[j] = apply_vec<T, kOpAdd>(acc[j], x[g][j], 0);
       }
     }
+  }
+  if (MORE_UNDIVIDED) {
+    // the further destinations take the sum itself (what a rank sends on), dst the quotient
+    for (int d = 0; d < n_more; d++) {  // uniform
+      VU* ov = reinterpret_cast<VU*>(static_cast<T*>(const_cast<void*>(more[d])) + head);
+#pragma unroll
+      for (int j = 0; j < UNROLL; j++)
+        if (ok[j]) RING_STORE_VEC(NT, &ov[v0 + j * kBlock], acc[j]);
+    }
+    n_more = 0;
   }
 #pragma unroll
   for (int j = 0; j < UNROLL; j++) {
@@ -798,6 +810,119 @@ fusion_span_kernel(const uint64_t* __restrict__ offsets, T* const* __restrict__ 
       }
       // several tensors: every lane finds the tensor of its 16-byte group
       multi_tensor_piece<T, GATHER, SOP, 0>(off_tab, ptr_tab, ta, tensors, b0, b1, lin_in, lin_out, tab.divisor);
+    }
+    if (staged) __syncthreads();  // before the next tile overwrites the table
+  }
+}
+
+// ---- the direct form of a fused allreduce in one launch ---------------------------------
+// One rank of a fused allreduce whose peers pushed their raw copies of the
+// rank's own segment into staging slots and whose other segments arrive
+// finished. Over the fused element space: inside the owned segment a piece of
+// a tensor is folded from the m staged copies and the tensor itself (the
+// rank's own copy, last in the ring's order for that segment), the sum goes to
+// the wire buffer the other ranks are sent from and the quotient back into the
+// tensor; everywhere else a finished segment is scattered into the tensors as
+// by fusion_span_kernel. The owned segment is read once and written once where
+// pack, fold and scatter as launches of their own read it three times.
+
+constexpr int kMaxDirectSpans = 32;  // ranks of a ring this kernel serves
+struct FusionDirectSpan {
+  uint64_t begin, end;  // elements of the fused space
+  const void* in;       // element `begin` of the finished segment
+};
+struct FusionDirectTable {
+  int n;        // finished spans (sorted, disjoint, none meets the fold span)
+  int divisor;  // > 0 divides what goes into the tensors
+  int m;        // staged copies of the fold span
+  uint64_t fold_begin, fold_end;
+  void* wire;   // element fold_begin of where the fold itself is stored
+  FusionDirectSpan span[kMaxDirectSpans];
+  const void* staged[kMaxDirectSpans];  // element fold_begin of every staged copy, in fold order
+};
+
+template <typename T, int NT, bool DIV>
+__global__ void __launch_bounds__(kBlock)
+fusion_direct_kernel(const uint64_t* __restrict__ offsets, T* const* __restrict__ ptrs,
+                     const FusionTile* __restrict__ tiles, uint32_t tile_lo, uint32_t tile_hi, uint64_t total,
+                     const FusionDirectTable tab) {
+  constexpr uint32_t VEC = 16 / sizeof(T);
+  constexpr uint64_t kTileElems = static_cast<uint64_t>(kFusionTileVecs) * VEC;
+  constexpr int SOP = DIV ? kOpDiv : kOpCopy;
+  __shared__ uint64_t s_off[kFusionLdsCap + 1];
+  __shared__ T* s_ptr[kFusionLdsCap];
+  __shared__ const void* s_src[kMaxDirectSpans + 1];
+  __shared__ const void* s_wire[1];
+
+  for (uint32_t tile = tile_lo + blockIdx.x; tile < tile_hi; tile += gridDim.x) {
+    const uint64_t e0 = static_cast<uint64_t>(tile) * kTileElems;
+    const uint64_t e1 = (e0 + kTileElems < total) ? e0 + kTileElems : total;
+    const FusionTile rec = load_tile(tiles, tile);
+    const uint32_t t0 = rec.first;
+    const uint32_t t1 = rec.last;
+    const uint32_t tensors = t1 - t0 + 1;
+    const uint64_t* off_tab = offsets + t0;
+    T* const* ptr_tab = ptrs + t0;
+    const bool staged = tensors > 1 && tensors <= kFusionLdsCap;  // uniform per workgroup
+    if (staged) {
+      for (uint32_t i = threadIdx.x; i <= tensors; i += kBlock) s_off[i] = offsets[t0 + i];
+      for (uint32_t i = threadIdx.x; i < tensors; i += kBlock) s_ptr[i] = ptrs[t0 + i];
+      __syncthreads();
+      off_tab = s_off;
+      ptr_tab = s_ptr;
+    }
+    // finished segments that meet the tile: scattered into the tensors
+    int lo = 0, hi = tab.n;
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (tab.span[mid].end <= e0) lo = mid + 1; else hi = mid;
+    }
+    for (int sp = lo; sp < tab.n && tab.span[sp].begin < e1; sp++) {
+      const FusionDirectSpan span = tab.span[sp];
+      const uint64_t b0 = span.begin > e0 ? span.begin : e0;
+      const uint64_t b1 = span.end < e1 ? span.end : e1;
+      if (b0 >= b1) continue;
+      const T* lin_in = static_cast<const T*>(span.in) + (b0 - span.begin);
+      uint32_t ta = 0;
+      if (tensors > 1)
+        while (off_tab[ta + 1] <= b0) ta++;
+      if (tensors == 1 || b1 <= off_tab[ta + 1]) {
+        T* tensor = tensors == 1 ? static_cast<T*>(rec.addr) + (b0 - e0) : ptr_tab[ta] + (b0 - off_tab[ta]);
+        row_tile<T, SOP, 4, NT>(tensor, lin_in, nullptr, b1 - b0, 0, 1, tab.divisor);
+        continue;
+      }
+      multi_tensor_piece<T, false, SOP, 0>(off_tab, ptr_tab, ta, tensors, b0, b1, lin_in, nullptr, tab.divisor);
+    }
+    // the part of the owned segment in the tile, cut where a tensor ends: every
+    // piece is one fold row over the staged copies and the tensor
+    uint64_t b0 = tab.fold_begin > e0 ? tab.fold_begin : e0;
+    const uint64_t fold_end = tab.fold_end < e1 ? tab.fold_end : e1;
+    uint32_t ta = 0;
+    while (b0 < fold_end) {
+      if (tensors > 1)
+        while (off_tab[ta + 1] <= b0) ta++;
+      uint64_t b1 = fold_end;
+      if (tensors > 1 && off_tab[ta + 1] < b1) b1 = off_tab[ta + 1];
+      T* tensor = tensors == 1 ? static_cast<T*>(rec.addr) + (b0 - e0) : ptr_tab[ta] + (b0 - off_tab[ta]);
+      const uint64_t within = b0 - tab.fold_begin;
+      if (threadIdx.x < static_cast<uint32_t>(tab.m))
+        s_src[threadIdx.x] = static_cast<const T*>(tab.staged[threadIdx.x]) + within;
+      if (threadIdx.x == static_cast<uint32_t>(tab.m)) {
+        s_src[tab.m] = tensor;
+        s_wire[0] = static_cast<T*>(tab.wire) + within;
+      }
+      __syncthreads();
+      const uint64_t count = b1 - b0;
+      uint64_t head = ((16u - (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(tensor)) & 15u)) & 15u) / sizeof(T);
+      if (head > count) head = count;
+      const uint64_t nvec = (count - head) / VEC;
+      uint32_t sub_tiles = static_cast<uint32_t>((nvec + kBlock - 1) / kBlock);
+      if (sub_tiles == 0) sub_tiles = 1;
+      for (uint32_t sub = 0; sub < sub_tiles; sub++)
+        fold_tile<T, 1, kFoldGroup, DIV, NT, true>(tensor, s_src, tab.m + 1, count, sub, sub_tiles, tab.divisor, DIV,
+                                                   s_wire, 1);
+      __syncthreads();  // before the next piece overwrites the pointers
+      b0 = b1;
     }
     if (staged) __syncthreads();  // before the next tile overwrites the table
   }
@@ -1994,6 +2119,77 @@ int fusion_spans_run(const ring_fusion_plan* p, const ring_fusion_span* spans, i
 }  // namespace
 
 extern "C" {
+
+int ring_fusion_fold_scatter(const ring_fusion_plan* plan, uint64_t fold_begin, uint64_t fold_count,
+                             const void* const* staged, int m, void* wire, const ring_fusion_span* finished,
+                             int n_finished, int divisor, void* stream) {
+  const ring_fusion_plan* p = plan;
+  if (!p || m < 0 || n_finished < 0 || divisor < 0 || (m > 0 && !staged) || (n_finished > 0 && !finished))
+    return RING_ERR_ARGUMENT;
+  if (m > kMaxDirectSpans || n_finished > kMaxDirectSpans) return RING_ERR_LIMIT;
+  const uint64_t fold_end = fold_begin + fold_count;
+  if (fold_end < fold_begin || fold_end > p->total) return RING_ERR_ARGUMENT;
+  FusionDirectTable tab;
+  tab.n = 0;
+  tab.divisor = divisor;
+  tab.m = m;
+  tab.fold_begin = fold_begin;
+  tab.fold_end = fold_end;
+  tab.wire = wire;
+  if (fold_count > 0) {
+    if (!wire || (reinterpret_cast<uintptr_t>(wire) & (p->esz - 1))) return RING_ERR_ARGUMENT;
+    for (int k = 0; k < m; k++)
+      if (!staged[k] || (reinterpret_cast<uintptr_t>(staged[k]) & (p->esz - 1))) return RING_ERR_ARGUMENT;
+  }
+  for (int k = 0; k < kMaxDirectSpans; k++) tab.staged[k] = (k < m && fold_count > 0) ? staged[k] : nullptr;
+  uint64_t lowest = fold_count > 0 ? fold_begin : p->total, highest = fold_count > 0 ? fold_end : 0;
+  uint64_t previous_end = 0;
+  for (int i = 0; i < n_finished; i++) {
+    const ring_fusion_span& sp = finished[i];
+    if (sp.count == 0) continue;
+    const uint64_t end = sp.begin + sp.count;
+    if (sp.begin < previous_end || end < sp.begin || end > p->total) return RING_ERR_ARGUMENT;
+    if (fold_count > 0 && sp.begin < fold_end && fold_begin < end) return RING_ERR_ARGUMENT;  // meets the fold span
+    if (!sp.incoming || (reinterpret_cast<uintptr_t>(sp.incoming) & (p->esz - 1))) return RING_ERR_ARGUMENT;
+    previous_end = end;
+    tab.span[tab.n++] = FusionDirectSpan{sp.begin, end, sp.incoming};
+    if (sp.begin < lowest) lowest = sp.begin;
+    if (end > highest) highest = end;
+  }
+  for (int k = tab.n; k < kMaxDirectSpans; k++) tab.span[k] = FusionDirectSpan{0, 0, nullptr};
+  if (highest <= lowest) return RING_OK;  // nothing to do
+  const uint64_t tile_elems = static_cast<uint64_t>(kFusionTileVecs) * (16 / p->esz);
+  const uint32_t tile_lo = static_cast<uint32_t>(lowest / tile_elems);
+  const uint32_t tile_hi = static_cast<uint32_t>((highest + tile_elems - 1) / tile_elems);
+  int nt = g_tuning.nt[kRoleUnpack];
+  if (nt < 0) nt = 3;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(tile_hi - tile_lo);
+#define RING_DIRECT(T, D, N)                                                                                  \
+  launch(fusion_direct_kernel<T, N, D>, grid, dim3(kBlock), s, static_cast<const uint64_t*>(p->d_offsets),    \
+         reinterpret_cast<T* const*>(p->d_ptrs), static_cast<const FusionTile*>(p->d_tiles), tile_lo, tile_hi, \
+         p->total, tab)
+#define RING_DIRECT_NT(T, D)                 \
+  switch (nt & 3) {                          \
+    case 0: RING_DIRECT(T, D, 0); break;     \
+    case 1: RING_DIRECT(T, D, 1); break;     \
+    case 2: RING_DIRECT(T, D, 2); break;     \
+    default: RING_DIRECT(T, D, 3); break;    \
+  }
+  if (divisor > 0) {
+    if (p->dtype == RING_F32) { RING_DIRECT_NT(float, true) }
+    else if (p->dtype == RING_I32) { RING_DIRECT_NT(int32_t, true) }
+    else { RING_DIRECT_NT(int64_t, true) }
+  } else {
+    if (p->dtype == RING_F32) { RING_DIRECT_NT(float, false) }
+    else if (p->dtype == RING_I32) { RING_DIRECT_NT(int32_t, false) }
+    else { RING_DIRECT_NT(int64_t, false) }
+  }
+#undef RING_DIRECT_NT
+#undef RING_DIRECT
+  RING_HIP(hipGetLastError());
+  return RING_OK;
+}
 
 int ring_fusion_allreduce_all(const ring_fusion_plan* const* in_plans, const ring_fusion_plan* const* out_plans, int n,
                               int divisor, void* stream) {

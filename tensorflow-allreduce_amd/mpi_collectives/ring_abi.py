@@ -25,7 +25,7 @@ EXPORTS = (
     "ring_allgather_steps", "ring_apply_rows", "ring_apply_rows_avg", "ring_fold_rows", "ring_fold_and_copy_rows", "ring_fold_to_all_rows", "ring_fusion_allreduce_all",
     "ring_fusion_plan_create", "ring_fusion_plan_destroy", "ring_fusion_plan_elements", "ring_fusion_plan_dtype",
     "ring_fusion_pack", "ring_fusion_unpack", "ring_fusion_unpack_scaled", "ring_fusion_gather",
-    "ring_fusion_scatter", "ring_scale", "ring_fusion_run_static",
+    "ring_fusion_scatter", "ring_fusion_fold_scatter", "ring_scale", "ring_fusion_run_static",
 )
 
 
@@ -138,6 +138,8 @@ def lib():
             "ring_fusion_unpack_scaled": (ci, [vp, vp, ci, vp]),
             "ring_fusion_gather": (ci, [vp, ctypes.POINTER(FusionSpan), ci, vp]),
             "ring_fusion_scatter": (ci, [vp, ctypes.POINTER(FusionSpan), ci, ci, vp]),
+            "ring_fusion_fold_scatter": (ci, [vp, ctypes.c_uint64, ctypes.c_uint64, ctypes.POINTER(vp), ci, vp,
+                                              ctypes.POINTER(FusionSpan), ci, ci, vp]),
             "ring_scale": (ci, [ci, vp, sz, ci, vp]),
             "ring_fusion_run_static": (ci, [ci, ctypes.POINTER(vp), psz, ci, ci, vp, ci, vp]),
         }
@@ -386,6 +388,15 @@ class FusionPlan:
     def scatter(self, spans, divisor, stream):
         """tensors = incoming (/ divisor) per span."""
         check(lib().ring_fusion_scatter(self._h, spans[0], spans[1], divisor, stream), "ring_fusion_scatter")
+
+    def fold_scatter(self, fold_begin, fold_count, staged, wire, finished, divisor, stream):
+        """The direct form in one launch: the owned span folded from `staged`
+        (pointers, in fold order) and the tensors, the sum to `wire`, the
+        tensors = sum (/ divisor); `finished` spans (make_spans) scattered."""
+        m = len(staged)
+        sp = (ctypes.c_void_p * max(m, 1))(*staged)
+        check(lib().ring_fusion_fold_scatter(self._h, fold_begin, fold_count, sp, m, wire, finished[0], finished[1],
+                                             divisor, stream), "ring_fusion_fold_scatter")
 
     def close(self):
         if self._h:

@@ -428,6 +428,44 @@ void test_fusion(const std::vector<size_t>& counts, int divisor, int n_ranks) {
     OK(ring_fusion_scatter(p2, spans.data(), n_ranks, divisor, nullptr));
     check_tensors(out, scattered, "scatter");
     OK(ring_fusion_plan_destroy(p2));
+    // the direct form in one launch: segment `own` folded from staged copies and the tensors (last), its sum
+    // to the wire buffer, the quotient into the tensors; the other segments scattered
+    for (int own : {0, n_ranks / 2, n_ranks - 1}) {
+      std::vector<Buf<T>> work;
+      std::vector<const void*> work_ptrs;
+      fresh(work, work_ptrs);
+      size_t at = 0;
+      for (auto& t : work) {
+        memcpy(t.p, packed.data() + at, t.count * sizeof(T));
+        at += t.count;
+      }
+      ring_fusion_plan* p3 = nullptr;
+      OK(ring_fusion_plan_create(work_ptrs.data(), counts.data(), static_cast<int>(counts.size()), code<T>(), &p3));
+      std::vector<Buf<T>> staged;
+      std::vector<const void*> staged_ptrs;
+      for (int k = 0; k < n_ranks - 1; k++) {
+        staged.emplace_back(sizes[own], (k + 1) % 4);
+        staged_ptrs.push_back(staged.back().p);
+      }
+      std::vector<T> sum(sizes[own]);
+      for (size_t e = 0; e < sizes[own]; e++) {
+        T acc = n_ranks > 1 ? staged[0].p[e] : packed[starts[own] + e];
+        for (int k = 1; k < n_ranks - 1; k++) acc = add(staged[k].p[e], acc);
+        if (n_ranks > 1) acc = add(packed[starts[own] + e], acc);
+        sum[e] = acc;
+      }
+      std::vector<ring_fusion_span> others;
+      std::vector<T> want_tensors(scattered);
+      for (int g = 0; g < n_ranks; g++)
+        if (g != own) others.push_back(ring_fusion_span{starts[g], sizes[g], incoming[g].p, nullptr});
+      for (size_t e = 0; e < sizes[own]; e++) want_tensors[starts[own] + e] = divisor ? divide(sum[e], divisor) : sum[e];
+      Buf<T> wire2(sizes[own], 1, false);
+      OK(ring_fusion_fold_scatter(p3, starts[own], sizes[own], staged_ptrs.data(), n_ranks - 1, wire2.p, others.data(),
+                                  n_ranks - 1, divisor, nullptr));
+      expect_equal(wire2.p, sum, "fold_scatter wire");
+      check_tensors(work, want_tensors, "fold_scatter tensors");
+      OK(ring_fusion_plan_destroy(p3));
+    }
   }
   OK(ring_fusion_plan_destroy(plan));
   for (auto& t : tensors) t.check_lead();

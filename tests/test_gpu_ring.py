@@ -552,6 +552,9 @@ def test_fused_allreduce_without_pack_and_unpack_passes(oracle, dtype):
                     G.assert_same_bits(G.host(dts[j][0]), want[at:at + c],
                                        "direct fused n=%d rank %d tensor %d /%d" % (n, r, j, divisor))
                     at += c
+                # the owned segment of the wire buffer: the sum itself, as the rank sends it on
+                a, b = starts[own], starts[own] + sizes[own]
+                G.assert_same_bits(G.host(wire)[a:b], outs[0][a:b], "direct fused wire n=%d rank %d" % (n, r))
             plan.close()
 
 
