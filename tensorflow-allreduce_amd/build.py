@@ -145,9 +145,30 @@ def build_launch_shape_probe(verbose=True):
     return exe
 
 
+def build_launch_bound_steps(verbose=True):
+    """examples/build/launch_bound_steps: a small tensor's allreduce step driven
+    from C++ through the C ABI, eager and as recorded HIP graphs (host clock)."""
+    cxx = shutil.which("g++") or shutil.which("c++")
+    out_dir = os.path.join(HERE, "examples", "build")
+    os.makedirs(out_dir, exist_ok=True)
+    exe = os.path.join(out_dir, "launch_bound_steps")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = [cxx, "-O2", "-std=c++17", "-Wall", "-Wextra", "-D__HIP_PLATFORM_AMD__",
+           "-I", os.path.join(rocm, "include"), "-I", os.path.join(ROOT, "include"),
+           "-o", exe, os.path.join(HERE, "examples", "launch_bound_steps.cc"),
+           "-L", LIB_DIR, "-lmpi_collectives", "-lring_hip", "-L", os.path.join(rocm, "lib"), "-lamdhip64",
+           "-Wl,-rpath," + LIB_DIR, "-Wl,-rpath," + os.path.join(rocm, "lib")]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("g++ failed:\n" + res.stdout)
+    return exe
+
+
 def build_all(verbose=True):
     return [build_ring_hip(verbose), build_plugin(verbose), build_cpp_gpu_test(verbose),
-            build_launch_shape_probe(verbose)]
+            build_launch_shape_probe(verbose), build_launch_bound_steps(verbose)]
 
 
 if __name__ == "__main__":

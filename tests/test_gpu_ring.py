@@ -558,6 +558,61 @@ def test_fused_allreduce_without_pack_and_unpack_passes(oracle, dtype):
             plan.close()
 
 
+@pytest.mark.parametrize("dtype", G.DTYPES)
+def test_direct_fused_form_split_at_the_exchange(oracle, dtype):
+    """With a real exchange the direct form is two launches: the fold of the
+    owned segment (ring_fusion_fold_scatter with no finished spans), whose sum
+    the rank then sends, and, once the peers' finished segments have arrived,
+    their scatter. Same tensors and the same wire segment as the one launch;
+    also the argument checks of the entry point."""
+    stream = torch.cuda.current_stream().cuda_stream
+    abi = G.NP2ABI[np.dtype(dtype)]
+    for n, counts, divisor in [(5, [3, 0, 9000, 17, 4096, 1, 5000], 5), (2, [70_001], 0), (33, [40] * 50, 3), (34, [40] * 50, 0)]:
+        total = sum(counts)
+        grads = [[G.random_array(np.random.default_rng(31 * r + j), c, dtype) for j, c in enumerate(counts)]
+                 for r in range(n)]
+        packed = [np.concatenate(g) for g in grads]
+        summed = oracle.ring_allreduce(packed)[0]
+        want = _tf_div(summed, divisor) if divisor else summed
+        sizes, starts = ring_abi.segment_table(total, n)
+        r = n - 2
+        own = (r + 1) % n
+        dts = [G.dev(t, (j + 1) % 4) for j, t in enumerate(grads[r])]
+        plan = ring_abi.FusionPlan([d[0].data_ptr() if c else None for d, c in zip(dts, counts)], counts, abi)
+        wire = torch.zeros(sizes[own] + 2, dtype=G.NP2TORCH[np.dtype(dtype)], device="cuda")[1:sizes[own] + 1]
+        raw = [cuda(packed[(own + k) % n][starts[own]:starts[own] + sizes[own]]) for k in range(n - 1)]
+        fin = {g: cuda(summed[starts[g]:starts[g] + sizes[g]]) for g in range(n) if g != own}
+        others = [(starts[g], sizes[g], fin[g].data_ptr(), None) for g in range(n) if g != own]
+        if n - 1 > 32:
+            with pytest.raises(ring_abi.RingError) as e:
+                plan.fold_scatter(starts[own], sizes[own], [t.data_ptr() for t in raw], wire.data_ptr(),
+                                  ring_abi.make_spans([]), divisor, stream)
+            assert e.value.status == 5            # beyond the capacity of one launch
+            plan.close()
+            continue
+        plan.fold_scatter(starts[own], sizes[own], [t.data_ptr() for t in raw], wire.data_ptr(),
+                          ring_abi.make_spans([]), divisor, stream)
+        torch.cuda.synchronize()
+        G.assert_same_bits(G.host(wire), summed[starts[own]:starts[own] + sizes[own]], "wire after the fold")
+        flat = np.concatenate([G.host(d[0]) for d in dts]) if total else np.zeros(0, dtype)
+        a, b = starts[own], starts[own] + sizes[own]
+        G.assert_same_bits(flat[a:b], want[a:b], "owned segment in the tensors")
+        G.assert_same_bits(np.concatenate([flat[:a], flat[b:]]), np.concatenate([packed[r][:a], packed[r][b:]]),
+                           "the other segments untouched by the fold")
+        plan.scatter(ring_abi.make_spans(others), divisor, stream)
+        torch.cuda.synchronize()
+        G.assert_same_bits(np.concatenate([G.host(d[0]) for d in dts]), want, "tensors after the scatter")
+        # a finished span that meets the fold span, a span beyond the plan, a null staged copy
+        for bad in ([(starts[own], 1, fin[(own + 1) % n].data_ptr(), None)], [(total, 1, fin[(own + 1) % n].data_ptr(), None)]):
+            with pytest.raises(ring_abi.RingError):
+                plan.fold_scatter(starts[own], sizes[own], [t.data_ptr() for t in raw], wire.data_ptr(),
+                                  ring_abi.make_spans(bad), divisor, stream)
+        with pytest.raises(ring_abi.RingError):
+            plan.fold_scatter(starts[own], sizes[own], [None] * (n - 1), wire.data_ptr(), ring_abi.make_spans([]),
+                              divisor, stream)
+        plan.close()
+
+
 def test_distributed_optimizer_fused_and_unfused(oracle):
     """DistributedOptimizer.compute_gradients averages every gradient across
     ranks (__init__.py:195-205); with fusion=True through one fused buffer."""
