@@ -54,7 +54,7 @@ TRAFFIC_PROFILES = {
     "allreduce_f32_1GiB_n64": "rows_kernel_f32_1GiB_n64.txt",
     "fused_resnet50_n8": "fusion_kernel_resnet50_161_tensors_n8.txt",
     "fused_resnet50_n8_no_passes": "fusion_span_kernel_resnet50_161_tensors_n8_no_passes.txt",
-    "fused_resnet50_n8_no_passes_direct": "fusion_span_kernel_resnet50_161_tensors_n8_direct.txt",
+    "fused_resnet50_n8_no_passes_direct": "fusion_direct_kernel_resnet50_161_tensors_n8.txt",
     "allreduce_f32_64MiB_n8_direct": "fold_kernel_f32_64MiB_n8_direct.txt",
     "allreduce_f32_64MiB_all_ranks_n8": "fold_kernel_f32_64MiB_all_ranks_n8.txt",
     "fused_resnet50_all_ranks_n8": "fusion_allreduce_kernel_resnet50_161_tensors_all_ranks_n8.txt",
