@@ -397,6 +397,100 @@ __global__ void __launch_bounds__(kBlock) rows_kernel_small(const SmallRowTable 
 }
 #undef RING_ROWS_KERNEL_BODY
 
+// The copies of an allgather phase as ONE read phase and ONE write phase of the
+// whole chip, the payload held in registers in between. One workgroup per CU,
+// every one resident (512 registers per lane leave room for one wave per
+// SIMD). The chip sweeps the rows one after the other, front to back: a lane
+// takes vectors base, base + stride, ... of a row's body (stride = workgroups
+// * 256), issues the loads of all rows, waits for the last, and stores in the
+// same order. HBM serves one direction at a time faster than the two
+// interleaved: measured stand-alone, a copy of 56-112 MiB runs at 76-78 % of
+// the roofline this way against 70-72 % as plain tiles.
+// What such a launch costs is its number of rounds (the most vectors any lane
+// takes), not its bytes: a row whose last round is a tenth full costs a whole
+// round. So the workgroup that takes the first 256 vectors of a row is not
+// workgroup 0 but the one after the last workgroup of the previous row's
+// last round (shift[row], set by the host): the rounds of successive rows
+// chain, every lane takes the same number of vectors to within one, and the
+// sweep over memory never restarts. Sweeping the rows side by side instead
+// (a grid of (x, rows)) ran 10-20 % slower than plain tiles.
+// ROWS is a template parameter so that a register's row is known at compile
+// time and the rows' pointers stay in scalar registers; a row has room for
+// kPhasedMax / ROWS vectors per lane.
+constexpr int kPhasedMax = 112;
+struct PhasedShape {
+  uint32_t rounds;             // most rounds any row needs (<= kPhasedMax / ROWS)
+  uint32_t shift[kSmallRows];  // the workgroup that starts row k
+};
+#ifdef HIP_CPU_SHIM_RUNTIME_H_
+#define RING_ONE_WAVE_PER_SIMD
+#else
+#define RING_ONE_WAVE_PER_SIMD __attribute__((amdgpu_waves_per_eu(1, 1)))
+#endif
+template <typename T, int ROWS>
+__global__ void __launch_bounds__(kBlock) RING_ONE_WAVE_PER_SIMD
+rows_phased_kernel(const SmallRowTable tab, const PhasedShape shape) {
+  if (tab.dry) return;
+  typedef typename VecOf<T>::type V;
+  typedef V VU __attribute__((aligned(sizeof(T))));
+  typedef T RING_GLOBAL GT;
+  typedef V RING_GLOBAL GV;
+  typedef VU RING_GLOBAL GVU;
+  constexpr uint32_t VEC = 16 / sizeof(T);
+  constexpr int PER = kPhasedMax / ROWS;
+  const uint32_t tid = threadIdx.x;
+  const uint32_t stride = gridDim.x * kBlock;
+  V s[ROWS * PER];
+  // where a row's body starts and how many vectors it has (uniform)
+  auto head_of = [](const Row& r) {
+    uint64_t head = ((kRowHeadAlign - (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(r.dst)) & (kRowHeadAlign - 1))) &
+                     (kRowHeadAlign - 1)) / sizeof(T);
+    return head > r.count ? r.count : head;
+  };
+  // the lane's first vector of row k: the workgroups take the row in the order shift[k], shift[k] + 1, ...
+  auto first_of = [&](int k) {
+    uint32_t w = blockIdx.x + gridDim.x - shape.shift[k];
+    if (w >= gridDim.x) w -= gridDim.x;
+    return w * kBlock + tid;
+  };
+#pragma unroll
+  for (int k = 0; k < ROWS; k++) {
+    const Row r = tab.row[k];
+    const uint64_t head = head_of(r);
+    const uint32_t nvec = static_cast<uint32_t>((r.count - head) / VEC);
+    const GT* a = (const GT*)static_cast<const T*>(r.a);
+    if (blockIdx.x == 0) {  // the row's scalar head and tail
+      GT* dst = (GT*)static_cast<T*>(r.dst);
+      if (tid < head) dst[tid] = a[tid];
+      const uint64_t e = head + static_cast<uint64_t>(nvec) * VEC + tid;
+      if (e < r.count) dst[e] = a[e];
+    }
+    const GVU* av = (const GVU*)(a + head);
+    const uint32_t base = first_of(k);
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+      if (static_cast<uint32_t>(j) < shape.rounds) {
+        if (base + j * stride < nvec) s[k * PER + j] = __builtin_nontemporal_load(&(av + j * stride)[base]);
+      }
+    }
+  }
+  RING_WAIT_VMEM();
+#pragma unroll
+  for (int k = 0; k < ROWS; k++) {
+    const Row r = tab.row[k];
+    const uint64_t head = head_of(r);
+    const uint32_t nvec = static_cast<uint32_t>((r.count - head) / VEC);
+    GV* dv = (GV*)((GT*)static_cast<T*>(r.dst) + head);
+    const uint32_t base = first_of(k);
+#pragma unroll
+    for (int j = 0; j < PER; j++) {
+      if (static_cast<uint32_t>(j) < shape.rounds) {
+        if (base + j * stride < nvec) __builtin_nontemporal_store(s[k * PER + j], &(dv + j * stride)[base]);
+      }
+    }
+  }
+}
+
 // Byte copy for operands that are not 4-byte compatible (never produced by the
 // three element types; kept so ring_copy_bytes is total).
 __global__ void __launch_bounds__(kBlock) bytes_kernel(uint8_t* __restrict__ dst,
@@ -1028,6 +1122,10 @@ struct Tuning {
   // phase and one write phase (rows_kernel's PACE): -1 chosen by the size of
   // the launch, 0 never, 1 always.
   int paced_copy = -1;
+  // The same idea with the whole payload of the launch in registers
+  // (rows_phased_kernel): -1 chosen by the size of the launch, 0 never, 1
+  // whenever the launch fits.
+  int phased_copy = -1;
   int blocks_per_cu = 0;   // 0: one workgroup per tile; >0: persistent grid of CUs x this
   int dry_launch = 0;      // measurement only: the step-table kernels return at entry (what a launch of that grid costs)
 };
@@ -1145,6 +1243,69 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
   // bound by memory rather than by its dispatch (2 per CU). Measured on 7 rows:
   // 21-56 MiB per side 1-10 % faster than the plain tiles (56 MiB: 19.6 against
   // 20.8 us), slower beyond (63 MiB: 25.3 against 23.7 us) and no different below.
+  // The copies of an allgather phase with the whole payload in registers
+  // between one read phase and one write phase (rows_phased_kernel): up to
+  // kSmallRows rows, each within its share of the registers, non-temporal both
+  // ways. By itself from 60 MiB per side on a whole chip, for rows whose source
+  // and destination are 16-byte aligned together.
+  if (role == kRoleAllgather && divisor <= 0 && n_rows >= 1 && n_rows <= static_cast<size_t>(kSmallRows) &&
+      (nt & 3) == 3 && g_tuning.phased_copy != 0 && g_tuning.blocks_per_cu == 0) {
+    int rc = device_info(&info);
+    if (rc != RING_OK) return rc;
+    const uint64_t wgs = static_cast<uint64_t>(info.cus), stride = wgs * kBlock;
+    const uint64_t room = static_cast<uint64_t>(kPhasedMax / static_cast<int>(n_rows));
+    SmallRowTable tab;
+    PhasedShape shape;
+    shape.rounds = 0;
+    uint64_t bytes = 0, start = 0;
+    bool fits = true;
+    for (size_t k = 0; k < static_cast<size_t>(kSmallRows); k++) {
+      shape.shift[k] = 0;
+      tab.row[k] = Row{nullptr, nullptr, nullptr, 0};
+      if (k >= n_rows || !fits) continue;
+      const HostRow& r = rows[k];
+      if (r.b != nullptr || r.count == 0) { fits = false; continue; }
+      const uintptr_t d = reinterpret_cast<uintptr_t>(r.dst);
+      uint64_t head = ((kRowHeadAlign - (d & (kRowHeadAlign - 1))) & (kRowHeadAlign - 1)) / esz;
+      if (head > r.count) head = r.count;
+      const uint64_t nvec = (r.count - head) / vec;
+      const uint64_t rounds = (nvec + stride - 1) / stride;
+      if (rounds > room) { fits = false; continue; }
+      // source and destination 16-byte aligned together: with one wave per SIMD the launch is bound by
+      // what a CU issues, and loads that straddle 16-byte groups cost it 15 % (the tiles lose 1 %)
+      if (g_tuning.phased_copy < 0 && ((reinterpret_cast<uintptr_t>(r.a) + head * esz) & 15u)) { fits = false; continue; }
+      if (rounds > shape.rounds) shape.rounds = static_cast<uint32_t>(rounds);
+      tab.row[k] = Row{r.dst, r.a, nullptr, r.count};
+      shape.shift[k] = static_cast<uint32_t>(start);
+      // the next row starts behind the last workgroup of this row's last round
+      start = (start + (nvec % stride + kBlock - 1) / kBlock) % wgs;
+      bytes += r.count * esz;
+    }
+    if (fits && (g_tuning.phased_copy > 0 || (bytes >= (60ull << 20) && info.cus >= 128))) {
+      tab.n_rows = static_cast<int>(n_rows);
+      tab.dry = g_tuning.dry_launch;
+      tab.uniform_tiles = 0;
+      tab.divisor = 0;
+      tab.div_mask = 0;
+      for (int k = 0; k <= kSmallRows; k++) tab.tile_begin[k] = 0;
+      const dim3 grid(static_cast<uint32_t>(wgs));
+#define RING_PHASED(T)                                                                                   \
+  switch (n_rows) {                                                                                      \
+    case 1: launch(rows_phased_kernel<T, 1>, grid, dim3(kBlock), stream, tab, shape); break;             \
+    case 2: launch(rows_phased_kernel<T, 2>, grid, dim3(kBlock), stream, tab, shape); break;             \
+    case 3: launch(rows_phased_kernel<T, 3>, grid, dim3(kBlock), stream, tab, shape); break;             \
+    case 4: launch(rows_phased_kernel<T, 4>, grid, dim3(kBlock), stream, tab, shape); break;             \
+    case 5: launch(rows_phased_kernel<T, 5>, grid, dim3(kBlock), stream, tab, shape); break;             \
+    case 6: launch(rows_phased_kernel<T, 6>, grid, dim3(kBlock), stream, tab, shape); break;             \
+    case 7: launch(rows_phased_kernel<T, 7>, grid, dim3(kBlock), stream, tab, shape); break;             \
+    default: launch(rows_phased_kernel<T, 8>, grid, dim3(kBlock), stream, tab, shape); break;            \
+  }
+      if (esz == 8) { RING_PHASED(uint64_t) } else { RING_PHASED(uint32_t) }
+#undef RING_PHASED
+      RING_HIP(hipGetLastError());
+      return RING_OK;
+    }
+  }
   bool paced = false;
   if (role == kRoleAllgather && divisor <= 0 && n_rows <= static_cast<size_t>(kMaxRows) && g_tuning.paced_copy != 0) {
     bool copy_only = true;
@@ -1471,6 +1632,9 @@ int ring_set_option(const char* name, int value) {
   } else if (!strcmp(name, "paced_copy")) {
     if (value < -1 || value > 1) return RING_ERR_ARGUMENT;
     g_tuning.paced_copy = value;
+  } else if (!strcmp(name, "phased_copy")) {
+    if (value < -1 || value > 1) return RING_ERR_ARGUMENT;
+    g_tuning.phased_copy = value;
   } else if (!strncmp(name, "nontemporal", 11)) {
     static const char* const kSuffix[kRoles] = {"_copy", "_accumulate", "_allgather", "_pack", "_unpack",
                                                 "_fold", "_broadcast", "_fold_all"};

@@ -491,6 +491,15 @@ void run_all(const char* name) {
   test_step_tables<T>(100003, 6);
   test_step_tables<T>(70001, 3);
   CHECK(ring_set_option("paced_copy", -1) == RING_OK);
+  CHECK(ring_set_option("phased_copy", 1) == RING_OK);  // ... and with the payload of the launch in registers
+  test_step_tables<T>(40013, 3);
+  test_step_tables<T>(100003, 4);
+  test_step_tables<T>(5, 4);
+  test_step_tables<T>(70001, 2);
+  test_step_tables<T>(65536, 8);
+  test_step_tables<T>(100003, 6);
+  test_step_tables<T>(900001, 9);   // 8 rows, each needing all of its share of the registers
+  CHECK(ring_set_option("phased_copy", -1) == RING_OK);
   printf("%s: fold\n", name); fflush(stdout);
   test_fold<T>(8, 10007, 0);
   test_fold<T>(3, 4096, 3);

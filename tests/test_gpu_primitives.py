@@ -6,6 +6,7 @@ import ctypes
 
 import numpy as np
 import pytest
+import torch
 
 import gpu_util as G
 from gpu_util import ring_abi
@@ -19,7 +20,7 @@ COUNTS = [0, 1, 2, 3, 4, 5, 7, 8, 1023, 1024, 1025, 4096, 4097, 3 * 4096 + 7, 26
 def _gpu():
     G.require_gpu()
     yield
-    for k, v in (("unroll", 4), ("nontemporal", -1), ("blocks_per_cu", 0), ("paced_copy", -1)):
+    for k, v in (("unroll", 4), ("nontemporal", -1), ("blocks_per_cu", 0), ("paced_copy", -1), ("phased_copy", -1)):
         ring_abi.set_option(k, v)
 
 
@@ -184,6 +185,46 @@ def test_paced_allgather_copies_match(dtype, paced):
             G.assert_same_bits(G.host(dbuf), want, "paced=%d rows=%d" % (paced, n_rows))
     finally:
         ring_abi.set_option("paced_copy", -1)
+
+
+@pytest.mark.parametrize("dtype", G.DTYPES)
+@pytest.mark.parametrize("phased", [1, 0, -1])
+def test_phased_allgather_copies_match(dtype, phased):
+    """The allgather copies with the whole payload in registers between one read
+    phase and one write phase of the chip (rows of near-equal length, at most
+    one workgroup per CU), forced on for every launch that fits and forced off:
+    the same bytes either way, ragged segments at any alignment, counts from
+    fewer elements than ranks up to all 112 vectors a lane has room for, and
+    counts that just no longer fit (they must fall back, not truncate)."""
+    rng = np.random.default_rng(43 + phased)
+    code = G.NP2ABI[np.dtype(dtype)]
+    vec = 16 // np.dtype(dtype).itemsize
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    ring_abi.set_option("phased_copy", phased)
+    try:
+        stride = cus * 256 * vec                                  # elements the chip takes per round
+        cases = [(8, 5), (6, 100_003), (8, 1_000_003), (3, 70_001), (64, 1_000_003), (2, 4_099), (9, 9_000_017),
+                 (8, 8 * 16 * stride),                            # 7 rows of 16 rounds: all the registers
+                 (8, 8 * (16 * stride + 128)),                    # a 17th round: must fall back, not truncate
+                 (5, 5 * 28 * stride + 3), (2, 2 * 112 * stride + 1)]
+        for n, count in cases:
+            sizes, starts = ring_abi.segment_table(count, n)
+            buf = G.random_array(rng, count + 5, dtype)
+            dbuf, _ = G.dev(buf, int(rng.integers(0, 4)))
+            want = buf.copy()
+            rows, keep = [], []
+            for g in range(1, n):                                 # n - 1 segments arrive, as in the allgather phase
+                src = G.random_array(rng, sizes[g], dtype)
+                ds, base = G.dev(src, int(rng.integers(0, 4)))
+                keep.append(base)
+                rows.append((starts[g], ds.data_ptr() if sizes[g] else None, sizes[g]))
+                want[starts[g]:starts[g] + sizes[g]] = src
+            steps, k = ring_abi.make_steps(rows)
+            ring_abi.allgather_steps(dbuf.data_ptr(), steps, k, code, None)
+            G.sync()
+            G.assert_same_bits(G.host(dbuf), want, "phased=%d n=%d count=%d" % (phased, n, count))
+    finally:
+        ring_abi.set_option("phased_copy", -1)
 
 
 @pytest.mark.parametrize("opt", [("unroll", 2), ("unroll", 8), ("nontemporal", 0),
