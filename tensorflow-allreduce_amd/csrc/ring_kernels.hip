@@ -404,8 +404,10 @@ __global__ void __launch_bounds__(kBlock) rows_kernel_small(const SmallRowTable 
 // takes vectors base, base + stride, ... of a row's body (stride = workgroups
 // * 256), issues the loads of all rows, waits for the last, and stores in the
 // same order. HBM serves one direction at a time faster than the two
-// interleaved: measured stand-alone, a copy of 56-112 MiB runs at 76-78 % of
-// the roofline this way against 70-72 % as plain tiles.
+// interleaved: measured stand-alone, a copy of 56-112 MiB runs at 76-79 % of
+// the roofline this way against 72-74 % as plain tiles; in a step, behind the
+// accumulate, the 7 ragged 12.2 MiB segments of the ResNet-50 set take 29.4 us
+// instead of 31.2 (76 %) and 5 int64 segments of 12.7 MiB 22.8 instead of 24.2.
 // What such a launch costs is its number of rounds (the most vectors any lane
 // takes), not its bytes: a row whose last round is a tenth full costs a whole
 // round. So the workgroup that takes the first 256 vectors of a row is not
@@ -413,7 +415,10 @@ __global__ void __launch_bounds__(kBlock) rows_kernel_small(const SmallRowTable 
 // last round (shift[row], set by the host): the rounds of successive rows
 // chain, every lane takes the same number of vectors to within one, and the
 // sweep over memory never restarts. Sweeping the rows side by side instead
-// (a grid of (x, rows)) ran 10-20 % slower than plain tiles.
+// (a grid of (x, rows)) ran 10-20 % slower than plain tiles. For the same
+// reason a row's scalar head and tail travel in registers like the rest: a
+// load, a wait and a store ahead of the loads held workgroup 0 back by a
+// memory latency per row, and the whole launch with it (32.5 us instead of 29.4).
 // ROWS is a template parameter so that a register's row is known at compile
 // time and the rows' pointers stay in scalar registers; a row has room for
 // kPhasedMax / ROWS vectors per lane.
@@ -441,6 +446,7 @@ rows_phased_kernel(const SmallRowTable tab, const PhasedShape shape) {
   const uint32_t tid = threadIdx.x;
   const uint32_t stride = gridDim.x * kBlock;
   V s[ROWS * PER];
+  T edge_head[ROWS], edge_tail[ROWS];
   // where a row's body starts and how many vectors it has (uniform)
   auto head_of = [](const Row& r) {
     uint64_t head = ((kRowHeadAlign - (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(r.dst)) & (kRowHeadAlign - 1))) &
@@ -459,11 +465,12 @@ rows_phased_kernel(const SmallRowTable tab, const PhasedShape shape) {
     const uint64_t head = head_of(r);
     const uint32_t nvec = static_cast<uint32_t>((r.count - head) / VEC);
     const GT* a = (const GT*)static_cast<const T*>(r.a);
-    if (blockIdx.x == 0) {  // the row's scalar head and tail
-      GT* dst = (GT*)static_cast<T*>(r.dst);
-      if (tid < head) dst[tid] = a[tid];
+    if (blockIdx.x == 0) {
+      // the row's scalar head and tail travel in registers too: a load, a wait and a store here
+      // would hold workgroup 0 back by a memory latency per row, and the launch ends with its last workgroup
+      if (tid < head) edge_head[k] = a[tid];
       const uint64_t e = head + static_cast<uint64_t>(nvec) * VEC + tid;
-      if (e < r.count) dst[e] = a[e];
+      if (e < r.count) edge_tail[k] = a[e];
     }
     const GVU* av = (const GVU*)(a + head);
     const uint32_t base = first_of(k);
@@ -487,6 +494,12 @@ rows_phased_kernel(const SmallRowTable tab, const PhasedShape shape) {
       if (static_cast<uint32_t>(j) < shape.rounds) {
         if (base + j * stride < nvec) __builtin_nontemporal_store(s[k * PER + j], &(dv + j * stride)[base]);
       }
+    }
+    if (blockIdx.x == 0) {
+      GT* dst = (GT*)static_cast<T*>(r.dst);
+      if (tid < head) dst[tid] = edge_head[k];
+      const uint64_t e = head + static_cast<uint64_t>(nvec) * VEC + tid;
+      if (e < r.count) dst[e] = edge_tail[k];
     }
   }
 }
@@ -1246,8 +1259,7 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
   // The copies of an allgather phase with the whole payload in registers
   // between one read phase and one write phase (rows_phased_kernel): up to
   // kSmallRows rows, each within its share of the registers, non-temporal both
-  // ways. By itself from 60 MiB per side on a whole chip, for rows whose source
-  // and destination are 16-byte aligned together.
+  // ways. By itself from 60 MiB per side on a whole chip.
   if (role == kRoleAllgather && divisor <= 0 && n_rows >= 1 && n_rows <= static_cast<size_t>(kSmallRows) &&
       (nt & 3) == 3 && g_tuning.phased_copy != 0 && g_tuning.blocks_per_cu == 0) {
     int rc = device_info(&info);
@@ -1271,9 +1283,6 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
       const uint64_t nvec = (r.count - head) / vec;
       const uint64_t rounds = (nvec + stride - 1) / stride;
       if (rounds > room) { fits = false; continue; }
-      // source and destination 16-byte aligned together: with one wave per SIMD the launch is bound by
-      // what a CU issues, and loads that straddle 16-byte groups cost it 15 % (the tiles lose 1 %)
-      if (g_tuning.phased_copy < 0 && ((reinterpret_cast<uintptr_t>(r.a) + head * esz) & 15u)) { fits = false; continue; }
       if (rounds > shape.rounds) shape.rounds = static_cast<uint32_t>(rounds);
       tab.row[k] = Row{r.dst, r.a, nullptr, r.count};
       shape.shift[k] = static_cast<uint32_t>(start);

@@ -10,7 +10,7 @@
 // use the library: every variant is a few lines here.
 //
 //   hipcc -O3 --offload-arch=gfx950 launch_shape_probe.hip -o launch_shape_probe
-//   ./launch_shape_probe [floor|pipeline|paced|rounds|timeline|all]
+//   ./launch_shape_probe [floor|pipeline|paced|rounds|registers|timeline|all]
 //
 // Buffers hold random data and rotate over 8 sets (1.9 GiB), so nothing a
 // launch reads is left in a cache by the one before. Durations come from HIP
@@ -180,6 +180,55 @@ __global__ void __launch_bounds__(256) k_paced(Rows r, unsigned tiles_per_row, u
   }
 }
 
+// The whole payload of a launch in registers between ONE read phase and ONE write phase: one
+// workgroup per CU (512 registers per lane: one wave per SIMD), a lane takes vectors base,
+// base + stride, ... (stride = workgroups * 256), issues all its loads, waits, stores.
+// SIDE_BY_SIDE: grid (x, rows), every row swept at the same time by its own x workgroups.
+// Otherwise grid (workgroups) and the rows one after the other; CHAIN: the workgroup that
+// takes a row's first 256 vectors is the one after the last workgroup of the previous row's
+// last round (shift[row]), so that every lane takes the same number of vectors to within one.
+// OFF: the sources are read 4 * OFF bytes further on (loads that straddle 16-byte groups).
+struct Shift {
+  unsigned s[kRows];
+};
+typedef f4 f4u __attribute__((aligned(4)));
+template <int PER, bool SIDE_BY_SIDE, bool CHAIN, int OFF>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+k_registers(Rows r, unsigned nvec, unsigned rounds, Shift sh) {
+  constexpr int ROWS = SIDE_BY_SIDE ? 1 : kRows;
+  const unsigned stride = gridDim.x * 256;
+  f4 s[ROWS * PER];
+#pragma unroll
+  for (int k = 0; k < ROWS; k++) {
+    const int row = SIDE_BY_SIDE ? blockIdx.y : k;
+    const f4u* src = (const f4u*)((const char*)r.src[row] + 4 * OFF);
+    unsigned w = blockIdx.x;
+    if (CHAIN) {
+      w += gridDim.x - sh.s[k];
+      if (w >= gridDim.x) w -= gridDim.x;
+    }
+    const unsigned base = w * 256 + threadIdx.x;
+#pragma unroll
+    for (int j = 0; j < PER; j++)
+      if (j < rounds && base + j * stride < nvec) s[k * PER + j] = LD(&src[base + j * stride]);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int k = 0; k < ROWS; k++) {
+    const int row = SIDE_BY_SIDE ? blockIdx.y : k;
+    f4* dst = r.dst[row];
+    unsigned w = blockIdx.x;
+    if (CHAIN) {
+      w += gridDim.x - sh.s[k];
+      if (w >= gridDim.x) w -= gridDim.x;
+    }
+    const unsigned base = w * 256 + threadIdx.x;
+#pragma unroll
+    for (int j = 0; j < PER; j++)
+      if (j < rounds && base + j * stride < nvec) ST(s[k * PER + j], &dst[base + j * stride]);
+  }
+}
+
 struct Buffers {
   static const int kSets = 8;
   size_t seg = 0;
@@ -203,6 +252,13 @@ struct Buffers {
         CK(hipMemcpy(staged[i][j], noise.data() + 1000 * j, seg + 4096, hipMemcpyHostToDevice));
       }
     }
+  }
+  void release() {
+    for (auto p : out) CK(hipFree(p));
+    for (auto& v : staged)
+      for (auto p : v) CK(hipFree(p));
+    out.clear();
+    staged.clear();
   }
   // the 7 segments of set s that an allgather / reduce-scatter phase of rank s touches
   Rows rows(int s) const {
@@ -412,6 +468,61 @@ int main(int argc, char** argv) {
   }
     ROUNDS(8, 1, 1, 0) ROUNDS(8, 1, 1, 7) ROUNDS(8, 1, 1, 4) ROUNDS(8, 1, 0, 4) ROUNDS(8, 0, 0, 7)
     ROUNDS(4, 1, 1, 0) ROUNDS(4, 1, 1, 8) ROUNDS(4, 0, 0, 8) ROUNDS(16, 1, 1, 0) ROUNDS(16, 1, 1, 3)
+  }
+
+  if (wanted("registers")) {
+    for (size_t seg_bytes : {(size_t)8 << 20, (size_t)9 << 20, (size_t)12800 << 10}) {
+      Buffers M;
+      M.init(seg_bytes);
+      const unsigned nvec = M.seg / 16, mt4 = (nvec + 1023) / 1024;
+      const double mbytes = 2.0 * kRows * M.seg;
+      printf("\n-- the payload of the launch in registers between one read phase and one write phase (7 x %.2f MiB)\n",
+             M.seg / 1048576.0);
+      for (int behind = 0; behind < 2; behind++) {
+        const char* where = behind ? ", behind acc" : "";
+        auto before = [&](int s) {
+          if (behind) PLAIN((k_tile<kAcc, 4>), dim3(mt4, kRows), M.rows(s), mt4, no_ts);
+        };
+        char nm[160];
+        snprintf(nm, sizeof nm, "copy%s: 16 KiB tiles, one workgroup per tile (reference point)", where);
+        run(nm, mbytes, [&](int s, hipEvent_t a, hipEvent_t b) {
+          before(s);
+          EXT((k_tile<kCopy, 4>), dim3(mt4, kRows), a, b, M.rows((s + 3) % 8), mt4, no_ts);
+        });
+        const unsigned gx = cus / kRows, side_rounds = (nvec + gx * 256 - 1) / (gx * 256);
+        snprintf(nm, sizeof nm, "copy%s: in registers, the 7 rows side by side, grid (%u, 7), %u rounds", where, gx, side_rounds);
+        if (side_rounds <= 112)
+          run(nm, mbytes, [&](int s, hipEvent_t a, hipEvent_t b) {
+            before(s);
+            EXT((k_registers<112, true, false, 0>), dim3(gx, kRows), a, b, M.rows((s + 3) % 8), nvec, side_rounds, Shift{});
+          });
+        const unsigned stride = cus * 256, rounds = (nvec + stride - 1) / stride;
+        Shift sh{};
+        unsigned at = 0;
+        for (int k = 0; k < kRows; k++) {
+          sh.s[k] = at;
+          at = (at + (nvec % stride + 255) / 256) % cus;
+        }
+        if (rounds <= 16) {
+          snprintf(nm, sizeof nm, "copy%s: in registers, rows one after the other, %u rounds per row", where, rounds);
+          run(nm, mbytes, [&](int s, hipEvent_t a, hipEvent_t b) {
+            before(s);
+            EXT((k_registers<16, false, false, 0>), dim3(cus), a, b, M.rows((s + 3) % 8), nvec, rounds, sh);
+          });
+          snprintf(nm, sizeof nm, "copy%s: in registers, rows one after the other, rounds chained across rows", where);
+          run(nm, mbytes, [&](int s, hipEvent_t a, hipEvent_t b) {
+            before(s);
+            EXT((k_registers<16, false, true, 0>), dim3(cus), a, b, M.rows((s + 3) % 8), nvec, rounds, sh);
+          });
+          snprintf(nm, sizeof nm, "copy%s: the same, sources 4 bytes off their 16-byte groups", where);
+          run(nm, mbytes, [&](int s, hipEvent_t a, hipEvent_t b) {
+            before(s);
+            EXT((k_registers<16, false, true, 1>), dim3(cus), a, b, M.rows((s + 3) % 8), nvec, rounds, sh);
+          });
+        }
+      }
+      M.release();
+    }
   }
 
   if (wanted("timeline")) {
