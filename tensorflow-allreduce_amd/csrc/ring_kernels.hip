@@ -1632,7 +1632,9 @@ size_t ring_dtype_size(int dtype) { return dtype_size(dtype); }
 // Tuning knobs for measurement runs; not part of the drop-in surface.
 // name: "unroll" (2|4|8), "blocks_per_cu" (0 = one workgroup per tile),
 // "nontemporal" (bit 0 stores, bit 1 loads; sets every role) and
-// "nontemporal_copy" / "_accumulate" / "_allgather" / "_pack" / "_unpack".
+// "nontemporal_copy" / "_accumulate" / "_allgather" / "_pack" / "_unpack",
+// "paced_copy" and "phased_copy" (the two forms of the allgather copies that
+// read first and write after: -1 by size, 0 never, 1 always), "dry_launch".
 int ring_set_option(const char* name, int value) {
   if (!name) return RING_ERR_ARGUMENT;
   if (!strcmp(name, "unroll")) {
