@@ -759,7 +759,7 @@ def main():
                          "time its replays; for launch-bound sizes. --steps is rounded down to a multiple of it")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="launch option of the kernel library (unroll, blocks_per_cu, nontemporal[_copy|_accumulate|"
-                         "_allgather|_pack|_unpack]), "
+                         "_allgather|_pack|_unpack], paced_copy, phased_copy, dry_launch), "
                          "for comparing launch shapes under a profiler")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
