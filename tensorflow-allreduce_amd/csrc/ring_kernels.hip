@@ -17,10 +17,17 @@
 //     launch, not n-1 launches and n-1 host syncs. Rows with equal tile counts
 //     (the segments of an allreduce) use a 2-D grid (tiles, rows); unequal rows
 //     share a 1-D grid and a workgroup finds its row by a scalar binary search;
-//   * stores are 16-byte aligned: up to 3 head elements are peeled per row so
-//     the destination is aligned, the sources are read with element-aligned
-//     (possibly 16-byte-unaligned) dwordx4 loads. Ragged segment starts only
-//     cost those few scalar elements;
+//   * stores are aligned: a scalar head is peeled per row so that the
+//     destination starts on a 128-byte line (16 bytes in the fold and fusion
+//     kernels), the sources are read with element-aligned (possibly
+//     16-byte-unaligned) dwordx4 loads. Ragged segment starts only cost those
+//     few scalar elements;
+//   * a copy runs faster when the chip reads first and writes after than with
+//     the two directions interleaved: the copies of an allgather phase wait
+//     for all their loads before their first store when every tile is resident
+//     at once (the paced tiles), and from 60 MiB they hold the whole payload
+//     of the launch in registers, one workgroup per CU (rows_phased_kernel).
+//     Accumulates and folds, which read more than they write, gain nothing from it;
 //   * what is touched once (accumulates, allgather copies, unpack) is loaded
 //     and stored non-temporally; the in->out copy and the fusion pack, whose
 //     output the reduce-scatter reads next, store with the ordinary policy;
