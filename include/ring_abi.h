@@ -86,7 +86,7 @@ size_t ring_dtype_size(int dtype);
  * (between 2 and 7 tiles of 32 KiB per CU). "phased_copy": the same copies
  * with the whole payload of the launch held in registers between the two
  * phases (one workgroup per CU, up to 8 rows and 112 MiB): 1 whenever the
- * launch fits, 0 never, -1 (default) from 60 MiB per side.
+ * launch fits, 0 never, -1 (default) above 56 MiB per side.
  * "dry_launch" = 1 makes the step-table / copy /
  * accumulate kernels return at entry: what is then timed is what a launch of
  * that grid costs by itself. No counterpart in the reference, whose launch

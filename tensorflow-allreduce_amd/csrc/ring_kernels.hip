@@ -25,7 +25,7 @@
 //   * a copy runs faster when the chip reads first and writes after than with
 //     the two directions interleaved: the copies of an allgather phase wait
 //     for all their loads before their first store when every tile is resident
-//     at once (the paced tiles), and from 60 MiB they hold the whole payload
+//     at once (the paced tiles), and above 56 MiB they hold the whole payload
 //     of the launch in registers, one workgroup per CU (rows_phased_kernel).
 //     Accumulates and folds, which read more than they write, gain nothing from it;
 //   * what is touched once (accumulates, allgather copies, unpack) is loaded
@@ -1266,7 +1266,8 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
   // The copies of an allgather phase with the whole payload in registers
   // between one read phase and one write phase (rows_phased_kernel): up to
   // kSmallRows rows, each within its share of the registers, non-temporal both
-  // ways. By itself from 60 MiB per side on a whole chip.
+  // ways. By itself above 56 MiB per side (where the paced tiles end) on a whole chip:
+  // 57 MiB take 19.9 us this way and 21.3 as plain tiles.
   if (role == kRoleAllgather && divisor <= 0 && n_rows >= 1 && n_rows <= static_cast<size_t>(kSmallRows) &&
       (nt & 3) == 3 && g_tuning.phased_copy != 0 && g_tuning.blocks_per_cu == 0) {
     int rc = device_info(&info);
@@ -1297,7 +1298,7 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
       start = (start + (nvec % stride + kBlock - 1) / kBlock) % wgs;
       bytes += r.count * esz;
     }
-    if (fits && (g_tuning.phased_copy > 0 || (bytes >= (60ull << 20) && info.cus >= 128))) {
+    if (fits && (g_tuning.phased_copy > 0 || (bytes > (56ull << 20) && info.cus >= 128))) {
       tab.n_rows = static_cast<int>(n_rows);
       tab.dry = g_tuning.dry_launch;
       tab.uniform_tiles = 0;
