@@ -186,6 +186,62 @@ def test_fusion_spans_with_boundaries_on_tiles_and_tensors(counts, dtype, seed, 
     plan.close()
 
 
+@settings(max_examples=40, **COMMON)
+@given(counts=st.lists(st.one_of(st.integers(0, 6), st.sampled_from([1023, 4095, 4096, 4097, 8192]),
+                                 st.integers(0, 20_000)), min_size=1, max_size=24),
+       dtype=st.sampled_from(G.DTYPES), seed=st.integers(0, 2**31), divisor=st.sampled_from([0, 3, 8]),
+       n=st.integers(1, 9), own_pick=st.integers(0, 8), with_others=st.booleans())
+def test_fusion_fold_scatter_is_fold_then_scatter(counts, dtype, seed, divisor, n, own_pick, with_others):
+    """ring_fusion_fold_scatter on any tensor set and ring size: the owned
+    segment of the packed layout folded from n - 1 staged copies and the
+    tensors (last), in that order; its sum in the send buffer, sum (/ divisor)
+    in the tensors; the other segments scattered (/ divisor) or, without them,
+    left untouched. Against numpy on the concatenation."""
+    rng = np.random.default_rng(seed)
+    total = sum(counts)
+    hosts = [G.random_array(rng, c, dtype, wide=True) for c in counts]
+    devs = [G.dev(h, int(rng.integers(0, 4))) for h in hosts]
+    plan = ring_abi.FusionPlan([d[0].data_ptr() if c else None for d, c in zip(devs, counts)], counts,
+                               G.NP2ABI[np.dtype(dtype)])
+    flat = np.concatenate(hosts) if hosts else np.empty(0, dtype=dtype)
+    sizes, starts = ring_abi.segment_table(total, n)
+    own = own_pick % n
+    a, b = starts[own], starts[own] + sizes[own]
+    staged = [G.random_array(rng, sizes[own], dtype, wide=True) for _ in range(n - 1)]
+    d_staged = [G.dev(x, (k + 1) % 4) for k, x in enumerate(staged)]
+    with np.errstate(all="ignore"):
+        acc = flat[a:b].copy() if n == 1 else staged[0].copy()
+        for x in staged[1:]:
+            acc = (x + acc).astype(dtype)
+        if n > 1:
+            acc = (flat[a:b] + acc).astype(dtype)
+
+        def div(x):
+            if not divisor:
+                return x
+            return (x / np.float32(divisor) if dtype == np.float32 else x // dtype(divisor)).astype(dtype)
+        want = flat.copy()
+        want[a:b] = div(acc)
+        finished, keep = [], []
+        if with_others:
+            for g in range(n):
+                if g == own or sizes[g] == 0:
+                    continue
+                x = G.random_array(rng, sizes[g], dtype, wide=True)
+                d = G.dev(x, g % 4)
+                keep.append(d)
+                finished.append((starts[g], sizes[g], d[0].data_ptr(), None))
+                want[starts[g]:starts[g] + sizes[g]] = div(x)
+    wire = G.dev(np.zeros(sizes[own], dtype=dtype), 3)
+    plan.fold_scatter(a, sizes[own], [d[0].data_ptr() if sizes[own] else d[1].data_ptr() for d in d_staged],
+                      wire[0].data_ptr() if sizes[own] else wire[1].data_ptr(), ring_abi.make_spans(finished), divisor, None)
+    torch.cuda.synchronize()
+    G.assert_same_bits(G.host(wire[0]), acc, "send buffer n=%d own=%d" % (n, own))
+    got = np.concatenate([G.host(d[0]) for d in devs]) if devs else np.empty(0, dtype=dtype)
+    G.assert_same_bits(got, want, "tensors n=%d own=%d /%d others=%s" % (n, own, divisor, with_others))
+    plan.close()
+
+
 @settings(max_examples=30, **COMMON)
 @given(m=st.integers(1, 12), count=counts, dtype=st.sampled_from(G.DTYPES), seed=st.integers(0, 2**31),
        divisor=st.sampled_from([0, 0, 2, 7]), in_place=st.integers(-1, 11), n_copies=st.integers(0, 3))
