@@ -85,8 +85,9 @@ size_t ring_dtype_size(int dtype);
  * -1 (default) when every tile of the launch is on the chip at the same time
  * (between 2 and 7 tiles of 32 KiB per CU). "phased_copy": the same copies
  * with the whole payload of the launch held in registers between the two
- * phases (one workgroup per CU, up to 8 rows and 112 MiB): 1 whenever the
- * launch fits, 0 never, -1 (default) above 56 MiB per side.
+ * phases (one or two workgroups per CU, up to 8 rows and 112 MiB): 1 whenever
+ * the launch fits, 0 never, -1 (default) above 56 MiB per side, and from
+ * 36 MiB when the paced tiles would not fill the chip's CUs evenly.
  * "dry_launch" = 1 makes the step-table / copy /
  * accumulate kernels return at entry: what is then timed is what a launch of
  * that grid costs by itself. No counterpart in the reference, whose launch

@@ -25,8 +25,9 @@
 //   * a copy runs faster when the chip reads first and writes after than with
 //     the two directions interleaved: the copies of an allgather phase wait
 //     for all their loads before their first store when every tile is resident
-//     at once (the paced tiles), and above 56 MiB they hold the whole payload
-//     of the launch in registers, one workgroup per CU (rows_phased_kernel).
+//     at once (the paced tiles), and from 36 MiB (unless those tiles fill the
+//     CUs evenly) they hold the whole payload of the launch in registers, one
+//     or two workgroups per CU (rows_phased_kernel).
 //     Accumulates and folds, which read more than they write, gain nothing from it;
 //   * what is touched once (accumulates, allgather copies, unpack) is loaded
 //     and stored non-temporally; the in->out copy and the fusion pack, whose
@@ -430,17 +431,22 @@ __global__ void __launch_bounds__(kBlock) rows_kernel_small(const SmallRowTable 
 // time and the rows' pointers stay in scalar registers; a row has room for
 // kPhasedMax / ROWS vectors per lane.
 constexpr int kPhasedMax = 112;
+constexpr int kPhasedMaxTwoWaves = 40;  // of a lane's 256 registers, with room for the rows' pointers and edges
 struct PhasedShape {
-  uint32_t rounds;             // most rounds any row needs (<= kPhasedMax / ROWS)
+  uint32_t rounds;             // most rounds any row needs (at most a row's share of the lane's vectors)
   uint32_t shift[kSmallRows];  // the workgroup that starts row k
 };
 #ifdef HIP_CPU_SHIM_RUNTIME_H_
-#define RING_ONE_WAVE_PER_SIMD
+#define RING_WAVES_PER_SIMD(n)
 #else
-#define RING_ONE_WAVE_PER_SIMD __attribute__((amdgpu_waves_per_eu(1, 1)))
+#define RING_WAVES_PER_SIMD(n) __attribute__((amdgpu_waves_per_eu(n, n)))
 #endif
-template <typename T, int ROWS>
-__global__ void __launch_bounds__(kBlock) RING_ONE_WAVE_PER_SIMD
+// WAVES: workgroups per CU (waves per SIMD). 1: 112 vectors per lane, the form
+// for 56-112 MiB. 2: twice the workgroups with 56 vectors per lane each, for
+// smaller launches, which want more loads in flight per CU than one wave per
+// SIMD issues in the few rounds they have.
+template <typename T, int ROWS, int WAVES>
+__global__ void __launch_bounds__(kBlock) RING_WAVES_PER_SIMD(WAVES)
 rows_phased_kernel(const SmallRowTable tab, const PhasedShape shape) {
   if (tab.dry) return;
   typedef typename VecOf<T>::type V;
@@ -449,7 +455,7 @@ rows_phased_kernel(const SmallRowTable tab, const PhasedShape shape) {
   typedef V RING_GLOBAL GV;
   typedef VU RING_GLOBAL GVU;
   constexpr uint32_t VEC = 16 / sizeof(T);
-  constexpr int PER = kPhasedMax / ROWS;
+  constexpr int PER = (WAVES == 1 ? kPhasedMax : kPhasedMaxTwoWaves) / ROWS;
   const uint32_t tid = threadIdx.x;
   const uint32_t stride = gridDim.x * kBlock;
   V s[ROWS * PER];
@@ -1266,19 +1272,25 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
   // The copies of an allgather phase with the whole payload in registers
   // between one read phase and one write phase (rows_phased_kernel): up to
   // kSmallRows rows, each within its share of the registers, non-temporal both
-  // ways. By itself above 56 MiB per side (where the paced tiles end) on a whole chip:
-  // 57 MiB take 19.9 us this way and 21.3 as plain tiles.
+  // ways.
   if (role == kRoleAllgather && divisor <= 0 && n_rows >= 1 && n_rows <= static_cast<size_t>(kSmallRows) &&
       (nt & 3) == 3 && g_tuning.phased_copy != 0 && g_tuning.blocks_per_cu == 0) {
     int rc = device_info(&info);
     if (rc != RING_OK) return rc;
-    const uint64_t wgs = static_cast<uint64_t>(info.cus), stride = wgs * kBlock;
-    const uint64_t room = static_cast<uint64_t>(kPhasedMax / static_cast<int>(n_rows));
     SmallRowTable tab;
     PhasedShape shape;
+    uint64_t bytes = 0;
+    for (size_t k = 0; k < n_rows; k++) bytes += rows[k].count * esz;
+    // The chip's registers hold 112 MiB either way; up to 56 MiB the launch runs as two workgroups per CU
+    // with half the vectors per lane each (a few rounds of one wave per SIMD keep too little in flight).
+    // (sizes per CU: 224 KiB per CU are the 56 MiB of 256 CUs, the 7 tiles of 32 KiB the paced form ends at)
+    const uint64_t per_cu = bytes / static_cast<uint64_t>(info.cus);
+    const int waves = per_cu > (224u << 10) ? 1 : 2;
+    const uint64_t wgs = static_cast<uint64_t>(info.cus) * waves, stride = wgs * kBlock;
+    const uint64_t room = static_cast<uint64_t>((waves == 1 ? kPhasedMax : kPhasedMaxTwoWaves) / static_cast<int>(n_rows));
     shape.rounds = 0;
-    uint64_t bytes = 0, start = 0;
-    bool fits = true;
+    uint64_t start = 0;
+    bool fits = room >= 1;
     for (size_t k = 0; k < static_cast<size_t>(kSmallRows); k++) {
       shape.shift[k] = 0;
       tab.row[k] = Row{nullptr, nullptr, nullptr, 0};
@@ -1296,9 +1308,18 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
       shape.shift[k] = static_cast<uint32_t>(start);
       // the next row starts behind the last workgroup of this row's last round
       start = (start + (nvec % stride + kBlock - 1) / kBlock) % wgs;
-      bytes += r.count * esz;
     }
-    if (fits && (g_tuning.phased_copy > 0 || (bytes > (56ull << 20) && info.cus >= 128))) {
+    // By itself: above 56 MiB per side (one workgroup per CU), and from 36 MiB (two per CU) unless the
+    // paced tiles fill the chip exactly (a whole number of 32 KiB tiles per CU), which is their best case
+    // and beats this form by 3-4 % (7 x 8 MiB: 19.7 against 20.4 us); with a CU or more left over they
+    // lose 3-8 % to it (7 x 7.5 MiB: 19.6 against 18.1 us).
+    bool by_itself = per_cu > (224u << 10);
+    if (!by_itself && per_cu >= (144u << 10)) {
+      uint64_t paced_tiles = 0;
+      for (size_t k = 0; k < n_rows; k++) paced_tiles += (rows[k].count / vec + kBlock * kPacedUnroll - 1) / (kBlock * kPacedUnroll);
+      by_itself = paced_tiles % static_cast<uint64_t>(info.cus) != 0;
+    }
+    if (fits && (g_tuning.phased_copy > 0 || (by_itself && info.cus >= 128))) {
       tab.n_rows = static_cast<int>(n_rows);
       tab.dry = g_tuning.dry_launch;
       tab.uniform_tiles = 0;
@@ -1306,18 +1327,22 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
       tab.div_mask = 0;
       for (int k = 0; k <= kSmallRows; k++) tab.tile_begin[k] = 0;
       const dim3 grid(static_cast<uint32_t>(wgs));
-#define RING_PHASED(T)                                                                                   \
+#define RING_PHASED(T, W)                                                                                \
   switch (n_rows) {                                                                                      \
-    case 1: launch(rows_phased_kernel<T, 1>, grid, dim3(kBlock), stream, tab, shape); break;             \
-    case 2: launch(rows_phased_kernel<T, 2>, grid, dim3(kBlock), stream, tab, shape); break;             \
-    case 3: launch(rows_phased_kernel<T, 3>, grid, dim3(kBlock), stream, tab, shape); break;             \
-    case 4: launch(rows_phased_kernel<T, 4>, grid, dim3(kBlock), stream, tab, shape); break;             \
-    case 5: launch(rows_phased_kernel<T, 5>, grid, dim3(kBlock), stream, tab, shape); break;             \
-    case 6: launch(rows_phased_kernel<T, 6>, grid, dim3(kBlock), stream, tab, shape); break;             \
-    case 7: launch(rows_phased_kernel<T, 7>, grid, dim3(kBlock), stream, tab, shape); break;             \
-    default: launch(rows_phased_kernel<T, 8>, grid, dim3(kBlock), stream, tab, shape); break;            \
+    case 1: launch(rows_phased_kernel<T, 1, W>, grid, dim3(kBlock), stream, tab, shape); break;          \
+    case 2: launch(rows_phased_kernel<T, 2, W>, grid, dim3(kBlock), stream, tab, shape); break;          \
+    case 3: launch(rows_phased_kernel<T, 3, W>, grid, dim3(kBlock), stream, tab, shape); break;          \
+    case 4: launch(rows_phased_kernel<T, 4, W>, grid, dim3(kBlock), stream, tab, shape); break;          \
+    case 5: launch(rows_phased_kernel<T, 5, W>, grid, dim3(kBlock), stream, tab, shape); break;          \
+    case 6: launch(rows_phased_kernel<T, 6, W>, grid, dim3(kBlock), stream, tab, shape); break;          \
+    case 7: launch(rows_phased_kernel<T, 7, W>, grid, dim3(kBlock), stream, tab, shape); break;          \
+    default: launch(rows_phased_kernel<T, 8, W>, grid, dim3(kBlock), stream, tab, shape); break;         \
   }
-      if (esz == 8) { RING_PHASED(uint64_t) } else { RING_PHASED(uint32_t) }
+      if (waves == 2) {
+        if (esz == 8) { RING_PHASED(uint64_t, 2) } else { RING_PHASED(uint32_t, 2) }
+      } else {
+        if (esz == 8) { RING_PHASED(uint64_t, 1) } else { RING_PHASED(uint32_t, 1) }
+      }
 #undef RING_PHASED
       RING_HIP(hipGetLastError());
       return RING_OK;

@@ -498,7 +498,9 @@ void run_all(const char* name) {
   test_step_tables<T>(70001, 2);
   test_step_tables<T>(65536, 8);
   test_step_tables<T>(100003, 6);
-  test_step_tables<T>(900001, 9);   // 8 rows, each needing all of its share of the registers
+  test_step_tables<T>(900001, 9);   // 8 rows beyond their share of the registers: falls back to tiles
+  test_step_tables<T>(300007, 4);   // one workgroup per CU (more than 224 KiB per CU)
+  test_step_tables<T>(400003, 8);
   CHECK(ring_set_option("phased_copy", -1) == RING_OK);
   printf("%s: fold\n", name); fflush(stdout);
   test_fold<T>(8, 10007, 0);
