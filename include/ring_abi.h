@@ -87,7 +87,7 @@ size_t ring_dtype_size(int dtype);
  * with the whole payload of the launch held in registers between the two
  * phases (one or two workgroups per CU, up to 8 rows and 112 MiB): 1 whenever
  * the launch fits, 0 never, -1 (default) above 56 MiB per side, and from
- * 36 MiB when the paced tiles would not fill the chip's CUs evenly.
+ * 31 MiB when the paced tiles would not fill the chip's CUs evenly.
  * "dry_launch" = 1 makes the step-table / copy /
  * accumulate kernels return at entry: what is then timed is what a launch of
  * that grid costs by itself. No counterpart in the reference, whose launch

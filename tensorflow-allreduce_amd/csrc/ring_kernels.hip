@@ -25,7 +25,7 @@
 //   * a copy runs faster when the chip reads first and writes after than with
 //     the two directions interleaved: the copies of an allgather phase wait
 //     for all their loads before their first store when every tile is resident
-//     at once (the paced tiles), and from 36 MiB (unless those tiles fill the
+//     at once (the paced tiles), and from 31 MiB (unless those tiles fill the
 //     CUs evenly) they hold the whole payload of the launch in registers, one
 //     or two workgroups per CU (rows_phased_kernel).
 //     Accumulates and folds, which read more than they write, gain nothing from it;
@@ -1309,12 +1309,13 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
       // the next row starts behind the last workgroup of this row's last round
       start = (start + (nvec % stride + kBlock - 1) / kBlock) % wgs;
     }
-    // By itself: above 56 MiB per side (one workgroup per CU), and from 36 MiB (two per CU) unless the
+    // By itself: above 56 MiB per side (one workgroup per CU), and from 31 MiB (two per CU; 5 ragged rows
+    // of 6.4 MiB: 11.7 against 12.7 us paced; at 28 MiB the paced tiles win, 10.2 against 11.2) unless the
     // paced tiles fill the chip exactly (a whole number of 32 KiB tiles per CU), which is their best case
     // and beats this form by 3-4 % (7 x 8 MiB: 19.7 against 20.4 us); with a CU or more left over they
     // lose 3-8 % to it (7 x 7.5 MiB: 19.6 against 18.1 us).
     bool by_itself = per_cu > (224u << 10);
-    if (!by_itself && per_cu >= (144u << 10)) {
+    if (!by_itself && per_cu >= (124u << 10)) {
       uint64_t paced_tiles = 0;
       for (size_t k = 0; k < n_rows; k++) paced_tiles += (rows[k].count / vec + kBlock * kPacedUnroll - 1) / (kBlock * kPacedUnroll);
       by_itself = paced_tiles % static_cast<uint64_t>(info.cus) != 0;
