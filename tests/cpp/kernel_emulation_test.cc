@@ -430,7 +430,7 @@ void test_fusion(const std::vector<size_t>& counts, int divisor, int n_ranks) {
     OK(ring_fusion_plan_destroy(p2));
     // the direct form in one launch: segment `own` folded from staged copies and the tensors (last), its sum
     // to the wire buffer, the quotient into the tensors; the other segments scattered
-    for (int own : {0, n_ranks / 2, n_ranks - 1}) {
+    for (int own : {n_ranks / 2, n_ranks - 1}) {
       std::vector<Buf<T>> work;
       std::vector<const void*> work_ptrs;
       fresh(work, work_ptrs);
