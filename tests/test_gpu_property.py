@@ -111,6 +111,44 @@ def test_all_ranks_allgather_is_the_concatenation(rows, epr, dtype, seed, direct
                            "allgather rows=%r epr=%d rank %d direct=%s /%d" % (rows, epr, r, direct, divisor))
 
 
+@settings(max_examples=40, **COMMON)
+@given(lens=st.lists(st.one_of(st.integers(0, 40), st.integers(0, 300_000), st.sampled_from([65_536, 131_072, 262_147])),
+                     min_size=1, max_size=9),
+       gaps=st.lists(st.integers(0, 37), min_size=9, max_size=9), dtype=st.sampled_from(G.DTYPES),
+       seed=st.integers(0, 2**31), phased=st.sampled_from([1, 1, -1, 0]), shift=st.integers(0, 3))
+def test_allgather_copy_rows_of_any_shape_in_every_form(lens, gaps, dtype, seed, phased, shift):
+    """The copies of an allgather phase through a step table whose rows have
+    any length (empty ones included), start anywhere in the destination and
+    read from sources at any element alignment: the form with the payload held
+    in registers forced on wherever it fits (one to eight rows; nine fall back
+    to tiles), left to the launcher, and off. Every byte outside the rows stays
+    as it was."""
+    rng = np.random.default_rng(seed)
+    starts, at = [], 0
+    for ln, gap in zip(lens, gaps):
+        at += gap
+        starts.append(at)
+        at += ln
+    buf = G.random_array(rng, at + 7, dtype)
+    dbuf, _ = G.dev(buf, shift)
+    want = buf.copy()
+    rows, keep = [], []
+    for ln, st_ in zip(lens, starts):
+        src = G.random_array(rng, ln, dtype)
+        ds, base = G.dev(src, int(rng.integers(0, 4)))
+        keep.append(base)
+        rows.append((st_, ds.data_ptr() if ln else None, ln))
+        want[st_:st_ + ln] = src
+    ring_abi.set_option("phased_copy", phased)
+    try:
+        steps, k = ring_abi.make_steps(rows)
+        ring_abi.allgather_steps(dbuf.data_ptr(), steps, k, G.NP2ABI[np.dtype(dtype)], None)
+        G.sync()
+    finally:
+        ring_abi.set_option("phased_copy", -1)
+    G.assert_same_bits(G.host(dbuf), want, "rows %r at %r phased=%d" % (lens, starts, phased))
+
+
 @settings(max_examples=30, **COMMON)
 @given(sizes=st.lists(st.integers(0, 9000), min_size=0, max_size=40), dtype=st.sampled_from(G.DTYPES),
        seed=st.integers(0, 2**31), divisor=st.integers(1, 9))
