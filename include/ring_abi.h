@@ -87,7 +87,11 @@ size_t ring_dtype_size(int dtype);
  * with the whole payload of the launch held in registers between the two
  * phases (one or two workgroups per CU, up to 8 rows and 112 MiB): 1 whenever
  * the launch fits, 0 never, -1 (default) above 56 MiB per side, and from
- * 31 MiB when the paced tiles would not fill the chip's CUs evenly.
+ * 31 MiB when the paced tiles would not fill the chip's CUs evenly. The same
+ * option governs the unpack of a fused buffer (ring_fusion_unpack,
+ * _unpack_scaled and the unpack of ring_fusion_run_static), which runs in that
+ * form by default between 56 and 112 MiB when the set has at most 512
+ * non-empty tensors and the divisor, if any, is a power of two.
  * "dry_launch" = 1 makes the step-table / copy /
  * accumulate kernels return at entry: what is then timed is what a launch of
  * that grid costs by itself. No counterpart in the reference, whose launch

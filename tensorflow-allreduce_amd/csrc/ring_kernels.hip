@@ -27,7 +27,8 @@
 //     for all their loads before their first store when every tile is resident
 //     at once (the paced tiles), and from 31 MiB (unless those tiles fill the
 //     CUs evenly) they hold the whole payload of the launch in registers, one
-//     or two workgroups per CU (rows_phased_kernel).
+//     or two workgroups per CU (rows_phased_kernel). The unpack of a fused
+//     buffer of 56-112 MiB runs the same way (unpack_phased_kernel).
 //     Accumulates and folds, which read more than they write, gain nothing from it;
 //   * what is touched once (accumulates, allgather copies, unpack) is loaded
 //     and stored non-temporally; the in->out copy and the fusion pack, whose
@@ -35,7 +36,8 @@
 //   * the average's divide rides on the accumulate that completes a segment
 //     (or on the unpack), never on a pass of its own;
 //   * LDS is used only by the fusion kernels, for the offset table of a tile
-//     that spans several small tensors.
+//     that spans several small tensors (and, in the unpack that holds its
+//     payload in registers, for where each round of a workgroup goes).
 // No MFMA: the path is one add per 12 bytes.
 
 #include <hip/hip_runtime.h>
@@ -47,6 +49,7 @@
 #include <algorithm>
 #include <mutex>
 #include <new>
+#include <type_traits>
 #include <vector>
 
 #include "ring_abi.h"
@@ -848,6 +851,148 @@ fusion_kernel(T* __restrict__ fused, const uint64_t* __restrict__ offsets, T* co
   }
 }
 
+// ---- the unpack with the payload in registers ------------------------------------
+// The unpack of a fused buffer of 56-112 MiB as rows_phased_kernel runs the
+// allgather copies: one workgroup per CU, one read phase and one write phase
+// of the whole chip. The fused side is one aligned run, so a lane's loads need
+// no table at all and go out first; where the 256 vectors a workgroup takes
+// in a round go (4 KiB of the fused space) is looked up while they are on
+// their way: lane j reads the record of round j's tile, and when that tile
+// lies inside one tensor the round's destination is an address, kept in LDS.
+// A round whose tile meets several tensors (a hundred of the 6240 tiles of a
+// ResNet-50 gradient set) is stored lane by lane: every lane finds the tensor
+// of its vector by binary search in the offset table, which the workgroup
+// staged in LDS next to the addresses. Nothing of this waits on memory a
+// second time: the records and the table arrive behind the payload.
+// DIV: the tensors receive value / divisor for a divisor that is a power of
+// two, the only ones this kernel takes: a multiplication by the exact
+// reciprocal for float32 and an arithmetic shift for the integers, which are
+// tf.div's true and floor division bit for bit (div_one does the same).
+template <typename T, bool DIV>
+__device__ __forceinline__ T divide_by_power_of_two(T x, float reciprocal, int shift) {
+  if constexpr (!DIV) {
+    (void)reciprocal;
+    (void)shift;
+    return x;
+  } else if constexpr (std::is_floating_point<T>::value) {
+    (void)shift;
+    return x * reciprocal;
+  } else {
+    (void)reciprocal;
+    return x >> shift;
+  }
+}
+
+// The tensor that holds element e of the fused space: off[l] <= e < off[l + 1], off[0] = 0, off[m] = total.
+__device__ __forceinline__ uint32_t tensor_of_element(const uint64_t* off, uint32_t m, uint64_t e) {
+  uint32_t l = 0, h = m;
+  while (h - l > 1) {
+    const uint32_t mid = (l + h) >> 1;
+    if (off[mid] <= e) l = mid; else h = mid;
+  }
+  return l;
+}
+
+template <typename T, bool DIV>
+__global__ void __launch_bounds__(kBlock) RING_WAVES_PER_SIMD(1)
+unpack_phased_kernel(const T* __restrict__ fused, const uint64_t* __restrict__ offsets, T* const* __restrict__ ptrs,
+                     const FusionTile* __restrict__ tiles, uint32_t m, uint64_t total, uint32_t rounds, int divisor) {
+  typedef typename VecOf<T>::type V;
+  typedef V VU __attribute__((aligned(sizeof(T))));
+  typedef T RING_GLOBAL GT;
+  typedef V RING_GLOBAL GV;
+  typedef VU RING_GLOBAL GVU;
+  constexpr uint32_t VEC = 16 / sizeof(T);
+  __shared__ uint64_t s_off[kFusionLdsCap + 1];
+  __shared__ T* s_ptr[kFusionLdsCap];
+  __shared__ T* s_to[kPhasedMax];  // where lane 0's vector of round j goes, or null: the round meets several tensors
+  const uint32_t tid = threadIdx.x;
+  const uint32_t stride = gridDim.x * kBlock;
+  const uint32_t base = blockIdx.x * kBlock + tid;
+  const uint32_t nvec = static_cast<uint32_t>(total / VEC);  // the host checked: at most kPhasedMax * stride
+  const uint32_t n_tail = static_cast<uint32_t>(total - static_cast<uint64_t>(nvec) * VEC);
+  const GV* fv = (const GV*)fused;
+  V s[kPhasedMax];
+  T tail = T();
+#pragma unroll
+  for (int j = 0; j < kPhasedMax; j++) {
+    if (static_cast<uint32_t>(j) < rounds) {
+      if (base + j * stride < nvec) s[j] = __builtin_nontemporal_load(&(fv + j * stride)[base]);
+    }
+  }
+  if (blockIdx.x == 0 && tid < n_tail) tail = ((const GT*)fused)[static_cast<uint64_t>(nvec) * VEC + tid];
+  // behind the payload: the destinations of this workgroup's rounds and the offset table (at most
+  // kFusionLdsCap tensors: three offsets and two pointers a lane). Every load is issued before the first
+  // is waited for, so the launch pays one memory latency for all of it, the one it pays for the payload.
+  static_assert(kFusionLdsCap == 2 * kBlock, "a lane stages offsets tid, tid + 256, tid + 512 and pointers tid, tid + 256");
+  T* to = nullptr;
+  const uint64_t v0 = static_cast<uint64_t>(blockIdx.x) * kBlock + static_cast<uint64_t>(tid) * stride;
+  const bool has_round = tid < rounds && v0 < nvec;
+  // (a lane without a round reads tile 0's record and drops it: a load under a branch would be waited for there)
+  const FusionTile rec = load_tile(tiles, has_round ? static_cast<uint32_t>(v0 / kFusionTileVecs) : 0u);
+  uint64_t off0 = 0, off1 = 0, off2 = 0;
+  T* ptr0 = nullptr;
+  T* ptr1 = nullptr;
+  if (tid <= m) off0 = offsets[tid];
+  if (tid + kBlock <= m) off1 = offsets[tid + kBlock];
+  if (tid + 2 * kBlock <= m) off2 = offsets[tid + 2 * kBlock];
+  if (tid < m) ptr0 = ptrs[tid];
+  if (tid + kBlock < m) ptr1 = ptrs[tid + kBlock];
+  if (has_round && rec.first == rec.last) to = static_cast<T*>(rec.addr) + (v0 % kFusionTileVecs) * VEC;
+  if (tid < kPhasedMax) s_to[tid] = to;
+  if (tid <= m) s_off[tid] = off0;
+  if (tid + kBlock <= m) s_off[tid + kBlock] = off1;
+  if (tid + 2 * kBlock <= m) s_off[tid + 2 * kBlock] = off2;
+  if (tid < m) s_ptr[tid] = ptr0;
+  if (tid + kBlock < m) s_ptr[tid + kBlock] = ptr1;
+  __syncthreads();
+  RING_WAIT_VMEM();
+  float reciprocal = 1.0f;
+  int shift = 0;
+  if (DIV) {
+    reciprocal = 1.0f / static_cast<float>(divisor);
+    while ((1 << shift) < divisor) shift++;
+  }
+#pragma unroll
+  for (int j = 0; j < kPhasedMax; j++) {
+    if (static_cast<uint32_t>(j) < rounds) {
+      const uint32_t idx = base + j * stride;
+      if (idx < nvec) {
+        V r = s[j];
+#pragma unroll
+        for (uint32_t c = 0; c < VEC; c++) r[c] = divide_by_power_of_two<T, DIV>(r[c], reciprocal, shift);
+        T* to = s_to[j];
+        if (to) {
+          __builtin_nontemporal_store(r, &((GVU*)(GT*)to)[tid]);
+        } else {
+          // small tensors share cache lines with their neighbours: ordinary stores
+          const uint64_t e = static_cast<uint64_t>(idx) * VEC;
+          uint32_t l = tensor_of_element(s_off, m, e);
+          if (e + VEC <= s_off[l + 1]) {
+            *(GVU*)(GT*)(s_ptr[l] + (e - s_off[l])) = r;
+          } else {
+            // a vector cut by the end of a tensor (one per end that is not 16-byte aligned): element by
+            // element, as a loop that stays a loop (this body is repeated for every round)
+#pragma unroll 1
+            for (uint32_t c = 0; c < VEC; c++) {
+              while (e + c >= s_off[l + 1]) l++;
+              T x = r[0];
+#pragma unroll
+              for (uint32_t k = 1; k < VEC; k++) x = (c == k) ? r[k] : x;
+              *(GT*)(s_ptr[l] + (e + c - s_off[l])) = x;
+            }
+          }
+        }
+      }
+    }
+  }
+  if (blockIdx.x == 0 && tid < n_tail) {
+    const uint64_t e = static_cast<uint64_t>(nvec) * VEC + tid;
+    const uint32_t l = tensor_of_element(s_off, m, e);
+    *(GT*)(s_ptr[l] + (e - s_off[l])) = divide_by_power_of_two<T, DIV>(tail, reciprocal, shift);
+  }
+}
+
 // ---- tensor fusion without passes of its own -------------------------------------
 // The pack before a fused allreduce and the unpack after it read and write the
 // whole set once each for nothing but a change of layout. Both fold into the
@@ -1501,14 +1646,35 @@ struct FusionView {
   const uint64_t* offsets;
   void* const* ptrs;
   const FusionTile* tiles;
+  uint32_t m;  // non-empty tensors: entries of ptrs, and of offsets less one
 };
 
 inline FusionView view_of(const ring_fusion_plan* p) {
-  return FusionView{p->dtype, p->esz, p->ntiles, p->total, p->d_offsets, p->d_ptrs, p->d_tiles};
+  return FusionView{p->dtype, p->esz, p->ntiles, p->total, p->d_offsets, p->d_ptrs, p->d_tiles, p->m};
 }
 
 template <typename T, bool PACK, bool DIV>
 int launch_fusion(const FusionView& p, void* fused, hipStream_t stream, int divisor) {
+  // The unpack of 56-112 MiB with the payload in registers (unpack_phased_kernel): by itself from 224 KiB per
+  // CU, where one workgroup per CU is the form that pays, up to the 112 vectors a lane holds.
+  if (!PACK && g_tuning.phased_copy != 0 && g_tuning.blocks_per_cu == 0 && (g_tuning.nt[kRoleUnpack] & 3) == 3 &&
+      p.m <= kFusionLdsCap && (!DIV || (divisor & (divisor - 1)) == 0)) {
+    DeviceInfo info;
+    int rc = device_info(&info);
+    if (rc != RING_OK) return rc;
+    const uint64_t stride = static_cast<uint64_t>(info.cus) * kBlock;
+    const uint64_t nvec = p.total / (16 / sizeof(T));
+    const uint64_t rounds = (nvec + stride - 1) / stride;
+    const uint64_t per_cu = p.total * sizeof(T) / static_cast<uint64_t>(info.cus);
+    if (rounds >= 1 && rounds <= static_cast<uint64_t>(kPhasedMax) &&
+        (g_tuning.phased_copy > 0 || (per_cu > (224u << 10) && info.cus >= 128))) {
+      launch(unpack_phased_kernel<T, DIV>, dim3(static_cast<uint32_t>(info.cus)), dim3(kBlock), stream,
+             static_cast<const T*>(fused), p.offsets, reinterpret_cast<T* const*>(p.ptrs), p.tiles, p.m, p.total,
+             static_cast<uint32_t>(rounds), divisor);
+      RING_HIP(hipGetLastError());
+      return RING_OK;
+    }
+  }
   uint32_t grid = p.ntiles;
   if (g_tuning.blocks_per_cu > 0) {
     DeviceInfo info;
@@ -2245,7 +2411,7 @@ int ring_fusion_run_static(int unpack, const void* const* tensors, const size_t*
   hipLaunchKernelGGL(table_tiles_kernel, dim3((ntiles + kBlock - 1) / kBlock), dim3(kBlock), 0, s, tab, m, ntiles,
                      tile_elems, total, static_cast<uint32_t>(esz));
   RING_HIP(hipGetLastError());
-  const FusionView view{dtype, esz, ntiles, total, tab->offsets, tab->ptrs, tab->tiles};
+  const FusionView view{dtype, esz, ntiles, total, tab->offsets, tab->ptrs, tab->tiles, m};
   return fusion_run(view, fused, stream, !unpack, divisor);
 }
 

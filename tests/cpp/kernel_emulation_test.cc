@@ -377,25 +377,31 @@ void test_fusion(const std::vector<size_t>& counts, int divisor, int n_ranks) {
   std::vector<T> divided(packed);
   if (divisor)
     for (auto& v : divided) v = divide(v, divisor);
-  {
-    std::vector<Buf<T>> out;
-    std::vector<const void*> out_ptrs;
-    fresh(out, out_ptrs);
-    ring_fusion_plan* p2 = nullptr;
-    OK(ring_fusion_plan_create(out_ptrs.data(), counts.data(), static_cast<int>(counts.size()), code<T>(), &p2));
-    if (divisor) OK(ring_fusion_unpack_scaled(p2, fused.p, divisor, nullptr));
-    else OK(ring_fusion_unpack(p2, fused.p, nullptr));
-    check_tensors(out, divided, "unpack");
-    OK(ring_fusion_plan_destroy(p2));
+  // as tiles, and with the payload in registers wherever that form takes the set (up to 512 tensors,
+  // 112 rounds of the chip, no divisor or a power of two)
+  for (int phased : {-1, 1}) {
+    CHECK(ring_set_option("phased_copy", phased) == RING_OK);
+    {
+      std::vector<Buf<T>> out;
+      std::vector<const void*> out_ptrs;
+      fresh(out, out_ptrs);
+      ring_fusion_plan* p2 = nullptr;
+      OK(ring_fusion_plan_create(out_ptrs.data(), counts.data(), static_cast<int>(counts.size()), code<T>(), &p2));
+      if (divisor) OK(ring_fusion_unpack_scaled(p2, fused.p, divisor, nullptr));
+      else OK(ring_fusion_unpack(p2, fused.p, nullptr));
+      check_tensors(out, divided, phased > 0 ? "unpack, payload in registers" : "unpack");
+      OK(ring_fusion_plan_destroy(p2));
+    }
+    {
+      std::vector<Buf<T>> out;
+      std::vector<const void*> out_ptrs;
+      fresh(out, out_ptrs);
+      OK(ring_fusion_run_static(1, out_ptrs.data(), counts.data(), static_cast<int>(counts.size()), code<T>(),
+                                total ? fused.p : nullptr, divisor, nullptr));
+      check_tensors(out, divided, phased > 0 ? "static unpack, payload in registers" : "static unpack");
+    }
   }
-  {
-    std::vector<Buf<T>> out;
-    std::vector<const void*> out_ptrs;
-    fresh(out, out_ptrs);
-    OK(ring_fusion_run_static(1, out_ptrs.data(), counts.data(), static_cast<int>(counts.size()), code<T>(),
-                              total ? fused.p : nullptr, divisor, nullptr));
-    check_tensors(out, divided, "static unpack");
-  }
+  CHECK(ring_set_option("phased_copy", -1) == RING_OK);
   // gather: wire[seg] = tensors[seg] + incoming (one segment only packed); scatter the result back
   if (total >= static_cast<size_t>(n_ranks)) {
     std::vector<size_t> sizes(n_ranks), starts(n_ranks);
@@ -518,6 +524,7 @@ void run_all(const char* name) {
   test_fusion<T>(tiny, 6, 4);
   test_fusion<T>({17}, 3, 2);
   test_fusion<T>({}, 0, 2);
+  test_fusion<T>({100003, 1, 2, 50001, 0, 4096, 3}, 4, 2);  // tensor ends that cut 16-byte groups, divided by a power of two
 }
 
 }  // namespace

@@ -492,7 +492,7 @@ def test_scale_is_tf_div(dtype):
             assert np.all(G.host(keep[:off]) == 0) and np.all(G.host(keep[off + count:]) == 0)
 
 
-def _fusion_roundtrip(counts, dtype, rng, offsets=None):
+def _fusion_roundtrip(counts, dtype, rng, offsets=None, divisors=(6,)):
     code = G.NP2ABI[np.dtype(dtype)]
     hosts, devs, keep = [], [], []
     for j, c in enumerate(counts):
@@ -524,16 +524,20 @@ def _fusion_roundtrip(counts, dtype, rng, offsets=None):
         assert int(torch.count_nonzero(base)) == int(np.count_nonzero(new[at:at + c]))  # nothing outside
         at += c
     # unpack with the average folded in: tf.div by the number of ranks
-    for base in keep:
-        base.zero_()
-    plan.unpack_scaled(fused.data_ptr(), 6, None)
-    G.sync()
-    with np.errstate(all="ignore"):
-        want = new / np.float32(6) if np.dtype(dtype) == np.float32 else new // np.dtype(dtype).type(6)
-    at = 0
-    for j, (d, c) in enumerate(zip(devs, counts)):
-        G.assert_same_bits(G.host(d), want[at:at + c].astype(dtype), "unpack_scaled tensor %d" % j)
-        at += c
+    if np.dtype(dtype) != np.float32 and total:
+        new[: total // 2] = -np.abs(new[: total // 2])               # negative values with remainders: floored
+        fused[:total].copy_(torch.from_numpy(new))
+    for divisor in divisors:
+        for base in keep:
+            base.zero_()
+        plan.unpack_scaled(fused.data_ptr(), divisor, None)
+        G.sync()
+        with np.errstate(all="ignore"):
+            want = new / np.float32(divisor) if np.dtype(dtype) == np.float32 else new // np.dtype(dtype).type(divisor)
+        at = 0
+        for j, (d, c) in enumerate(zip(devs, counts)):
+            G.assert_same_bits(G.host(d), want[at:at + c].astype(dtype), "unpack_scaled /%d tensor %d" % (divisor, j))
+            at += c
     plan.close()
 
 
@@ -548,6 +552,40 @@ def test_fusion_pack_unpack(dtype):
     # thousands of tiny tensors inside one tile: more than the LDS table holds
     _fusion_roundtrip([int(c) for c in rng.integers(0, 4, 3000)], dtype, rng)
     _fusion_roundtrip([int(c) for c in rng.integers(1, 200, 700)], dtype, rng)
+
+
+@pytest.mark.parametrize("dtype", G.DTYPES)
+@pytest.mark.parametrize("phased", [1, -1, 0])
+def test_fusion_unpack_with_the_payload_in_registers(dtype, phased):
+    """The unpack as one read phase and one write phase of the chip (every lane
+    holds its share of the fused buffer in registers; rounds whose tile meets
+    several tensors are stored lane by lane after a search of the offset
+    table), forced on for every set it can take, left to the launcher (the
+    ResNet-50 set of 4-byte elements is in its range) and off: the same bytes
+    in the tensors and nothing outside them, with no divisor, with powers of
+    two (the form divides by them itself) and with 6 (it must leave that to
+    the tiles), tensor ends that cut 16-byte groups, hundreds of tiny tensors,
+    more tensors than its table holds, and a buffer of exactly and of just
+    over the 112 rounds a lane has registers for."""
+    import torch
+    rng = np.random.default_rng(51 + phased)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    vec = 16 // np.dtype(dtype).itemsize
+    full = cus * 256 * 112 * vec                                     # elements of 112 rounds
+    ring_abi.set_option("phased_copy", phased)
+    try:
+        _fusion_roundtrip([int(np.prod(s)) for s in G.resnet50_shapes()], dtype, rng, divisors=(8, 6))
+        _fusion_roundtrip([5, 0, 4096, 1, 0, 3, 8191, 2, 70_001], dtype, rng, divisors=(1, 2, 6, 1024))
+        _fusion_roundtrip([1], dtype, rng, divisors=(4,))
+        _fusion_roundtrip([3, 2_000_003, 1, 1, 7, 999_999], dtype, rng, divisors=(8,))
+        _fusion_roundtrip([int(c) for c in rng.integers(1, 200, 500)], dtype, rng, divisors=(4, 3))
+        _fusion_roundtrip([int(c) for c in rng.integers(0, 9000, 512)], dtype, rng, divisors=(16,))
+        _fusion_roundtrip([int(c) for c in rng.integers(1, 300, 513)], dtype, rng, divisors=(8,))   # one too many
+        if np.dtype(dtype).itemsize == 4:
+            _fusion_roundtrip([full - 5, 5], dtype, rng, divisors=(8,))                             # all the registers
+            _fusion_roundtrip([full - 5, 5 + vec], dtype, rng, divisors=(8,))                       # a 113th round
+    finally:
+        ring_abi.set_option("phased_copy", -1)
 
 
 @pytest.mark.parametrize("dtype", G.DTYPES)

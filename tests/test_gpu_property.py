@@ -151,8 +151,12 @@ def test_allgather_copy_rows_of_any_shape_in_every_form(lens, gaps, dtype, seed,
 
 @settings(max_examples=30, **COMMON)
 @given(sizes=st.lists(st.integers(0, 9000), min_size=0, max_size=40), dtype=st.sampled_from(G.DTYPES),
-       seed=st.integers(0, 2**31), divisor=st.integers(1, 9))
-def test_fusion_pack_unpack_roundtrip(sizes, dtype, seed, divisor):
+       seed=st.integers(0, 2**31), divisor=st.one_of(st.integers(1, 9), st.sampled_from([2, 4, 8, 64])),
+       phased=st.sampled_from([-1, 1, 1]))
+def test_fusion_pack_unpack_roundtrip(sizes, dtype, seed, divisor, phased):
+    """pack, then unpack and divide, as tiles and (phased = 1) with the fused
+    buffer held in registers between one read phase and one write phase, the
+    form that takes no divisor but a power of two."""
     rng = np.random.default_rng(seed)
     hosts = [G.random_array(rng, c, dtype, wide=True) for c in sizes]
     devs = [G.dev(h, int(rng.integers(0, 4))) for h in hosts]
@@ -166,8 +170,12 @@ def test_fusion_pack_unpack_roundtrip(sizes, dtype, seed, divisor):
     G.assert_same_bits(G.host(fused)[:total], want, "pack")
     for d in devs:
         d[1].zero_()
-    plan.unpack_scaled(fused.data_ptr(), divisor, None)
-    torch.cuda.synchronize()
+    ring_abi.set_option("phased_copy", phased)
+    try:
+        plan.unpack_scaled(fused.data_ptr(), divisor, None)
+        torch.cuda.synchronize()
+    finally:
+        ring_abi.set_option("phased_copy", -1)
     with np.errstate(all="ignore"):
         scaled = want / np.float32(divisor) if dtype == np.float32 else want // dtype(divisor)
     at = 0
