@@ -326,7 +326,7 @@ class FusedResnet50(Workload):
             ("pack", total * 8, "fusion_kernel<unsigned int, pack> (161 tensors, 25,557,032 elements)"),
             ("reduce_scatter", 7 * seg * 12, "rows_kernel<float, kAdd> (7 rows x 3,194,629 elements, in place)"),
             ("allgather", 7 * seg * 8, "rows_kernel<unsigned int, kCopy> (7 rows x 3,194,629 elements)"),
-            ("unpack_scaled", total * 8, "fusion_kernel<float, unpack, divide> (161 tensors, /8)"))
+            ("unpack_scaled", total * 8, "unpack_phased_kernel<float, divide> (161 tensors, /8; fusion_kernel<float, unpack, divide> with phased_copy=0)"))
         self.dominant = 1
         self.description = ("tensor-fusion allreduce of a ResNet-50 v1 gradient set: 161 float32 tensors "
                             "(25,557,032 elements, values ~N(0,1e-3)) packed into one fusion buffer, ring-reduced in "
