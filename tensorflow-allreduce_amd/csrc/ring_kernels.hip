@@ -28,7 +28,7 @@
 //     at once (the paced tiles), and from 31 MiB (unless those tiles fill the
 //     CUs evenly) they hold the whole payload of the launch in registers, one
 //     or two workgroups per CU (rows_phased_kernel). The unpack of a fused
-//     buffer of 56-112 MiB runs the same way (unpack_phased_kernel).
+//     buffer of 1-112 MiB runs the same way (unpack_phased_kernel).
 //     Accumulates and folds, which read more than they write, gain nothing from it;
 //   * what is touched once (accumulates, allgather copies, unpack) is loaded
 //     and stored non-temporally; the in->out copy and the fusion pack, whose
@@ -852,9 +852,9 @@ fusion_kernel(T* __restrict__ fused, const uint64_t* __restrict__ offsets, T* co
 }
 
 // ---- the unpack with the payload in registers ------------------------------------
-// The unpack of a fused buffer of 56-112 MiB as rows_phased_kernel runs the
-// allgather copies: one workgroup per CU, one read phase and one write phase
-// of the whole chip. The fused side is one aligned run, so a lane's loads need
+// The unpack of a fused buffer of up to 112 MiB as rows_phased_kernel runs the
+// allgather copies: one or two workgroups per CU, one read phase and one write
+// phase of the whole chip. The fused side is one aligned run, so a lane's loads need
 // no table at all and go out first; where the 256 vectors a workgroup takes
 // in a round go (4 KiB of the fused space) is looked up while they are on
 // their way: lane j reads the record of round j's tile, and when that tile
@@ -893,8 +893,9 @@ __device__ __forceinline__ uint32_t tensor_of_element(const uint64_t* off, uint3
   return l;
 }
 
-template <typename T, bool DIV>
-__global__ void __launch_bounds__(kBlock) RING_WAVES_PER_SIMD(1)
+// WAVES: workgroups per CU, as in rows_phased_kernel (2: buffers of up to 56 MiB, 40 groups a lane).
+template <typename T, bool DIV, int WAVES>
+__global__ void __launch_bounds__(kBlock) RING_WAVES_PER_SIMD(WAVES)
 unpack_phased_kernel(const T* __restrict__ fused, const uint64_t* __restrict__ offsets, T* const* __restrict__ ptrs,
                      const FusionTile* __restrict__ tiles, uint32_t m, uint64_t total, uint32_t rounds, int divisor) {
   typedef typename VecOf<T>::type V;
@@ -903,19 +904,20 @@ unpack_phased_kernel(const T* __restrict__ fused, const uint64_t* __restrict__ o
   typedef V RING_GLOBAL GV;
   typedef VU RING_GLOBAL GVU;
   constexpr uint32_t VEC = 16 / sizeof(T);
+  constexpr int PER = WAVES == 1 ? kPhasedMax : kPhasedMaxTwoWaves;  // groups a lane holds
   __shared__ uint64_t s_off[kFusionLdsCap + 1];
   __shared__ T* s_ptr[kFusionLdsCap];
-  __shared__ T* s_to[kPhasedMax];  // where lane 0's vector of round j goes, or null: the round meets several tensors
+  __shared__ T* s_to[PER];  // where lane 0's vector of round j goes, or null: the round meets several tensors
   const uint32_t tid = threadIdx.x;
   const uint32_t stride = gridDim.x * kBlock;
   const uint32_t base = blockIdx.x * kBlock + tid;
-  const uint32_t nvec = static_cast<uint32_t>(total / VEC);  // the host checked: at most kPhasedMax * stride
+  const uint32_t nvec = static_cast<uint32_t>(total / VEC);  // the host checked: at most PER * stride
   const uint32_t n_tail = static_cast<uint32_t>(total - static_cast<uint64_t>(nvec) * VEC);
   const GV* fv = (const GV*)fused;
-  V s[kPhasedMax];
+  V s[PER];
   T tail = T();
 #pragma unroll
-  for (int j = 0; j < kPhasedMax; j++) {
+  for (int j = 0; j < PER; j++) {
     if (static_cast<uint32_t>(j) < rounds) {
       if (base + j * stride < nvec) s[j] = __builtin_nontemporal_load(&(fv + j * stride)[base]);
     }
@@ -939,7 +941,7 @@ unpack_phased_kernel(const T* __restrict__ fused, const uint64_t* __restrict__ o
   if (tid < m) ptr0 = ptrs[tid];
   if (tid + kBlock < m) ptr1 = ptrs[tid + kBlock];
   if (has_round && rec.first == rec.last) to = static_cast<T*>(rec.addr) + (v0 % kFusionTileVecs) * VEC;
-  if (tid < kPhasedMax) s_to[tid] = to;
+  if (tid < static_cast<uint32_t>(PER)) s_to[tid] = to;
   if (tid <= m) s_off[tid] = off0;
   if (tid + kBlock <= m) s_off[tid + kBlock] = off1;
   if (tid + 2 * kBlock <= m) s_off[tid + 2 * kBlock] = off2;
@@ -954,7 +956,7 @@ unpack_phased_kernel(const T* __restrict__ fused, const uint64_t* __restrict__ o
     while ((1 << shift) < divisor) shift++;
   }
 #pragma unroll
-  for (int j = 0; j < kPhasedMax; j++) {
+  for (int j = 0; j < PER; j++) {
     if (static_cast<uint32_t>(j) < rounds) {
       const uint32_t idx = base + j * stride;
       if (idx < nvec) {
@@ -1653,24 +1655,39 @@ inline FusionView view_of(const ring_fusion_plan* p) {
   return FusionView{p->dtype, p->esz, p->ntiles, p->total, p->d_offsets, p->d_ptrs, p->d_tiles, p->m};
 }
 
+// Bytes of the fused buffer per CU: from where the unpack holds its payload in registers by itself (1 MiB on
+// 256 CUs), and up to where it runs as two workgroups per CU (75 MiB on 256 CUs).
+constexpr uint64_t kUnpackPhasedMinPerCu = 4u << 10;
+constexpr uint64_t kUnpackTwoWorkgroupsMaxPerCu = 300u << 10;
+
 template <typename T, bool PACK, bool DIV>
 int launch_fusion(const FusionView& p, void* fused, hipStream_t stream, int divisor) {
-  // The unpack of 56-112 MiB with the payload in registers (unpack_phased_kernel): by itself from 224 KiB per
-  // CU, where one workgroup per CU is the form that pays, up to the 112 vectors a lane holds.
+  // The unpack with the payload in registers (unpack_phased_kernel), by itself from 1 MiB up to what the
+  // registers hold. Measured behind the allgather that wrote the buffer, float32, sets of 79-155 tensors,
+  // against the tiles: 2-12 MiB 4.4-5.8 us against 6.7-7.8; 24 MiB 10.0 / 13.4; 40 MiB 16.1 / 18.3;
+  // 56 MiB 23.0 / 24.3 (two workgroups per CU); 80 MiB 31.4 / 32.9 and 97 MiB 34.8 / 39.4 (one per CU).
+  // Between the two, the form with two workgroups per CU holds up to 80 MiB and is the better one up to 72
+  // (64 MiB: 26.4 against 27.7 as one workgroup per CU and 27.0 as tiles; 80 MiB: 33.4 against 31.4).
   if (!PACK && g_tuning.phased_copy != 0 && g_tuning.blocks_per_cu == 0 && (g_tuning.nt[kRoleUnpack] & 3) == 3 &&
       p.m <= kFusionLdsCap && (!DIV || (divisor & (divisor - 1)) == 0)) {
     DeviceInfo info;
     int rc = device_info(&info);
     if (rc != RING_OK) return rc;
-    const uint64_t stride = static_cast<uint64_t>(info.cus) * kBlock;
+    const uint64_t per_cu = p.total * sizeof(T) / static_cast<uint64_t>(info.cus);
+    const int waves = per_cu > kUnpackTwoWorkgroupsMaxPerCu ? 1 : 2;
+    const uint64_t wgs = static_cast<uint64_t>(info.cus) * waves, stride = wgs * kBlock;
     const uint64_t nvec = p.total / (16 / sizeof(T));
     const uint64_t rounds = (nvec + stride - 1) / stride;
-    const uint64_t per_cu = p.total * sizeof(T) / static_cast<uint64_t>(info.cus);
-    if (rounds >= 1 && rounds <= static_cast<uint64_t>(kPhasedMax) &&
-        (g_tuning.phased_copy > 0 || (per_cu > (224u << 10) && info.cus >= 128))) {
-      launch(unpack_phased_kernel<T, DIV>, dim3(static_cast<uint32_t>(info.cus)), dim3(kBlock), stream,
-             static_cast<const T*>(fused), p.offsets, reinterpret_cast<T* const*>(p.ptrs), p.tiles, p.m, p.total,
-             static_cast<uint32_t>(rounds), divisor);
+    if (rounds >= 1 && rounds <= static_cast<uint64_t>(waves == 1 ? kPhasedMax : kPhasedMaxTwoWaves) &&
+        (g_tuning.phased_copy > 0 || (per_cu >= kUnpackPhasedMinPerCu && info.cus >= 128))) {
+      if (waves == 1)
+        launch(unpack_phased_kernel<T, DIV, 1>, dim3(static_cast<uint32_t>(wgs)), dim3(kBlock), stream,
+               static_cast<const T*>(fused), p.offsets, reinterpret_cast<T* const*>(p.ptrs), p.tiles, p.m, p.total,
+               static_cast<uint32_t>(rounds), divisor);
+      else
+        launch(unpack_phased_kernel<T, DIV, 2>, dim3(static_cast<uint32_t>(wgs)), dim3(kBlock), stream,
+               static_cast<const T*>(fused), p.offsets, reinterpret_cast<T* const*>(p.ptrs), p.tiles, p.m, p.total,
+               static_cast<uint32_t>(rounds), divisor);
       RING_HIP(hipGetLastError());
       return RING_OK;
     }

@@ -560,8 +560,9 @@ def test_fusion_unpack_with_the_payload_in_registers(dtype, phased):
     """The unpack as one read phase and one write phase of the chip (every lane
     holds its share of the fused buffer in registers; rounds whose tile meets
     several tensors are stored lane by lane after a search of the offset
-    table), forced on for every set it can take, left to the launcher (the
-    ResNet-50 set of 4-byte elements is in its range) and off: the same bytes
+    table), forced on for every set it can take, left to the launcher (which
+    takes it from 1 MiB, as two workgroups per CU up to 75 MiB and as one
+    beyond) and off: the same bytes
     in the tensors and nothing outside them, with no divisor, with powers of
     two (the form divides by them itself) and with 6 (it must leave that to
     the tiles), tensor ends that cut 16-byte groups, hundreds of tiny tensors,
@@ -582,6 +583,9 @@ def test_fusion_unpack_with_the_payload_in_registers(dtype, phased):
         _fusion_roundtrip([int(c) for c in rng.integers(0, 9000, 512)], dtype, rng, divisors=(16,))
         _fusion_roundtrip([int(c) for c in rng.integers(1, 300, 513)], dtype, rng, divisors=(8,))   # one too many
         if np.dtype(dtype).itemsize == 4:
+            switch = cus * 300 * 1024 // 4                                                           # elements at the change of form
+            _fusion_roundtrip([switch - 7, 7], dtype, rng, divisors=(2,))                           # two workgroups per CU, 38 rounds
+            _fusion_roundtrip([switch - 7, 7 + 1024], dtype, rng, divisors=(2,))                    # one per CU
             _fusion_roundtrip([full - 5, 5], dtype, rng, divisors=(8,))                             # all the registers
             _fusion_roundtrip([full - 5, 5 + vec], dtype, rng, divisors=(8,))                       # a 113th round
     finally:
