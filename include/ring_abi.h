@@ -90,7 +90,7 @@ size_t ring_dtype_size(int dtype);
  * 31 MiB when the paced tiles would not fill the chip's CUs evenly. The same
  * option governs the unpack of a fused buffer (ring_fusion_unpack,
  * _unpack_scaled and the unpack of ring_fusion_run_static), which runs in that
- * form by default between 1 and 112 MiB when the set has at most 512
+ * form by default between 1 and 112 MiB when the set has at most 1024
  * non-empty tensors and the divisor, if any, is a power of two.
  * "dry_launch" = 1 makes the step-table / copy /
  * accumulate kernels return at entry: what is then timed is what a launch of

@@ -706,6 +706,7 @@ __global__ void __launch_bounds__(kBlock) fold_kernel(const FoldTable tab) {
 
 constexpr uint32_t kFusionTileVecs = 1024;
 constexpr uint32_t kFusionLdsCap = 512;  // tensors of one tile staged in LDS
+constexpr uint32_t kUnpackPhasedTensors = 1024;  // tensors of a set whose unpack holds its payload in registers
 
 // What a workgroup needs to know about its tile, in one 16-byte scalar load:
 // the first and last tensor that overlap it and, when that is one tensor (all
@@ -905,8 +906,8 @@ unpack_phased_kernel(const T* __restrict__ fused, const uint64_t* __restrict__ o
   typedef VU RING_GLOBAL GVU;
   constexpr uint32_t VEC = 16 / sizeof(T);
   constexpr int PER = WAVES == 1 ? kPhasedMax : kPhasedMaxTwoWaves;  // groups a lane holds
-  __shared__ uint64_t s_off[kFusionLdsCap + 1];
-  __shared__ T* s_ptr[kFusionLdsCap];
+  __shared__ uint64_t s_off[kUnpackPhasedTensors + 1];
+  __shared__ T* s_ptr[kUnpackPhasedTensors];
   __shared__ T* s_to[PER];  // where lane 0's vector of round j goes, or null: the round meets several tensors
   const uint32_t tid = threadIdx.x;
   const uint32_t stride = gridDim.x * kBlock;
@@ -924,29 +925,35 @@ unpack_phased_kernel(const T* __restrict__ fused, const uint64_t* __restrict__ o
   }
   if (blockIdx.x == 0 && tid < n_tail) tail = ((const GT*)fused)[static_cast<uint64_t>(nvec) * VEC + tid];
   // behind the payload: the destinations of this workgroup's rounds and the offset table (at most
-  // kFusionLdsCap tensors: three offsets and two pointers a lane). Every load is issued before the first
-  // is waited for, so the launch pays one memory latency for all of it, the one it pays for the payload.
-  static_assert(kFusionLdsCap == 2 * kBlock, "a lane stages offsets tid, tid + 256, tid + 512 and pointers tid, tid + 256");
+  // kUnpackPhasedTensors tensors: five offsets and four pointers a lane). Every load is issued before the
+  // first is waited for, so the launch pays one memory latency for all of it, the one it pays for the payload.
+  constexpr uint32_t kPtrsPerLane = kUnpackPhasedTensors / kBlock, kOffsPerLane = kPtrsPerLane + 1;
+  static_assert(kUnpackPhasedTensors % kBlock == 0, "whole rounds of the workgroup over the pointer table");
   T* to = nullptr;
   const uint64_t v0 = static_cast<uint64_t>(blockIdx.x) * kBlock + static_cast<uint64_t>(tid) * stride;
   const bool has_round = tid < rounds && v0 < nvec;
   // (a lane without a round reads tile 0's record and drops it: a load under a branch would be waited for there)
   const FusionTile rec = load_tile(tiles, has_round ? static_cast<uint32_t>(v0 / kFusionTileVecs) : 0u);
-  uint64_t off0 = 0, off1 = 0, off2 = 0;
-  T* ptr0 = nullptr;
-  T* ptr1 = nullptr;
-  if (tid <= m) off0 = offsets[tid];
-  if (tid + kBlock <= m) off1 = offsets[tid + kBlock];
-  if (tid + 2 * kBlock <= m) off2 = offsets[tid + 2 * kBlock];
-  if (tid < m) ptr0 = ptrs[tid];
-  if (tid + kBlock < m) ptr1 = ptrs[tid + kBlock];
+  uint64_t off[kOffsPerLane];
+  T* ptr[kPtrsPerLane];
+#pragma unroll
+  for (uint32_t i = 0; i < kOffsPerLane; i++) {
+    off[i] = 0;
+    if (tid + i * kBlock <= m) off[i] = offsets[tid + i * kBlock];
+  }
+#pragma unroll
+  for (uint32_t i = 0; i < kPtrsPerLane; i++) {
+    ptr[i] = nullptr;
+    if (tid + i * kBlock < m) ptr[i] = ptrs[tid + i * kBlock];
+  }
   if (has_round && rec.first == rec.last) to = static_cast<T*>(rec.addr) + (v0 % kFusionTileVecs) * VEC;
   if (tid < static_cast<uint32_t>(PER)) s_to[tid] = to;
-  if (tid <= m) s_off[tid] = off0;
-  if (tid + kBlock <= m) s_off[tid + kBlock] = off1;
-  if (tid + 2 * kBlock <= m) s_off[tid + 2 * kBlock] = off2;
-  if (tid < m) s_ptr[tid] = ptr0;
-  if (tid + kBlock < m) s_ptr[tid + kBlock] = ptr1;
+#pragma unroll
+  for (uint32_t i = 0; i < kOffsPerLane; i++)
+    if (tid + i * kBlock <= m) s_off[tid + i * kBlock] = off[i];
+#pragma unroll
+  for (uint32_t i = 0; i < kPtrsPerLane; i++)
+    if (tid + i * kBlock < m) s_ptr[tid + i * kBlock] = ptr[i];
   __syncthreads();
   RING_WAIT_VMEM();
   float reciprocal = 1.0f;
@@ -1669,7 +1676,7 @@ int launch_fusion(const FusionView& p, void* fused, hipStream_t stream, int divi
   // Between the two, the form with two workgroups per CU holds up to 80 MiB and is the better one up to 72
   // (64 MiB: 26.4 against 27.7 as one workgroup per CU and 27.0 as tiles; 80 MiB: 33.4 against 31.4).
   if (!PACK && g_tuning.phased_copy != 0 && g_tuning.blocks_per_cu == 0 && (g_tuning.nt[kRoleUnpack] & 3) == 3 &&
-      p.m <= kFusionLdsCap && (!DIV || (divisor & (divisor - 1)) == 0)) {
+      p.m <= kUnpackPhasedTensors && (!DIV || (divisor & (divisor - 1)) == 0)) {
     DeviceInfo info;
     int rc = device_info(&info);
     if (rc != RING_OK) return rc;

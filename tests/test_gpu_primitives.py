@@ -562,12 +562,12 @@ def test_fusion_unpack_with_the_payload_in_registers(dtype, phased):
     several tensors are stored lane by lane after a search of the offset
     table), forced on for every set it can take, left to the launcher (which
     takes it from 1 MiB, as two workgroups per CU up to 75 MiB and as one
-    beyond) and off: the same bytes
-    in the tensors and nothing outside them, with no divisor, with powers of
-    two (the form divides by them itself) and with 6 (it must leave that to
-    the tiles), tensor ends that cut 16-byte groups, hundreds of tiny tensors,
-    more tensors than its table holds, and a buffer of exactly and of just
-    over the 112 rounds a lane has registers for."""
+    beyond) and off: the same bytes in the tensors and nothing outside them,
+    with no divisor, with powers of two (the form divides by them itself) and
+    with 6 (it must leave that to the tiles), tensor ends that cut 16-byte
+    groups, hundreds of tiny tensors, as many tensors as its table holds
+    (1024) and one more, and a buffer of exactly and of just over the 112
+    rounds a lane has registers for."""
     import torch
     rng = np.random.default_rng(51 + phased)
     cus = torch.cuda.get_device_properties(0).multi_processor_count
@@ -581,7 +581,8 @@ def test_fusion_unpack_with_the_payload_in_registers(dtype, phased):
         _fusion_roundtrip([3, 2_000_003, 1, 1, 7, 999_999], dtype, rng, divisors=(8,))
         _fusion_roundtrip([int(c) for c in rng.integers(1, 200, 500)], dtype, rng, divisors=(4, 3))
         _fusion_roundtrip([int(c) for c in rng.integers(0, 9000, 512)], dtype, rng, divisors=(16,))
-        _fusion_roundtrip([int(c) for c in rng.integers(1, 300, 513)], dtype, rng, divisors=(8,))   # one too many
+        _fusion_roundtrip([int(c) for c in rng.integers(1, 300, 1024)], dtype, rng, divisors=(8,))  # all its table holds
+        _fusion_roundtrip([int(c) for c in rng.integers(1, 300, 1025)], dtype, rng, divisors=(8,))  # one too many
         if np.dtype(dtype).itemsize == 4:
             switch = cus * 300 * 1024 // 4                                                           # elements at the change of form
             _fusion_roundtrip([switch - 7, 7], dtype, rng, divisors=(2,))                           # two workgroups per CU, 38 rounds
