@@ -521,8 +521,7 @@ void run_all(const char* name) {
   std::vector<size_t> tiny(600);
   for (auto& c : tiny) c = g_rng() % 40;
   tiny[77] = 9000;
-  test_fusion<T>(tiny, 6, 4);
-  test_fusion<T>(tiny, 8, 4);  // a divisor the unpack that holds its payload in registers takes, on 600 tensors
+  test_fusion<T>(tiny, 8, 4);  // (a divisor the unpack that holds its payload in registers takes, here on 600 tensors)
   test_fusion<T>({17}, 3, 2);
   test_fusion<T>({}, 0, 2);
   test_fusion<T>({100003, 1, 2, 50001, 0, 4096, 3}, 4, 2);  // tensor ends that cut 16-byte groups, divided by a power of two
