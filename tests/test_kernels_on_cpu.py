@@ -97,5 +97,29 @@ def test_no_scalar_select_on_a_stale_condition_code():
     cmd = [hipcc] + HIP_FLAGS + ["-I", os.path.join(ROOT, "include"), "-S", "--cuda-device-only", "-o", asm, SRC]
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     assert res.returncode == 0, res.stdout[-4000:]
-    found = stale_selects(open(asm).read())
+    text = open(asm).read()
+    found = stale_selects(text)
     assert not found, "scalar selects on a stale condition code: %r" % (found[:5],)
+    # The kernels that hold a launch's payload in registers must really hold it there: a body too large to
+    # unroll, or one lane too many registers, and the compiler moves the array to scratch memory (a kernel
+    # several times slower with the same results, which no parity test would notice).
+    in_registers = kernels_in_scratch(text, ("rows_phased_kernel", "unpack_phased_kernel"))
+    assert in_registers["seen"] >= 20, in_registers
+    assert not in_registers["scratch"], "payload in scratch memory: %r" % (in_registers["scratch"][:5],)
+
+
+def kernels_in_scratch(asm_text, names):
+    """Of the kernels whose mangled name contains one of `names`: how many the
+    code object's metadata lists, and which of them have a private segment or
+    spilled vector registers."""
+    seen, scratch = 0, []
+    for block in asm_text.split("- .agpr_count:")[1:]:
+        name = re.search(r"\.name:\s+(\S+)", block)
+        if not name or not any(n in name.group(1) for n in names):
+            continue
+        seen += 1
+        private = int(re.search(r"\.private_segment_fixed_size:\s+(\d+)", block).group(1))
+        spilled = int(re.search(r"\.vgpr_spill_count:\s+(\d+)", block).group(1))
+        if private or spilled:
+            scratch.append((name.group(1), private, spilled))
+    return {"seen": seen, "scratch": scratch}
