@@ -91,7 +91,8 @@ size_t ring_dtype_size(int dtype);
  * option governs the unpack of a fused buffer (ring_fusion_unpack,
  * _unpack_scaled and the unpack of ring_fusion_run_static), which runs in that
  * form by default between 1 and 112 MiB when the set has at most 1024
- * non-empty tensors and the divisor, if any, is a power of two.
+ * non-empty tensors and the divisor, if any, is a power of two (float32: any
+ * divisor up to 64 MiB).
  * "dry_launch" = 1 makes the step-table / copy /
  * accumulate kernels return at entry: what is then timed is what a launch of
  * that grid costs by itself. No counterpart in the reference, whose launch

@@ -865,21 +865,24 @@ fusion_kernel(T* __restrict__ fused, const uint64_t* __restrict__ offsets, T* co
 // of its vector by binary search in the offset table, which the workgroup
 // staged in LDS next to the addresses. Nothing of this waits on memory a
 // second time: the records and the table arrive behind the payload.
-// DIV: the tensors receive value / divisor for a divisor that is a power of
-// two, the only ones this kernel takes: a multiplication by the exact
-// reciprocal for float32 and an arithmetic shift for the integers, which are
-// tf.div's true and floor division bit for bit (div_one does the same).
-template <typename T, bool DIV>
-__device__ __forceinline__ T divide_by_power_of_two(T x, float reciprocal, int shift) {
-  if constexpr (!DIV) {
-    (void)reciprocal;
-    (void)shift;
+// DIV 1: the tensors receive value / divisor for a divisor that is a power of
+// two: a multiplication by the exact reciprocal for float32 and an arithmetic
+// shift for the integers, which are tf.div's true and floor division bit for
+// bit (div_one does the same). DIV 2: float32 by any divisor, the IEEE
+// division of div_one (a dozen instructions an element, which the write phase
+// has the time for); the integers' general division is left to the tiles.
+template <typename T, int DIV>
+__device__ __forceinline__ T divide_in_registers(T x, float reciprocal, int shift, float divisor) {
+  (void)reciprocal;
+  (void)shift;
+  (void)divisor;
+  if constexpr (DIV == 0) {
     return x;
   } else if constexpr (std::is_floating_point<T>::value) {
-    (void)shift;
-    return x * reciprocal;
+    if constexpr (DIV == 2) return x / divisor;
+    else return x * reciprocal;
   } else {
-    (void)reciprocal;
+    static_assert(DIV == 1, "integers: powers of two only");
     return x >> shift;
   }
 }
@@ -895,7 +898,7 @@ __device__ __forceinline__ uint32_t tensor_of_element(const uint64_t* off, uint3
 }
 
 // WAVES: workgroups per CU, as in rows_phased_kernel (2: buffers of up to 56 MiB, 40 groups a lane).
-template <typename T, bool DIV, int WAVES>
+template <typename T, int DIV, int WAVES>
 __global__ void __launch_bounds__(kBlock) RING_WAVES_PER_SIMD(WAVES)
 unpack_phased_kernel(const T* __restrict__ fused, const uint64_t* __restrict__ offsets, T* const* __restrict__ ptrs,
                      const FusionTile* __restrict__ tiles, uint32_t m, uint64_t total, uint32_t rounds, int divisor) {
@@ -958,8 +961,9 @@ unpack_phased_kernel(const T* __restrict__ fused, const uint64_t* __restrict__ o
   RING_WAIT_VMEM();
   float reciprocal = 1.0f;
   int shift = 0;
-  if (DIV) {
-    reciprocal = 1.0f / static_cast<float>(divisor);
+  const float fdivisor = static_cast<float>(divisor);
+  if (DIV == 1) {
+    reciprocal = 1.0f / fdivisor;
     while ((1 << shift) < divisor) shift++;
   }
 #pragma unroll
@@ -969,7 +973,7 @@ unpack_phased_kernel(const T* __restrict__ fused, const uint64_t* __restrict__ o
       if (idx < nvec) {
         V r = s[j];
 #pragma unroll
-        for (uint32_t c = 0; c < VEC; c++) r[c] = divide_by_power_of_two<T, DIV>(r[c], reciprocal, shift);
+        for (uint32_t c = 0; c < VEC; c++) r[c] = divide_in_registers<T, DIV>(r[c], reciprocal, shift, fdivisor);
         T* to = s_to[j];
         if (to) {
           __builtin_nontemporal_store(r, &((GVU*)(GT*)to)[tid]);
@@ -998,7 +1002,7 @@ unpack_phased_kernel(const T* __restrict__ fused, const uint64_t* __restrict__ o
   if (blockIdx.x == 0 && tid < n_tail) {
     const uint64_t e = static_cast<uint64_t>(nvec) * VEC + tid;
     const uint32_t l = tensor_of_element(s_off, m, e);
-    *(GT*)(s_ptr[l] + (e - s_off[l])) = divide_by_power_of_two<T, DIV>(tail, reciprocal, shift);
+    *(GT*)(s_ptr[l] + (e - s_off[l])) = divide_in_registers<T, DIV>(tail, reciprocal, shift, fdivisor);
   }
 }
 
@@ -1676,7 +1680,7 @@ int launch_fusion(const FusionView& p, void* fused, hipStream_t stream, int divi
   // Between the two, the form with two workgroups per CU holds up to 80 MiB and is the better one up to 72
   // (64 MiB: 26.4 against 27.7 as one workgroup per CU and 27.0 as tiles; 80 MiB: 33.4 against 31.4).
   if (!PACK && g_tuning.phased_copy != 0 && g_tuning.blocks_per_cu == 0 && (g_tuning.nt[kRoleUnpack] & 3) == 3 &&
-      p.m <= kUnpackPhasedTensors && (!DIV || (divisor & (divisor - 1)) == 0)) {
+      p.m <= kUnpackPhasedTensors && (!DIV || (divisor & (divisor - 1)) == 0 || std::is_floating_point<T>::value)) {
     DeviceInfo info;
     int rc = device_info(&info);
     if (rc != RING_OK) return rc;
@@ -1687,16 +1691,29 @@ int launch_fusion(const FusionView& p, void* fused, hipStream_t stream, int divi
     const uint64_t rounds = (nvec + stride - 1) / stride;
     if (rounds >= 1 && rounds <= static_cast<uint64_t>(waves == 1 ? kPhasedMax : kPhasedMaxTwoWaves) &&
         (g_tuning.phased_copy > 0 || (per_cu >= kUnpackPhasedMinPerCu && info.cus >= 128))) {
-      if (waves == 1)
-        launch(unpack_phased_kernel<T, DIV, 1>, dim3(static_cast<uint32_t>(wgs)), dim3(kBlock), stream,
-               static_cast<const T*>(fused), p.offsets, reinterpret_cast<T* const*>(p.ptrs), p.tiles, p.m, p.total,
-               static_cast<uint32_t>(rounds), divisor);
-      else
-        launch(unpack_phased_kernel<T, DIV, 2>, dim3(static_cast<uint32_t>(wgs)), dim3(kBlock), stream,
-               static_cast<const T*>(fused), p.offsets, reinterpret_cast<T* const*>(p.ptrs), p.tiles, p.m, p.total,
-               static_cast<uint32_t>(rounds), divisor);
-      RING_HIP(hipGetLastError());
-      return RING_OK;
+#define RING_UNPACK_PHASED(D, W)                                                                              \
+  launch(unpack_phased_kernel<T, D, W>, dim3(static_cast<uint32_t>(wgs)), dim3(kBlock), stream,               \
+         static_cast<const T*>(fused), p.offsets, reinterpret_cast<T* const*>(p.ptrs), p.tiles, p.m, p.total, \
+         static_cast<uint32_t>(rounds), divisor)
+      constexpr int kPowerOfTwo = DIV ? 1 : 0;
+      bool launched = true;
+      if (!DIV || (divisor & (divisor - 1)) == 0) {
+        if (waves == 1) RING_UNPACK_PHASED(kPowerOfTwo, 1); else RING_UNPACK_PHASED(kPowerOfTwo, 2);
+      } else if constexpr (DIV && std::is_floating_point<T>::value) {
+        // float32 by any other divisor: the IEEE division in the kernel, as two workgroups per CU only
+        // (with 112 rounds to unroll the division makes the body too large for the compiler to keep the
+        // payload in registers) and up to 64 MiB (by 6, behind the allgather: 4 MiB 5.4 against 7.2 us as
+        // tiles, 32 MiB 13.1 / 15.5, 64 MiB 26.1 / 27.2, 72 MiB 30.1 / 28.9); beyond, the tiles
+        if (waves == 2 && (g_tuning.phased_copy > 0 || per_cu <= (256u << 10))) RING_UNPACK_PHASED(2, 2);
+        else launched = false;
+      } else {
+        launched = false;
+      }
+#undef RING_UNPACK_PHASED
+      if (launched) {
+        RING_HIP(hipGetLastError());
+        return RING_OK;
+      }
     }
   }
   uint32_t grid = p.ntiles;

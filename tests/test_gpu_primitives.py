@@ -563,8 +563,9 @@ def test_fusion_unpack_with_the_payload_in_registers(dtype, phased):
     table), forced on for every set it can take, left to the launcher (which
     takes it from 1 MiB, as two workgroups per CU up to 75 MiB and as one
     beyond) and off: the same bytes in the tensors and nothing outside them,
-    with no divisor, with powers of two (the form divides by them itself) and
-    with 6 (it must leave that to the tiles), tensor ends that cut 16-byte
+    with no divisor, with powers of two and with 6 and 3 (float32 divides by
+    them in the form as two workgroups per CU; the integers and the larger
+    float32 sets must leave them to the tiles), tensor ends that cut 16-byte
     groups, hundreds of tiny tensors, as many tensors as its table holds
     (1024) and one more, and a buffer of exactly and of just over the 112
     rounds a lane has registers for."""
