@@ -41,9 +41,14 @@ for p in (ROOT, os.path.join(ROOT, "tensorflow-allreduce_amd")):
         sys.path.insert(0, p)
 
 HBM_PEAK_GBS = 8000.0
-SAMPLE_EVERY = 16                   # steps between launches that carry timing events
-MIN_SAMPLES = 16                    # timed launches per phase, whatever --steps is
+FRESH_STAGING = False               # --fresh-staging: see FusedResnet50NoPasses.coaligned
+REGIONS = 9                         # wall-clock regions of --steps steps each; ms_per_step is their median
+SAMPLE_EVERY = 4                    # steps between launches that carry timing events (sampling pass only)
+MIN_SAMPLES = 32                    # timed launches per phase, whatever --steps is
+MAX_SAMPLES = 128
 COLD_SAMPLES = 32                   # timed launches of the cold-operand accumulate
+EXTRA_MIN_STEPS = 200               # the extras (hot, fused_copy, direct_form) run at least this many steps per region
+EXTRA_REGIONS = 3
 METRIC = "per-rank ring allreduce GB/s & % of HBM peak, 64 MiB fp32, N=8 virtual ranks"
 # committed rocprofv3 counter summaries holding a `traffic_bytes_per_launch:` line for a workload's dominant kernel
 TRAFFIC_PROFILES = {
@@ -222,6 +227,65 @@ class RingAllreducePerStep(RingAllreduce):
                 A.check(R.ring_accumulate(self.code, dst, t.data_ptr(), self.sizes[g], stream), "accumulate")
             else:
                 A.check(R.ring_copy_bytes(dst, t.data_ptr(), self.sizes[g] * self.esz, stream), "copy")
+
+
+class StreamFloors(Workload):
+    """What the chip gives ONE direction at the sizes of an allreduce's two copy
+    launches, next to the launches themselves: the copy source read and nothing
+    written, the copy destination written and nothing read, the in->out copy;
+    the same three for the rows of the allgather phase. A copy runs no faster
+    than its two directions one after the other, so read-only + write-only is
+    the floor of the copy at that size on this chip. Buffers rotate as in the
+    allreduce workload; every phase is one launch (ring_probe_stream for the
+    one-directional ones), timed by events in its dispatch."""
+
+    def __init__(self, name, np_name, count, n, nsets, what):
+        self.inner = r = RingAllreduce(name, np_name, count, n, nsets, what)
+        self.name, self.dtype, self.count, self.n, self.nsets, self.esz = name, np_name, count, n, nsets, r.esz
+        self.ring_abi, self.R = r.ring_abi, r.R
+        esz = r.esz
+        up = lambda p: (p + 15) & ~15       # the probe wants 16-byte aligned pointers; a ragged start loses < 16 bytes
+        for s in r.sets:
+            out = s["out"].data_ptr()
+            s["probe_copy"] = [(out, s["inp"].data_ptr(), None, count)]
+            s["probe_ag"] = [(up(out + r.starts[g] * esz), t.data_ptr(), None, r.sizes[g] - 16 // esz)
+                             for g, t in zip(s["ag_seg"], s["ag"])]
+        ag_bytes = sum(r.sizes[g] for g in r.sets[0]["ag_seg"]) * esz
+        self.phases = (
+            ("read_only_copy_source", count * esz, "stream_probe_kernel<read> (1 row, %d bytes)" % (count * esz)),
+            ("write_only_copy_destination", count * esz, "stream_probe_kernel<write> (1 row, %d bytes)" % (count * esz)),
+            r.phases[0],
+            ("read_only_allgather_sources", ag_bytes, "stream_probe_kernel<read> (%d rows, %d bytes)" % (n - 1, ag_bytes)),
+            ("write_only_allgather_destinations", ag_bytes,
+             "stream_probe_kernel<write> (%d rows, %d bytes)" % (n - 1, ag_bytes)),
+            r.phases[2])
+        self.dominant = 2
+        self.description = ("one direction at a time against the copy launches of: " + what)
+
+    def launch_phase(self, k, i, stream):
+        # the probes work on another buffer set than the copies of the same step, so that no copy
+        # finds in a cache what a probe has just touched
+        s, A = self.inner.sets[(k + self.nsets // 2) % self.nsets], self.ring_abi
+        if i in (0, 1):
+            A.probe_stream(s["probe_copy"], self.inner.code, i, stream)
+        elif i == 2:
+            self.inner.launch_phase(k, 0, stream)
+        elif i in (3, 4):
+            A.probe_stream(s["probe_ag"], self.inner.code, i - 3, stream)
+        else:
+            self.inner.launch_phase(k, 2, stream)
+
+    def launch_step(self, k, stream, fused=False):
+        for i in range(6):
+            self.launch_phase(k, i, stream)
+
+    def check(self, k):
+        s = self.inner.sets[k % self.nsets]
+        ok = True
+        for g, t in zip(s["ag_seg"], s["ag"]):
+            a = self.inner.starts[g]
+            ok = ok and self.inner.torch.equal(s["out"][a:a + self.inner.sizes[g]], t)
+        return bool(ok)
 
 
 class RingAllreduceDirect(Workload):
@@ -405,6 +469,11 @@ class FusedResnet50NoPasses(FusedResnet50):
             r = s % 8
             rs_seg = [A.schedule(0, 8, r, i)[1] for i in range(7)]
             ag_seg = [A.schedule(1, 8, r, i)[1] for i in range(7)]
+            # Where a finished segment lands is the receiver's choice, and the reference receives it in place,
+            # at buffer + starts[segment] (ring.h:211-225): 16-byte groups of the arrival are then groups of the
+            # fused space. The slots here keep that: each starts starts[segment] % 4 elements into its allocation
+            # (3,194,629-element segments begin at every residue), so the scatter's loads are aligned like its stores.
+            st["ag"] = [self.coaligned(t, starts[g]) for g, t in zip(ag_seg, st["ag"])]
             rs_of = {g: t for g, t in zip(rs_seg, st["rs"])}
             ag_of = {g: t for g, t in zip(ag_seg, st["ag"])}
             own, wire = (r + 1) % 8, st["fused"].data_ptr()
@@ -426,6 +495,15 @@ class FusedResnet50NoPasses(FusedResnet50):
                             "elements, values ~N(0,1e-3)) at N=8 virtual ranks WITHOUT pack and unpack passes: the 7 "
                             "accumulates read their local operand from the tensors and write the wire buffer, the 8 "
                             "finished segments go straight into the tensors with the divide by 8; 2 launches per step")
+
+    def coaligned(self, t, begin):
+        """A copy of segment `t` whose element 0 lies `begin` % 4 elements behind a 16-byte boundary."""
+        if FRESH_STAGING:      # --fresh-staging: the slots as fresh allocations, for comparison
+            return t
+        room = self.torch.empty(t.numel() + 4, device="cuda")
+        view = room[begin % 4: begin % 4 + t.numel()]
+        view.copy_(t)
+        return view
 
     def launch_phase(self, k, i, stream):
         s = self.sets[k % self.nsets]
@@ -458,7 +536,8 @@ class FusedResnet50NoPassesDirect(FusedResnet50NoPasses):
         for st in self.sets:
             own = (st["r"] + 1) % 8
             gen = torch.Generator(device="cuda").manual_seed(77 + st["r"])
-            st["raw"] = [torch.randn(sizes[own], device="cuda", generator=gen) * 1e-3 for _ in range(7)]
+            st["raw"] = [self.coaligned(torch.randn(sizes[own], device="cuda", generator=gen) * 1e-3, starts[own])
+                         for _ in range(7)]
             st["raw_ptrs"] = (ctypes.c_void_p * 7)(*[t.data_ptr() for t in st["raw"]])
             st["own"], st["mine"] = own, st["fused"].data_ptr() + starts[own] * 4
             ag_of = {g: t for g, t in zip(st["ag_seg"], st["ag"])}
@@ -652,6 +731,13 @@ def make_workload(name):
                              "%s ring allreduce of a ragged 10,000,019-element tensor, N=6 virtual ranks (segments "
                              "1,666,670 x5 + 1,666,669): copy + 5 accumulates + 5 copies per step, peers pre-staged, "
                              "12 buffer sets rotated" % {"i32": "int32", "i64": "int64"}[dt])
+    if name.startswith("floors_"):
+        _, dt, size, ranks = name.split("_")
+        count = {"64MiB": 16 * 1024 * 1024, "10000019": 10_000_019}[size]
+        n = int(ranks[1:])
+        return StreamFloors(name, dt, count, n, 8 if n == 8 else 12,
+                            "%s ring allreduce of %d elements at N=%d (in->out copy of %d bytes; allgather copies of %d rows)"
+                            % (dt, count, n, count * (8 if dt == "i64" else 4), n - 1))
     if name == "allreduce_f32_1MiB_n8":
         return RingAllreduce(name, "f32", 262_144, 8, 8,
                              "float32 ring allreduce of one 262,144-element (1 MiB) tensor, N=8 virtual ranks: a "
@@ -678,7 +764,8 @@ WORKLOADS = ("allreduce_f32_64MiB_n8", "allreduce_i32_10000019_n6", "allreduce_i
              "allreduce_f32_1MiB_n8", "allreduce_f32_1MiB_n8_direct",
              "allreduce_f32_64MiB_n8_direct", "fused_resnet50_n8_no_passes",
              "fused_resnet50_n8_no_passes_direct", "allreduce_f32_64MiB_all_ranks_n8",
-             "fused_resnet50_all_ranks_n8")
+             "fused_resnet50_all_ranks_n8",
+             "floors_f32_64MiB_n8", "floors_i32_10000019_n6", "floors_i64_10000019_n6")
 
 
 def cpu_baseline(w):
@@ -749,6 +836,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--workload", default=WORKLOADS[0], choices=WORKLOADS)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--fresh-staging", action="store_true",
+                    help="fused workloads without passes: stage every finished segment at the start of a fresh "
+                         "allocation instead of where its 16-byte groups line up with the fused space")
     ap.add_argument("--variant", choices=("all", "reference", "fused"), default="all",
                     help="all: the reference-shaped path (the reported value), then the extras: the same job with "
                          "the in->out copy folded into the accumulate, and the hot (one buffer set) rate. "
@@ -759,9 +849,11 @@ def main():
                          "time its replays; for launch-bound sizes. --steps is rounded down to a multiple of it")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="launch option of the kernel library (unroll, blocks_per_cu, nontemporal[_copy|_accumulate|"
-                         "_allgather|_pack|_unpack], paced_copy, phased_copy, dry_launch), "
+                         "_allgather|_pack|_unpack], paced_copy, phased_copy, dry_launch, flat_grid), "
                          "for comparing launch shapes under a profiler")
     args = ap.parse_args()
+    global FRESH_STAGING
+    FRESH_STAGING = args.fresh_staging
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures the per-rank data path on ONE GPU (the ring's N ranks are virtual); "
                  "--gpus %d is not supported" % args.gpus)
@@ -790,59 +882,86 @@ def main():
     # the dedicated stream every ring kernel is launched on (CudaStreamForMPI)
     stream = ring_abi.stream_create()
     nph = len(w.phases)
-    # events are created before the timed region: creating them inside it would
-    # let the queue drain and the sampled launches start on an idle GPU
-    sample_every = max(1, min(SAMPLE_EVERY, steps))
+    # events are created ahead of the passes that use them: creating them between launches
+    # would let the queue drain and the sampled launches start on an idle GPU
     # (a set = one pair per launch of the sampled step and one per launch of the step before it)
     npairs = max(nph, 2)
+    n_samples = max(MIN_SAMPLES, min(steps // 16, MAX_SAMPLES))
     event_pool = [[ring_abi.event_create() for _ in range(4 * npairs)]
-                  for _ in range(steps // sample_every + 1 + MIN_SAMPLES + COLD_SAMPLES)]
+                  for _ in range(n_samples + 1 + COLD_SAMPLES)]
 
-    def timed(nsteps, nwarm, fused=False, with_samples=False, hot=False, sample_every=sample_every):
+    def launcher(hot):
         # hot: the same buffer set every step (what fits stays in the last-level
         # cache); otherwise the sets rotate and every step starts cold
         if hot:
-            def launch_step(k, stream, fused):
-                w.launch_step(0, stream, fused)
-        else:
-            launch_step = w.launch_step
-        for k in range(nwarm):
+            return lambda k, stream, fused: w.launch_step(0, stream, fused)
+        return w.launch_step
+
+    def region(nsteps, nwarm, fused=False, hot=False, first=0):
+        """Wall-clock seconds of `nsteps` steps, bracketed by a synchronize on both sides,
+        after `nwarm` untimed steps. Nothing inside the region carries an event: a dispatch
+        that carries one ends only when its stores have drained, which serialises it against
+        the launch behind it."""
+        launch_step = launcher(hot)
+        for k in range(first, first + nwarm):
             launch_step(k, stream, fused)
         ring_abi.stream_synchronize(stream)
         torch.cuda.synchronize()
-        samples = []
-        # a collection of the interpreter's garbage in the middle of the region stalls the
-        # launching thread for tens of milliseconds; workloads whose step is one short launch
-        # have no queue of launches ahead of the GPU to hide that behind
+        t0 = time.perf_counter()
+        for k in range(first + nwarm, first + nwarm + nsteps):
+            launch_step(k, stream, fused)
+        ring_abi.stream_synchronize(stream)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    def regions(count, nsteps, nwarm, **kw):
+        """`count` such regions back to back, each behind its own `nwarm` warm-up steps;
+        returns their seconds per step, in the order measured. The interpreter's garbage is
+        collected once, ahead of the first region, and the collector is off until the last
+        has ended: a collection in the middle of a region stalls the launching thread for
+        tens of milliseconds (a step that is one short launch has no queue of launches ahead
+        of the GPU to hide that behind), and one between two regions leaves the GPU idle for
+        as long, after which a region of a millisecond runs 5 % slower from its first step to
+        its last than the same steps do in a longer one."""
+        out, first = [], 0
         gc.collect()
         gc.disable()
-        t0 = time.perf_counter()
-        launches = 2 if fused else nph
-        for k in range(nsteps):
-            if with_samples and sample_every > 1 and (k + 1) % sample_every == sample_every // 2:
-                # the step before a sampled one is timed as well (its figures are not used): a timed
-                # dispatch ends when its stores have drained, so the sampled step's first launch does
-                # not pay for its predecessor's, as under a profiler's kernel trace
+        try:
+            for _ in range(count):
+                out.append(region(nsteps, nwarm, first=first, **kw) / nsteps)
+                first += nsteps + nwarm
+        finally:
+            gc.enable()
+        return out
+
+    def sampling_pass(count):
+        """Per-launch durations, outside every wall-clock region: the same steps on the same
+        rotating buffers, every SAMPLE_EVERY-th one launched phase by phase, each launch
+        carrying its own pair of HIP events in the dispatch (on the stream the kernels run
+        on). The step before a sampled one carries (unused) events too: a timed dispatch ends
+        when its stores have drained, so the sampled step's first launch does not pay for its
+        predecessor's, as under a profiler's kernel trace, where every dispatch is timed."""
+        samples = []
+        for k in range(8):
+            w.launch_step(k, stream)
+        for k in range(8, 8 + count * SAMPLE_EVERY):
+            if k % SAMPLE_EVERY == SAMPLE_EVERY - 2:
                 spare = event_pool[-1]
-                for i in range(launches):
+                for i in range(nph):
                     ring_abi.time_next_launch(spare[2 * (npairs + i)], spare[2 * (npairs + i) + 1])
-                launch_step(k, stream, fused)
+                w.launch_step(k, stream)
                 ring_abi.time_next_launch(None, None)       # a step of fewer launches leaves none armed
-            elif with_samples and k % sample_every == sample_every // 2:
-                # the same launches, one ABI call each, every one carrying its own
-                # pair of HIP events in the dispatch (on the stream the kernels run on)
+            elif k % SAMPLE_EVERY == SAMPLE_EVERY - 1:
                 e = event_pool.pop()
                 for i in range(nph):
                     ring_abi.time_next_launch(e[2 * i], e[2 * i + 1])
                     w.launch_phase(k, i, stream)
                 samples.append(e)
             else:
-                launch_step(k, stream, fused)
+                w.launch_step(k, stream)
         ring_abi.stream_synchronize(stream)
         torch.cuda.synchronize()
-        elapsed = time.perf_counter() - t0
-        gc.enable()
-        return elapsed, samples
+        return samples
 
     if args.recorded:
         # `recorded` consecutive steps (rotating over the buffer sets) as one HIP graph, replayed
@@ -882,8 +1001,9 @@ def main():
     if args.variant == "fused":
         if not isinstance(w, RingAllreduce) or isinstance(w, RingAllreducePerStep):
             sys.exit("bench.py: --variant fused applies to the allreduce workloads")
-        fused_elapsed, _ = timed(steps, warmup, fused=True)
-        if not w.check(steps - 1):
+        per_step = regions(REGIONS, steps, warmup, fused=True)
+        fused_elapsed = statistics.median(per_step) * steps
+        if not w.check(REGIONS * (steps + warmup) - 1):
             sys.exit("bench.py: the output of the fused-copy path is wrong; refusing to report a number")
         print(json.dumps({"metric": "per-rank ring data path GB/s, %s, in->out copy folded into the accumulate" % w.name,
                           "value": round(w.fused_bytes * steps / fused_elapsed / 1e9, 1), "unit": "GB/s", "n_gpus": 1,
@@ -892,17 +1012,12 @@ def main():
                           "config": {"workload": w.description, "name": w.name, "bytes_per_step": w.fused_bytes,
                                      "launches_per_step": 2}}))
         return
-    elapsed, samples = timed(steps, warmup, with_samples=True)
-    in_region = len(samples)
-    if in_region < MIN_SAMPLES:
-        # a short timed region carries too few timed launches: a sampling pass of its own, the same
-        # steps on the same rotating buffers, every 4th one timed; not part of the wall clock
-        _, more = timed((MIN_SAMPLES - in_region) * 4, 4, with_samples=True, sample_every=4)
-        samples += more
-    if not w.check(steps - 1):
+    per_step = regions(REGIONS, steps, warmup)
+    if not w.check(REGIONS * (steps + warmup) - 1):
         sys.exit("bench.py: the output of the timed path is wrong; refusing to report a number")
-    ms_per_step = elapsed / steps * 1e3
-    value = w.bytes_per_step * steps / elapsed / 1e9
+    ms_per_step = statistics.median(per_step) * 1e3
+    value = w.bytes_per_step / statistics.median(per_step) / 1e9
+    samples = sampling_pass(n_samples)
     phase_times = [[ring_abi.event_elapsed_us(e[2 * i], e[2 * i + 1]) for e in samples] for i in range(nph)]
     phase_us = [statistics.mean(t) for t in phase_times]
     dom = w.phases[w.dominant]
@@ -918,7 +1033,7 @@ def main():
         cold_events = []
         for k in range(COLD_SAMPLES * 4):
             if k % 4 == 1:
-                # the step before, timed too (see timed())
+                # the step before, timed too (see sampling_pass())
                 spare = event_pool[-1]
                 for i in range(2):
                     ring_abi.time_next_launch(spare[2 * (npairs + i)], spare[2 * (npairs + i) + 1])
@@ -946,6 +1061,12 @@ def main():
         "steps": steps,
         "warmup": warmup,
         "ms_per_step": round(ms_per_step, 5),
+        "regions": {"count": REGIONS, "steps_each": steps, "warmup_before_each": warmup,
+                    "ms_per_step_each": [round(t * 1e3, 5) for t in per_step],
+                    "min_ms_per_step": round(min(per_step) * 1e3, 5),
+                    "note": "ms_per_step and value are the MEDIAN of %d wall-clock regions of %d steps each, run back "
+                            "to back, every region bracketed by a stream synchronize on both sides and free of "
+                            "event-carrying launches" % (REGIONS, steps)},
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -967,7 +1088,7 @@ def main():
             "median_launch_us": round(dom_median, 3),
             "avg_launch_us": round(phase_us[w.dominant], 3),
             "launches_timed": len(samples),
-            "launches_timed_inside_the_wall_clock_region": in_region,
+            "launches_timed_inside_the_wall_clock_region": 0,
             "note": "achieved = algorithmic bytes / median launch duration (HIP events carried in the dispatch)."
                     + (" In the reference-shaped step the accumulate reads the buffer the in->out copy has just "
                        "written with ordinary stores, so part of its reads are served by the last-level cache: `frac` "
@@ -981,9 +1102,9 @@ def main():
                           "min_us": round(min(phase_times[i]), 3), "GBps": round(p[1] / t / 1e3, 1),
                           "bytes": p[1]}
                    for i, (p, t) in enumerate(zip(w.phases, phase_us))},
-        "phases_note": "HIP events carried by each launch of every %dth step of the timed region%s; us = mean"
-                       % (sample_every, "" if in_region >= MIN_SAMPLES else
-                          " plus a sampling pass after it (every 4th step) to reach %d timed launches" % MIN_SAMPLES),
+        "phases_note": "HIP events carried by each launch of every %dth step of a sampling pass of %d steps that "
+                       "follows the wall-clock regions (none of their launches carries an event); us = mean"
+                       % (SAMPLE_EVERY, n_samples * SAMPLE_EVERY),
     }
     if cold is not None:
         result["roofline"]["frac_cold"] = round(dom[1] / cold["accumulate_median_us"] / 1e3 / HBM_PEAK_GBS, 4)
@@ -992,8 +1113,9 @@ def main():
     # the same steps on ONE buffer set: at the headline size the working set fits the
     # last-level cache, so this is the cache-resident rate, not the HBM one
     if args.variant == "all":
-        hot_steps = max(steps // 4, 1)
-        hot_elapsed, _ = timed(hot_steps, min(warmup, 50), hot=True)
+        extra_steps = max(steps, EXTRA_MIN_STEPS)
+        hot_steps = extra_steps
+        hot_elapsed = statistics.median(regions(EXTRA_REGIONS, hot_steps, min(max(warmup, 20), 50), hot=True)) * hot_steps
         result["hot"] = {"ms_per_step": round(hot_elapsed / hot_steps * 1e3, 5),
                          "GBps": round(w.bytes_per_step * hot_steps / hot_elapsed / 1e9, 1),
                          "note": "every step on the same buffers (%.0f MiB touched per step); `value` is the cold "
@@ -1001,13 +1123,15 @@ def main():
     if isinstance(w, RingAllreduce) and not isinstance(w, RingAllreducePerStep):
         # the same job with the in->out copy folded into the accumulate (fewer bytes, same result)
         if args.variant == "all":
-            fused_elapsed, _ = timed(steps, min(warmup, 50), fused=True)
-            if not w.check(steps - 1):
+            fwarm = min(max(warmup, 20), 50)
+            fused_per_step = statistics.median(regions(EXTRA_REGIONS, extra_steps, fwarm, fused=True))
+            if not w.check(EXTRA_REGIONS * (extra_steps + fwarm) - 1):
                 sys.exit("bench.py: the output of the fused-copy path is wrong; refusing to report a number")
             result["fused_copy"] = {
-                "ms_per_step": round(fused_elapsed / steps * 1e3, 5),
+                "ms_per_step": round(fused_per_step * 1e3, 5),
+                "steps": extra_steps, "regions": EXTRA_REGIONS,
                 "bytes_per_step": w.fused_bytes,
-                "GBps": round(w.fused_bytes * steps / fused_elapsed / 1e9, 1),
+                "GBps": round(w.fused_bytes / fused_per_step / 1e9, 1),
                 "launches_per_step": 2,
                 "note": "same allreduce with the in->out copy folded into the accumulate (out = in + received; the "
                         "segment that is only sent is written by the first allgather step and never copied)",
@@ -1017,18 +1141,22 @@ def main():
             d = make_workload("allreduce_f32_64MiB_n8_direct")
             for k in range(50):
                 d.launch_step(k, stream)
-            ring_abi.stream_synchronize(stream)
-            t0 = time.perf_counter()
-            for k in range(steps):
-                d.launch_step(k, stream)
-            ring_abi.stream_synchronize(stream)
-            direct_elapsed = time.perf_counter() - t0
-            if not d.check(steps - 1):
+            direct = []
+            for _ in range(EXTRA_REGIONS):
+                ring_abi.stream_synchronize(stream)
+                t0 = time.perf_counter()
+                for k in range(extra_steps):
+                    d.launch_step(k, stream)
+                ring_abi.stream_synchronize(stream)
+                direct.append((time.perf_counter() - t0) / extra_steps)
+            if not d.check(extra_steps - 1):
                 sys.exit("bench.py: the output of the direct form is wrong; refusing to report a number")
+            direct_per_step = statistics.median(direct)
             result["direct_form"] = {
-                "ms_per_step": round(direct_elapsed / steps * 1e3, 5),
+                "ms_per_step": round(direct_per_step * 1e3, 5),
+                "steps": extra_steps, "regions": EXTRA_REGIONS,
                 "bytes_per_step": d.bytes_per_step,
-                "GBps": round(d.bytes_per_step * steps / direct_elapsed / 1e9, 1),
+                "GBps": round(d.bytes_per_step / direct_per_step / 1e9, 1),
                 "launches_per_step": 1,
                 "note": "same tensor and ranks, peers push raw copies of the owned segment instead of passing partial "
                         "sums round: the owner folds the 8 copies in ring order in one pass and copies the 7 finished "
@@ -1048,6 +1176,13 @@ def main():
                                             "direct form and no ranks that share a device, and its allgather moves "
                                             "bytes only): the default workload carries the CPU baseline"}
     ring_abi.stream_destroy(stream)
+    try:
+        # what this process started and has not reaped (the cpu_baseline's mpirun legs run in process
+        # groups of their own, which are ended when each returns)
+        import psutil
+        result["child_processes_at_exit"] = len(psutil.Process().children(recursive=True))
+    except Exception:
+        result["child_processes_at_exit"] = None
     print(json.dumps(result))
 
 

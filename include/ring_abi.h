@@ -67,7 +67,8 @@ int ring_last_hip_error(void);
 size_t ring_dtype_size(int dtype);
 
 /* Launch-shape knobs for measurement runs (process-wide; not needed for
- * normal use): "unroll" = 16-byte vectors per lane per tile (2, 4, 8),
+ * normal use; may be set from one thread while others launch: every launch
+ * reads the options once, at entry): "unroll" = 16-byte vectors per lane per tile (2, 4, 8),
  * "blocks_per_cu" = 0 for one workgroup per tile, k > 0 for a persistent grid
  * of CUs x k workgroups that stride over the tiles. Cache policy per kind of
  * launch: "nontemporal_copy" (ring_copy_bytes), "nontemporal_accumulate"
@@ -95,7 +96,9 @@ size_t ring_dtype_size(int dtype);
  * divisor up to 64 MiB).
  * "dry_launch" = 1 makes the step-table / copy /
  * accumulate kernels return at entry: what is then timed is what a launch of
- * that grid costs by itself. No counterpart in the reference, whose launch
+ * that grid costs by itself. "flat_grid" = 1 gives rows of equal length the
+ * 1-D grid of unequal rows (a workgroup finds its row by counting) instead of
+ * the 2-D grid (tiles, rows). No counterpart in the reference, whose launch
  * shape is the constant <<<32, 256>>> (ring.cu.cc:64). */
 int ring_set_option(const char* name, int value);
 
@@ -172,6 +175,13 @@ int ring_allgather_table(const size_t* rows, int n, size_t elems_per_row,
  * (ring.h:171-174). */
 enum ring_phase { RING_PHASE_REDUCE_SCATTER = 0, RING_PHASE_ALLGATHER = 1, RING_PHASE_GATHER = 2 };
 int ring_schedule(int phase, int n, int r, int step, int* send_seg, int* recv_seg);
+
+/* The GPU of the calling thread, for host code that includes no HIP header:
+ * the reference remembers the device MPI was initialised on (cudaGetDevice,
+ * mpi_ops.cc:805-809) and makes it current on its background thread before it
+ * creates the stream there (cudaSetDevice, mpi_ops.cc:582). */
+int ring_get_device(int* device);
+int ring_set_device(int device);
 
 /* ---- the dedicated stream — CudaStreamForMPI(), mpi_ops.cc:213-230, 582-583,
  * 872-876: one non-default stream for all ring copies and accumulates, so a
@@ -265,6 +275,44 @@ int ring_apply_rows(const ring_row* rows, int n_rows, int dtype, void* stream);
  * `rows` and `divide` are HOST arrays. */
 int ring_apply_rows_avg(const ring_row* rows, int n_rows, const unsigned char* divide, int divisor,
                         int dtype, void* stream);
+
+/* Which form a launch takes, as a query that needs no GPU (no counterpart in
+ * the reference, whose one launch shape is the constant <<<32, 256>>>,
+ * ring.cu.cc:64). The copies of an allgather phase and the unpack of a fused
+ * buffer run in one of several forms, chosen from the shape of the launch and
+ * the number of compute units; every form gives the same bytes, so only this
+ * query (and a profiler) tells which one a shape takes, and a test can pin
+ * the choice for the shapes that were measured.
+ * ring_describe_rows_launch: `rows` as ring_apply_rows takes them (pointers
+ * are looked at for their alignment only, never dereferenced), `role` the
+ * entry point they come from: RING_ROLE_COPY (ring_copy_bytes),
+ * RING_ROLE_ACCUMULATE (accumulates, reduce-scatter tables, row tables) or
+ * RING_ROLE_ALLGATHER (ring_allgather_steps: the only one with a choice).
+ * ring_describe_unpack_launch: a fused buffer of `total_elements` elements in
+ * `n_tensors` non-empty tensors, unpacked with `divisor` (0: no divide).
+ * `cus`: compute units of the GPU (256 on an MI355X). Both answer for the
+ * options currently set (ring_set_option). */
+enum ring_form {
+  RING_FORM_TILES = 0,       /* one workgroup per tile of 16 KiB */
+  RING_FORM_PACED = 1,       /* tiles of 32 KiB: all loads, one wait, then one store in flight per wave */
+  RING_FORM_REGISTERS_2 = 2, /* the launch's payload in registers, two workgroups per CU */
+  RING_FORM_REGISTERS_1 = 3  /* the same, one workgroup per CU (one wave per SIMD, 112 vectors per lane) */
+};
+enum ring_role { RING_ROLE_COPY = 0, RING_ROLE_ACCUMULATE = 1, RING_ROLE_ALLGATHER = 2 };
+int ring_describe_rows_launch(const ring_row* rows, int n_rows, int dtype, int role, int cus, int* form);
+int ring_describe_unpack_launch(uint64_t total_elements, int n_tensors, int dtype, int divisor, int cus,
+                                int* form);
+
+/* Measurement only (no counterpart in the reference): ONE direction of a copy
+ * launch in the tile shape and grid of the step-table kernel. mode 0: every
+ * row's `a` is read (non-temporal loads) and nothing is written; mode 1:
+ * every row's `dst` is written (non-temporal stores) and nothing is read;
+ * modes 2 and 3: the same with the ordinary cache policy. Up to 8 rows;
+ * the pointer used must be 16-byte aligned; counts are rounded down to whole
+ * 16-byte vectors. A copy runs no faster than its two directions one after
+ * the other, so these two launches give the floor of a copy of that shape.
+ * Timed like any other launch (ring_time_next_launch). */
+int ring_probe_stream(const ring_row* rows, int n_rows, int dtype, int mode, void* stream);
 
 /* A segment reduced in one pass. After its n-1 reduce-scatter steps the ring
  * holds in segment s the left fold over the ranks in ring order,
@@ -367,7 +415,15 @@ int ring_fusion_run_static(int unpack, const void* const* tensors, const size_t*
  * straight to the tensors. Elements outside the spans are not touched. Spans
  * must be sorted by `begin` and disjoint; `spans` is a HOST array. Together
  * the two calls do what pack, n-1 accumulates, and unpack do, minus one read
- * and one write of the whole set. */
+ * and one write of the whole set. `incoming` and `out` need only be aligned
+ * to an element. The kernels align their stores; the loads of `incoming` are
+ * aligned too when its 16-byte groups are groups of the fused space, i.e.
+ * when (address of incoming / element size - begin) is a multiple of
+ * 16 / element size, as it is for a segment received in place at
+ * wire + begin (where ring.h:211-225 receives it). A slot that starts at a
+ * fresh allocation instead costs a segment with begin % 4 != 0 about 4 % more
+ * bytes fetched (every 1 KiB a wave loads touches 33 sectors of 32 bytes
+ * instead of 32) and as much time. */
 typedef struct ring_fusion_span {
   uint64_t begin;       /* first element in the fused space */
   uint64_t count;       /* elements */

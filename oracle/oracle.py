@@ -10,6 +10,7 @@ import ctypes
 import json
 import os
 import shutil
+import signal
 import subprocess
 
 import numpy as np
@@ -201,26 +202,44 @@ def mpirun_path():
     return None
 
 
+def _run_mpi(argv, timeout):
+    """mpirun with its proxies and ranks in a process group of their own, which is
+    ended once mpirun has returned (or timed out): nothing it started outlives the call."""
+    proc = subprocess.Popen(argv, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True,
+                            start_new_session=True)
+    try:
+        out, err = proc.communicate(timeout=timeout)
+    except subprocess.TimeoutExpired:
+        proc.kill()
+        proc.communicate()
+        raise
+    finally:
+        try:
+            os.killpg(proc.pid, signal.SIGKILL)   # the group this call created, whatever is left of it
+        except (ProcessLookupError, PermissionError):
+            pass
+    if proc.returncode != 0:
+        raise subprocess.CalledProcessError(proc.returncode, argv, out, err)
+    return out, err
+
+
 def mpi_check(inputs, workdir, timeout=120):
     """Run the per-rank restatement over real MPI; returns the outputs."""
     inputs, code, cnt = _check_inputs(inputs)
     n = len(inputs)
     for r, x in enumerate(inputs):
         x.tofile(os.path.join(workdir, "in_%d.bin" % r))
-    subprocess.run([mpirun_path(), "-np", str(n), _MPI_BIN, "check",
-                    DTYPE_NAME[code], str(cnt), workdir],
-                   check=True, timeout=timeout)
+    _run_mpi([mpirun_path(), "-np", str(n), _MPI_BIN, "check", DTYPE_NAME[code], str(cnt), workdir], timeout)
     return [np.fromfile(os.path.join(workdir, "out_%d.bin" % r), dtype=inputs[0].dtype)
             for r in range(n)]
 
 
 def mpi_time(n, code, count, warmup, reps, timeout=300):
     """Time RingAllreduce over real MPI; returns the parsed JSON line."""
-    out = subprocess.run([mpirun_path(), "-np", str(n), _MPI_BIN, "time",
-                          DTYPE_NAME[code], str(count), str(warmup), str(reps)],
-                         check=True, timeout=timeout, capture_output=True, text=True)
-    for line in out.stdout.splitlines():
+    stdout, stderr = _run_mpi([mpirun_path(), "-np", str(n), _MPI_BIN, "time",
+                               DTYPE_NAME[code], str(count), str(warmup), str(reps)], timeout)
+    for line in stdout.splitlines():
         line = line.strip()
         if line.startswith("{"):
             return json.loads(line)
-    raise RuntimeError("ring_mpi printed no result: " + out.stdout + out.stderr)
+    raise RuntimeError("ring_mpi printed no result: " + stdout + stderr)

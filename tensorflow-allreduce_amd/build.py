@@ -127,24 +127,6 @@ def build_cpp_gpu_test(verbose=True):
     return exe
 
 
-def build_launch_shape_probe(verbose=True):
-    """examples/build/launch_shape_probe: the stand-alone program that times
-    launch shapes of a 56 MiB copy and accumulate (it does not use the library)."""
-    out_dir = os.path.join(HERE, "examples", "build")
-    os.makedirs(out_dir, exist_ok=True)
-    exe = os.path.join(out_dir, "launch_shape_probe")
-    cmd = [hipcc(), "--offload-arch=gfx950", "-O3", "-std=c++17",
-           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
-           "-o", exe, os.path.join(HERE, "examples", "launch_shape_probe.hip")]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
-    if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + out)
-    return exe
-
-
 def build_launch_bound_steps(verbose=True):
     """examples/build/launch_bound_steps: a small tensor's allreduce step driven
     from C++ through the C ABI, eager and as recorded HIP graphs (host clock)."""
@@ -168,7 +150,7 @@ def build_launch_bound_steps(verbose=True):
 
 def build_all(verbose=True):
     return [build_ring_hip(verbose), build_plugin(verbose), build_cpp_gpu_test(verbose),
-            build_launch_shape_probe(verbose), build_launch_bound_steps(verbose)]
+            build_launch_bound_steps(verbose)]
 
 
 if __name__ == "__main__":

@@ -1,11 +1,46 @@
 #include "ring_driver.h"
 
+#include <memory>
 #include <string>
 
 #include "ring_abi.h"
 
 namespace mpic {
 namespace {
+
+// A call's small tables (segment sizes, step rows, pointers): on the stack up
+// to N items, which covers a ring of 64 ranks, on the heap beyond. The driver
+// runs once per collective on the thread that feeds the stream; at small
+// tensors a step costs what that thread spends, and a handful of heap
+// allocations per call were a measurable part of it.
+template <typename T, size_t N>
+class Table {
+ public:
+  explicit Table(size_t capacity) : data_(stack_) {
+    if (capacity > N) {
+      heap_.reset(new T[capacity]);
+      data_ = heap_.get();
+    }
+  }
+  Table(size_t n, const T& fill) : Table(n) {
+    for (size_t i = 0; i < n; i++) data_[i] = fill;
+    size_ = n;
+  }
+  void push_back(const T& v) { data_[size_++] = v; }  // within the capacity given at construction
+  T* data() { return data_; }
+  const T* data() const { return data_; }
+  size_t size() const { return size_; }
+  T& operator[](size_t i) { return data_[i]; }
+  const T& operator[](size_t i) const { return data_[i]; }
+
+ private:
+  T stack_[N];
+  std::unique_ptr<T[]> heap_;
+  T* data_;
+  size_t size_ = 0;
+};
+constexpr size_t kStackRanks = 64;
+constexpr size_t kStackPointers = 256;  // the n x n tables of resident ranks: 16 ranks on the stack
 
 // The reference's MPI_REQUIRES_OK (ring.h:36-39) for the device layer.
 Status FromRing(int rc, const char* what) {
@@ -55,7 +90,7 @@ Status RingAllreducePrestaged(int n, int r, DataType dt, const void* input, void
   if (!input || !output) return errors::InvalidArgument("null tensor with a non-zero element count");
   if (n > 1 && (!rs_recv || !ag_recv)) return errors::InvalidArgument("no staged peer segments");
 
-  std::vector<size_t> sizes(static_cast<size_t>(n)), starts(static_cast<size_t>(n));
+  Table<size_t, kStackRanks> sizes(static_cast<size_t>(n), 0), starts(static_cast<size_t>(n), 0);
   RING_RETURN_IF_ERROR(ring_segment_table(count, n, sizes.data(), starts.data()), "ring_segment_table");
 
   const int divisor = opts.divisor;
@@ -74,12 +109,12 @@ Status RingAllreducePrestaged(int n, int r, DataType dt, const void* input, void
     RING_RETURN_IF_ERROR(ring_copy_bytes(output, input, count * esz, stream), "ring_copy_bytes");
   // the segment whose sum completes at the last step (n-2) is the one this rank
   // owns and sends first in the allgather: the only one it divides
-  std::vector<unsigned char> divide(static_cast<size_t>(n), 0);
+  Table<unsigned char, kStackRanks> divide(static_cast<size_t>(n), 0);
   divide[static_cast<size_t>(n - 2)] = 1;
 
   // ring.h:183-205: step i receives segment (r-i-1) and adds it into the buffer
   if (fuse) {
-    std::vector<ring_row> rows;
+    Table<ring_row, kStackRanks> rows(static_cast<size_t>(n));
     for (int i = 0; i < n - 1; i++) {
       const size_t seg = static_cast<size_t>(Seg(RING_PHASE_REDUCE_SCATTER, n, r, i, true));
       rows.push_back(ring_row{at(output, starts[seg], esz), rs_recv[i], at(input, starts[seg], esz), sizes[seg]});
@@ -91,7 +126,7 @@ Status RingAllreducePrestaged(int n, int r, DataType dt, const void* input, void
                                              code, stream),
                          "ring_apply_rows_avg");
   } else if (opts.batched && divisor > 0) {
-    std::vector<ring_row> rows;
+    Table<ring_row, kStackRanks> rows(static_cast<size_t>(n));
     for (int i = 0; i < n - 1; i++) {
       const size_t seg = static_cast<size_t>(Seg(RING_PHASE_REDUCE_SCATTER, n, r, i, true));
       char* dst = at(output, starts[seg], esz);
@@ -100,7 +135,7 @@ Status RingAllreducePrestaged(int n, int r, DataType dt, const void* input, void
     RING_RETURN_IF_ERROR(ring_apply_rows_avg(rows.data(), n - 1, divide.data(), divisor, code, stream),
                          "ring_apply_rows_avg");
   } else if (opts.batched) {
-    std::vector<ring_step> steps;
+    Table<ring_step, kStackRanks> steps(static_cast<size_t>(n));
     for (int i = 0; i < n - 1; i++) {
       const size_t seg = static_cast<size_t>(Seg(RING_PHASE_REDUCE_SCATTER, n, r, i, true));
       steps.push_back(ring_step{starts[seg], rs_recv[i], sizes[seg]});
@@ -123,7 +158,7 @@ Status RingAllreducePrestaged(int n, int r, DataType dt, const void* input, void
 
   // ring.h:211-225: step i receives segment (r-i) straight into the buffer
   if (opts.batched) {
-    std::vector<ring_step> steps;
+    Table<ring_step, kStackRanks> steps(static_cast<size_t>(n));
     for (int i = 0; i < n - 1; i++) {
       const size_t seg = static_cast<size_t>(Seg(RING_PHASE_ALLGATHER, n, r, i, true));
       steps.push_back(ring_step{starts[seg], ag_recv[i], sizes[seg]});
@@ -156,12 +191,12 @@ Status RingAllreduceDirectPrestaged(int n, int r, DataType dt, const void* input
   if (count == 0) return Status::OK();
   if (!input || !output) return errors::InvalidArgument("null tensor with a non-zero element count");
   if (n > 1 && (!peers || !ag_recv)) return errors::InvalidArgument("no staged peer segments");
-  std::vector<size_t> sizes(static_cast<size_t>(n)), starts(static_cast<size_t>(n));
+  Table<size_t, kStackRanks> sizes(static_cast<size_t>(n), 0), starts(static_cast<size_t>(n), 0);
   RING_RETURN_IF_ERROR(ring_segment_table(count, n, sizes.data(), starts.data()), "ring_segment_table");
 
   // the owned segment: x_s, x_{s+1}, ..., x_{s+n-1} = this rank's own, folded in that order
   const size_t own = static_cast<size_t>((r + 1) % n);
-  std::vector<const void*> srcs;
+  Table<const void*, kStackRanks> srcs(static_cast<size_t>(n));
   for (int k = 0; k < n - 1; k++) {
     if (sizes[own] && !peers[k]) return errors::InvalidArgument("null staged peer segment");
     srcs.push_back(peers[k]);
@@ -169,7 +204,7 @@ Status RingAllreduceDirectPrestaged(int n, int r, DataType dt, const void* input
   srcs.push_back(at(input, starts[own], esz));
   ring_fold_row fold{at(output, starts[own], esz), srcs.data(), sizes[own]};
   // every other segment arrives finished (ring.h:211-225 delivers the same values step by step)
-  std::vector<ring_row> copies;
+  Table<ring_row, kStackRanks> copies(static_cast<size_t>(n));
   for (int i = 0; i < n - 1; i++) {
     const size_t seg = static_cast<size_t>(Seg(RING_PHASE_ALLGATHER, n, r, i, true));
     copies.push_back(ring_row{at(output, starts[seg], esz), ag_recv[i], nullptr, sizes[seg]});
@@ -197,7 +232,7 @@ Status RingAllreduceFusedPrestaged(const ring_fusion_plan* plan, int n, int r, v
   if (!wire) return errors::InvalidArgument("no wire buffer");
   if (n > 1 && (!rs_recv || !ag_recv)) return errors::InvalidArgument("no staged peer segments");
   const size_t esz = ring_dtype_size(code);
-  std::vector<size_t> sizes(static_cast<size_t>(n)), starts(static_cast<size_t>(n));
+  Table<size_t, kStackRanks> sizes(static_cast<size_t>(n), 0), starts(static_cast<size_t>(n), 0);
   RING_RETURN_IF_ERROR(ring_segment_table(count, n, sizes.data(), starts.data()), "ring_segment_table");
 
   const size_t own = static_cast<size_t>((r + 1) % n);
@@ -209,19 +244,19 @@ Status RingAllreduceFusedPrestaged(const ring_fusion_plan* plan, int n, int r, v
     // (packed layout). The rank packs its own copy of that segment into the
     // wire buffer, folds the n copies there in ring order, and scatters the
     // finished segments into the tensors.
-    std::vector<const void*> ag_direct(static_cast<size_t>(n), nullptr);
+    Table<const void*, kStackRanks> ag_direct(static_cast<size_t>(n), nullptr);
     for (int i = 0; i < n - 1; i++)
       ag_direct[static_cast<size_t>(Seg(RING_PHASE_ALLGATHER, n, r, i, true))] = ag_recv[i];
     char* mine = at(wire, starts[own], esz);
     if (n - 1 <= kMaxOneLaunchDirectRanks) {
       // one launch: the owned segment folded from the staged copies and the
       // tensors, its sum left in the wire buffer, everything scattered
-      std::vector<const void*> staged;
+      Table<const void*, kStackRanks> staged(static_cast<size_t>(n));
       for (int k = 0; k < n - 1; k++) {
         if (sizes[own] && !rs_recv[k]) return errors::InvalidArgument("null staged peer segment");
         staged.push_back(rs_recv[k]);
       }
-      std::vector<ring_fusion_span> others;
+      Table<ring_fusion_span, kStackRanks> others(static_cast<size_t>(n));
       for (size_t seg = 0; seg < static_cast<size_t>(n); seg++) {
         if (seg == own) continue;
         if (sizes[seg] && !ag_direct[seg]) return errors::InvalidArgument("null staged peer segment");
@@ -234,7 +269,7 @@ Status RingAllreduceFusedPrestaged(const ring_fusion_plan* plan, int n, int r, v
     }
     ring_fusion_span pack{starts[own], sizes[own], nullptr, mine};
     RING_RETURN_IF_ERROR(ring_fusion_gather(plan, &pack, 1, stream), "ring_fusion_gather");
-    std::vector<const void*> srcs;
+    Table<const void*, kStackRanks> srcs(static_cast<size_t>(n));
     for (int k = 0; k < n - 1; k++) {
       if (sizes[own] && !rs_recv[k]) return errors::InvalidArgument("null staged peer segment");
       srcs.push_back(rs_recv[k]);
@@ -242,7 +277,7 @@ Status RingAllreduceFusedPrestaged(const ring_fusion_plan* plan, int n, int r, v
     srcs.push_back(mine);
     ring_fold_row fold{mine, srcs.data(), sizes[own]};
     RING_RETURN_IF_ERROR(ring_fold_rows(&fold, 1, n, 0, code, stream), "ring_fold_rows");
-    std::vector<ring_fusion_span> finished;
+    Table<ring_fusion_span, kStackRanks> finished(static_cast<size_t>(n));
     for (size_t seg = 0; seg < static_cast<size_t>(n); seg++) {
       const void* from = seg == own ? static_cast<const void*>(mine) : ag_direct[seg];
       if (sizes[seg] && !from) return errors::InvalidArgument("null staged peer segment");
@@ -253,12 +288,12 @@ Status RingAllreduceFusedPrestaged(const ring_fusion_plan* plan, int n, int r, v
   }
 
   // what arrives for each segment in either phase (ring.h:183-205, :211-225)
-  std::vector<const void*> rs_of(static_cast<size_t>(n), nullptr), ag_of(static_cast<size_t>(n), nullptr);
+  Table<const void*, kStackRanks> rs_of(static_cast<size_t>(n), nullptr), ag_of(static_cast<size_t>(n), nullptr);
   for (int i = 0; i < n - 1; i++) {
     rs_of[static_cast<size_t>(Seg(RING_PHASE_REDUCE_SCATTER, n, r, i, true))] = rs_recv[i];
     ag_of[static_cast<size_t>(Seg(RING_PHASE_ALLGATHER, n, r, i, true))] = ag_recv[i];
   }
-  std::vector<ring_fusion_span> gather, scatter;
+  Table<ring_fusion_span, kStackRanks> gather(static_cast<size_t>(n)), scatter(static_cast<size_t>(n));
   for (size_t seg = 0; seg < static_cast<size_t>(n); seg++) {
     // segment r has no arrival in the reduce-scatter: packed, as the first send needs it
     gather.push_back(ring_fusion_span{starts[seg], sizes[seg], rs_of[seg], at(wire, starts[seg], esz)});
@@ -283,7 +318,7 @@ Status RingAllgatherPrestaged(int n, int r, DataType dt, const void* input, cons
   if (n < 1 || r < 0 || r >= n || rows.size() != static_cast<size_t>(n))
     return errors::InvalidArgument("rank or sizes do not match the ring");
   const size_t esz = ring_dtype_size(code);
-  std::vector<size_t> starts(static_cast<size_t>(n));
+  Table<size_t, kStackRanks> starts(static_cast<size_t>(n), 0);
   RING_RETURN_IF_ERROR(ring_allgather_table(rows.data(), n, elems_per_row, starts.data()), "ring_allgather_table");
 
   // ring.h:263-266: own slice to its offset
@@ -295,8 +330,8 @@ Status RingAllgatherPrestaged(int n, int r, DataType dt, const void* input, cons
   // the own-slice copy is one more row of the same launch.
   if (opts.divisor < 0) return errors::InvalidArgument("negative divisor");
   if (opts.batched && opts.divisor > 0) {
-    std::vector<ring_row> table;
-    std::vector<unsigned char> divide(static_cast<size_t>(n), 0);
+    Table<ring_row, kStackRanks> table(static_cast<size_t>(n));
+    Table<unsigned char, kStackRanks> divide(static_cast<size_t>(n), 0);
     divide[0] = 1;  // the own slice; what arrives was divided by its owner
     table.push_back(ring_row{own ? at(output, starts[static_cast<size_t>(r)], esz) : nullptr, input, nullptr, own});
     for (int i = 0; i < n - 1; i++) {
@@ -307,7 +342,7 @@ Status RingAllgatherPrestaged(int n, int r, DataType dt, const void* input, cons
     RING_RETURN_IF_ERROR(ring_apply_rows_avg(table.data(), n, divide.data(), opts.divisor, code, stream),
                          "ring_apply_rows_avg");
   } else if (opts.batched) {
-    std::vector<ring_step> steps;
+    Table<ring_step, kStackRanks> steps(static_cast<size_t>(n));
     steps.push_back(ring_step{starts[static_cast<size_t>(r)], input, own});
     for (int i = 0; i < n - 1; i++) {
       const size_t seg = static_cast<size_t>(Seg(RING_PHASE_GATHER, n, r, i, true));
@@ -340,10 +375,10 @@ Status RingAllreduceAllRanks(int n, DataType dt, const void* const* inputs, void
   if (opts.divisor < 0) return errors::InvalidArgument("negative divisor");
   if (count == 0) return Status::OK();
   const size_t esz = ring_dtype_size(code);
-  std::vector<size_t> sizes(static_cast<size_t>(n)), starts(static_cast<size_t>(n));
+  Table<size_t, kStackRanks> sizes(static_cast<size_t>(n), 0), starts(static_cast<size_t>(n), 0);
   RING_RETURN_IF_ERROR(ring_segment_table(count, n, sizes.data(), starts.data()), "ring_segment_table");
 
-  std::vector<ring_row> rows(static_cast<size_t>(n));
+  Table<ring_row, kStackRanks> rows(static_cast<size_t>(n), ring_row{nullptr, nullptr, nullptr, 0});
   for (int r = 0; r < n; r++)
     if (!inputs[r] || !outputs[r]) return errors::InvalidArgument("null tensor with a non-zero element count");
 
@@ -353,17 +388,18 @@ Status RingAllreduceAllRanks(int n, DataType dt, const void* const* inputs, void
     // One launch for the whole allreduce: the owner of every segment folds the n
     // copies in ring order and stores the result into every rank's output. Rank
     // (seg-1) owns segment seg; its own output leads the destinations.
-    std::vector<std::vector<const void*>> srcs(static_cast<size_t>(n));
-    std::vector<std::vector<void*>> dsts(static_cast<size_t>(n));
-    std::vector<ring_fold_to_all_row> folds;
+    const size_t un = static_cast<size_t>(n);
+    Table<const void*, kStackPointers> srcs(un * un);  // row j's n sources at [j * n, (j + 1) * n)
+    Table<void*, kStackPointers> dsts(un * un);
+    Table<ring_fold_to_all_row, kStackRanks> folds(un);
     for (int j = 0; j < n; j++) {
       const size_t seg = static_cast<size_t>((j + 1) % n);
       for (int k = 0; k < n; k++) {
-        srcs[static_cast<size_t>(j)].push_back(at(inputs[(static_cast<int>(seg) + k) % n], starts[seg], esz));
-        dsts[static_cast<size_t>(j)].push_back(at(outputs[(j + k) % n], starts[seg], esz));
+        srcs.push_back(at(inputs[(static_cast<int>(seg) + k) % n], starts[seg], esz));
+        dsts.push_back(at(outputs[(j + k) % n], starts[seg], esz));
       }
-      folds.push_back(ring_fold_to_all_row{dsts[static_cast<size_t>(j)].data(), srcs[static_cast<size_t>(j)].data(),
-                                           sizes[seg]});
+      folds.push_back(ring_fold_to_all_row{dsts.data() + static_cast<size_t>(j) * un,
+                                           srcs.data() + static_cast<size_t>(j) * un, sizes[seg]});
     }
     if (!(n == 1 && inputs[0] == outputs[0] && opts.divisor == 0))
       RING_RETURN_IF_ERROR(ring_fold_to_all_rows(folds.data(), n, n, n, opts.divisor, code, stream),
@@ -373,17 +409,18 @@ Status RingAllreduceAllRanks(int n, DataType dt, const void* const* inputs, void
   if (opts.direct && n <= kMaxDirectRanks) {
     // More ranks than one row's pointers hold twice over: the owner of every
     // segment folds the n copies in ring order (one launch) ...
-    std::vector<std::vector<const void*>> srcs(static_cast<size_t>(n));
-    std::vector<ring_fold_row> folds;
+    const size_t un = static_cast<size_t>(n);
+    Table<const void*, kStackPointers> srcs(un * un);
+    Table<ring_fold_row, kStackRanks> folds(un);
     for (int j = 0; j < n; j++) {
       const size_t seg = static_cast<size_t>((j + 1) % n);
       for (int k = 0; k < n; k++)
-        srcs[static_cast<size_t>(j)].push_back(at(inputs[(static_cast<int>(seg) + k) % n], starts[seg], esz));
-      folds.push_back(ring_fold_row{at(outputs[j], starts[seg], esz), srcs[static_cast<size_t>(j)].data(), sizes[seg]});
+        srcs.push_back(at(inputs[(static_cast<int>(seg) + k) % n], starts[seg], esz));
+      folds.push_back(ring_fold_row{at(outputs[j], starts[seg], esz), srcs.data() + static_cast<size_t>(j) * un, sizes[seg]});
     }
     RING_RETURN_IF_ERROR(ring_fold_rows(folds.data(), n, n, opts.divisor, code, stream), "ring_fold_rows");
     // ... and every rank copies each finished segment from its owner (one more).
-    std::vector<ring_row> copies;
+    Table<ring_row, kStackPointers> copies(un * un);
     for (int r = 0; r < n; r++) {
       for (int seg = 0; seg < n; seg++) {
         const int owner = (seg - 1 + n) % n;
@@ -452,7 +489,7 @@ Status RingAllgatherAllRanks(int n, DataType dt, const void* const* inputs, cons
   if (!s.ok()) return s;
   if (n < 1 || rows_per_rank.size() != static_cast<size_t>(n)) return errors::InvalidArgument("sizes do not match the ring");
   const size_t esz = ring_dtype_size(code);
-  std::vector<size_t> starts(static_cast<size_t>(n));
+  Table<size_t, kStackRanks> starts(static_cast<size_t>(n), 0);
   RING_RETURN_IF_ERROR(ring_allgather_table(rows_per_rank.data(), n, elems_per_row, starts.data()), "ring_allgather_table");
 
   if (opts.direct) {
@@ -460,7 +497,7 @@ Status RingAllgatherAllRanks(int n, DataType dt, const void* const* inputs, cons
     // launch: the values a ring allgather delivers after n-1 steps (it only
     // moves bytes). A divisor divides every copy, which gives each rank what
     // the owner's one division would have sent round.
-    std::vector<ring_row> all;
+    Table<ring_row, kStackPointers> all(static_cast<size_t>(n) * static_cast<size_t>(n));
     for (int r = 0; r < n; r++) {
       for (int k = 0; k < n; k++) {
         const size_t cnt = elems_per_row * rows_per_rank[static_cast<size_t>(k)];
@@ -475,7 +512,7 @@ Status RingAllgatherAllRanks(int n, DataType dt, const void* const* inputs, cons
     return Status::OK();
   }
 
-  std::vector<ring_row> rows(static_cast<size_t>(n));
+  Table<ring_row, kStackRanks> rows(static_cast<size_t>(n), ring_row{nullptr, nullptr, nullptr, 0});
   for (int r = 0; r < n; r++) {  // ring.h:263-266
     const size_t own = elems_per_row * rows_per_rank[static_cast<size_t>(r)];
     if (own && (!inputs[r] || !outputs[r])) return errors::InvalidArgument("null tensor with a non-zero element count");

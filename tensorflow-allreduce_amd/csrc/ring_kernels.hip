@@ -47,6 +47,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <atomic>
 #include <mutex>
 #include <new>
 #include <type_traits>
@@ -527,6 +528,42 @@ __global__ void __launch_bounds__(kBlock) bytes_kernel(uint8_t* __restrict__ dst
   for (uint64_t i = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x; i < n;
        i += static_cast<uint64_t>(gridDim.x) * kBlock)
     dst[i] = src[i];
+}
+
+// Measurement only (ring_probe_stream): ONE direction of a copy launch, in the
+// tile shape of rows_kernel (256 lanes x 4 vectors of 16 bytes, one workgroup
+// per tile, grid (tiles, rows)): every lane loads its four vectors and stores
+// nothing, or stores four vectors and loads nothing. What the chip gives one
+// direction at a given size is the floor of a copy of that size, which runs no
+// faster than its two directions one after the other. count: 16-byte vectors.
+template <int WRITE, int NT>
+__global__ void __launch_bounds__(kBlock) stream_probe_kernel(const SmallRowTable tab) {
+  typedef VecOf<uint32_t>::type V;
+  typedef V RING_GLOBAL GV;
+  const Row r = tab.row[blockIdx.y];
+  const uint64_t base = static_cast<uint64_t>(blockIdx.x) * (kBlock * 4);
+  if (base >= r.count) return;
+  const uint64_t left = r.count - base;
+  const uint32_t tid = threadIdx.x;
+  if (WRITE) {
+    GV* d = (GV*)static_cast<uint32_t*>(r.dst) + base;
+    const V v = {1u, 2u, 3u, tid};
+#pragma unroll
+    for (uint32_t j = 0; j < 4; j++)
+      if (tid + j * kBlock < left) RING_STORE_VEC(NT ? 1 : 0, &d[tid + j * kBlock], v);
+  } else {
+    const GV* a = (const GV*)static_cast<const uint32_t*>(r.a) + base;
+    V x[4];
+#pragma unroll
+    for (uint32_t j = 0; j < 4; j++) {
+      x[j] = V{0u, 0u, 0u, 0u};
+      if (tid + j * kBlock < left) x[j] = RING_LOAD_VEC(NT ? 2 : 0, &a[tid + j * kBlock]);
+    }
+    const V acc = x[0] ^ x[1] ^ x[2] ^ x[3];
+    // keeps the loads alive; four given words out of 2^128, and then the store goes where the loads came from
+    if (acc[0] == 0x9e3779b9u && acc[1] == 0x7f4a7c15u && acc[2] == 0xf39cc060u && acc[3] == 0x5cedc834u)
+      ((GV*)static_cast<const uint32_t*>(r.a))[base + tid] = acc;
+  }
 }
 
 // ---- fold: a segment reduced in one pass, in ring order ---------------------------
@@ -1288,6 +1325,7 @@ enum Role {
   kRoleCopy, kRoleAccumulate, kRoleAllgather, kRolePack, kRoleUnpack, kRoleFold, kRoleBroadcast, kRoleFoldAll, kRoles
 };
 
+// Launch options (ring_set_option), as one launch sees them: a snapshot.
 struct Tuning {
   int unroll = 4;          // 16-byte vectors per lane per tile: 2, 4 or 8
   // Cache policy per role; bit 0: non-temporal stores, bit 1: non-temporal
@@ -1312,8 +1350,41 @@ struct Tuning {
   int phased_copy = -1;
   int blocks_per_cu = 0;   // 0: one workgroup per tile; >0: persistent grid of CUs x this
   int dry_launch = 0;      // measurement only: the step-table kernels return at entry (what a launch of that grid costs)
+  int flat_grid = 0;       // measurement only: rows of equal tile counts share the 1-D grid of unequal rows instead of (tiles, rows)
 };
-Tuning g_tuning;
+
+// Where the options live: one atomic cell each, so that ring_set_option on one
+// thread and launches on others (one thread per rank drives its own stream)
+// are no data race. A launch reads them once, at entry (tuning()), and works
+// on that snapshot; an option set while a launch is being prepared applies to
+// that launch or to the next one.
+enum OptionCell { kCellUnroll, kCellPaced, kCellPhased, kCellBlocksPerCu, kCellDry, kCellFlat, kCellNt, kCells = kCellNt + kRoles };
+struct OptionCells {
+  std::atomic<int> v[kCells];
+  OptionCells() { store(Tuning()); }
+  void store(const Tuning& t) {
+    v[kCellUnroll].store(t.unroll, std::memory_order_relaxed);
+    v[kCellPaced].store(t.paced_copy, std::memory_order_relaxed);
+    v[kCellPhased].store(t.phased_copy, std::memory_order_relaxed);
+    v[kCellBlocksPerCu].store(t.blocks_per_cu, std::memory_order_relaxed);
+    v[kCellDry].store(t.dry_launch, std::memory_order_relaxed);
+    v[kCellFlat].store(t.flat_grid, std::memory_order_relaxed);
+    for (int r = 0; r < kRoles; r++) v[kCellNt + r].store(t.nt[r], std::memory_order_relaxed);
+  }
+};
+OptionCells g_options;
+
+inline Tuning tuning() {
+  Tuning t;
+  t.unroll = g_options.v[kCellUnroll].load(std::memory_order_relaxed);
+  t.paced_copy = g_options.v[kCellPaced].load(std::memory_order_relaxed);
+  t.phased_copy = g_options.v[kCellPhased].load(std::memory_order_relaxed);
+  t.blocks_per_cu = g_options.v[kCellBlocksPerCu].load(std::memory_order_relaxed);
+  t.dry_launch = g_options.v[kCellDry].load(std::memory_order_relaxed);
+  t.flat_grid = g_options.v[kCellFlat].load(std::memory_order_relaxed);
+  for (int r = 0; r < kRoles; r++) t.nt[r] = g_options.v[kCellNt + r].load(std::memory_order_relaxed);
+  return t;
+}
 
 struct DeviceInfo {
   bool ok = false;
@@ -1406,81 +1477,129 @@ struct HostRow {
   bool divide;     // with a divisor: this row also divides
 };
 
+// ---- which form a launch of copy rows takes ----------------------------------------------
+// The thresholds, in one place. All of them are per CU, so that they scale
+// with the chip; they were measured on the 256 CUs of an MI355X, where
+// 4 KiB per CU are 1 MiB.
+//
+// The paced tiles: every tile of the launch on the chip at the same time (at
+// most 7 workgroups per CU of 32 KiB tiles, 56 MiB per side on 256 CUs) and the
+// launch large enough to be bound by memory rather than by its dispatch (2 per
+// CU). Measured on 7 rows: 21-56 MiB per side 1-10 % faster than the plain
+// tiles (56 MiB: 19.6 against 20.8 us), slower beyond (63 MiB: 25.3 against
+// 23.7 us) and no different below.
+constexpr uint64_t kPacedMinTilesPerCu = 2;
+constexpr uint64_t kPacedMaxTilesPerCu = 7;
+// The payload in registers (rows_phased_kernel). The chip's registers hold
+// 112 MiB as one workgroup per CU; up to 224 KiB per side per CU (56 MiB, where
+// the 7 paced tiles per CU end) the launch runs as TWO workgroups per CU with
+// fewer vectors per lane each (a few rounds of one wave per SIMD keep too
+// little in flight). By itself the launcher takes the form above that size,
+// and from 124 KiB per CU (31 MiB; 5 ragged rows of 6.4 MiB: 11.7 against
+// 12.7 us paced; at 28 MiB the paced tiles win, 10.2 against 11.2) unless the
+// paced tiles fill the chip exactly (a whole number of 32 KiB tiles per CU),
+// which is their best case and beats this form by 3-4 % (7 x 8 MiB: 19.7
+// against 20.4 us); with a CU or more left over they lose 3-8 % to it
+// (7 x 7.5 MiB: 19.6 against 18.1 us). Not on chips of fewer than 128 CUs,
+// where none of this was measured.
+constexpr uint64_t kRegistersOnePerCuAbove = 224u << 10;
+constexpr uint64_t kRegistersTwoPerCuFrom = 124u << 10;
+constexpr int kRegistersMinCus = 128;
+
+struct RowsChoice {
+  int form;           // RING_FORM_*
+  PhasedShape shape;  // the forms in registers: rounds, and the workgroup that starts each row
+};
+
+// The form of one launch of `rows` (what launch_rows was handed: rows of `esz`-byte
+// elements for `role`), from the shape of the launch, the options and the
+// number of CUs alone. Only the copies of an allgather phase have a choice.
+RowsChoice choose_rows_form(const HostRow* rows, size_t n_rows, size_t esz, Role role, int divisor, int nt,
+                            const Tuning& tun, int cus) {
+  RowsChoice c;
+  c.form = RING_FORM_TILES;
+  c.shape.rounds = 0;
+  for (int k = 0; k < kSmallRows; k++) c.shape.shift[k] = 0;
+  if (role != kRoleAllgather || divisor > 0 || n_rows < 1 || cus < 1) return c;
+  const uint64_t vec = 16 / esz, ucus = static_cast<uint64_t>(cus);
+  bool copies = true;           // no row has a second operand (empty rows aside)
+  bool copies_not_empty = true;  // and none is empty
+  uint64_t bytes = 0, paced_tiles = 0;
+  for (size_t k = 0; k < n_rows; k++) {
+    const bool empty = rows[k].count == 0;
+    copies = copies && (rows[k].b == nullptr || empty);
+    copies_not_empty = copies_not_empty && rows[k].b == nullptr && !empty;
+    bytes += rows[k].count * esz;
+    paced_tiles += (rows[k].count / vec + kBlock * kPacedUnroll - 1) / (kBlock * kPacedUnroll);
+  }
+  // In registers: up to kSmallRows rows, each within its share of a lane's vectors, non-temporal both ways.
+  if (n_rows <= static_cast<size_t>(kSmallRows) && (nt & 3) == 3 && tun.phased_copy != 0 && tun.blocks_per_cu == 0 &&
+      copies_not_empty) {
+    const uint64_t per_cu = bytes / ucus;
+    const int waves = per_cu > kRegistersOnePerCuAbove ? 1 : 2;
+    const uint64_t wgs = ucus * waves, stride = wgs * kBlock;
+    const uint64_t room = static_cast<uint64_t>((waves == 1 ? kPhasedMax : kPhasedMaxTwoWaves) / static_cast<int>(n_rows));
+    PhasedShape shape = c.shape;
+    uint64_t start = 0;
+    bool fits = room >= 1;
+    for (size_t k = 0; k < n_rows && fits; k++) {
+      const HostRow& r = rows[k];
+      const uintptr_t d = reinterpret_cast<uintptr_t>(r.dst);
+      uint64_t head = ((kRowHeadAlign - (d & (kRowHeadAlign - 1))) & (kRowHeadAlign - 1)) / esz;
+      if (head > r.count) head = r.count;
+      const uint64_t nvec = (r.count - head) / vec;
+      const uint64_t rounds = (nvec + stride - 1) / stride;
+      if (rounds > room) { fits = false; break; }
+      if (rounds > shape.rounds) shape.rounds = static_cast<uint32_t>(rounds);
+      shape.shift[k] = static_cast<uint32_t>(start);
+      // the next row starts behind the last workgroup of this row's last round
+      start = (start + (nvec % stride + kBlock - 1) / kBlock) % wgs;
+    }
+    bool by_itself = per_cu > kRegistersOnePerCuAbove;
+    if (!by_itself && per_cu >= kRegistersTwoPerCuFrom) by_itself = paced_tiles % ucus != 0;
+    if (fits && (tun.phased_copy > 0 || (by_itself && cus >= kRegistersMinCus))) {
+      c.form = waves == 1 ? RING_FORM_REGISTERS_1 : RING_FORM_REGISTERS_2;
+      c.shape = shape;
+      return c;
+    }
+  }
+  if (n_rows <= static_cast<size_t>(kMaxRows) && tun.paced_copy != 0 && copies &&
+      (tun.paced_copy > 0 || (tun.blocks_per_cu == 0 && paced_tiles >= kPacedMinTilesPerCu * ucus &&
+                              paced_tiles <= kPacedMaxTilesPerCu * ucus)))
+    c.form = RING_FORM_PACED;
+  return c;
+}
+
 // Launches rows (any number) in groups of kMaxRows. esz: 4 or 8. A table with
 // no add row runs the copy-only kernel.
 // divisor > 0: rows marked `divide` also divide by it (kAvg) and the element
 // type is signed.
 int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, hipStream_t stream,
                 Role role, int divisor = 0) {
-  int nt = g_tuning.nt[role];
+  const Tuning tun = tuning();
+  int nt = tun.nt[role];
   if (nt < 0) {
     uint64_t bytes = 0;
     for (size_t k = 0; k < n_rows; k++) bytes += rows[k].count * esz;
     nt = bytes <= kCacheResidentBytes ? 0 : 2;
   }
-  int unroll = (g_tuning.unroll == 2 || g_tuning.unroll == 8) ? g_tuning.unroll : 4;
+  int unroll = (tun.unroll == 2 || tun.unroll == 8) ? tun.unroll : 4;
   const uint64_t vec = 16 / esz;
   DeviceInfo info;
-  // The paced form for the copies of an allgather phase, where every tile of
-  // the launch is on the chip at the same time (at most 7 workgroups per CU
-  // of 32 KiB tiles, 56 MiB on 256 CUs) and the launch is large enough to be
-  // bound by memory rather than by its dispatch (2 per CU). Measured on 7 rows:
-  // 21-56 MiB per side 1-10 % faster than the plain tiles (56 MiB: 19.6 against
-  // 20.8 us), slower beyond (63 MiB: 25.3 against 23.7 us) and no different below.
-  // The copies of an allgather phase with the whole payload in registers
-  // between one read phase and one write phase (rows_phased_kernel): up to
-  // kSmallRows rows, each within its share of the registers, non-temporal both
-  // ways.
-  if (role == kRoleAllgather && divisor <= 0 && n_rows >= 1 && n_rows <= static_cast<size_t>(kSmallRows) &&
-      (nt & 3) == 3 && g_tuning.phased_copy != 0 && g_tuning.blocks_per_cu == 0) {
+  bool paced = false;
+  if (role == kRoleAllgather && divisor <= 0 && n_rows >= 1) {
     int rc = device_info(&info);
     if (rc != RING_OK) return rc;
-    SmallRowTable tab;
-    PhasedShape shape;
-    uint64_t bytes = 0;
-    for (size_t k = 0; k < n_rows; k++) bytes += rows[k].count * esz;
-    // The chip's registers hold 112 MiB either way; up to 56 MiB the launch runs as two workgroups per CU
-    // with half the vectors per lane each (a few rounds of one wave per SIMD keep too little in flight).
-    // (sizes per CU: 224 KiB per CU are the 56 MiB of 256 CUs, the 7 tiles of 32 KiB the paced form ends at)
-    const uint64_t per_cu = bytes / static_cast<uint64_t>(info.cus);
-    const int waves = per_cu > (224u << 10) ? 1 : 2;
-    const uint64_t wgs = static_cast<uint64_t>(info.cus) * waves, stride = wgs * kBlock;
-    const uint64_t room = static_cast<uint64_t>((waves == 1 ? kPhasedMax : kPhasedMaxTwoWaves) / static_cast<int>(n_rows));
-    shape.rounds = 0;
-    uint64_t start = 0;
-    bool fits = room >= 1;
-    for (size_t k = 0; k < static_cast<size_t>(kSmallRows); k++) {
-      shape.shift[k] = 0;
-      tab.row[k] = Row{nullptr, nullptr, nullptr, 0};
-      if (k >= n_rows || !fits) continue;
-      const HostRow& r = rows[k];
-      if (r.b != nullptr || r.count == 0) { fits = false; continue; }
-      const uintptr_t d = reinterpret_cast<uintptr_t>(r.dst);
-      uint64_t head = ((kRowHeadAlign - (d & (kRowHeadAlign - 1))) & (kRowHeadAlign - 1)) / esz;
-      if (head > r.count) head = r.count;
-      const uint64_t nvec = (r.count - head) / vec;
-      const uint64_t rounds = (nvec + stride - 1) / stride;
-      if (rounds > room) { fits = false; continue; }
-      if (rounds > shape.rounds) shape.rounds = static_cast<uint32_t>(rounds);
-      tab.row[k] = Row{r.dst, r.a, nullptr, r.count};
-      shape.shift[k] = static_cast<uint32_t>(start);
-      // the next row starts behind the last workgroup of this row's last round
-      start = (start + (nvec % stride + kBlock - 1) / kBlock) % wgs;
-    }
-    // By itself: above 56 MiB per side (one workgroup per CU), and from 31 MiB (two per CU; 5 ragged rows
-    // of 6.4 MiB: 11.7 against 12.7 us paced; at 28 MiB the paced tiles win, 10.2 against 11.2) unless the
-    // paced tiles fill the chip exactly (a whole number of 32 KiB tiles per CU), which is their best case
-    // and beats this form by 3-4 % (7 x 8 MiB: 19.7 against 20.4 us); with a CU or more left over they
-    // lose 3-8 % to it (7 x 7.5 MiB: 19.6 against 18.1 us).
-    bool by_itself = per_cu > (224u << 10);
-    if (!by_itself && per_cu >= (124u << 10)) {
-      uint64_t paced_tiles = 0;
-      for (size_t k = 0; k < n_rows; k++) paced_tiles += (rows[k].count / vec + kBlock * kPacedUnroll - 1) / (kBlock * kPacedUnroll);
-      by_itself = paced_tiles % static_cast<uint64_t>(info.cus) != 0;
-    }
-    if (fits && (g_tuning.phased_copy > 0 || (by_itself && info.cus >= 128))) {
+    const RowsChoice choice = choose_rows_form(rows, n_rows, esz, role, divisor, nt, tun, info.cus);
+    if (choice.form == RING_FORM_REGISTERS_1 || choice.form == RING_FORM_REGISTERS_2) {
+      const int waves = choice.form == RING_FORM_REGISTERS_1 ? 1 : 2;
+      const uint64_t wgs = static_cast<uint64_t>(info.cus) * waves;
+      SmallRowTable tab;
+      for (size_t k = 0; k < static_cast<size_t>(kSmallRows); k++)
+        tab.row[k] = k < n_rows ? Row{rows[k].dst, rows[k].a, nullptr, rows[k].count} : Row{nullptr, nullptr, nullptr, 0};
+      const PhasedShape shape = choice.shape;
       tab.n_rows = static_cast<int>(n_rows);
-      tab.dry = g_tuning.dry_launch;
+      tab.dry = tun.dry_launch;
       tab.uniform_tiles = 0;
       tab.divisor = 0;
       tab.div_mask = 0;
@@ -1506,23 +1625,7 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
       RING_HIP(hipGetLastError());
       return RING_OK;
     }
-  }
-  bool paced = false;
-  if (role == kRoleAllgather && divisor <= 0 && n_rows <= static_cast<size_t>(kMaxRows) && g_tuning.paced_copy != 0) {
-    bool copy_only = true;
-    uint64_t tiles = 0;
-    for (size_t k = 0; k < n_rows; k++) {
-      copy_only = copy_only && (rows[k].b == nullptr || rows[k].count == 0);
-      tiles += (rows[k].count / vec + kBlock * kPacedUnroll - 1) / (kBlock * kPacedUnroll);
-    }
-    if (copy_only && g_tuning.paced_copy > 0) {
-      paced = true;
-    } else if (copy_only && g_tuning.blocks_per_cu == 0) {
-      int rc = device_info(&info);
-      if (rc != RING_OK) return rc;
-      const uint64_t cus = static_cast<uint64_t>(info.cus);
-      paced = tiles >= 2 * cus && tiles <= 7 * cus;
-    }
+    paced = choice.form == RING_FORM_PACED;
   }
   if (paced) unroll = kPacedUnroll;
   const uint64_t tile_vecs = static_cast<uint64_t>(kBlock) * unroll;
@@ -1530,7 +1633,7 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
   while (i < n_rows) {
     RowTable tab;
     tab.n_rows = 0;
-    tab.dry = g_tuning.dry_launch;
+    tab.dry = tun.dry_launch;
     tab.divisor = divisor;
     tab.div_mask = 0;
     tab.tile_begin[0] = 0;
@@ -1563,13 +1666,13 @@ int launch_rows(const HostRow* rows, size_t n_rows, size_t esz, bool is_float, h
     }
     if (tab.n_rows == 0) continue;
     uint64_t cap = tiles;
-    if (g_tuning.blocks_per_cu > 0) {
+    if (tun.blocks_per_cu > 0) {
       int rc = device_info(&info);
       if (rc != RING_OK) return rc;
-      cap = static_cast<uint64_t>(info.cus) * g_tuning.blocks_per_cu;
+      cap = static_cast<uint64_t>(info.cus) * tun.blocks_per_cu;
     }
     dim3 grid;
-    if (uniform && tab.n_rows <= 65535) {
+    if (uniform && !tun.flat_grid && tab.n_rows <= 65535) {
       uint64_t per_row = cap / static_cast<uint64_t>(tab.n_rows);
       if (per_row < 1) per_row = 1;
       if (per_row > first_tiles) per_row = first_tiles;
@@ -1666,68 +1769,87 @@ inline FusionView view_of(const ring_fusion_plan* p) {
   return FusionView{p->dtype, p->esz, p->ntiles, p->total, p->d_offsets, p->d_ptrs, p->d_tiles, p->m};
 }
 
-// Bytes of the fused buffer per CU: from where the unpack holds its payload in registers by itself (1 MiB on
-// 256 CUs), and up to where it runs as two workgroups per CU (75 MiB on 256 CUs).
+// ---- which form an unpack takes -------------------------------------------------------
+// The unpack with the payload in registers (unpack_phased_kernel), by itself from 4 KiB of the fused buffer
+// per CU (1 MiB on 256 CUs) up to what the registers hold. Measured behind the allgather that wrote the
+// buffer, float32, sets of 79-155 tensors, against the tiles: 2-12 MiB 4.4-5.8 us against 6.7-7.8; 24 MiB
+// 10.0 / 13.4; 40 MiB 16.1 / 18.3; 56 MiB 23.0 / 24.3 (two workgroups per CU); 80 MiB 31.4 / 32.9 and 97 MiB
+// 34.8 / 39.4 (one per CU). Between the two, the form with two workgroups per CU holds up to 80 MiB and is
+// the better one up to 72 (64 MiB: 26.4 against 27.7 as one workgroup per CU and 27.0 as tiles; 80 MiB: 33.4
+// against 31.4): two per CU up to 300 KiB per CU (75 MiB).
+// float32 by a divisor that is no power of two: the IEEE division in the kernel, as two workgroups per CU
+// only (with 112 rounds to unroll the division makes the body too large for the compiler to keep the payload
+// in registers) and up to 256 KiB per CU (64 MiB; by 6, behind the allgather: 4 MiB 5.4 against 7.2 us as
+// tiles, 32 MiB 13.1 / 15.5, 64 MiB 26.1 / 27.2, 72 MiB 30.1 / 28.9); beyond, and for the integer types
+// (floor division), the tiles.
 constexpr uint64_t kUnpackPhasedMinPerCu = 4u << 10;
 constexpr uint64_t kUnpackTwoWorkgroupsMaxPerCu = 300u << 10;
+constexpr uint64_t kUnpackDivideMaxPerCu = 256u << 10;
+
+struct UnpackChoice {
+  int form;         // RING_FORM_TILES, RING_FORM_REGISTERS_1 or RING_FORM_REGISTERS_2
+  uint32_t rounds;  // the forms in registers: 16-byte groups per lane
+};
+
+// total: elements of the fused buffer; m: non-empty tensors; divisor 0: no divide.
+UnpackChoice choose_unpack_form(uint64_t total, uint32_t m, size_t esz, bool is_float, int divisor, const Tuning& tun,
+                                int cus) {
+  UnpackChoice c{RING_FORM_TILES, 0};
+  const bool power_of_two = divisor <= 0 || (divisor & (divisor - 1)) == 0;
+  if (tun.phased_copy == 0 || tun.blocks_per_cu != 0 || (tun.nt[kRoleUnpack] & 3) != 3 || m > kUnpackPhasedTensors ||
+      cus < 1 || !(power_of_two || is_float))
+    return c;
+  const uint64_t per_cu = total * esz / static_cast<uint64_t>(cus);
+  const int waves = per_cu > kUnpackTwoWorkgroupsMaxPerCu ? 1 : 2;
+  const uint64_t stride = static_cast<uint64_t>(cus) * waves * kBlock;
+  const uint64_t rounds = (total / (16 / esz) + stride - 1) / stride;
+  if (rounds < 1 || rounds > static_cast<uint64_t>(waves == 1 ? kPhasedMax : kPhasedMaxTwoWaves)) return c;
+  if (!(tun.phased_copy > 0 || (per_cu >= kUnpackPhasedMinPerCu && cus >= kRegistersMinCus))) return c;
+  if (!power_of_two && !(waves == 2 && (tun.phased_copy > 0 || per_cu <= kUnpackDivideMaxPerCu))) return c;
+  c.form = waves == 1 ? RING_FORM_REGISTERS_1 : RING_FORM_REGISTERS_2;
+  c.rounds = static_cast<uint32_t>(rounds);
+  return c;
+}
 
 template <typename T, bool PACK, bool DIV>
 int launch_fusion(const FusionView& p, void* fused, hipStream_t stream, int divisor) {
-  // The unpack with the payload in registers (unpack_phased_kernel), by itself from 1 MiB up to what the
-  // registers hold. Measured behind the allgather that wrote the buffer, float32, sets of 79-155 tensors,
-  // against the tiles: 2-12 MiB 4.4-5.8 us against 6.7-7.8; 24 MiB 10.0 / 13.4; 40 MiB 16.1 / 18.3;
-  // 56 MiB 23.0 / 24.3 (two workgroups per CU); 80 MiB 31.4 / 32.9 and 97 MiB 34.8 / 39.4 (one per CU).
-  // Between the two, the form with two workgroups per CU holds up to 80 MiB and is the better one up to 72
-  // (64 MiB: 26.4 against 27.7 as one workgroup per CU and 27.0 as tiles; 80 MiB: 33.4 against 31.4).
-  if (!PACK && g_tuning.phased_copy != 0 && g_tuning.blocks_per_cu == 0 && (g_tuning.nt[kRoleUnpack] & 3) == 3 &&
-      p.m <= kUnpackPhasedTensors && (!DIV || (divisor & (divisor - 1)) == 0 || std::is_floating_point<T>::value)) {
+  const Tuning tun = tuning();
+  if (!PACK) {
     DeviceInfo info;
     int rc = device_info(&info);
     if (rc != RING_OK) return rc;
-    const uint64_t per_cu = p.total * sizeof(T) / static_cast<uint64_t>(info.cus);
-    const int waves = per_cu > kUnpackTwoWorkgroupsMaxPerCu ? 1 : 2;
-    const uint64_t wgs = static_cast<uint64_t>(info.cus) * waves, stride = wgs * kBlock;
-    const uint64_t nvec = p.total / (16 / sizeof(T));
-    const uint64_t rounds = (nvec + stride - 1) / stride;
-    if (rounds >= 1 && rounds <= static_cast<uint64_t>(waves == 1 ? kPhasedMax : kPhasedMaxTwoWaves) &&
-        (g_tuning.phased_copy > 0 || (per_cu >= kUnpackPhasedMinPerCu && info.cus >= 128))) {
+    const UnpackChoice choice = choose_unpack_form(p.total, p.m, sizeof(T), std::is_floating_point<T>::value,
+                                                   DIV ? divisor : 0, tun, info.cus);
+    if (choice.form != RING_FORM_TILES) {
+      const int waves = choice.form == RING_FORM_REGISTERS_1 ? 1 : 2;
+      const uint64_t wgs = static_cast<uint64_t>(info.cus) * waves;
 #define RING_UNPACK_PHASED(D, W)                                                                              \
   launch(unpack_phased_kernel<T, D, W>, dim3(static_cast<uint32_t>(wgs)), dim3(kBlock), stream,               \
          static_cast<const T*>(fused), p.offsets, reinterpret_cast<T* const*>(p.ptrs), p.tiles, p.m, p.total, \
-         static_cast<uint32_t>(rounds), divisor)
+         choice.rounds, divisor)
       constexpr int kPowerOfTwo = DIV ? 1 : 0;
-      bool launched = true;
       if (!DIV || (divisor & (divisor - 1)) == 0) {
         if (waves == 1) RING_UNPACK_PHASED(kPowerOfTwo, 1); else RING_UNPACK_PHASED(kPowerOfTwo, 2);
       } else if constexpr (DIV && std::is_floating_point<T>::value) {
-        // float32 by any other divisor: the IEEE division in the kernel, as two workgroups per CU only
-        // (with 112 rounds to unroll the division makes the body too large for the compiler to keep the
-        // payload in registers) and up to 64 MiB (by 6, behind the allgather: 4 MiB 5.4 against 7.2 us as
-        // tiles, 32 MiB 13.1 / 15.5, 64 MiB 26.1 / 27.2, 72 MiB 30.1 / 28.9); beyond, the tiles
-        if (waves == 2 && (g_tuning.phased_copy > 0 || per_cu <= (256u << 10))) RING_UNPACK_PHASED(2, 2);
-        else launched = false;
-      } else {
-        launched = false;
+        RING_UNPACK_PHASED(2, 2);  // choose_unpack_form gives this divisor the form with two workgroups per CU only
       }
 #undef RING_UNPACK_PHASED
-      if (launched) {
-        RING_HIP(hipGetLastError());
-        return RING_OK;
-      }
+      RING_HIP(hipGetLastError());
+      return RING_OK;
     }
   }
   uint32_t grid = p.ntiles;
-  if (g_tuning.blocks_per_cu > 0) {
+  if (tun.blocks_per_cu > 0) {
     DeviceInfo info;
     int rc = device_info(&info);
     if (rc != RING_OK) return rc;
-    const uint64_t cap = static_cast<uint64_t>(info.cus) * g_tuning.blocks_per_cu;
+    const uint64_t cap = static_cast<uint64_t>(info.cus) * tun.blocks_per_cu;
     if (grid > cap) grid = static_cast<uint32_t>(cap);
   }
 #define RING_FUSION(N)                                                                                   \
   launch(fusion_kernel<T, PACK, N, DIV>, dim3(grid), dim3(kBlock), stream, static_cast<T*>(fused),       \
          p.offsets, reinterpret_cast<T* const*>(p.ptrs), p.tiles, p.ntiles, p.total, divisor)
-  int nt = g_tuning.nt[PACK ? kRolePack : kRoleUnpack];
+  int nt = tun.nt[PACK ? kRolePack : kRoleUnpack];
   if (nt < 0) nt = 2;
   switch (nt & 3) {
     case 0: RING_FUSION(0); break;
@@ -1875,18 +1997,20 @@ size_t ring_dtype_size(int dtype) { return dtype_size(dtype); }
 // "nontemporal" (bit 0 stores, bit 1 loads; sets every role) and
 // "nontemporal_copy" / "_accumulate" / "_allgather" / "_pack" / "_unpack",
 // "paced_copy" and "phased_copy" (the two forms of the allgather copies that
-// read first and write after: -1 by size, 0 never, 1 always), "dry_launch".
+// read first and write after: -1 by size, 0 never, 1 always), "dry_launch",
+// "flat_grid".
 int ring_set_option(const char* name, int value) {
   if (!name) return RING_ERR_ARGUMENT;
+  auto set = [](int cell, int v) { g_options.v[cell].store(v, std::memory_order_relaxed); };
   if (!strcmp(name, "unroll")) {
     if (value != 2 && value != 4 && value != 8) return RING_ERR_ARGUMENT;
-    g_tuning.unroll = value;
+    set(kCellUnroll, value);
   } else if (!strcmp(name, "paced_copy")) {
     if (value < -1 || value > 1) return RING_ERR_ARGUMENT;
-    g_tuning.paced_copy = value;
+    set(kCellPaced, value);
   } else if (!strcmp(name, "phased_copy")) {
     if (value < -1 || value > 1) return RING_ERR_ARGUMENT;
-    g_tuning.phased_copy = value;
+    set(kCellPhased, value);
   } else if (!strncmp(name, "nontemporal", 11)) {
     static const char* const kSuffix[kRoles] = {"_copy", "_accumulate", "_allgather", "_pack", "_unpack",
                                                 "_fold", "_broadcast", "_fold_all"};
@@ -1895,19 +2019,53 @@ int ring_set_option(const char* name, int value) {
     bool known = name[11] == 0;
     for (int r = 0; r < kRoles; r++) {
       if (name[11] == 0 || !strcmp(name + 11, kSuffix[r])) {
-        g_tuning.nt[r] = value < 0 ? defaults.nt[r] : value;  // -1: back to the default
+        set(kCellNt + r, value < 0 ? defaults.nt[r] : value);  // -1: back to the default
         known = true;
       }
     }
     if (!known) return RING_ERR_ARGUMENT;
   } else if (!strcmp(name, "blocks_per_cu")) {
     if (value < 0 || value > 64) return RING_ERR_ARGUMENT;
-    g_tuning.blocks_per_cu = value;
+    set(kCellBlocksPerCu, value);
   } else if (!strcmp(name, "dry_launch")) {
-    g_tuning.dry_launch = value != 0;
+    set(kCellDry, value != 0);
+  } else if (!strcmp(name, "flat_grid")) {
+    set(kCellFlat, value != 0);
   } else {
     return RING_ERR_ARGUMENT;
   }
+  return RING_OK;
+}
+
+// ---- which form a launch takes, as a query --------------------------------------------
+
+int ring_describe_rows_launch(const ring_row* rows, int n_rows, int dtype, int role, int cus, int* form) {
+  if (!dtype_ok(dtype)) return RING_ERR_DTYPE;
+  if (!form || n_rows < 0 || (n_rows > 0 && !rows) || cus < 1) return RING_ERR_ARGUMENT;
+  if (role != RING_ROLE_COPY && role != RING_ROLE_ACCUMULATE && role != RING_ROLE_ALLGATHER) return RING_ERR_ARGUMENT;
+  const size_t esz = dtype_size(dtype);
+  // the rows as the entry points hand them to the launcher: empty ones dropped
+  RowBuffer<HostRow, kMaxRows> host(static_cast<size_t>(n_rows));
+  size_t n_host = 0;
+  uint64_t bytes = 0;
+  for (int i = 0; i < n_rows; i++) {
+    if (rows[i].count == 0) continue;
+    host.data[n_host++] = HostRow{rows[i].dst, rows[i].a, rows[i].b, rows[i].count, false};
+    bytes += rows[i].count * esz;
+  }
+  const Tuning tun = tuning();
+  const Role r = role == RING_ROLE_COPY ? kRoleCopy : role == RING_ROLE_ACCUMULATE ? kRoleAccumulate : kRoleAllgather;
+  int nt = tun.nt[r];
+  if (nt < 0) nt = bytes <= kCacheResidentBytes ? 0 : 2;
+  *form = choose_rows_form(host.data, n_host, esz, r, 0, nt, tun, cus).form;
+  return RING_OK;
+}
+
+int ring_describe_unpack_launch(uint64_t total_elements, int n_tensors, int dtype, int divisor, int cus, int* form) {
+  if (!dtype_ok(dtype)) return RING_ERR_DTYPE;
+  if (!form || n_tensors < 0 || divisor < 0 || cus < 1) return RING_ERR_ARGUMENT;
+  *form = choose_unpack_form(total_elements, static_cast<uint32_t>(n_tensors), dtype_size(dtype), dtype == RING_F32,
+                             divisor, tuning(), cus).form;
   return RING_OK;
 }
 
@@ -1996,6 +2154,42 @@ int ring_time_next_launch(void* start_event, void* stop_event) {
   return RING_OK;
 }
 
+int ring_probe_stream(const ring_row* rows, int n_rows, int dtype, int mode, void* stream) {
+  if (!dtype_ok(dtype)) return RING_ERR_DTYPE;
+  if (!rows || n_rows < 1 || n_rows > kSmallRows || mode < 0 || mode > 3) return RING_ERR_ARGUMENT;
+  const size_t esz = dtype_size(dtype);
+  const bool write = (mode & 1) != 0;
+  SmallRowTable tab;
+  tab.n_rows = n_rows;
+  tab.dry = 0;
+  tab.uniform_tiles = 0;
+  tab.divisor = 0;
+  tab.div_mask = 0;
+  for (int k = 0; k <= kSmallRows; k++) tab.tile_begin[k] = 0;
+  uint64_t tiles = 1;
+  for (int k = 0; k < kSmallRows; k++) {
+    tab.row[k] = Row{nullptr, nullptr, nullptr, 0};
+    if (k >= n_rows) continue;
+    const void* p = write ? rows[k].dst : rows[k].a;
+    if (!p || (reinterpret_cast<uintptr_t>(p) & 15u)) return RING_ERR_ARGUMENT;
+    const uint64_t nvec = rows[k].count * esz / 16;  // whole 16-byte vectors; a probe has no scalar edges
+    tab.row[k] = Row{rows[k].dst, rows[k].a, nullptr, nvec};
+    const uint64_t t = (nvec + kBlock * 4 - 1) / (kBlock * 4);
+    if (t > tiles) tiles = t;
+  }
+  if (tiles > 0x7fffffffull) return RING_ERR_ARGUMENT;
+  const dim3 grid(static_cast<uint32_t>(tiles), static_cast<uint32_t>(n_rows));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (mode) {
+    case 0: launch(stream_probe_kernel<0, 1>, grid, dim3(kBlock), s, tab); break;
+    case 1: launch(stream_probe_kernel<1, 1>, grid, dim3(kBlock), s, tab); break;
+    case 2: launch(stream_probe_kernel<0, 0>, grid, dim3(kBlock), s, tab); break;
+    default: launch(stream_probe_kernel<1, 0>, grid, dim3(kBlock), s, tab); break;
+  }
+  RING_HIP(hipGetLastError());
+  return RING_OK;
+}
+
 // ---- host tables ------------------------------------------------------------
 
 int ring_segment_table(size_t count, int n, size_t* sizes, size_t* starts) {
@@ -2045,6 +2239,17 @@ int ring_schedule(int phase, int n, int r, int step, int* send_seg, int* recv_se
 }
 
 // ---- stream -------------------------------------------------------------------
+
+int ring_get_device(int* device) {
+  if (!device) return RING_ERR_ARGUMENT;
+  RING_HIP(hipGetDevice(device));
+  return RING_OK;
+}
+
+int ring_set_device(int device) {
+  RING_HIP(hipSetDevice(device));
+  return RING_OK;
+}
 
 int ring_stream_create(void** stream) {
   if (!stream) return RING_ERR_ARGUMENT;
@@ -2175,7 +2380,7 @@ int launch_fold(const HostFoldRow* rows, size_t n_rows, int divisor, int dtype, 
   bool to_all = false;
   for (size_t k = 0; k < n_rows; k++) to_all = to_all || rows[k].n_more > 0;
   const uint64_t kTileVecs = static_cast<uint64_t>(kBlock) * (to_all ? kFoldToAllUnroll : kFoldUnroll);
-  int nt = g_tuning.nt[to_all ? kRoleFoldAll : kRoleFold];
+  int nt = tuning().nt[to_all ? kRoleFoldAll : kRoleFold];
   if (nt < 0) nt = to_all ? 3 : 2;
   size_t i = 0;
   while (i < n_rows) {
@@ -2464,7 +2669,7 @@ template <typename T, bool GATHER, bool DIV>
 int launch_fusion_spans(const ring_fusion_plan* p, const FusionSpanTable& tab, uint32_t tile_lo, uint32_t tile_hi,
                         hipStream_t stream, Role role) {
   uint32_t grid = tile_hi - tile_lo;
-  int nt = g_tuning.nt[role];
+  int nt = tuning().nt[role];
   if (nt < 0) nt = 3;
 #define RING_SPANS(N)                                                                                        \
   launch(fusion_span_kernel<T, GATHER, N, DIV>, dim3(grid), dim3(kBlock), stream,                            \
@@ -2577,7 +2782,7 @@ int ring_fusion_fold_scatter(const ring_fusion_plan* plan, uint64_t fold_begin, 
   const uint64_t tile_elems = static_cast<uint64_t>(kFusionTileVecs) * (16 / p->esz);
   const uint32_t tile_lo = static_cast<uint32_t>(lowest / tile_elems);
   const uint32_t tile_hi = static_cast<uint32_t>((highest + tile_elems - 1) / tile_elems);
-  int nt = g_tuning.nt[kRoleUnpack];
+  int nt = tuning().nt[kRoleUnpack];
   if (nt < 0) nt = 3;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid(tile_hi - tile_lo);
@@ -2630,7 +2835,7 @@ int ring_fusion_allreduce_all(const ring_fusion_plan* const* in_plans, const rin
     ranks.in[k] = k < n ? in_plans[k]->d_ptrs : nullptr;
     ranks.out[k] = k < n ? out_plans[k]->d_ptrs : nullptr;
   }
-  int nt = g_tuning.nt[kRoleFoldAll];
+  int nt = tuning().nt[kRoleFoldAll];
   if (nt < 0) nt = 3;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid(first->ntiles);

@@ -10,6 +10,11 @@ import os
 F32, I32, I64 = 0, 1, 2
 DTYPE_SIZE = {F32: 4, I32: 4, I64: 8}
 PHASE_REDUCE_SCATTER, PHASE_ALLGATHER, PHASE_GATHER = 0, 1, 2
+# enum ring_form / ring_role: which form a launch takes (describe_rows_launch, describe_unpack_launch)
+FORM_TILES, FORM_PACED, FORM_REGISTERS_2, FORM_REGISTERS_1 = 0, 1, 2, 3
+FORM_NAMES = {FORM_TILES: "tiles", FORM_PACED: "paced tiles", FORM_REGISTERS_2: "in registers, two workgroups per CU",
+              FORM_REGISTERS_1: "in registers, one workgroup per CU"}
+ROLE_COPY, ROLE_ACCUMULATE, ROLE_ALLGATHER = 0, 1, 2
 
 _PKG_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB_PATH = os.path.join(_PKG_ROOT, "lib", "libring_hip.so")
@@ -26,6 +31,8 @@ EXPORTS = (
     "ring_fusion_plan_create", "ring_fusion_plan_destroy", "ring_fusion_plan_elements", "ring_fusion_plan_dtype",
     "ring_fusion_pack", "ring_fusion_unpack", "ring_fusion_unpack_scaled", "ring_fusion_gather",
     "ring_fusion_scatter", "ring_fusion_fold_scatter", "ring_scale", "ring_fusion_run_static",
+    "ring_describe_rows_launch", "ring_describe_unpack_launch", "ring_probe_stream",
+    "ring_get_device", "ring_set_device",
 )
 
 
@@ -142,6 +149,11 @@ def lib():
                                               ctypes.POINTER(FusionSpan), ci, ci, vp]),
             "ring_scale": (ci, [ci, vp, sz, ci, vp]),
             "ring_fusion_run_static": (ci, [ci, ctypes.POINTER(vp), psz, ci, ci, vp, ci, vp]),
+            "ring_describe_rows_launch": (ci, [ctypes.POINTER(Row), ci, ci, ci, ci, pint]),
+            "ring_describe_unpack_launch": (ci, [ctypes.c_uint64, ci, ci, ci, ci, pint]),
+            "ring_probe_stream": (ci, [ctypes.POINTER(Row), ci, ci, ci, vp]),
+            "ring_get_device": (ci, [pint]),
+            "ring_set_device": (ci, [ci]),
         }
         for name in EXPORTS:
             fn = getattr(L, name)          # AttributeError if the symbol is missing
@@ -163,6 +175,39 @@ def check(status, where):
 
 def set_option(name, value):
     check(lib().ring_set_option(name.encode(), int(value)), "ring_set_option(%s)" % name)
+
+
+def make_rows(rows):
+    """rows: iterable of (dst_ptr, a_ptr, b_ptr_or_None, count) -> ctypes array, length."""
+    rows = list(rows)
+    arr = (Row * max(len(rows), 1))()
+    for i, (dst, a, b, cnt) in enumerate(rows):
+        arr[i].dst, arr[i].a, arr[i].b, arr[i].count = dst, a, b, cnt
+    return arr, len(rows)
+
+
+def describe_rows_launch(rows, dtype, role, cus=256):
+    """The form (FORM_*) a launch of `rows` (dst, a, b, count) takes on a GPU of
+    `cus` compute units; needs no GPU, pointers only matter for their alignment."""
+    arr, n = make_rows(rows)
+    form = ctypes.c_int(-1)
+    check(lib().ring_describe_rows_launch(arr, n, dtype, role, cus, ctypes.byref(form)), "ring_describe_rows_launch")
+    return form.value
+
+
+def describe_unpack_launch(total_elements, n_tensors, dtype, divisor=0, cus=256):
+    """The form (FORM_*) the unpack of such a fused buffer takes; needs no GPU."""
+    form = ctypes.c_int(-1)
+    check(lib().ring_describe_unpack_launch(total_elements, n_tensors, dtype, divisor, cus, ctypes.byref(form)),
+          "ring_describe_unpack_launch")
+    return form.value
+
+
+def probe_stream(rows, dtype, mode, stream):
+    """Measurement only: one direction of a copy launch. rows: (dst, a, None, count);
+    mode 0 reads every `a`, mode 1 writes every `dst` (2 / 3: ordinary cache policy)."""
+    arr, n = make_rows(rows)
+    check(lib().ring_probe_stream(arr, n, dtype, mode, stream), "ring_probe_stream")
 
 
 # ---- timing of single launches -----------------------------------------------------

@@ -28,6 +28,18 @@ namespace contrib {
 namespace mpi {
 template <typename Device> void CopyTensorData(void* destination, void* source, size_t size);
 template <typename Device, typename T> void AccumulateTensorData(T* destination, T* source, size_t size);
+int RingDeviceStatusTake();
+
+// What the patched mpi_ops.cc provides (mpi_ops.cc:213-230 the stream member, :582-583 its creation on the
+// background thread after the device has been made current, :872-876 the accessor ring.h:55-57 declares):
+// here the test is the owner of the stream.
+static void* g_stream_for_mpi = nullptr;
+void* CudaStreamForMPI() { return g_stream_for_mpi; }
+static bool CreateStreamForMPI() {
+  int device = -1;
+  return ring_get_device(&device) == RING_OK && ring_set_device(device) == RING_OK &&
+         ring_stream_create(&g_stream_for_mpi) == RING_OK && g_stream_for_mpi != nullptr;
+}
 }  // namespace mpi
 }  // namespace contrib
 }  // namespace tensorflow
@@ -147,7 +159,25 @@ static void reference_loop(int n, size_t count) {
   }
 }
 
+// A failed device call is not dropped (the reference's seam is void and drops them): the first status is
+// kept for the thread and handed out once.
+static void failures_are_remembered() {
+  using tensorflow::contrib::mpi::RingDeviceStatusTake;
+  CHECK(RingDeviceStatusTake() == RING_OK);
+  std::vector<float> a(64, 1.f);
+  float* da = device_copy(a, 0);
+  AccumulateTensorData<GPUDevice, float>(nullptr, da, 64);                        // no destination
+  AccumulateTensorData<GPUDevice, float>(da, da, 64);                             // a good call does not clear it
+  CHECK(RingDeviceStatusTake() == RING_ERR_ARGUMENT);
+  CHECK(RingDeviceStatusTake() == RING_OK);
+  CopyTensorData<GPUDevice>(nullptr, da, 16);
+  CHECK(RingDeviceStatusTake() == RING_ERR_ARGUMENT);
+  HIP_OK(hipFree(da));
+}
+
 int main() {
+  CHECK(tensorflow::contrib::mpi::CreateStreamForMPI());
+  failures_are_remembered();
   primitives<float>();
   primitives<int>();
   primitives<long long>();
@@ -156,6 +186,7 @@ int main() {
   reference_loop<int>(6, 100019);
   reference_loop<long long>(5, 4099);
   reference_loop<float>(4, 2);       // fewer elements than ranks: empty segments
+  CHECK(tensorflow::contrib::mpi::RingDeviceStatusTake() == RING_OK);
   std::printf("ok\n");
   return 0;
 }

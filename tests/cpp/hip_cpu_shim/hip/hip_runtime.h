@@ -163,6 +163,7 @@ inline void __syncthreads() { hip_cpu_shim::Pool::get().barrier(); }
 
 inline hipError_t hipGetLastError() { return hipSuccess; }
 inline hipError_t hipGetDevice(int* dev) { *dev = 0; return hipSuccess; }
+inline hipError_t hipSetDevice(int dev) { return dev == 0 ? hipSuccess : hipErrorInvalidValue; }
 inline hipError_t hipDeviceGetAttribute(int* value, int, int) { *value = 4; return hipSuccess; }
 // exact-size heap blocks: an access one byte outside is an AddressSanitizer error
 inline hipError_t hipMalloc(void** p, size_t bytes) { *p = malloc(bytes ? bytes : 1); return *p ? hipSuccess : hipErrorInvalidValue; }

@@ -123,3 +123,21 @@ def kernels_in_scratch(asm_text, names):
         if private or spilled:
             scratch.append((name.group(1), private, spilled))
     return {"seen": seen, "scratch": scratch}
+
+
+def test_options_set_while_another_thread_launches_under_thread_sanitizer():
+    """ring_set_option from one thread while another launches copies, accumulates and
+    unpacks through the CPU stand-in: no data race, and every output right."""
+    clang = _clang()
+    if clang is None:
+        pytest.skip("no clang++ (the kernels use clang vector extensions)")
+    os.makedirs(BUILD, exist_ok=True)
+    exe = os.path.join(BUILD, "options_race_test")
+    cmd = [clang, "-x", "c++", "-std=c++17", "-O1", "-g", "-fsanitize=thread", "-fno-omit-frame-pointer", "-pthread",
+           "-I", os.path.join(ROOT, "tests", "cpp", "hip_cpu_shim"), "-I", os.path.join(ROOT, "include"),
+           "-o", exe, SRC, os.path.join(ROOT, "tests", "cpp", "options_race_test.cc")]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert res.returncode == 0, res.stdout[-4000:]
+    env = dict(os.environ, TSAN_OPTIONS="halt_on_error=1:report_signal_unsafe=0")
+    res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600, env=env)
+    assert res.returncode == 0 and "options race test: ok" in res.stdout, res.stdout[-4000:]

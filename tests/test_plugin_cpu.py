@@ -464,3 +464,109 @@ def test_direct_form_refuses_more_ranks_than_a_fold_addresses():
     rc = L.mpic_ring_allreduce_direct_prestaged(n, 0, _plugin.DT_FLOAT, 0x1000, 0x2000, 1000, ptrs, ptrs, None, 1)
     assert rc == _plugin.INVALID_ARGUMENT
     assert b"at most 256 copies" in L.mpic_last_error()
+
+
+# ---- which form a launch takes (host-only query; every form gives the same bytes, so only this pins the choice)
+
+def _allgather_rows(count, n, rank, esz, misalign=0):
+    """The copy rows of rank `rank`'s allgather phase on a `count`-element tensor at n ranks, as
+    ring_allgather_steps hands them to the launcher (addresses made up: only their alignment matters)."""
+    sizes, starts = ring_abi.segment_table(count, n)
+    segs = [ring_abi.schedule(ring_abi.PHASE_ALLGATHER, n, rank, i)[1] for i in range(n - 1)]
+    out, staged = 1 << 32, 1 << 40
+    return [(out + misalign + starts[g] * esz, staged + (i << 30), None, sizes[g]) for i, g in enumerate(segs)]
+
+
+def _equal_rows(n_rows, elems, esz=4):
+    return [((1 << 32) + k * elems * esz, (1 << 40) + (k << 30), None, elems) for k in range(n_rows)]
+
+
+def test_launch_forms_of_the_benchmark_shapes_on_256_compute_units():
+    A = ring_abi
+    form = lambda rows, dt: A.describe_rows_launch(rows, dt, A.ROLE_ALLGATHER, 256)
+    # float32 64 MiB, N=8: 7 x 8 MiB fill the chip with exactly 7 paced tiles of 32 KiB per CU
+    for rank in range(8):
+        assert form(_allgather_rows(16 * 1024 * 1024, 8, rank, 4), A.F32) == A.FORM_PACED
+    # int32 / int64 ragged 10,000,019 at N=6: 5 rows of 6.4 / 12.7 MiB
+    for rank in range(6):
+        assert form(_allgather_rows(10_000_019, 6, rank, 4), A.I32) == A.FORM_REGISTERS_2
+        assert form(_allgather_rows(10_000_019, 6, rank, 8), A.I64) == A.FORM_REGISTERS_1
+    # the fused ResNet-50 buffer at N=8: 7 rows of 12.2 MiB; and its unpack with the divide by 8 (97.5 MiB)
+    assert form(_allgather_rows(25_557_032, 8, 0, 4), A.F32) == A.FORM_REGISTERS_1
+    assert A.describe_unpack_launch(25_557_032, 161, A.F32, 8, 256) == A.FORM_REGISTERS_1
+    assert A.describe_unpack_launch(25_557_032, 161, A.F32, 0, 256) == A.FORM_REGISTERS_1
+    # float32 1 GiB at N=64: 63 rows of 16 MiB, far beyond what is resident at once
+    assert form(_allgather_rows(268_435_456, 64, 0, 4), A.F32) == A.FORM_TILES
+    # the variable allgather at N=16 (16 unequal rows, about 130 MiB)
+    rows = [(1 << 32, 1 << 40, None, r * 1024) for r in (3000, 17, 4096, 2222, 1, 999, 4000, 3100, 2900, 12, 3500, 2048, 77,
+                                                       4095, 1800, 2600)]
+    assert form(rows, A.F32) == A.FORM_TILES
+    # the in->out copy and the accumulates have one form
+    assert A.describe_rows_launch(_equal_rows(1, 16 * 1024 * 1024), A.F32, A.ROLE_COPY, 256) == A.FORM_TILES
+    acc = [(d, a, d, c) for d, a, _, c in _equal_rows(7, 2 * 1024 * 1024)]
+    assert A.describe_rows_launch(acc, A.F32, A.ROLE_ACCUMULATE, 256) == A.FORM_TILES
+
+
+def test_launch_forms_change_where_they_were_measured_to():
+    A = ring_abi
+    MiB = 1 << 18   # float32 elements
+    form = lambda rows, cus=256, dt=A.F32: A.describe_rows_launch(rows, dt, A.ROLE_ALLGATHER, cus)
+    assert form(_equal_rows(7, 2 * MiB)) == A.FORM_TILES                 # 14 MiB, under 2 paced tiles per CU: bound by the dispatch
+    assert form(_equal_rows(8, 2 * MiB)) == A.FORM_PACED                 # 16 MiB: 2 tiles of 32 KiB per CU
+    assert form(_equal_rows(7, 4 * MiB)) == A.FORM_PACED                 # 28 MiB: under 124 KiB per CU the paced tiles win
+    assert form(_equal_rows(7, 7 * MiB + MiB // 2)) == A.FORM_REGISTERS_2  # 52.5 MiB: the paced tiles leave CUs over
+    assert form(_equal_rows(7, 8 * MiB)) == A.FORM_PACED                 # 56 MiB: exactly 7 tiles per CU
+    assert form(_equal_rows(7, 8 * MiB + 8192)) == A.FORM_REGISTERS_1    # one tile per row more: above 224 KiB per CU
+    assert form(_equal_rows(7, 16 * MiB)) == A.FORM_REGISTERS_1          # 112 MiB: all the registers hold
+    assert form(_equal_rows(7, 16 * MiB + 65536 * 4)) == A.FORM_TILES    # a 17th round per row does not fit
+    assert form(_equal_rows(8, 14 * MiB)) == A.FORM_REGISTERS_1          # 8 rows of 14 rounds
+    assert form(_equal_rows(9, 8 * MiB)) == A.FORM_TILES                 # more than 8 rows: not in registers, too many tiles to pace
+    assert form(_equal_rows(9, 6 * MiB)) == A.FORM_PACED                 # 9 rows, 54 MiB: all tiles resident
+    assert form(_equal_rows(1, 60 * MiB)) == A.FORM_REGISTERS_1          # one row (ring_allgather_steps of one step)
+    assert form(_equal_rows(7, 8 * MiB), cus=64) == A.FORM_TILES         # a chip none of this was measured on
+    assert form(_equal_rows(7, 2 * MiB), cus=64) == A.FORM_PACED
+    # a row with a second operand, or an empty row kept by the caller, leaves the registers form
+    mixed = _equal_rows(7, 12 * MiB)
+    mixed[3] = (mixed[3][0], mixed[3][1], mixed[3][0], mixed[3][3])
+    assert form(mixed) == A.FORM_TILES
+    # the unpack: by itself from 1 MiB, two workgroups per CU up to 75 MiB, one up to 112 MiB
+    unpack = lambda elems, k=100, dt=A.F32, div=0, cus=256: A.describe_unpack_launch(elems, k, dt, div, cus)
+    assert unpack(MiB // 2) == A.FORM_TILES
+    assert unpack(MiB) == A.FORM_REGISTERS_2
+    assert unpack(75 * MiB) == A.FORM_REGISTERS_2
+    assert unpack(75 * MiB + 1024) == A.FORM_REGISTERS_1
+    assert unpack(112 * MiB) == A.FORM_REGISTERS_1
+    assert unpack(112 * MiB + 4) == A.FORM_TILES
+    assert unpack(64 * MiB, k=1024) == A.FORM_REGISTERS_2 and unpack(64 * MiB, k=1025) == A.FORM_TILES
+    assert unpack(64 * MiB, cus=64) == A.FORM_TILES
+    # divisors: a power of two everywhere; any other one for float32 up to 64 MiB; the integers' floor division as tiles
+    assert unpack(97 * MiB, div=8) == A.FORM_REGISTERS_1 and unpack(97 * MiB, dt=A.I32, div=8) == A.FORM_REGISTERS_1
+    assert unpack(64 * MiB, div=6) == A.FORM_REGISTERS_2 and unpack(64 * MiB + 1024, div=6) == A.FORM_TILES
+    assert unpack(32 * MiB, dt=A.I32, div=6) == A.FORM_TILES and unpack(16 * MiB, dt=A.I64, div=3) == A.FORM_TILES
+
+
+def test_launch_form_query_follows_the_options_and_checks_its_arguments():
+    A = ring_abi
+    rows = _allgather_rows(10_000_019, 6, 0, 4)
+    try:
+        A.set_option("phased_copy", 0)
+        assert A.describe_rows_launch(rows, A.I32, A.ROLE_ALLGATHER, 256) == A.FORM_PACED
+        assert A.describe_unpack_launch(25_557_032, 161, A.F32, 8, 256) == A.FORM_TILES
+        A.set_option("paced_copy", 0)
+        assert A.describe_rows_launch(rows, A.I32, A.ROLE_ALLGATHER, 256) == A.FORM_TILES
+        A.set_option("paced_copy", 1)
+        assert A.describe_rows_launch(_equal_rows(3, 1000), A.F32, A.ROLE_ALLGATHER, 256) == A.FORM_PACED
+        A.set_option("phased_copy", 1)
+        assert A.describe_rows_launch(_equal_rows(3, 1000), A.F32, A.ROLE_ALLGATHER, 256) == A.FORM_REGISTERS_2
+    finally:
+        A.set_option("phased_copy", -1)
+        A.set_option("paced_copy", -1)
+    assert A.describe_rows_launch(rows, A.I32, A.ROLE_ALLGATHER, 256) == A.FORM_REGISTERS_2
+    with pytest.raises(A.RingError):
+        A.describe_rows_launch(rows, 7, A.ROLE_ALLGATHER, 256)
+    with pytest.raises(A.RingError):
+        A.describe_rows_launch(rows, A.I32, 5, 256)
+    with pytest.raises(A.RingError):
+        A.describe_rows_launch(rows, A.I32, A.ROLE_ALLGATHER, 0)
+    with pytest.raises(A.RingError):
+        A.describe_unpack_launch(1 << 20, 10, A.F32, -1, 256)
