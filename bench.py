@@ -41,7 +41,7 @@ for p in (ROOT, os.path.join(ROOT, "tensorflow-allreduce_amd")):
         sys.path.insert(0, p)
 
 HBM_PEAK_GBS = 8000.0
-FRESH_STAGING = False               # --fresh-staging: see FusedResnet50NoPasses.coaligned
+FRESH_STAGING = False               # --fresh-staging: see coaligned()
 REGIONS = 9                         # wall-clock regions of --steps steps each; ms_per_step is their median
 SAMPLE_EVERY = 4                    # steps between launches that carry timing events (sampling pass only)
 MIN_SAMPLES = 32                    # timed launches per phase, whatever --steps is
@@ -79,6 +79,25 @@ def resnet50_counts():
                 counts += [cin * 4 * width, 4 * width, 4 * width]
             cin = 4 * width
     return counts + [2048 * 1000, 1000]
+
+
+def coaligned(torch, t, begin_bytes):
+    """A copy of the finished segment `t` that lies in its allocation where it would lie in a neighbour's buffer:
+    `begin_bytes` mod 128 behind a 128-byte line. The reference receives an allgather segment in place, at
+    buffer + starts[segment] (ring.h:211-225), and a virtual rank copies it from the neighbour's buffer at that
+    same offset, so the 128-byte lines of the source are the lines of the destination; staged at the start of a
+    fresh allocation instead, a ragged segment's source is shifted against its destination and every 1 KiB a
+    wave loads straddles one more line (1.5-4.5 % more bytes fetched, measured). --fresh-staging keeps the
+    fresh allocations, for comparison. Reduce-scatter arrivals stay at the start of theirs, like the reference's
+    temp tensor (ring.h:189-204)."""
+    if FRESH_STAGING:
+        return t
+    esz = t.element_size()
+    lead = (begin_bytes % 128) // esz
+    room = torch.empty(t.numel() + 128 // esz, dtype=t.dtype, device=t.device)
+    view = room[lead: lead + t.numel()]
+    view.copy_(t)
+    return view
 
 
 class Workload:
@@ -141,7 +160,7 @@ class RingAllreduce(Workload):
             rs_seg = [ring_abi.schedule(ring_abi.PHASE_REDUCE_SCATTER, n, r, i)[1] for i in range(n - 1)]
             ag_seg = [ring_abi.schedule(ring_abi.PHASE_ALLGATHER, n, r, i)[1] for i in range(n - 1)]
             rs = [rnd(self.sizes[g], left) for g in rs_seg]
-            ag = [rnd(self.sizes[g], left) for g in ag_seg]
+            ag = [coaligned(torch, rnd(self.sizes[g], left), self.starts[g] * esz) for g in ag_seg]
             self.sets.append(dict(
                 r=r, inp=inp, out=out, rs=rs, ag=ag, rs_seg=rs_seg, ag_seg=ag_seg,
                 rs_ptrs=(ctypes.c_void_p * max(n - 1, 1))(*[t.data_ptr() for t in rs]),
@@ -380,7 +399,7 @@ class FusedResnet50(Workload):
             rs_seg = [ring_abi.schedule(0, 8, r, i)[1] for i in range(7)]
             ag_seg = [ring_abi.schedule(1, 8, r, i)[1] for i in range(7)]
             rs = [torch.randn(sizes[g], device="cuda", generator=gen) * 1e-3 for g in rs_seg]
-            ag = [torch.randn(sizes[g], device="cuda", generator=gen) * 1e-3 for g in ag_seg]
+            ag = [coaligned(torch, torch.randn(sizes[g], device="cuda", generator=gen) * 1e-3, starts[g] * 4) for g in ag_seg]
             self.sets.append(dict(grads=grads, plan=plan, fused=fused, rs=rs, ag=ag, r=r, rs_seg=rs_seg, ag_seg=ag_seg,
                                   rs_steps=ring_abi.make_steps([(starts[g], t.data_ptr(), sizes[g]) for g, t in zip(rs_seg, rs)]),
                                   ag_steps=ring_abi.make_steps([(starts[g], t.data_ptr(), sizes[g]) for g, t in zip(ag_seg, ag)])))
@@ -469,11 +488,6 @@ class FusedResnet50NoPasses(FusedResnet50):
             r = s % 8
             rs_seg = [A.schedule(0, 8, r, i)[1] for i in range(7)]
             ag_seg = [A.schedule(1, 8, r, i)[1] for i in range(7)]
-            # Where a finished segment lands is the receiver's choice, and the reference receives it in place,
-            # at buffer + starts[segment] (ring.h:211-225): 16-byte groups of the arrival are then groups of the
-            # fused space. The slots here keep that: each starts starts[segment] % 4 elements into its allocation
-            # (3,194,629-element segments begin at every residue), so the scatter's loads are aligned like its stores.
-            st["ag"] = [self.coaligned(t, starts[g]) for g, t in zip(ag_seg, st["ag"])]
             rs_of = {g: t for g, t in zip(rs_seg, st["rs"])}
             ag_of = {g: t for g, t in zip(ag_seg, st["ag"])}
             own, wire = (r + 1) % 8, st["fused"].data_ptr()
@@ -495,15 +509,6 @@ class FusedResnet50NoPasses(FusedResnet50):
                             "elements, values ~N(0,1e-3)) at N=8 virtual ranks WITHOUT pack and unpack passes: the 7 "
                             "accumulates read their local operand from the tensors and write the wire buffer, the 8 "
                             "finished segments go straight into the tensors with the divide by 8; 2 launches per step")
-
-    def coaligned(self, t, begin):
-        """A copy of segment `t` whose element 0 lies `begin` % 4 elements behind a 16-byte boundary."""
-        if FRESH_STAGING:      # --fresh-staging: the slots as fresh allocations, for comparison
-            return t
-        room = self.torch.empty(t.numel() + 4, device="cuda")
-        view = room[begin % 4: begin % 4 + t.numel()]
-        view.copy_(t)
-        return view
 
     def launch_phase(self, k, i, stream):
         s = self.sets[k % self.nsets]
@@ -536,7 +541,8 @@ class FusedResnet50NoPassesDirect(FusedResnet50NoPasses):
         for st in self.sets:
             own = (st["r"] + 1) % 8
             gen = torch.Generator(device="cuda").manual_seed(77 + st["r"])
-            st["raw"] = [self.coaligned(torch.randn(sizes[own], device="cuda", generator=gen) * 1e-3, starts[own])
+            # the slots peers push their raw copies of the owned segment into are the receiver's to place
+            st["raw"] = [coaligned(torch, torch.randn(sizes[own], device="cuda", generator=gen) * 1e-3, starts[own] * 4)
                          for _ in range(7)]
             st["raw_ptrs"] = (ctypes.c_void_p * 7)(*[t.data_ptr() for t in st["raw"]])
             st["own"], st["mine"] = own, st["fused"].data_ptr() + starts[own] * 4
@@ -837,8 +843,8 @@ def main():
     ap.add_argument("--workload", default=WORKLOADS[0], choices=WORKLOADS)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--fresh-staging", action="store_true",
-                    help="fused workloads without passes: stage every finished segment at the start of a fresh "
-                         "allocation instead of where its 16-byte groups line up with the fused space")
+                    help="stage every finished (allgather) segment at the start of a fresh allocation instead of "
+                         "where it lies in a neighbour's buffer (see coaligned())")
     ap.add_argument("--variant", choices=("all", "reference", "fused"), default="all",
                     help="all: the reference-shaped path (the reported value), then the extras: the same job with "
                          "the in->out copy folded into the accumulate, and the hot (one buffer set) rate. "

@@ -416,14 +416,14 @@ int ring_fusion_run_static(int unpack, const void* const* tensors, const size_t*
  * must be sorted by `begin` and disjoint; `spans` is a HOST array. Together
  * the two calls do what pack, n-1 accumulates, and unpack do, minus one read
  * and one write of the whole set. `incoming` and `out` need only be aligned
- * to an element. The kernels align their stores; the loads of `incoming` are
- * aligned too when its 16-byte groups are groups of the fused space, i.e.
- * when (address of incoming / element size - begin) is a multiple of
- * 16 / element size, as it is for a segment received in place at
- * wire + begin (where ring.h:211-225 receives it). A slot that starts at a
- * fresh allocation instead costs a segment with begin % 4 != 0 about 4 % more
- * bytes fetched (every 1 KiB a wave loads touches 33 sectors of 32 bytes
- * instead of 32) and as much time. */
+ * to an element. The kernels align their stores to the tensors; a wave's
+ * loads of `incoming` cover whole 128-byte lines as well when the arrival is
+ * shifted against the fused space by a multiple of 128 bytes, i.e. when
+ * (address of incoming - begin * element size) is a multiple of 128, as it is
+ * for a segment received in place at wire + begin in a 128-byte aligned wire
+ * buffer (where ring.h:211-225 receives it). A slot at the start of a fresh
+ * allocation instead costs a ragged segment 3.6 % more bytes fetched (every
+ * 1 KiB a wave loads straddles one more line) and 1.5 % of the launch. */
 typedef struct ring_fusion_span {
   uint64_t begin;       /* first element in the fused space */
   uint64_t count;       /* elements */

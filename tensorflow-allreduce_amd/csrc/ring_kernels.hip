@@ -1253,6 +1253,11 @@ fusion_direct_kernel(const uint64_t* __restrict__ offsets, T* const* __restrict_
 // whose pointers the first lanes look up in the ranks' tensor tables.
 
 constexpr int kMaxFusedRanks = 16;
+// A tile of the fused space (1024 16-byte groups) is worked on by this many
+// workgroups, a quarter each: the fold that stores to every rank wants short
+// tiles (kFoldToAllUnroll), and what a workgroup has to look up before its
+// first load is one round trip to memory, so there is nothing to share.
+constexpr uint32_t kFusedAllSplit = kFusionTileVecs / (kBlock * kFoldToAllUnroll);
 struct FusedRanks {
   int n;
   int divisor;
@@ -1261,7 +1266,20 @@ struct FusedRanks {
   uint64_t rem;     // total % n: the first rem segments hold one more
   const void* const* in[kMaxFusedRanks];   // rank k's input tensor table
   void* const* out[kMaxFusedRanks];        // rank k's output tensor table
+  const FusionTile* in_tiles[kMaxFusedRanks];   // rank k's tile records: where a tile inside one tensor starts
+  const FusionTile* out_tiles[kMaxFusedRanks];
 };
+
+// The pointer of rank r out of a table in the kernel arguments, r different per
+// lane: a run of selects on scalar registers instead of a load from the
+// argument segment (one more trip to memory ahead of the loads that matter).
+template <typename P>
+__device__ __forceinline__ P pick_rank(const P (&table)[kMaxFusedRanks], int r) {
+  P p = table[0];
+#pragma unroll
+  for (int j = 1; j < kMaxFusedRanks; j++) p = (r == j) ? table[j] : p;
+  return p;
+}
 
 template <typename T, bool DIV, int NT>
 __global__ void __launch_bounds__(kBlock)
@@ -1269,22 +1287,69 @@ fusion_allreduce_kernel(const uint64_t* __restrict__ offsets, const FusionTile* 
                         const FusedRanks ranks) {
   constexpr uint32_t VEC = 16 / sizeof(T);
   constexpr uint64_t kTileElems = static_cast<uint64_t>(kFusionTileVecs) * VEC;
+  constexpr uint64_t kPartElems = kTileElems / kFusedAllSplit;
   __shared__ const void* s_src[kMaxFusedRanks];
   __shared__ const void* s_dst[kMaxFusedRanks];
   const int n = ranks.n;
   auto seg_start = [&](uint64_t s) { return s * ranks.seg + (s < ranks.rem ? s : ranks.rem); };
+  auto seg_of = [&](uint64_t e) {  // segments 0..rem-1 have seg+1 elements
+    const uint64_t big = ranks.rem * (ranks.seg + 1);
+    return e < big ? e / (ranks.seg + 1) : ranks.rem + (ranks.seg ? (e - big) / ranks.seg : 0);
+  };
+  // one piece: fold row with n sources (rank (s + k) mod n is source k, the ring's order for segment s)
+  // and n destinations, whose pointers lie in s_src / s_dst
+  auto fold_piece = [&](uint64_t count) {
+    T* dst = static_cast<T*>(const_cast<void*>(s_dst[0]));
+    uint64_t head = ((16u - (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(dst)) & 15u)) & 15u) / sizeof(T);
+    if (head > count) head = count;
+    const uint64_t nvec = (count - head) / VEC;
+    uint32_t sub_tiles = static_cast<uint32_t>((nvec + kBlock * kFoldToAllUnroll - 1) / (kBlock * kFoldToAllUnroll));
+    if (sub_tiles == 0) sub_tiles = 1;
+    for (uint32_t sub = 0; sub < sub_tiles; sub++)
+      fold_tile<T, kFoldToAllUnroll, kFoldGroup, DIV, NT>(dst, s_src, n, count, sub, sub_tiles, ranks.divisor, DIV,
+                                                          s_dst + 1, n - 1);
+  };
 
-  for (uint32_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+  for (uint32_t item = blockIdx.x; item < ntiles * kFusedAllSplit; item += gridDim.x) {
+    const uint32_t tile = item / kFusedAllSplit, part = item % kFusedAllSplit;
     const uint64_t e0 = static_cast<uint64_t>(tile) * kTileElems;
     const uint64_t e1 = (e0 + kTileElems < ranks.total) ? e0 + kTileElems : ranks.total;
+    // Issued together, one trip to memory: the tile's record (uniform) and, by lane k < n, where the tile
+    // starts in rank k's input and output tensors (meaningful when the tile lies inside one tensor).
     const FusionTile rec = load_tile(tiles, tile);
-    uint32_t t = rec.first;  // the tensor holding the current position (all uniform over the workgroup)
-    // the segment holding e0: segments 0..rem-1 have seg+1 elements
-    uint64_t s;
-    {
-      const uint64_t big = ranks.rem * (ranks.seg + 1);
-      s = e0 < big ? e0 / (ranks.seg + 1) : ranks.rem + (ranks.seg ? (e0 - big) / ranks.seg : 0);
+    FusionTile mine_in{nullptr, 0, 0}, mine_out{nullptr, 0, 0};
+    const int k = static_cast<int>(threadIdx.x);
+    if (k < n) {
+      mine_in = load_tile(pick_rank(ranks.in_tiles, k), tile);
+      mine_out = load_tile(pick_rank(ranks.out_tiles, k), tile);
     }
+    if (rec.first == rec.last) {
+      // inside one tensor: this workgroup's quarter of the tile, cut where a ring segment ends
+      uint64_t b0 = e0 + part * kPartElems;
+      const uint64_t end = b0 + kPartElems < e1 ? b0 + kPartElems : e1;
+      uint64_t s = b0 < end ? seg_of(b0) : 0;
+      while (b0 < end) {
+        while (seg_start(s + 1) <= b0) s++;
+        const uint64_t b1 = seg_start(s + 1) < end ? seg_start(s + 1) : end;
+        if (k < n) {
+          // rank k is source (k - s) mod n of this segment's fold, and destination k
+          const int j = static_cast<int>((static_cast<uint64_t>(k) + static_cast<uint64_t>(n) - s % static_cast<uint64_t>(n)) %
+                                         static_cast<uint64_t>(n));
+          s_src[j] = static_cast<const T*>(mine_in.addr) + (b0 - e0);
+          s_dst[k] = static_cast<T*>(mine_out.addr) + (b0 - e0);
+        }
+        __syncthreads();
+        fold_piece(b1 - b0);
+        __syncthreads();  // before the next piece overwrites the pointers
+        b0 = b1;
+      }
+      continue;
+    }
+    // several tensors meet in the tile (a few hundred KiB of a ResNet-sized set): one workgroup takes all of
+    // it, cut where a tensor or a segment ends, the pointers looked up in the ranks' tensor tables
+    if (part != 0) continue;
+    uint32_t t = rec.first;  // the tensor holding the current position (all uniform over the workgroup)
+    uint64_t s = seg_of(e0);
     uint64_t b0 = e0;
     while (b0 < e1) {
       while (offsets[t + 1] <= b0) t++;
@@ -1293,24 +1358,13 @@ fusion_allreduce_kernel(const uint64_t* __restrict__ offsets, const FusionTile* 
       if (offsets[t + 1] < b1) b1 = offsets[t + 1];
       if (seg_start(s + 1) < b1) b1 = seg_start(s + 1);
       const uint64_t within = b0 - offsets[t];
-      // rank (s + k) mod n is source k (the ring's order for segment s); rank k is destination k
-      if (threadIdx.x < static_cast<uint32_t>(n)) {
-        const int k = static_cast<int>(threadIdx.x);
+      if (k < n) {
         const int r = static_cast<int>((s + static_cast<uint64_t>(k)) % static_cast<uint64_t>(n));
-        s_src[k] = static_cast<const T*>(ranks.in[r][t]) + within;
-        s_dst[k] = static_cast<T*>(ranks.out[k][t]) + within;
+        s_src[k] = static_cast<const T*>(pick_rank(ranks.in, r)[t]) + within;
+        s_dst[k] = static_cast<T*>(pick_rank(ranks.out, k)[t]) + within;
       }
       __syncthreads();
-      T* dst = static_cast<T*>(const_cast<void*>(s_dst[0]));
-      const uint64_t count = b1 - b0;
-      uint64_t head = ((16u - (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(dst)) & 15u)) & 15u) / sizeof(T);
-      if (head > count) head = count;
-      const uint64_t nvec = (count - head) / VEC;
-      uint32_t sub_tiles = static_cast<uint32_t>((nvec + kBlock * kFoldToAllUnroll - 1) / (kBlock * kFoldToAllUnroll));
-      if (sub_tiles == 0) sub_tiles = 1;
-      for (uint32_t sub = 0; sub < sub_tiles; sub++)
-        fold_tile<T, kFoldToAllUnroll, kFoldGroup, DIV, NT>(dst, s_src, n, count, sub, sub_tiles, ranks.divisor, DIV,
-                                                            s_dst + 1, n - 1);
+      fold_piece(b1 - b0);
       __syncthreads();  // before the next piece overwrites the pointers
       b0 = b1;
     }
@@ -2834,11 +2888,14 @@ int ring_fusion_allreduce_all(const ring_fusion_plan* const* in_plans, const rin
   for (int k = 0; k < kMaxFusedRanks; k++) {
     ranks.in[k] = k < n ? in_plans[k]->d_ptrs : nullptr;
     ranks.out[k] = k < n ? out_plans[k]->d_ptrs : nullptr;
+    ranks.in_tiles[k] = k < n ? in_plans[k]->d_tiles : nullptr;
+    ranks.out_tiles[k] = k < n ? out_plans[k]->d_tiles : nullptr;
   }
   int nt = tuning().nt[kRoleFoldAll];
   if (nt < 0) nt = 3;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const dim3 grid(first->ntiles);
+  const uint64_t items = static_cast<uint64_t>(first->ntiles) * kFusedAllSplit;
+  const dim3 grid(static_cast<uint32_t>(items < 0x7fffffffull ? items : 0x7fffffffull));
 #define RING_FUSED_ALL(T, D, N)                                                                              \
   launch(fusion_allreduce_kernel<T, D, N>, grid, dim3(kBlock), s, static_cast<const uint64_t*>(first->d_offsets), \
          static_cast<const FusionTile*>(first->d_tiles), first->ntiles, ranks)
