@@ -142,6 +142,10 @@ const char* mpic_context_message(const mpic_context* ctx);
 int mpic_context_num_outputs(const mpic_context* ctx);
 int mpic_context_output(const mpic_context* ctx, int index, int* dtype, int* ndims,
                         int64_t* dims /* room for 8 */, void** data);
+/* 1 when the op's done() has run (or the op was never started), else 0: whether
+ * mpic_context_destroy would return at once. */
+int mpic_context_done(mpic_context* ctx);
+/* Waits for a started op's done() before it frees the context. */
 int mpic_context_destroy(mpic_context* ctx);
 
 /* k MPIAllreduce nodes of one rank in one call: what k rounds of
@@ -177,7 +181,13 @@ int mpic_context_wait_batch(mpic_context** contexts, int k, int destroy_ok, int*
  * submission is still running); mpic_batch_wait blocks until all of them have
  * finished, returns the first status that is not OK and fills codes[j] (when
  * given) with node j's; mpic_batch_message(batch, j) is node j's message
- * until the next submit. mpic_batch_destroy waits for a running submission. */
+ * until the next submit. mpic_batch_destroy waits for a running submission
+ * (mpic_batch_busy: 1 while one is running). Lifetime: a batch may be
+ * destroyed before or after its world; once mpic_world_destroy has returned
+ * (which fails whatever was still running), mpic_batch_submit answers
+ * FAILED_PRECONDITION and only mpic_batch_wait / _message / _destroy remain
+ * meaningful. The contexts handed out by mpic_allreduce_batch follow the rule
+ * of single contexts: wait for them, or destroy the world first. */
 typedef struct mpic_batch mpic_batch;
 int mpic_batch_create(mpic_world* world, int rank, int k, const char* const* node_names, const int* dtypes,
                       const int* ndims, const int64_t* dims, const void* const* inputs, void* const* outputs,
@@ -186,6 +196,7 @@ int mpic_batch_size(const mpic_batch* batch);
 int mpic_batch_submit(mpic_batch* batch);
 int mpic_batch_wait(mpic_batch* batch, int* codes);
 const char* mpic_batch_message(const mpic_batch* batch, int index);
+int mpic_batch_busy(mpic_batch* batch);
 int mpic_batch_destroy(mpic_batch* batch);
 
 /* ---- the ring driver, callable without the op layer ------------------------

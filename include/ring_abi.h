@@ -399,9 +399,15 @@ int ring_fusion_unpack_scaled(const ring_fusion_plan* plan, const void* fused, i
  * process ends. Limits: 1024 non-empty tensors and 268,435,456 four-byte
  * (134,217,728 eight-byte) elements per call, beyond which the call returns
  * RING_ERR_LIMIT and launches nothing. All calls on one GPU share that GPU's
- * array: calls on the same stream are ordered, calls that overlap on
- * different streams of one GPU race. Calls no hipMalloc / hipFree / hipMemcpy
- * (the first call on a device looks up the array's address). */
+ * array. Calls on the same stream are ordered by it; a call on another stream
+ * than the call before it on that GPU makes its stream wait, on the device,
+ * for an event recorded behind that call's kernels, so eager calls from
+ * several streams (one per rank, say) are safe, one after the other. A call
+ * on a stream that is being captured neither waits nor records (a wait would
+ * pull the other stream into the graph, and replays run whenever their owner
+ * launches them): whoever captures a call orders its replays against calls on
+ * other streams. Calls no hipMalloc / hipFree / hipMemcpy; the first call on
+ * a device looks up the array's address and creates the one event. */
 int ring_fusion_run_static(int unpack, const void* const* tensors, const size_t* counts, int k, int dtype,
                            void* fused, int divisor, void* stream);
 

@@ -15,6 +15,7 @@
 //     from a pre-staged one;
 //   * collectives only have GPU kernels. A CPU tensor is an error, not a
 //     silent host path.
+#include <algorithm>
 #include <atomic>
 #include <condition_variable>
 #include <cstring>
@@ -68,6 +69,13 @@ typedef std::unordered_map<std::string, std::vector<MPIRequest>> MessageTable;
 }  // namespace mpic
 
 // mpi_ops.cc:165-240 (MPIGlobalState), one per world instead of one per process.
+struct mpic_batch;
+// Links between worlds and the batches built on them (either may be destroyed first).
+static std::mutex g_batch_registry_mu;
+// The batches built on a world outlive it as objects (their owner destroys them), but can no
+// longer be submitted: mpic_batch_submit answers FAILED_PRECONDITION once this has run.
+static void DetachBatches(mpic_world* w);
+
 struct mpic_world {
   std::atomic_flag initialized_flag = ATOMIC_FLAG_INIT;
   std::condition_variable cv;       // initialisation
@@ -98,6 +106,9 @@ struct mpic_world {
   size_t fusion_bytes = 0;     // per rank
   bool flush_requested = false;  // with fusion on, a tick starts when the embedder asks
   std::map<std::string, ring_fusion_plan*> fusion_plans;  // keyed by the tensors' addresses and sizes
+  // the batches built on this world (mpic_batch_create), so that destroying the world can tell them:
+  // guarded by g_batch_registry_mu, not by mu
+  std::vector<mpic_batch*> batches;
 
   int expected_requests() const { return real_rank >= 0 ? 1 : size; }
 };
@@ -959,6 +970,7 @@ int mpic_world_destroy(mpic_world* w) {
     w->work_cv.notify_all();
     w->background_thread.join();
   }
+  DetachBatches(w);
   delete w;
   return MPIC_OK;
 }
@@ -1092,6 +1104,13 @@ int mpic_context_output(const mpic_context* c, int index, int* dtype, int* ndims
   return MPIC_OK;
 }
 
+int mpic_context_done(mpic_context* c) {
+  if (!c) return 1;
+  if (!c->started) return 1;
+  std::lock_guard<std::mutex> lock(c->mu);
+  return c->done ? 1 : 0;
+}
+
 int mpic_context_destroy(mpic_context* c) {
   if (!c) return MPIC_OK;
   if (c->started) {  // never free a context the background thread may still call back into
@@ -1156,7 +1175,9 @@ int mpic_context_wait_batch(mpic_context** contexts, int k, int destroy_ok, int*
 // ---- a rank's MPIAllreduce nodes, built once and run every step ---------------------------
 
 struct mpic_batch {
-  mpic_world* world = nullptr;
+  // null once the world has been destroyed: the nodes' contexts still point at it, so the batch
+  // may only be waited for and destroyed from then on
+  std::atomic<mpic_world*> world{nullptr};
   int rank = 0;
   // the graph's nodes: kernels are constructed once, as a TensorFlow graph's are,
   // and every submission is one execution of each
@@ -1166,6 +1187,14 @@ struct mpic_batch {
   std::condition_variable cv;
   int outstanding = 0;  // nodes of the current submission that have not called done()
 };
+
+}  // extern "C"
+static void DetachBatches(mpic_world* w) {
+  std::lock_guard<std::mutex> registry(g_batch_registry_mu);
+  for (mpic_batch* b : w->batches) b->world.store(nullptr);
+  w->batches.clear();
+}
+extern "C" {
 
 int mpic_batch_create(mpic_world* world, int rank, int k, const char* const* node_names, const int* dtypes,
                       const int* ndims, const int64_t* dims, const void* const* inputs, void* const* outputs,
@@ -1193,6 +1222,10 @@ int mpic_batch_create(mpic_world* world, int rank, int k, const char* const* nod
                                               const_cast<void*>(inputs[j]), false));
     b->contexts.back()->set_fused_divisor(divisor);
   }
+  {
+    std::lock_guard<std::mutex> registry(g_batch_registry_mu);
+    world->batches.push_back(b.get());
+  }
   *batch = b.release();
   return MPIC_OK;
 }
@@ -1201,6 +1234,10 @@ int mpic_batch_size(const mpic_batch* b) { return b ? static_cast<int>(b->kernel
 
 int mpic_batch_submit(mpic_batch* b) {
   if (!b) return MPIC_INVALID_ARGUMENT;
+  if (b->world.load() == nullptr) {
+    mpic::g_last_error = "the world this batch was built on has been destroyed";
+    return MPIC_FAILED_PRECONDITION;
+  }
   {
     std::lock_guard<std::mutex> guard(b->mu);
     if (b->outstanding != 0) {
@@ -1241,11 +1278,24 @@ const char* mpic_batch_message(const mpic_batch* b, int index) {
   return b->contexts[static_cast<size_t>(index)]->status().error_message().c_str();
 }
 
+int mpic_batch_busy(mpic_batch* b) {
+  if (!b) return 0;
+  std::lock_guard<std::mutex> guard(b->mu);
+  return b->outstanding != 0;
+}
+
 int mpic_batch_destroy(mpic_batch* b) {
   if (!b) return MPIC_OK;
   {  // never free nodes the background thread may still call back into
     std::unique_lock<std::mutex> lock(b->mu);
     b->cv.wait(lock, [b] { return b->outstanding == 0; });
+  }
+  {
+    std::lock_guard<std::mutex> registry(g_batch_registry_mu);
+    if (mpic_world* w = b->world.load()) {
+      auto it = std::find(w->batches.begin(), w->batches.end(), b);
+      if (it != w->batches.end()) w->batches.erase(it);
+    }
   }
   delete b;
   return MPIC_OK;

@@ -1955,22 +1955,35 @@ static __device__ __align__(256) unsigned char scratch[sizeof(StaticFusionTable)
 
 // `scratch` is a host-side stand-in in host code: the array's device address is
 // looked up once per device and only that pointer is ever handed to a kernel.
+// With it, per device: an event recorded behind the last call's launches and
+// the stream they went to, so that a call on another stream can be ordered
+// behind them (every call on a GPU works in the same array).
+struct ScratchState {
+  StaticFusionTable* ptr = nullptr;
+  hipEvent_t last_done = nullptr;   // created with the address, once per device
+  hipStream_t last_stream = nullptr;
+  bool recorded = false;            // last_done marks a call
+};
 std::mutex g_scratch_mutex;
-StaticFusionTable* g_scratch_ptr[64] = {};
+ScratchState g_scratch_state[64];
 
-int scratch_of_current_device(StaticFusionTable** out) {
+// g_scratch_mutex held.
+int scratch_of_current_device(ScratchState** out) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) { hip_fail(e); return RING_ERR_NO_DEVICE; }
   if (dev < 0 || dev >= 64) return RING_ERR_NO_DEVICE;
-  std::lock_guard<std::mutex> lock(g_scratch_mutex);
-  if (!g_scratch_ptr[dev]) {
+  ScratchState& st = g_scratch_state[dev];
+  if (!st.ptr) {
     void* p = nullptr;
     RING_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
     if (!p) return RING_ERR_HIP;
-    g_scratch_ptr[dev] = static_cast<StaticFusionTable*>(p);
+    hipEvent_t ev = nullptr;
+    RING_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+    st.last_done = ev;
+    st.ptr = static_cast<StaticFusionTable*>(p);
   }
-  *out = g_scratch_ptr[dev];
+  *out = &st;
   return RING_OK;
 }
 
@@ -2683,10 +2696,22 @@ int ring_fusion_run_static(int unpack, const void* const* tensors, const size_t*
   if (!fused || (reinterpret_cast<uintptr_t>(fused) & 15u)) return RING_ERR_ARGUMENT;
   const uint32_t ntiles = static_cast<uint32_t>((total + tile_elems - 1) / tile_elems);
 
-  StaticFusionTable* tab = nullptr;
-  int rc = scratch_of_current_device(&tab);
+  // One call at a time prepares launches on the array (the lock covers enqueueing, not execution).
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  ScratchState* st = nullptr;
+  int rc = scratch_of_current_device(&st);
   if (rc != RING_OK) return rc;
+  StaticFusionTable* tab = st->ptr;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  // The last call's kernels may still be reading the table this call is about to rewrite. On the same
+  // stream they are ordered ahead of it; on another stream this call's launches wait for the event recorded
+  // behind them. A stream that is being captured is left alone (a wait would pull the other stream's work
+  // into its graph, and a graph's replays run whenever its owner launches them): ordering a captured call
+  // against calls on other streams stays with the caller.
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  RING_HIP(hipStreamIsCapturing(s, &capture));
+  const bool eager = capture == hipStreamCaptureStatusNone;
+  if (eager && st->recorded && st->last_stream != s) RING_HIP(hipStreamWaitEvent(s, st->last_done, 0));
 
   // the table, kTableChunk tensors per launch; the fused-buffer offsets are the running sum of the counts
   TableChunk chunk;
@@ -2712,7 +2737,15 @@ int ring_fusion_run_static(int unpack, const void* const* tensors, const size_t*
                      tile_elems, total, static_cast<uint32_t>(esz));
   RING_HIP(hipGetLastError());
   const FusionView view{dtype, esz, ntiles, total, tab->offsets, tab->ptrs, tab->tiles, m};
-  return fusion_run(view, fused, stream, !unpack, divisor);
+  rc = fusion_run(view, fused, stream, !unpack, divisor);
+  if (eager) {
+    // also after a failed launch: the table kernels above are enqueued and the next call must not overtake them
+    const hipError_t e = hipEventRecord(st->last_done, s);
+    if (e != hipSuccess) return rc != RING_OK ? rc : hip_fail(e);
+    st->last_stream = s;
+    st->recorded = true;
+  }
+  return rc;
 }
 
 }  // extern "C"

@@ -271,6 +271,8 @@ class Session:
         Returns one handle per tensor."""
         inputs = [t.contiguous() for t in tensors]
         self._order_after_producers(inputs)
+        with self._lock:
+            counters_before = dict(self._counters)
         node_names = [self._node_name(r, 'MPIAllreduce', name) for name in names]
         # the outputs: one allocation per element type, cut into the tensors' shapes
         outputs = [None] * len(inputs)
@@ -281,7 +283,18 @@ class Session:
             flat = torch.empty(sum(inputs[j].numel() for j in idx), dtype=dtype, device=device)
             for j, piece in zip(idx, flat.split([inputs[j].numel() for j in idx])):
                 outputs[j] = piece.view(inputs[j].shape)
-        batch = _plugin.PendingBatch(self._world, r, node_names, inputs, outputs, divisor)
+        try:
+            batch = _plugin.PendingBatch(self._world, r, node_names, inputs, outputs, divisor)
+        except OpError:
+            # nothing was filed: give the names back, or this rank's next unnamed op would carry another
+            # name than the same op on the ranks whose call succeeded
+            with self._lock:
+                for key in [k for k in self._counters if k[0] == r]:
+                    if key in counters_before:
+                        self._counters[key] = counters_before[key]
+                    else:
+                        del self._counters[key]
+            raise
         batch.rank = r
         batch.next_op = batch.on_done = batch.handle = batch.fail_handle = None
         batch.lock = threading.Lock()
@@ -645,6 +658,12 @@ class AllreduceBatch:
         if self in self.session._batches:
             self.session._batches.remove(self)
 
+    def __del__(self):
+        try:
+            self._c.close(wait=False)
+        except Exception:
+            pass
+
 
 def prepare_allreduce_batch(tensors, average=True, inplace=False):
     """An AllreduceBatch for the current rank (not in the reference, where
@@ -677,6 +696,8 @@ class DistributedOptimizer:
         self._fused = None      # (FusionPlan, fused buffer, grads) while a fused allreduce is in flight
         self._batch = None      # the dense gradients' allreduces, built once (AllreduceBatch)
         self._batch_key = None
+        self._stale = []        # batches replaced while their last submission was still pending
+        self._rebuilt = 0       # steps in a row that presented other gradient tensors than the step before
 
     @property
     def param_groups(self):
@@ -720,12 +741,28 @@ class DistributedOptimizer:
         if session._immediate or not grads or not all(g.is_cuda and g.is_contiguous() for g in grads):
             return allreduce_batch(grads)
         key = (id(session),) + tuple(g.data_ptr() for g in grads) + tuple(g.shape for g in grads)
-        if self._batch is None or self._batch_key != key:
-            if self._batch is not None and self._batch.completed:
+        for old in [b for b in self._stale if b.completed]:
+            old.close()
+            self._stale.remove(old)
+        if self._batch is not None and self._batch_key == key:
+            self._rebuilt = 0
+            return self._batch.submit()
+        if self._batch is not None:
+            # other tensors than last step's: the nodes built for those are of no further use
+            if self._batch.completed:
                 self._batch.close()
-            # in place: the averaged gradient takes the gradient's memory, so tensors that stay
-            # where they are between steps (zero_grad(set_to_none=False)) keep the batch valid
-            self._batch, self._batch_key = AllreduceBatch(grads, inplace=True), key
+            else:
+                self._stale.append(self._batch)
+            self._batch = self._batch_key = None
+            self._rebuilt += 1
+        if self._rebuilt >= 2:
+            # the gradients move every step (zero_grad(set_to_none=True) frees them): building nodes for
+            # tensors that will not be seen again costs more than it saves, and would keep them alive
+            return allreduce_batch(grads)
+        # in place: the averaged gradient takes the gradient's memory (p.grad then holds the average
+        # already when compute_gradients returns), so tensors that stay where they are between steps
+        # (zero_grad(), whose default here is set_to_none=False) keep the batch valid
+        self._batch, self._batch_key = AllreduceBatch(grads, inplace=True), key
         return self._batch.submit()
 
     def _compute_fused(self, params):
@@ -782,8 +819,18 @@ class DistributedOptimizer:
             closure()
         return self.apply_gradients(self.compute_gradients())
 
-    def zero_grad(self, *args, **kwargs):
-        return self._optimizer.zero_grad(*args, **kwargs)
+    def zero_grad(self, set_to_none=False):
+        """Clears the gradients. Unlike torch's own default the tensors are kept
+        and zeroed: gradients that stay where they are let the next step run the
+        allreduce nodes built for them again instead of building new ones."""
+        return self._optimizer.zero_grad(set_to_none=set_to_none)
+
+    def close(self):
+        """Destroys the allreduce nodes this optimizer has built (a closing session does the same)."""
+        for b in self._stale + ([self._batch] if self._batch is not None else []):
+            if b.completed:
+                b.close()
+        self._stale, self._batch, self._batch_key = [], None, None
 
     def state_dict(self):
         return self._optimizer.state_dict()

@@ -30,10 +30,10 @@ EXPORTS = (
     "mpic_world_size", "mpic_world_stream", "mpic_world_set_option", "mpic_world_set_fusion_buffer",
     "mpic_world_flush", "mpic_stage_peers",
     "mpic_context_create", "mpic_context_add_input", "mpic_context_set_divisor", "mpic_context_compute", "mpic_context_wait",
-    "mpic_context_message", "mpic_context_num_outputs", "mpic_context_output", "mpic_context_destroy",
+    "mpic_context_message", "mpic_context_num_outputs", "mpic_context_output", "mpic_context_destroy", "mpic_context_done",
     "mpic_allreduce_batch", "mpic_context_wait_batch",
     "mpic_batch_create", "mpic_batch_size", "mpic_batch_submit", "mpic_batch_wait", "mpic_batch_message",
-    "mpic_batch_destroy",
+    "mpic_batch_destroy", "mpic_batch_busy",
     "mpic_ring_allreduce_prestaged", "mpic_ring_allreduce_direct_prestaged", "mpic_ring_allreduce_fused_prestaged",
     "mpic_ring_allgather_prestaged", "mpic_ring_allreduce_all_ranks",
     "mpic_ring_allgather_all_ranks", "mpic_ring_allreduce_transport", "mpic_ring_allgather_transport",
@@ -140,6 +140,7 @@ def load_library(name="libmpi_collectives.so", op_list=None):
             "mpic_context_num_outputs": (ci, [vp]),
             "mpic_context_output": (ci, [vp, ci, pint, pint, p64, pvp]),
             "mpic_context_destroy": (ci, [vp]),
+            "mpic_context_done": (ci, [vp]),
             "mpic_allreduce_batch": (ci, [vp, ci, ci, ctypes.POINTER(cp), pint, pint, p64, pvp, pvp, ci, pvp]),
             "mpic_context_wait_batch": (ci, [pvp, ci, ci, pint]),
             "mpic_batch_create": (ci, [vp, ci, ci, ctypes.POINTER(cp), pint, pint, p64, pvp, pvp, ci, pvp]),
@@ -148,6 +149,7 @@ def load_library(name="libmpi_collectives.so", op_list=None):
             "mpic_batch_wait": (ci, [vp, pint]),
             "mpic_batch_message": (cp, [vp, ci]),
             "mpic_batch_destroy": (ci, [vp]),
+            "mpic_batch_busy": (ci, [vp]),
             "mpic_ring_allreduce_prestaged": (ci, [ci, ci, ci, vp, vp, sz, pvp, pvp, vp, ci]),
             "mpic_ring_allreduce_direct_prestaged": (ci, [ci, ci, ci, vp, vp, sz, pvp, pvp, vp, ci]),
             "mpic_ring_allreduce_fused_prestaged": (ci, [vp, ci, ci, vp, pvp, pvp, vp, ci]),
@@ -358,6 +360,22 @@ class PendingBatch:
     def outputs(self):
         return self._outputs
 
+    def close(self, wait=True):
+        """Destroys the contexts that wait() has not destroyed (a batch that was never waited
+        for). mpic_context_destroy waits for a node that is still running; with wait=False such
+        a node is left alone (and leaks until its world goes)."""
+        L = lib()
+        for j in range(self._k):
+            if self._contexts[j] and (wait or L.mpic_context_done(self._contexts[j])):
+                L.mpic_context_destroy(self._contexts[j])
+                self._contexts[j] = None
+
+    def __del__(self):
+        try:
+            self.close(wait=False)      # a finaliser must not block on ranks that never submitted
+        except Exception:
+            pass
+
 
 class Batch:
     """k MPIAllreduce nodes of one rank built once and run every step
@@ -404,7 +422,13 @@ class Batch:
     def outputs(self):
         return self._outputs
 
-    def close(self):
-        if self._handle:
+    def close(self, wait=True):
+        if self._handle and (wait or not lib().mpic_batch_busy(self._handle)):
             lib().mpic_batch_destroy(self._handle)      # waits for a submission that is still running
             self._handle = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close(wait=False)      # a finaliser must not block on ranks that never submitted
+        except Exception:
+            pass

@@ -1226,6 +1226,56 @@ def test_distributed_optimizer_builds_its_nodes_once(oracle):
         assert built[1] == built[2], "the nodes were rebuilt although the gradients stayed in place"
 
 
+@pytest.mark.parametrize("set_to_none", [None, True])
+def test_distributed_optimizer_with_default_and_freed_gradients(oracle, set_to_none):
+    """zero_grad() as a training loop calls it. The wrapper's default keeps the
+    gradient tensors (set_to_none=False), so the nodes are built once; with
+    set_to_none=True every backward allocates new gradients, and after two
+    steps of rebuilding the optimizer stops building nodes for tensors it will
+    not see again. Either way every step's gradients are the ring's averages,
+    and the session's list of batches does not grow with the steps."""
+    n, steps = 2, 5
+    torch.manual_seed(5)
+    base = torch.nn.Linear(11, 7).cuda()
+    replicas, opts = [], []
+    for r in range(n):
+        m = torch.nn.Linear(11, 7).cuda()
+        m.load_state_dict(base.state_dict())
+        replicas.append(m)
+        opts.append(mpi.DistributedOptimizer(torch.optim.SGD(m.parameters(), lr=0.05)))
+    with mpi.Session(size=n) as session:
+        live = []
+        for step in range(steps):
+            local, gvs = [], []
+            for r in range(n):
+                with session.as_rank(r):
+                    if set_to_none is None:
+                        opts[r].zero_grad()
+                    else:
+                        opts[r].zero_grad(set_to_none=set_to_none)
+                    x = torch.randn(9, 11, generator=torch.Generator().manual_seed(10 * step + r)).cuda()
+                    replicas[r](x).square().mean().backward()
+                    local.append([G.host(p.grad).reshape(-1).copy() for p in replicas[r].parameters()])
+                    gvs.append(opts[r].compute_gradients())
+            session.run()
+            for r in range(n):
+                with session.as_rank(r):
+                    opts[r].apply_gradients(gvs[r])
+            live.append(len(session._batches))
+            for j in range(len(local[0])):
+                want = oracle.ring_allreduce([local[r][j] for r in range(n)])[0] / np.float32(n)
+                for r in range(n):
+                    G.assert_same_bits(G.host(list(replicas[r].parameters())[j].grad).reshape(-1), want,
+                                       "step %d rank %d gradient %d" % (step, r, j))
+        if set_to_none is None:
+            assert live == [n] * steps, live                  # one batch per rank, built at the first step
+        else:
+            assert max(live) <= 2 * n and live[-1] <= n, live  # replaced, closed, and given up after two rebuilds
+        for o in opts:
+            o.close()
+        assert session._batches == []
+
+
 @pytest.mark.parametrize("dtype", G.DTYPES)
 def test_fused_allreduce_of_resident_ranks_without_a_fused_buffer(oracle, dtype):
     """ring_fusion_allreduce_all: one launch over the tensors of all ranks gives

@@ -570,3 +570,43 @@ def test_launch_form_query_follows_the_options_and_checks_its_arguments():
         A.describe_rows_launch(rows, A.I32, A.ROLE_ALLGATHER, 0)
     with pytest.raises(A.RingError):
         A.describe_unpack_launch(1 << 20, 10, A.F32, -1, 256)
+
+
+def test_a_batch_outlives_its_world_but_cannot_be_submitted():
+    """mpic_batch_submit after mpic_world_destroy answers FAILED_PRECONDITION instead of
+    walking into the freed world; the batch can still be waited for and destroyed."""
+    L = _plugin.lib()
+    world = ctypes.c_void_p()
+    assert L.mpic_world_create(2, ctypes.byref(world)) == _plugin.OK
+    names = (ctypes.c_char_p * 1)(b"grad")
+    dtypes = (ctypes.c_int * 1)(_plugin.DT_FLOAT)
+    ndims = (ctypes.c_int * 1)(1)
+    dims = (ctypes.c_int64 * 1)(16)
+    ins = (ctypes.c_void_p * 1)(0x1000)          # never dereferenced: nothing is submitted
+    outs = (ctypes.c_void_p * 1)(0x2000)
+    batches = []
+    for _ in range(2):
+        b = ctypes.c_void_p()
+        assert L.mpic_batch_create(world, 0, 1, names, dtypes, ndims, dims, ins, outs, 0, ctypes.byref(b)) == _plugin.OK
+        batches.append(b)
+    assert L.mpic_batch_busy(batches[0]) == 0
+    assert L.mpic_batch_destroy(batches[0]) == _plugin.OK      # before its world: unregisters itself
+    assert L.mpic_world_destroy(world) == _plugin.OK
+    rc = L.mpic_batch_submit(batches[1])
+    assert _plugin.error_for(rc, "").__class__ is mpi.FailedPreconditionError
+    assert b"destroyed" in L.mpic_last_error()
+    assert L.mpic_batch_wait(batches[1], None) == _plugin.OK
+    assert L.mpic_batch_destroy(batches[1]) == _plugin.OK      # after its world
+
+
+def test_a_batch_that_fails_gives_its_node_names_back():
+    """An entry the plugin cannot describe (more than 8 dimensions) fails the whole allreduce_batch
+    call and files nothing; the auto-generated node names it took are given back, so the rank's
+    next unnamed op still matches the other ranks'."""
+    with mpi.Session(size=2) as session:
+        with session.as_rank(0):
+            good = torch.zeros(4)
+            with pytest.raises(mpi.OpError):
+                mpi.allreduce_batch([good, torch.zeros((1,) * 9), good])
+            assert session._node_name(0, 'MPIAllreduce', None) == 'MPIAllreduce'
+            assert session._node_name(0, 'MPIAllreduce', None) == 'MPIAllreduce_1'

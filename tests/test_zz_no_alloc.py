@@ -117,3 +117,42 @@ def test_limits_and_arguments():
     ring_abi.fusion_run_static(False, [], [], ring_abi.F32, 0, 0, None)
     ring_abi.fusion_run_static(True, [0, 0], [0, 0], ring_abi.I64, 0, 4, None)
     sync()
+
+
+def test_calls_on_different_streams_are_ordered_and_nothing_is_allocated():
+    """Two streams take turns on the one array with no synchronisation in between: every
+    call's stream waits (on the device) for the call before it, so a table is never rewritten
+    under a running pack. And the property the entry point exists for: free device memory is
+    the same after warmed-up calls as before them."""
+    require_gpu()
+    rng = np.random.default_rng(21)
+    big = [int(np.prod(s)) for s in resnet50_shapes()]
+    small = [int(c) for c in rng.integers(1, 3000, 200)]
+    sets = []
+    for counts in (big, small):
+        views, keep = _tensor_set(rng, counts, np.float32)
+        ptrs = [v.data_ptr() for v in views]
+        want = torch.cat([v.reshape(-1) for v in views])
+        sets.append((counts, ptrs, want, keep))
+    streams = [ring_abi.stream_create(), ring_abi.stream_create()]
+    outs = [[torch.zeros(int(sum(c)), device="cuda") for _ in range(6)] for c, _, _, _ in sets]
+    try:
+        # warm-up: the array's address and the event exist from here on
+        for which, (counts, ptrs, _w, _k) in enumerate(sets):
+            ring_abi.fusion_run_static(False, ptrs, counts, ring_abi.F32, outs[which][0].data_ptr(), 0, streams[which])
+        for s in streams:
+            ring_abi.stream_synchronize(s)
+        sync()
+        free_before = torch.cuda.mem_get_info()[0]
+        for i in range(6):
+            for which, (counts, ptrs, _w, _k) in enumerate(sets):
+                ring_abi.fusion_run_static(False, ptrs, counts, ring_abi.F32, outs[which][i].data_ptr(), 0, streams[which])
+        for s in streams:
+            ring_abi.stream_synchronize(s)
+        assert torch.cuda.mem_get_info()[0] == free_before, "a call allocated or freed device memory"
+        for which, (_c, _p, want, _k) in enumerate(sets):
+            for i in range(6):
+                assert torch.equal(outs[which][i], want), "pack %d of set %d, calls interleaved on two streams" % (i, which)
+    finally:
+        for s in streams:
+            ring_abi.stream_destroy(s)
