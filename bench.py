@@ -252,11 +252,13 @@ class StreamFloors(Workload):
     """What the chip gives ONE direction at the sizes of an allreduce's two copy
     launches, next to the launches themselves: the copy source read and nothing
     written, the copy destination written and nothing read, the in->out copy;
-    the same three for the rows of the allgather phase. A copy runs no faster
-    than its two directions one after the other, so read-only + write-only is
-    the floor of the copy at that size on this chip. Buffers rotate as in the
-    allreduce workload; every phase is one launch (ring_probe_stream for the
-    one-directional ones), timed by events in its dispatch."""
+    the same three for the rows of the allgather phase (up to 8 rows: a larger
+    ring shows its allgather without the one-directional launches). A copy runs
+    no faster than its two directions one after the other, so read-only +
+    write-only is the floor of the copy at that size on this chip. Buffers
+    rotate as in the allreduce workload; every phase is one launch
+    (ring_probe_stream for the one-directional ones), timed by events in its
+    dispatch."""
 
     def __init__(self, name, np_name, count, n, nsets, what):
         self.inner = r = RingAllreduce(name, np_name, count, n, nsets, what)
@@ -264,38 +266,42 @@ class StreamFloors(Workload):
         self.ring_abi, self.R = r.ring_abi, r.R
         esz = r.esz
         up = lambda p: (p + 15) & ~15       # the probe wants 16-byte aligned pointers; a ragged start loses < 16 bytes
+        self.probe_rows = n - 1 <= 8
         for s in r.sets:
             out = s["out"].data_ptr()
             s["probe_copy"] = [(out, s["inp"].data_ptr(), None, count)]
-            s["probe_ag"] = [(up(out + r.starts[g] * esz), t.data_ptr(), None, r.sizes[g] - 16 // esz)
+            s["probe_ag"] = [(up(out + r.starts[g] * esz), up(t.data_ptr()), None, r.sizes[g] - 16 // esz)
                              for g, t in zip(s["ag_seg"], s["ag"])]
         ag_bytes = sum(r.sizes[g] for g in r.sets[0]["ag_seg"]) * esz
-        self.phases = (
+        # (what runs, phase of the inner workload or probe mode, rows)
+        self.plan = [("probe", 0, "probe_copy"), ("probe", 1, "probe_copy"), ("phase", 0, None)]
+        self.phases = [
             ("read_only_copy_source", count * esz, "stream_probe_kernel<read> (1 row, %d bytes)" % (count * esz)),
             ("write_only_copy_destination", count * esz, "stream_probe_kernel<write> (1 row, %d bytes)" % (count * esz)),
-            r.phases[0],
-            ("read_only_allgather_sources", ag_bytes, "stream_probe_kernel<read> (%d rows, %d bytes)" % (n - 1, ag_bytes)),
-            ("write_only_allgather_destinations", ag_bytes,
-             "stream_probe_kernel<write> (%d rows, %d bytes)" % (n - 1, ag_bytes)),
-            r.phases[2])
+            r.phases[0]]
+        if self.probe_rows:
+            self.plan += [("probe", 0, "probe_ag"), ("probe", 1, "probe_ag")]
+            self.phases += [
+                ("read_only_allgather_sources", ag_bytes, "stream_probe_kernel<read> (%d rows, %d bytes)" % (n - 1, ag_bytes)),
+                ("write_only_allgather_destinations", ag_bytes,
+                 "stream_probe_kernel<write> (%d rows, %d bytes)" % (n - 1, ag_bytes))]
+        self.plan.append(("phase", 2, None))
+        self.phases = tuple(self.phases + [r.phases[2]])
         self.dominant = 2
         self.description = ("one direction at a time against the copy launches of: " + what)
 
     def launch_phase(self, k, i, stream):
-        # the probes work on another buffer set than the copies of the same step, so that no copy
-        # finds in a cache what a probe has just touched
-        s, A = self.inner.sets[(k + self.nsets // 2) % self.nsets], self.ring_abi
-        if i in (0, 1):
-            A.probe_stream(s["probe_copy"], self.inner.code, i, stream)
-        elif i == 2:
-            self.inner.launch_phase(k, 0, stream)
-        elif i in (3, 4):
-            A.probe_stream(s["probe_ag"], self.inner.code, i - 3, stream)
+        kind, arg, rows = self.plan[i]
+        if kind == "phase":
+            self.inner.launch_phase(k, arg, stream)
         else:
-            self.inner.launch_phase(k, 2, stream)
+            # the probes work on another buffer set than the copies of the same step, so that no copy
+            # finds in a cache what a probe has just touched
+            s = self.inner.sets[(k + self.nsets // 2) % self.nsets]
+            self.ring_abi.probe_stream(s[rows], self.inner.code, arg, stream)
 
     def launch_step(self, k, stream, fused=False):
-        for i in range(6):
+        for i in range(len(self.plan)):
             self.launch_phase(k, i, stream)
 
     def check(self, k):
@@ -739,9 +745,9 @@ def make_workload(name):
                              "12 buffer sets rotated" % {"i32": "int32", "i64": "int64"}[dt])
     if name.startswith("floors_"):
         _, dt, size, ranks = name.split("_")
-        count = {"64MiB": 16 * 1024 * 1024, "10000019": 10_000_019}[size]
+        count = {"64MiB": 16 * 1024 * 1024, "10000019": 10_000_019, "1GiB": 268_435_456}[size]
         n = int(ranks[1:])
-        return StreamFloors(name, dt, count, n, 8 if n == 8 else 12,
+        return StreamFloors(name, dt, count, n, {8: 8, 6: 12, 64: 2}[n],
                             "%s ring allreduce of %d elements at N=%d (in->out copy of %d bytes; allgather copies of %d rows)"
                             % (dt, count, n, count * (8 if dt == "i64" else 4), n - 1))
     if name == "allreduce_f32_1MiB_n8":
@@ -771,7 +777,7 @@ WORKLOADS = ("allreduce_f32_64MiB_n8", "allreduce_i32_10000019_n6", "allreduce_i
              "allreduce_f32_64MiB_n8_direct", "fused_resnet50_n8_no_passes",
              "fused_resnet50_n8_no_passes_direct", "allreduce_f32_64MiB_all_ranks_n8",
              "fused_resnet50_all_ranks_n8",
-             "floors_f32_64MiB_n8", "floors_i32_10000019_n6", "floors_i64_10000019_n6")
+             "floors_f32_64MiB_n8", "floors_i32_10000019_n6", "floors_i64_10000019_n6", "floors_f32_1GiB_n64")
 
 
 def cpu_baseline(w):
@@ -863,7 +869,7 @@ def main():
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures the per-rank data path on ONE GPU (the ring's N ranks are virtual); "
                  "--gpus %d is not supported" % args.gpus)
-    big = args.workload == "allreduce_f32_1GiB_n64"
+    big = args.workload in ("allreduce_f32_1GiB_n64", "floors_f32_1GiB_n64")
     steps = args.steps if args.steps is not None else (200 if big else 2000)
     warmup = args.warmup if args.warmup is not None else (20 if big else 200)
 
