@@ -437,6 +437,17 @@ typedef struct ring_fusion_span {
   void* out;            /* gather: element 0 of the span's destination; scatter: unused */
 } ring_fusion_span;
 int ring_fusion_gather(const ring_fusion_plan* plan, const ring_fusion_span* spans, int n_spans, void* stream);
+/* The form (enum ring_form) ring_fusion_scatter takes for these spans on a GPU
+ * of `cus` compute units, without a GPU. Finished segments that were received
+ * in place lie in one buffer, each at its own offset (every `incoming` less
+ * `begin` elements is the same 16-byte aligned address, and the spans, empty
+ * ones aside, cover the fused space end to end): the scatter is then the
+ * unpack of that buffer and takes the unpack's launch
+ * (ring_describe_unpack_launch: in registers from 1 to 112 MiB). Segments in
+ * slots of their own are scattered as tiles (RING_FORM_TILES). Same results
+ * either way. */
+int ring_describe_scatter_launch(const ring_fusion_plan* plan, const ring_fusion_span* spans, int n_spans,
+                                 int divisor, int cus, int* form);
 int ring_fusion_scatter(const ring_fusion_plan* plan, const ring_fusion_span* spans, int n_spans, int divisor,
                         void* stream);
 

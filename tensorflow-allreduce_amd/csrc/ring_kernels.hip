@@ -2773,6 +2773,31 @@ int launch_fusion_spans(const ring_fusion_plan* p, const FusionSpanTable& tab, u
   return RING_OK;
 }
 
+// The finished segments of a scatter that were received in place lie in ONE buffer, each at its own offset
+// (piece k at buffer + begin[k]): the scatter is then the unpack of that buffer, and takes the unpack's
+// launch, in registers where the unpack would (a scatter from separate slots was built in that form twice,
+// its source per round looked up in LDS or worked out on the scalar unit from the kernel arguments: 37.8 and
+// 42.5 us for the ResNet-50 set against 36.6-36.9 us as tiles and 33.4 us for the unpack, because a lane's
+// 112 loads then wait for a lookup each instead of going out back to back; not kept). Returns that buffer when
+// the spans (empty ones aside) cover the plan's fused space end to end and every `incoming` less `begin`
+// elements is the same 16-byte aligned address, else null.
+const void* scatter_in_place_buffer(const ring_fusion_plan* p, const ring_fusion_span* spans, int n) {
+  uintptr_t buffer = 0;
+  uint64_t at = 0;
+  bool any = false;
+  for (int i = 0; i < n; i++) {
+    const ring_fusion_span& sp = spans[i];
+    if (sp.count == 0) continue;
+    if (sp.begin != at || !sp.incoming) return nullptr;
+    const uintptr_t base = reinterpret_cast<uintptr_t>(sp.incoming) - sp.begin * p->esz;
+    if ((base & 15u) || (any && base != buffer)) return nullptr;
+    buffer = base;
+    any = true;
+    at = sp.begin + sp.count;
+  }
+  return (any && at == p->total) ? reinterpret_cast<const void*>(buffer) : nullptr;
+}
+
 // Checks the spans (sorted, disjoint, inside the plan, operands present and
 // element-aligned) and launches them in tables of kMaxFusionSpans.
 int fusion_spans_run(const ring_fusion_plan* p, const ring_fusion_span* spans, int n, bool gather, int divisor,
@@ -2781,6 +2806,10 @@ int fusion_spans_run(const ring_fusion_plan* p, const ring_fusion_span* spans, i
   const uint64_t tile_elems = static_cast<uint64_t>(kFusionTileVecs) * (16 / p->esz);
   hipStream_t s = static_cast<hipStream_t>(stream);
   uint64_t previous_end = 0;
+  if (!gather) {
+    if (const void* buffer = scatter_in_place_buffer(p, spans, n))
+      return fusion_run(p, const_cast<void*>(buffer), stream, false, divisor);
+  }
   int i = 0;
   while (i < n) {
     FusionSpanTable tab;
@@ -2951,6 +2980,15 @@ int ring_fusion_allreduce_all(const ring_fusion_plan* const* in_plans, const rin
 #undef RING_FUSED_ALL_NT
 #undef RING_FUSED_ALL
   RING_HIP(hipGetLastError());
+  return RING_OK;
+}
+
+int ring_describe_scatter_launch(const ring_fusion_plan* plan, const ring_fusion_span* spans, int n_spans, int divisor,
+                                 int cus, int* form) {
+  if (!plan || !form || n_spans < 0 || (n_spans > 0 && !spans) || divisor < 0 || cus < 1) return RING_ERR_ARGUMENT;
+  *form = RING_FORM_TILES;
+  if (scatter_in_place_buffer(plan, spans, n_spans))
+    *form = choose_unpack_form(plan->total, plan->m, plan->esz, plan->dtype == RING_F32, divisor, tuning(), cus).form;
   return RING_OK;
 }
 

@@ -32,7 +32,7 @@ EXPORTS = (
     "ring_fusion_pack", "ring_fusion_unpack", "ring_fusion_unpack_scaled", "ring_fusion_gather",
     "ring_fusion_scatter", "ring_fusion_fold_scatter", "ring_scale", "ring_fusion_run_static",
     "ring_describe_rows_launch", "ring_describe_unpack_launch", "ring_probe_stream",
-    "ring_get_device", "ring_set_device",
+    "ring_get_device", "ring_set_device", "ring_describe_scatter_launch",
 )
 
 
@@ -152,6 +152,7 @@ def lib():
             "ring_describe_rows_launch": (ci, [ctypes.POINTER(Row), ci, ci, ci, ci, pint]),
             "ring_describe_unpack_launch": (ci, [ctypes.c_uint64, ci, ci, ci, ci, pint]),
             "ring_probe_stream": (ci, [ctypes.POINTER(Row), ci, ci, ci, vp]),
+            "ring_describe_scatter_launch": (ci, [vp, ctypes.POINTER(FusionSpan), ci, ci, ci, pint]),
             "ring_get_device": (ci, [pint]),
             "ring_set_device": (ci, [ci]),
         }

@@ -29,6 +29,7 @@
 namespace {
 
 std::mt19937_64 g_rng(12345);
+int g_scatters_in_registers = 0;  // scatters that took the form with their payload in registers
 
 template <typename T> int code();
 template <> int code<float>() { return RING_F32; }
@@ -434,6 +435,29 @@ void test_fusion(const std::vector<size_t>& counts, int divisor, int n_ranks) {
     OK(ring_fusion_scatter(p2, spans.data(), n_ranks, divisor, nullptr));
     check_tensors(out, scattered, "scatter");
     OK(ring_fusion_plan_destroy(p2));
+    {
+      // the finished segments received in place, all in one buffer at their own offsets: the scatter is
+      // the unpack of that buffer and takes its launch (here forced into the form with the payload in registers)
+      Buf<T> arrivals(total, 0, false);
+      std::vector<ring_fusion_span> in_place;
+      for (int g = 0; g < n_ranks; g++) {
+        memcpy(arrivals.p + starts[g], incoming[g].p, sizes[g] * sizeof(T));
+        in_place.push_back(ring_fusion_span{starts[g], sizes[g], arrivals.p + starts[g], nullptr});
+      }
+      std::vector<Buf<T>> out2;
+      std::vector<const void*> out2_ptrs;
+      fresh(out2, out2_ptrs);
+      ring_fusion_plan* p4 = nullptr;
+      OK(ring_fusion_plan_create(out2_ptrs.data(), counts.data(), static_cast<int>(counts.size()), code<T>(), &p4));
+      CHECK(ring_set_option("phased_copy", 1) == RING_OK);
+      int form = -1;
+      OK(ring_describe_scatter_launch(p4, in_place.data(), n_ranks, divisor, 4, &form));
+      if (form != RING_FORM_TILES) g_scatters_in_registers++;
+      OK(ring_fusion_scatter(p4, in_place.data(), n_ranks, divisor, nullptr));
+      CHECK(ring_set_option("phased_copy", -1) == RING_OK);
+      check_tensors(out2, scattered, "scatter of segments received in place");
+      OK(ring_fusion_plan_destroy(p4));
+    }
     // the direct form in one launch: segment `own` folded from staged copies and the tensors (last), its sum
     // to the wire buffer, the quotient into the tensors; the other segments scattered
     for (int own : {n_ranks / 2, n_ranks - 1}) {
@@ -525,6 +549,10 @@ void run_all(const char* name) {
   test_fusion<T>({17}, 3, 2);
   test_fusion<T>({}, 0, 2);
   test_fusion<T>({100003, 1, 2, 50001, 0, 4096, 3}, 4, 2);  // tensor ends that cut 16-byte groups, divided by a power of two
+  // segments whose ends cut 16-byte groups (154,107 elements in 3, 5 and 7 segments), received in place and scattered from there
+  test_fusion<T>({100003, 1, 2, 50001, 0, 4096, 3, 1}, 0, 3);
+  test_fusion<T>({100003, 1, 2, 50001, 0, 4096, 3, 1}, 2, 5);
+  test_fusion<T>({7, 100003, 1, 2, 50001, 0, 4096, 1}, 4, 7);
 }
 
 }  // namespace
@@ -534,6 +562,7 @@ int main() {
   run_all<float>("float32");
   run_all<int32_t>("int32");
   run_all<int64_t>("int64");
+  CHECK(g_scatters_in_registers >= 9);  // the three cases made for it, per element type, at least
   printf("kernel emulation: ok\n");
   return 0;
 }

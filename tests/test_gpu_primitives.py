@@ -655,6 +655,77 @@ def test_fusion_gather_and_scatter_spans(dtype):
         plan.close()
 
 
+@pytest.mark.parametrize("dtype", G.DTYPES)
+def test_scatter_of_segments_received_in_place(dtype):
+    """Finished segments that lie in one buffer, each at its own offset (received in
+    place), are scattered by the unpack of that buffer, in registers where the
+    unpack would be; segments in slots of their own, a gap, or a buffer that is not
+    16-byte aligned take the tiles. Same tensors either way, against numpy on the
+    concatenation: segment ends that cut 16-byte groups, the full ResNet-50 set at
+    N=8 with the divide, a divisor the registers do not take."""
+    import torch
+    rng = np.random.default_rng(47)
+    code = G.NP2ABI[np.dtype(dtype)]
+    tdt = G.NP2TORCH[np.dtype(dtype)]
+    esz = np.dtype(dtype).itemsize
+    resnet = [int(np.prod(s)) for s in G.resnet50_shapes()]
+    cases = [(resnet, 8, 8), (resnet[:60], 6, 0), ([100_003, 1, 2, 50_001, 0, 4096, 3, 1], 5, 2),
+             ([7, 300_017, 64, 64, 99_991], 3, 4), (resnet[:100], 7, 6)]
+    for counts, n, divisor in cases:
+        total = sum(counts)
+        hosts = [G.random_array(rng, c, dtype) for c in counts]
+        if dtype != np.float32:
+            for h in hosts:
+                h[: h.size // 2] = -np.abs(h[: h.size // 2])              # negative values for the floor division
+        devs = [G.dev(h, int(rng.integers(0, 4))) for h in hosts]
+        plan = ring_abi.FusionPlan([d[0].data_ptr() if c else None for d, c in zip(devs, counts)], counts, code)
+        sizes, starts = ring_abi.segment_table(total, n)
+        incoming = [G.random_array(rng, c, dtype) for c in sizes]
+        want = np.concatenate(incoming)
+        if divisor:
+            with np.errstate(all="ignore"):
+                want = (want / np.float32(divisor) if dtype == np.float32 else want // dtype(divisor)).astype(dtype)
+        unpack_form = ring_abi.describe_unpack_launch(total, sum(1 for c in counts if c), code, divisor, 256)
+
+        def form_of(spans):
+            form = ctypes.c_int(-1)
+            ring_abi.check(ring_abi.lib().ring_describe_scatter_launch(plan._h, spans[0], spans[1], divisor, 256,
+                                                                        ctypes.byref(form)), "describe")
+            return form.value
+
+        def run(pointers, what, expect_form):
+            spans = ring_abi.make_spans([(starts[g], sizes[g], pointers[g], None) for g in range(n)])
+            assert form_of(spans) == expect_form, (what, form_of(spans), expect_form)
+            for d in devs:
+                d[0].zero_()
+            plan.scatter(spans, divisor, None)
+            G.sync()
+            got = np.concatenate([G.host(d[0]) for d in devs])
+            G.assert_same_bits(got, want, "%s: %d elements in %d tensors, %d segments, /%d" % (what, total, len(counts), n, divisor))
+
+        buffer = torch.from_numpy(np.concatenate(incoming)).cuda()
+        run([buffer.data_ptr() + starts[g] * esz for g in range(n)], "received in place", unpack_form)
+        shifted = torch.zeros(total + 8, dtype=tdt, device="cuda")
+        shifted[1:total + 1].copy_(buffer)
+        run([shifted.data_ptr() + (starts[g] + 1) * esz for g in range(n)], "in place in a buffer an element off 16 bytes",
+            ring_abi.FORM_TILES)
+        slots = [G.dev(x, starts[g] % 32, pad=40) for g, x in enumerate(incoming)]
+        run([s[0].data_ptr() for s in slots], "slots of their own", ring_abi.FORM_TILES)
+        if n > 2:
+            # a gap: the second piece is left out, and its elements keep their values
+            spans = ring_abi.make_spans([(starts[g], sizes[g], buffer.data_ptr() + starts[g] * esz, None)
+                                         for g in range(n) if g != 1])
+            assert form_of(spans) == ring_abi.FORM_TILES
+            for d, h in zip(devs, hosts):
+                d[0].copy_(torch.from_numpy(h))
+            plan.scatter(spans, divisor, None)
+            G.sync()
+            expect = want.copy()
+            expect[starts[1]:starts[1] + sizes[1]] = np.concatenate(hosts)[starts[1]:starts[1] + sizes[1]]
+            G.assert_same_bits(np.concatenate([G.host(d[0]) for d in devs]), expect, "a gap in the pieces")
+        plan.close()
+
+
 def test_fusion_errors():
     L = ring_abi.lib()
     h = ctypes.c_void_p()
