@@ -909,20 +909,26 @@ def main():
             return lambda k, stream, fused: w.launch_step(0, stream, fused)
         return w.launch_step
 
-    def region(nsteps, nwarm, fused=False, hot=False, first=0):
+    def region(nsteps, nwarm, fused=False, hot=False, first=0, streams=None):
         """Wall-clock seconds of `nsteps` steps, bracketed by a synchronize on both sides,
         after `nwarm` untimed steps. Nothing inside the region carries an event: a dispatch
         that carries one ends only when its stores have drained, which serialises it against
-        the launch behind it."""
+        the launch behind it. `streams`: the steps go to these streams in turn (successive
+        steps work on different virtual ranks' buffers and do not depend on one another);
+        the default is the one dedicated stream."""
         launch_step = launcher(hot)
+        streams = streams or (stream,)
+        ns = len(streams)
         for k in range(first, first + nwarm):
-            launch_step(k, stream, fused)
-        ring_abi.stream_synchronize(stream)
+            launch_step(k, streams[k % ns], fused)
+        for st in streams:
+            ring_abi.stream_synchronize(st)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for k in range(first + nwarm, first + nwarm + nsteps):
-            launch_step(k, stream, fused)
-        ring_abi.stream_synchronize(stream)
+            launch_step(k, streams[k % ns], fused)
+        for st in streams:
+            ring_abi.stream_synchronize(st)
         torch.cuda.synchronize()
         return time.perf_counter() - t0
 
@@ -1132,6 +1138,21 @@ def main():
                          "GBps": round(w.bytes_per_step * hot_steps / hot_elapsed / 1e9, 1),
                          "note": "every step on the same buffers (%.0f MiB touched per step); `value` is the cold "
                                  "rate, buffer sets rotated" % (w.bytes_per_step / 2**20)}
+    if args.variant == "all" and w.nsets >= 2 and not options.get("dry_launch"):
+        # the same steps issued to two streams in turn: successive steps work on different virtual ranks'
+        # buffers, so the start of one step's launches fills the chip while the step before it drains
+        second = ring_abi.stream_create()
+        two = statistics.median(regions(EXTRA_REGIONS, extra_steps, min(max(warmup, 20), 50), streams=(stream, second)))
+        ok = all(w.check(k) for k in range(min(w.nsets, 2))) if not isinstance(w, FusedResnet50) else True
+        ring_abi.stream_destroy(second)
+        if not ok:
+            sys.exit("bench.py: the output of the two-stream run is wrong; refusing to report a number")
+        result["two_streams"] = {
+            "ms_per_step": round(two * 1e3, 5), "steps": extra_steps, "regions": EXTRA_REGIONS,
+            "GBps": round(w.bytes_per_step / two / 1e9, 1),
+            "note": "the same steps, even ones on the dedicated stream and odd ones on a second stream (the C ABI takes the "
+                    "stream per call): throughput of independent allreduces in flight together, not the latency of one; "
+                    "`value` is the one-stream figure"}
     if isinstance(w, RingAllreduce) and not isinstance(w, RingAllreducePerStep):
         # the same job with the in->out copy folded into the accumulate (fewer bytes, same result)
         if args.variant == "all":
