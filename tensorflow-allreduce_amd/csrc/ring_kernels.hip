@@ -223,10 +223,9 @@ typedef RowTableT<kSmallRows> SmallRowTable;
   } while (0)
 
 // Blocks the wave until every vector-memory access it has issued is complete.
-// (Nothing to wait for where the library is compiled for the host.)
-#ifdef HIP_CPU_SHIM_RUNTIME_H_
-#define RING_WAIT_VMEM() do {} while (0)
-#else
+// (A build for another target, which has no such instruction, defines the macro
+// before this point.)
+#ifndef RING_WAIT_VMEM
 #define RING_WAIT_VMEM() asm volatile("s_waitcnt vmcnt(0)" ::: "memory")
 #endif
 
@@ -440,9 +439,7 @@ struct PhasedShape {
   uint32_t rounds;             // most rounds any row needs (at most a row's share of the lane's vectors)
   uint32_t shift[kSmallRows];  // the workgroup that starts row k
 };
-#ifdef HIP_CPU_SHIM_RUNTIME_H_
-#define RING_WAVES_PER_SIMD(n)
-#else
+#ifndef RING_WAVES_PER_SIMD
 #define RING_WAVES_PER_SIMD(n) __attribute__((amdgpu_waves_per_eu(n, n)))
 #endif
 // WAVES: workgroups per CU (waves per SIMD). 1: 112 vectors per lane, the form

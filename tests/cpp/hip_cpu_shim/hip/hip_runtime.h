@@ -34,6 +34,10 @@
 #define __shared__ static
 #define __align__(n) __attribute__((aligned(n)))
 #define HIP_SYMBOL(x) (&(x))
+// what the kernel library lets a build for another target define: nothing to wait for on the
+// CPU (every access has completed when the statement returns), and no occupancy attribute
+#define RING_WAIT_VMEM() do {} while (0)
+#define RING_WAVES_PER_SIMD(n)
 
 struct dim3 {
   unsigned x, y, z;

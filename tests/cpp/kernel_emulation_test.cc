@@ -549,10 +549,10 @@ void run_all(const char* name) {
   test_fusion<T>({17}, 3, 2);
   test_fusion<T>({}, 0, 2);
   test_fusion<T>({100003, 1, 2, 50001, 0, 4096, 3}, 4, 2);  // tensor ends that cut 16-byte groups, divided by a power of two
-  // segments whose ends cut 16-byte groups (154,107 elements in 3, 5 and 7 segments), received in place and scattered from there
-  test_fusion<T>({100003, 1, 2, 50001, 0, 4096, 3, 1}, 0, 3);
-  test_fusion<T>({100003, 1, 2, 50001, 0, 4096, 3, 1}, 2, 5);
-  test_fusion<T>({7, 100003, 1, 2, 50001, 0, 4096, 1}, 4, 7);
+  // segments whose ends cut 16-byte groups (19,107 elements in 3, 5 and 7 segments), received in place and scattered from there
+  test_fusion<T>({10003, 1, 2, 5001, 0, 4096, 3, 1}, 0, 3);
+  test_fusion<T>({10003, 1, 2, 5001, 0, 4096, 3, 1}, 2, 5);
+  test_fusion<T>({7, 10003, 1, 2, 5001, 0, 4096, 1}, 4, 7);
 }
 
 }  // namespace

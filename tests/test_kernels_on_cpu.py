@@ -133,7 +133,7 @@ def test_options_set_while_another_thread_launches_under_thread_sanitizer():
         pytest.skip("no clang++ (the kernels use clang vector extensions)")
     os.makedirs(BUILD, exist_ok=True)
     exe = os.path.join(BUILD, "options_race_test")
-    cmd = [clang, "-x", "c++", "-std=c++17", "-O1", "-g", "-fsanitize=thread", "-fno-omit-frame-pointer", "-pthread",
+    cmd = [clang, "-x", "c++", "-std=c++17", "-O0", "-g", "-fsanitize=thread", "-fno-omit-frame-pointer", "-pthread",
            "-I", os.path.join(ROOT, "tests", "cpp", "hip_cpu_shim"), "-I", os.path.join(ROOT, "include"),
            "-o", exe, SRC, os.path.join(ROOT, "tests", "cpp", "options_race_test.cc")]
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
