@@ -20,8 +20,6 @@
 #include <condition_variable>
 #include <cstring>
 #include <mutex>
-#include <queue>
-#include <sstream>
 #include <thread>
 #include <unordered_map>
 
@@ -41,7 +39,17 @@ template <typename T> bool IsGPUDevice();
 template <> bool IsGPUDevice<GPUDevice>() { return true; }
 template <> bool IsGPUDevice<CPUDevice>() { return false; }
 
-typedef std::function<void(const Status&)> CommunicationDoneCallback;
+// What ends a rank's part of a collective (mpi_ops.cc:119-121: a function of the
+// status; here the two things every op's callback does, mpi_ops.cc:1084-1087,
+// held in place: a std::function over them would allocate for every request).
+struct CommunicationDoneCallback {
+  OpKernelContext* context = nullptr;
+  AsyncOpKernel::DoneCallback done;
+  void operator()(const Status& status) const {
+    context->SetStatus(status);
+    done();
+  }
+};
 
 // mpi_ops.cc:123-153
 struct CollectiveOpRecord {
@@ -62,7 +70,37 @@ struct StagedPeers {
   std::vector<const void*> rs, ag;
 };
 
-typedef std::unordered_map<std::string, std::map<int, CollectiveOpRecord>> TensorTable;
+// The records of one collective, one per rank that lives in this process, in
+// rank order: the contents of a map from rank to record, in one array.
+class RankRecords {
+ public:
+  typedef std::pair<int, CollectiveOpRecord> value_type;
+  typedef std::vector<value_type>::iterator iterator;
+  typedef std::vector<value_type>::const_iterator const_iterator;
+  iterator begin() { return v_.begin(); }
+  iterator end() { return v_.end(); }
+  const_iterator begin() const { return v_.begin(); }
+  const_iterator end() const { return v_.end(); }
+  size_t size() const { return v_.size(); }
+  bool empty() const { return v_.empty(); }
+  void clear() { v_.clear(); }
+  void reserve(size_t n) { v_.reserve(n); }
+  CollectiveOpRecord& operator[](int rank) {
+    auto it = std::lower_bound(v_.begin(), v_.end(), rank, [](const value_type& e, int r) { return e.first < r; });
+    if (it == v_.end() || it->first != rank) it = v_.emplace(it, rank, CollectiveOpRecord());
+    return it->second;
+  }
+  // the record of a rank that is known to have one
+  const CollectiveOpRecord& at(int rank) const {
+    auto it = std::lower_bound(v_.begin(), v_.end(), rank, [](const value_type& e, int r) { return e.first < r; });
+    return it->second;
+  }
+
+ private:
+  std::vector<value_type> v_;
+};
+
+typedef std::unordered_map<std::string, RankRecords> TensorTable;
 typedef std::unordered_map<std::string, std::vector<MPIRequest>> MessageTable;
 
 }  // namespace
@@ -85,8 +123,8 @@ struct mpic_world {
   std::mutex mu;
   mpic::TensorTable tensor_table;
   // requests on their way to the coordinator, in wire format (the bytes a rank
-  // in another process would send)
-  std::queue<std::string> message_queue;
+  // in another process would send), each behind its length
+  std::string message_bytes;
   std::thread background_thread;
   bool shut_down = false;
   mpic::MessageTable message_table;  // coordinator side
@@ -119,7 +157,14 @@ namespace {
 // mpi_ops.cc:255-269
 bool IncrementTensorCount(MessageTable* table, const MPIRequest& msg, int expected) {
   std::vector<MPIRequest>& v = (*table)[msg.tensor_name];
-  v.push_back(msg);
+  if (v.empty()) v.reserve(static_cast<size_t>(expected));
+  // the table's key is the name: the stored requests do not repeat it
+  v.emplace_back();
+  MPIRequest& stored = v.back();
+  stored.request_rank = msg.request_rank;
+  stored.request_type = msg.request_type;
+  stored.tensor_type = msg.tensor_type;
+  stored.tensor_shape = msg.tensor_shape;
   return static_cast<int>(v.size()) == expected;
 }
 
@@ -129,14 +174,17 @@ TensorShape ShapeOf(const MPIRequest& r) { return TensorShape(r.tensor_shape); }
 MPIResponse ConstructMPIResponse(MessageTable* table, const std::string& name) {
   bool error = false;
   const std::vector<MPIRequest>& requests = (*table)[name];
-  std::ostringstream err;
+  std::string message;  // of the first check that fails
+  auto fail = [&error, &message](std::string text) {
+    error = true;
+    message = std::move(text);
+  };
 
   const MPIDataType data_type = requests[0].tensor_type;
   for (size_t i = 1; i < requests.size(); i++) {
     if (data_type != requests[i].tensor_type) {
-      error = true;
-      err << "Mismatched data types: One rank had type " << MPIDataType_Name(data_type)
-          << ", but another rank had type " << MPIDataType_Name(requests[i].tensor_type) << ".";
+      fail(std::string("Mismatched data types: One rank had type ") + MPIDataType_Name(data_type) +
+           ", but another rank had type " + MPIDataType_Name(requests[i].tensor_type) + ".");
       break;
     }
   }
@@ -144,44 +192,38 @@ MPIResponse ConstructMPIResponse(MessageTable* table, const std::string& name) {
   const MPIRequest::RequestType message_type = requests[0].request_type;
   for (size_t i = 1; i < requests.size() && !error; i++) {
     if (message_type != requests[i].request_type) {
-      error = true;
-      err << "Mismatched MPI operations: One rank did an " << static_cast<int>(message_type)
-          << ", but another rank did an " << static_cast<int>(requests[i].request_type) << ".";
+      fail("Mismatched MPI operations: One rank did an " + std::to_string(static_cast<int>(message_type)) +
+           ", but another rank did an " + std::to_string(static_cast<int>(requests[i].request_type)) + ".");
     }
   }
 
   if (message_type == MPIRequest::ALLREDUCE) {
     for (size_t i = 1; i < requests.size() && !error; i++) {
       if (requests[0].tensor_shape != requests[i].tensor_shape) {
-        error = true;
-        err << "Mismatched allreduce tensor shapes: One rank reduced a tensor of shape "
-            << ShapeOf(requests[0]).DebugString() << ", but another rank sent a tensor of shape "
-            << ShapeOf(requests[i]).DebugString() << ".";
+        fail("Mismatched allreduce tensor shapes: One rank reduced a tensor of shape " +
+             ShapeOf(requests[0]).DebugString() + ", but another rank sent a tensor of shape " +
+             ShapeOf(requests[i]).DebugString() + ".");
       }
     }
   }
 
   if (message_type == MPIRequest::ALLGATHER) {
     const TensorShape tensor_shape = ShapeOf(requests[0]);
-    if (tensor_shape.dims() == 0 && !error) {
-      error = true;
-      err << "Rank zero tried to gather a rank-zero tensor.";
-    }
+    if (tensor_shape.dims() == 0 && !error) fail("Rank zero tried to gather a rank-zero tensor.");
     for (size_t i = 1; i < requests.size() && !error; i++) {
       const TensorShape request_shape = ShapeOf(requests[i]);
       if (tensor_shape.dims() != request_shape.dims()) {
-        error = true;
-        err << "Mismatched allgather tensor shapes: One rank gathered a tensor of rank "
-            << tensor_shape.dims() << ", but another rank sent a tensor of rank " << request_shape.dims() << ".";
+        fail("Mismatched allgather tensor shapes: One rank gathered a tensor of rank " +
+             std::to_string(tensor_shape.dims()) + ", but another rank sent a tensor of rank " +
+             std::to_string(request_shape.dims()) + ".");
         break;
       }
       for (int dim = 1; dim < tensor_shape.dims(); dim++) {
         if (tensor_shape.dim_size(dim) != request_shape.dim_size(dim)) {
-          error = true;
-          err << "Mismatched allgather tensor shapes: One rank gathered a tensor with dimension " << dim
-              << " equal to " << tensor_shape.dim_size(dim)
-              << ", but another rank sent a tensor with dimension " << dim << " equal to "
-              << request_shape.dim_size(dim) << ".";
+          fail("Mismatched allgather tensor shapes: One rank gathered a tensor with dimension " +
+               std::to_string(dim) + " equal to " + std::to_string(tensor_shape.dim_size(dim)) +
+               ", but another rank sent a tensor with dimension " + std::to_string(dim) + " equal to " +
+               std::to_string(request_shape.dim_size(dim)) + ".");
           break;
         }
       }
@@ -192,7 +234,7 @@ MPIResponse ConstructMPIResponse(MessageTable* table, const std::string& name) {
   response.tensor_name = name;
   if (error) {
     response.response_type = MPIResponse::ERROR;
-    response.error_message = err.str();
+    response.error_message = std::move(message);
   } else {
     response.response_type =
         message_type == MPIRequest::ALLREDUCE ? MPIResponse::ALLREDUCE : MPIResponse::ALLGATHER;
@@ -231,13 +273,13 @@ void FinishRecords(Records* records, std::vector<CommunicationDoneCallback>* cal
   records->clear();
   for (auto& done : *callbacks) {
     done(status);
-    done = nullptr;  // and its captured state, while the waiters still wait for the last ones
+    done = CommunicationDoneCallback();  // and its captured state, while the waiters still wait for the last ones
   }
 }
 
 void PerformCollectiveOp(mpic_world* w, const MPIResponse& response) {
   const WorldOptions opt = SnapshotOptions(w);
-  std::map<int, CollectiveOpRecord> records;
+  RankRecords records;
   StagedPeers peers;
   bool have_peers = false;
   {
@@ -370,7 +412,8 @@ constexpr int kMaxFusedDirectRanks = 16;
 // the reference ring applied to the packed buffer.
 void PerformFusedAllreduce(mpic_world* w, const std::vector<std::string>& names, const WorldOptions& opt) {
   const int n = w->size;
-  std::vector<std::map<int, CollectiveOpRecord>> records;
+  std::vector<RankRecords> records;
+  records.reserve(names.size());
   {
     std::lock_guard<std::mutex> guard(w->mu);
     for (const std::string& name : names) {
@@ -414,6 +457,8 @@ void PerformFusedAllreduce(mpic_world* w, const std::vector<std::string>& names,
     std::vector<const ring_fusion_plan*> in_plans, out_plans;
     for (int r = 0; r < n; r++) {
       std::vector<const void*> ins, outs;
+      ins.reserve(records.size());
+      outs.reserve(records.size());
       for (auto& rec : records) {
         ins.push_back(rec.at(r).in_t->data());
         outs.push_back(rec.at(r).out_t->data());
@@ -428,6 +473,7 @@ void PerformFusedAllreduce(mpic_world* w, const std::vector<std::string>& names,
     if (status.ok() && opt.sync_on_done && ring_stream_synchronize(w->stream) != RING_OK)
       status = errors::Unknown("MPI operation failed unexpectedly.");
     std::vector<CommunicationDoneCallback> callbacks;
+    callbacks.reserve(records.size() * static_cast<size_t>(n));
     for (auto& rec : records)
       for (auto& kv : rec) callbacks.push_back(std::move(kv.second.callback));
     FinishRecords(&records, &callbacks, status);
@@ -536,28 +582,35 @@ void BackgroundThreadLoop(mpic_world* w) {
   if (!init.ok()) return;
 
   bool should_shut_down = false;
+  // this tick's requests; the buffer goes back to the ranks at the next swap, so
+  // that neither side allocates per request
+  std::string message_bytes;
   do {
-    std::queue<std::string> message_queue;
+    message_bytes.clear();
     {
       std::unique_lock<std::mutex> lock(w->mu);
       // With fusion on a tick starts when the embedder asks for one (so the set of
       // tensors fused together, and with it the rounding of the sums, does not
-      // depend on timing); otherwise every arrival starts one.
+      // depend on timing); otherwise every arrival starts one. (Counting the
+      // requests while the ranks still submit them, ahead of the flush, was
+      // measured and not kept: the two threads then compete for the allocator
+      // and the queue, and a step's submission slows by more than its tick gains.)
       w->work_cv.wait(lock, [w] {
         const bool hold = w->fusion_bytes > 0 && !w->flush_requested;
-        return w->shut_down || (!w->message_queue.empty() && !hold);
+        return w->shut_down || (!w->message_bytes.empty() && !hold);
       });
-      std::swap(message_queue, w->message_queue);
+      std::swap(message_bytes, w->message_bytes);
       w->flush_requested = false;
       should_shut_down = w->shut_down;
     }
     std::vector<std::string> ready_to_reduce;
-    while (!message_queue.empty()) {
-      MPIRequest message;
-      if (message.ParseFromString(message_queue.front()) &&
+    size_t at = 0, size = 0;
+    const char* data = nullptr;
+    MPIRequest message;  // one for the whole tick: the storage of its name is reused
+    while (NextRequestFrame(message_bytes, &at, &data, &size)) {
+      if (message.ParseFromArray(data, size) &&
           IncrementTensorCount(&w->message_table, message, w->expected_requests()))
         ready_to_reduce.push_back(message.tensor_name);
-      message_queue.pop();
     }
     PerformReady(w, ready_to_reduce);
   } while (!should_shut_down);
@@ -612,20 +665,16 @@ Status DataTypeToMPIType(DataType tf_dtype, MPIDataType* mpi_dtype) {
 
 // mpi_ops.cc:853-868
 void EnqueueTensorCollective(mpic_world* w, CollectiveOpRecord record, MPIRequest::RequestType rtype) {
-  MPIRequest message;
-  message.request_rank = record.rank;
-  message.tensor_name = record.name;
-  message.tensor_type = record.dtype;
-  message.request_type = rtype;
-  message.tensor_shape = record.in_t->shape().dim_sizes();
-  std::string wire = message.SerializeAsString();
   bool wake;
   {
     std::lock_guard<std::mutex> guard(w->mu);
-    std::map<int, CollectiveOpRecord>& by_rank = w->tensor_table[record.name];
+    // the MPIRequest of mpi_ops.cc:855-863, written straight into its wire form
+    AppendRequestFrame(&w->message_bytes, record.rank, rtype, record.dtype, record.name,
+                       record.in_t->shape().dim_sizes());
+    RankRecords& by_rank = w->tensor_table[record.name];
+    if (by_rank.empty()) by_rank.reserve(static_cast<size_t>(w->expected_requests()));
     const int rank = record.rank;
     by_rank[rank] = std::move(record);
-    w->message_queue.push(std::move(wire));
     // with fusion on, requests wait for a flush: waking the thread for each
     // would only have it look at the queue and go back to sleep
     wake = !(w->fusion_bytes > 0 && !w->flush_requested);
@@ -763,10 +812,8 @@ class MPIAllreduceOp : public AsyncOpKernel {
     record.on_gpu = IsGPUDevice<Device>() && !input_tensor->host_memory();
     record.temp_elements = ring_temp_elements(static_cast<size_t>(input_tensor->NumElements()), world->size);
     record.divisor = context->fused_divisor();
-    record.callback = [done, context](const Status& status) {
-      context->SetStatus(status);
-      done();
-    };
+    record.callback.context = context;
+    record.callback.done = done;
     // The caller's producer work is ordered before the collective by the
     // embedding framework (the reference defers this call with a stream host
     // callback, mpi_ops.cc:1099-1105).
@@ -850,10 +897,8 @@ class MPIAllgatherOp : public AsyncOpKernel {
                          context->allocate_output(0, output_shape, input_tensor->dtype(), false, &output_tensor), done);
     record.out_t = output_tensor;
     record.divisor = context->fused_divisor();
-    record.callback = [done, context](const Status& status) {
-      context->SetStatus(status);
-      done();
-    };
+    record.callback.context = context;
+    record.callback.done = done;
     EnqueueTensorCollective(world, std::move(record), MPIRequest::ALLGATHER);
   }
 };

@@ -80,7 +80,13 @@ Status OpKernelContext::allocate_output(int index, const TensorShape& shape, Dat
   if (!mem && shape.num_elements() > 0)
     return errors::Internal("allocate_output failed for a tensor of shape " + shape.DebugString());
   if (outputs_.size() <= static_cast<size_t>(index)) outputs_.resize(static_cast<size_t>(index) + 1);
-  outputs_[static_cast<size_t>(index)].reset(new Tensor(dt, shape, mem, host_memory));
+  std::unique_ptr<Tensor>& slot = outputs_[static_cast<size_t>(index)];
+  if (!slot && !spare_.empty()) {
+    slot = std::move(spare_.back());
+    spare_.pop_back();
+  }
+  if (slot) *slot = Tensor(dt, shape, mem, host_memory);
+  else slot.reset(new Tensor(dt, shape, mem, host_memory));
   *out = outputs_[static_cast<size_t>(index)].get();
   return Status::OK();
 }

@@ -17,6 +17,8 @@
 #include <utility>
 #include <vector>
 
+#include "dims.h"
+
 namespace mpic {
 
 // ---- Status (tensorflow/core/lib/core/status.h, error_codes.proto) ----------
@@ -55,7 +57,7 @@ size_t DataTypeSize(DataType dt);  // 0 for types the MPI ops do not handle
 class TensorShape {
  public:
   TensorShape() {}
-  explicit TensorShape(std::vector<int64_t> dims) : dims_(std::move(dims)) {}
+  explicit TensorShape(Dims dims) : dims_(std::move(dims)) {}  // also from a std::vector<int64_t>
   void AddDim(int64_t d) { dims_.push_back(d); }
   int dims() const { return static_cast<int>(dims_.size()); }
   int64_t dim_size(int i) const { return dims_[static_cast<size_t>(i)]; }
@@ -64,13 +66,13 @@ class TensorShape {
     for (int64_t d : dims_) n *= d;
     return n;
   }
-  const std::vector<int64_t>& dim_sizes() const { return dims_; }
+  const Dims& dim_sizes() const { return dims_; }
   std::string DebugString() const;  // "[17,17,17]"
   bool operator==(const TensorShape& o) const { return dims_ == o.dims_; }
   bool operator!=(const TensorShape& o) const { return dims_ != o.dims_; }
 
  private:
-  std::vector<int64_t> dims_;
+  Dims dims_;
 };
 
 // A view of memory owned by the embedding framework (device memory unless
@@ -211,6 +213,7 @@ class OpKernelContext {
   // For a node that runs again with the same inputs (a step of a training
   // loop): forgets the last run's outputs and status.
   void Reset() {
+    for (auto& t : outputs_) spare_.push_back(std::move(t));  // their objects serve the next run's outputs
     outputs_.clear();
     status_ = Status();
   }
@@ -237,6 +240,7 @@ class OpKernelContext {
   OutputAllocator alloc_;
   std::vector<Tensor> inputs_;
   std::vector<std::unique_ptr<Tensor>> outputs_;
+  std::vector<std::unique_ptr<Tensor>> spare_;  // Tensor objects of earlier runs, reused by allocate_output
   Status status_;
 };
 

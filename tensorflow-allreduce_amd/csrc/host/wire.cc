@@ -25,6 +25,7 @@ void PutBytes(std::string* out, const std::string& s) {
 class Reader {
  public:
   explicit Reader(const std::string& s) : p_(s.data()), end_(s.data() + s.size()) {}
+  Reader(const char* data, size_t size) : p_(data), end_(data + size) {}
   template <typename T>
   bool Get(T* v) {
     if (static_cast<size_t>(end_ - p_) < sizeof(T)) return false;
@@ -59,21 +60,49 @@ const char* MPIDataType_Name(MPIDataType t) {
   }
 }
 
+void MPIRequest::AppendTo(std::string* out, int32_t rank, RequestType type, MPIDataType dtype,
+                          const std::string& name, const Dims& shape) {
+  Put<uint32_t>(out, kRequestMagic);
+  Put<uint8_t>(out, kVersion);
+  Put<int32_t>(out, rank);
+  Put<uint8_t>(out, static_cast<uint8_t>(type));
+  Put<uint8_t>(out, static_cast<uint8_t>(dtype));
+  PutBytes(out, name);
+  Put<uint32_t>(out, static_cast<uint32_t>(shape.size()));
+  for (int64_t d : shape) Put<int64_t>(out, d);
+}
+
 std::string MPIRequest::SerializeAsString() const {
   std::string out;
-  Put<uint32_t>(&out, kRequestMagic);
-  Put<uint8_t>(&out, kVersion);
-  Put<int32_t>(&out, request_rank);
-  Put<uint8_t>(&out, static_cast<uint8_t>(request_type));
-  Put<uint8_t>(&out, static_cast<uint8_t>(tensor_type));
-  PutBytes(&out, tensor_name);
-  Put<uint32_t>(&out, static_cast<uint32_t>(tensor_shape.size()));
-  for (int64_t d : tensor_shape) Put<int64_t>(&out, d);
+  out.reserve(4 + 1 + 4 + 1 + 1 + 4 + tensor_name.size() + 4 + 8 * tensor_shape.size());  // one allocation
+  AppendTo(&out, request_rank, request_type, tensor_type, tensor_name, tensor_shape);
   return out;
 }
 
-bool MPIRequest::ParseFromString(const std::string& bytes) {
-  Reader r(bytes);
+void AppendRequestFrame(std::string* stream, int32_t rank, MPIRequest::RequestType type, MPIDataType dtype,
+                        const std::string& name, const Dims& shape) {
+  const size_t at = stream->size();
+  Put<uint32_t>(stream, 0);
+  MPIRequest::AppendTo(stream, rank, type, dtype, name, shape);
+  const uint32_t size = static_cast<uint32_t>(stream->size() - at - 4);
+  for (size_t i = 0; i < 4; i++) (*stream)[at + i] = static_cast<char>((size >> (8 * i)) & 0xff);
+}
+
+bool NextRequestFrame(const std::string& stream, size_t* at, const char** data, size_t* size) {
+  if (*at > stream.size() || stream.size() - *at < 4) return false;
+  uint32_t n = 0;
+  for (size_t i = 0; i < 4; i++) n |= static_cast<uint32_t>(static_cast<unsigned char>(stream[*at + i])) << (8 * i);
+  if (stream.size() - *at - 4 < n) return false;
+  *data = stream.data() + *at + 4;
+  *size = n;
+  *at += 4 + static_cast<size_t>(n);
+  return true;
+}
+
+bool MPIRequest::ParseFromString(const std::string& bytes) { return ParseFromArray(bytes.data(), bytes.size()); }
+
+bool MPIRequest::ParseFromArray(const char* data, size_t size) {
+  Reader r(data, size);
   uint32_t magic = 0, ndims = 0;
   uint8_t version = 0, rtype = 0, dtype = 0;
   if (!r.Get(&magic) || magic != kRequestMagic || !r.Get(&version) || version != kVersion) return false;
@@ -90,6 +119,7 @@ bool MPIRequest::ParseFromString(const std::string& bytes) {
 
 std::string MPIResponse::SerializeAsString() const {
   std::string out;
+  out.reserve(4 + 1 + 1 + 4 + tensor_name.size() + 4 + error_message.size());
   Put<uint32_t>(&out, kResponseMagic);
   Put<uint8_t>(&out, kVersion);
   Put<uint8_t>(&out, static_cast<uint8_t>(response_type));

@@ -22,6 +22,8 @@
 #include <string>
 #include <vector>
 
+#include "dims.h"
+
 namespace mpic {
 
 // mpi_message.proto:12-17
@@ -35,11 +37,25 @@ struct MPIRequest {
   RequestType request_type = ALLREDUCE;
   MPIDataType tensor_type = TF_MPI_INVALID_TYPE;
   std::string tensor_name;
-  std::vector<int64_t> tensor_shape;
+  Dims tensor_shape;
 
   std::string SerializeAsString() const;
   bool ParseFromString(const std::string& bytes);
+  bool ParseFromArray(const char* data, size_t size);
+  // The bytes SerializeAsString gives for a request of these fields, appended to
+  // `out` without building the request.
+  static void AppendTo(std::string* out, int32_t rank, RequestType type, MPIDataType dtype, const std::string& name,
+                       const Dims& shape);
 };
+
+// A stream of requests, each behind its length (u32, little endian): how the
+// requests of one process travel to its coordinator thread, in one buffer that
+// is filled, handed over and reused, instead of one string per request.
+void AppendRequestFrame(std::string* stream, int32_t rank, MPIRequest::RequestType type, MPIDataType dtype,
+                        const std::string& name, const Dims& shape);
+// The frame that starts at *at: its bytes, and *at moved behind it. False at
+// the end of the stream or when the stream is cut short inside a frame.
+bool NextRequestFrame(const std::string& stream, size_t* at, const char** data, size_t* size);
 
 // mpi_message.proto:49-63
 struct MPIResponse {
