@@ -277,7 +277,17 @@ void FinishRecords(Records* records, std::vector<CommunicationDoneCallback>* cal
   }
 }
 
-void PerformCollectiveOp(mpic_world* w, const MPIResponse& response) {
+// A collective whose launches are on the stream and whose ops wait for the
+// stream to be synchronised.
+struct EnqueuedCollective {
+  RankRecords records;
+  std::vector<CommunicationDoneCallback> callbacks;
+};
+
+// With `enqueued`, a collective that has been launched is left there for the
+// caller to synchronise and finish (one synchronisation for all the collectives
+// of a tick instead of one each); without, it is finished here.
+void PerformCollectiveOp(mpic_world* w, const MPIResponse& response, std::vector<EnqueuedCollective>* enqueued) {
   const WorldOptions opt = SnapshotOptions(w);
   RankRecords records;
   StagedPeers peers;
@@ -367,12 +377,17 @@ void PerformCollectiveOp(mpic_world* w, const MPIResponse& response) {
     }
   }
 
+  std::vector<CommunicationDoneCallback> callbacks;
+  callbacks.reserve(records.size());
+  for (auto& kv : records) callbacks.push_back(std::move(kv.second.callback));
   if (status.ok() && opt.sync_on_done && response.response_type != MPIResponse::ERROR) {
+    if (enqueued) {
+      enqueued->push_back(EnqueuedCollective{std::move(records), std::move(callbacks)});
+      return;
+    }
     const int rc = ring_stream_synchronize(w->stream);
     if (rc != RING_OK) status = errors::Unknown("MPI operation failed unexpectedly.");  // ring.h:36-39
   }
-  std::vector<CommunicationDoneCallback> callbacks;
-  for (auto& kv : records) callbacks.push_back(std::move(kv.second.callback));
   FinishRecords(&records, &callbacks, status);
 }
 
@@ -530,6 +545,12 @@ void PerformReady(mpic_world* w, const std::vector<std::string>& ready) {
   }
   const WorldOptions opt = SnapshotOptions(w);
   const bool fusing = opt.fusion_bytes > 0 && opt.fusion_buffer && w->real_rank < 0 && w->size > 1;
+  // The reference synchronises the stream inside every device primitive
+  // (ring.cu.cc:41-45, 60-69). Here a tick's collectives are all enqueued first
+  // and the stream is synchronised once, before any of their ops is told: an op
+  // still completes only when its result is there, and a tick of 161 small
+  // gradients waits for the GPU once instead of 161 times.
+  std::vector<EnqueuedCollective> enqueued;
   size_t i = 0;
   while (i < responses.size()) {
     std::vector<std::string> group;
@@ -558,9 +579,16 @@ void PerformReady(mpic_world* w, const std::vector<std::string>& ready) {
       PerformFusedAllreduce(w, group, opt);
       i += group.size();
     } else {
-      PerformCollectiveOp(w, responses[i]);
+      PerformCollectiveOp(w, responses[i], &enqueued);
       i++;
     }
+  }
+  if (!enqueued.empty()) {
+    Status status;
+    if (ring_stream_synchronize(w->stream) != RING_OK)
+      status = errors::Unknown("MPI operation failed unexpectedly.");  // ring.h:36-39
+    for (EnqueuedCollective& e : enqueued) e.records.clear();  // all of them, before any waiter is told
+    for (EnqueuedCollective& e : enqueued) FinishRecords(&e.records, &e.callbacks, status);
   }
 }
 
