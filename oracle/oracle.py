@@ -61,6 +61,8 @@ def lib():
         pvp = ctypes.POINTER(vp)
         L.oracle_ring_allreduce_threads.restype = ci
         L.oracle_ring_allreduce_threads.argtypes = [ci, ci, sz, pvp, pvp, ctypes.POINTER(Tap)]
+        L.oracle_ring_allreduce_rank_prestaged.restype = ci
+        L.oracle_ring_allreduce_rank_prestaged.argtypes = [ci, ci, ci, vp, vp, sz, pvp, pvp]
         L.oracle_ring_allreduce_lockstep.restype = ci
         L.oracle_ring_allreduce_lockstep.argtypes = [ci, ci, sz, pvp, pvp]
         L.oracle_ring_allgather_threads.restype = ci
@@ -147,6 +149,25 @@ def ring_allreduce(inputs, tap=False):
     if rc:
         raise RuntimeError("oracle allreduce failed: %d" % rc)
     return (outs, rs, ag) if tap else outs
+
+
+def ring_allreduce_rank_prestaged(n, r, inp, rs_segments, ag_segments):
+    """One rank of the reference ring on given incoming segments (the per-rank
+    data path): rs_segments[i] / ag_segments[i] are what rank r receives at
+    step i of the reduce-scatter / allgather. Returns that rank's output."""
+    inp = np.ascontiguousarray(inp).reshape(-1)
+    rs = [np.ascontiguousarray(x, dtype=inp.dtype).reshape(-1) for x in rs_segments]
+    ag = [np.ascontiguousarray(x, dtype=inp.dtype).reshape(-1) for x in ag_segments]
+    assert len(rs) == n - 1 and len(ag) == n - 1
+    sizes, _ = segment_table(inp.size, n)
+    for i in range(n - 1):
+        assert rs[i].size >= sizes[(r - i - 1) % n] and ag[i].size >= sizes[(r - i) % n]
+    out = np.empty_like(inp)
+    rc = lib().oracle_ring_allreduce_rank_prestaged(n, r, dtype_code(inp.dtype), _ptr(inp), _ptr(out), inp.size,
+                                                    _ptr_array(rs), _ptr_array(ag))
+    if rc != 0:
+        raise RuntimeError("oracle_ring_allreduce_rank_prestaged failed: %d" % rc)
+    return out
 
 
 def ring_allreduce_lockstep(inputs):

@@ -11,6 +11,9 @@
  *   - whole ring: an independent closed form (element of segment s is the
  *     left fold x_s, x_{s+1}, ... x_{s+n-1 mod n}) evaluated in numpy, the
  *     lockstep evaluator below, and the same per-rank code run over real MPI;
+ *   - one rank on given incoming segments (the replay transport): what the
+ *     threaded ring's taps recorded, replayed to each rank alone, must give
+ *     that rank's output of the threaded ring;
  *   - the reference tests' own invariants: allreduce(x) == x*size exactly for
  *     size <= 3 (mpi_ops_test.py:92-112), rank-stamped allgather
  *     (mpi_ops_test.py:204-263), the 13-stage chained closed form
@@ -141,6 +144,60 @@ int oracle_ring_allreduce_rank(int n, int r, int dtype, const void* input,
                   buffer + starts[recv_seg] * esz, sizes[recv_seg] * esz);
   }
   free(sizes);
+  return rc;
+}
+
+/* A transport that replays what one rank of a ring receives: the i-th receive
+ * of the reduce-scatter delivers rs[i], the i-th of the allgather ag[i]; what
+ * the rank sends goes nowhere. */
+typedef struct replay_state {
+  const void* const* rs;
+  const void* const* ag;
+  int next_rs, next_ag, steps;
+} replay_state;
+
+static int replay_irecv(void* self, void* buf, size_t bytes, int from) {
+  replay_state* st = (replay_state*)self;
+  (void)from;
+  if (st->next_rs >= st->steps) return -3;
+  oracle_copy(buf, st->rs[st->next_rs++], bytes);
+  return 0;
+}
+static int replay_send(void* self, const void* buf, size_t bytes, int to) {
+  (void)self; (void)buf; (void)bytes; (void)to;
+  return 0;
+}
+static int replay_wait(void* self) {
+  (void)self;
+  return 0;
+}
+static int replay_sendrecv(void* self, const void* sbuf, size_t sbytes, int to,
+                           void* rbuf, size_t rbytes, int from) {
+  replay_state* st = (replay_state*)self;
+  (void)sbuf; (void)sbytes; (void)to; (void)from;
+  if (st->next_ag >= st->steps) return -3;
+  oracle_copy(rbuf, st->ag[st->next_ag++], rbytes);
+  return 0;
+}
+
+/* ring.h:136-228 for ONE rank whose incoming segments are given: the same
+ * oracle_ring_allreduce_rank, over the replay transport. */
+int oracle_ring_allreduce_rank_prestaged(int n, int r, int dtype,
+                                         const void* input, void* output,
+                                         size_t count,
+                                         const void* const* rs_segments,
+                                         const void* const* ag_segments) {
+  const size_t esz = oracle_dtype_size(dtype);
+  if (!esz || n < 1) return -1;
+  replay_state st = {rs_segments, ag_segments, 0, 0, n - 1};
+  oracle_transport tp = {&st, replay_irecv, replay_send, replay_wait,
+                         replay_sendrecv};
+  const size_t temp_elems = oracle_temp_elements(count, n);
+  void* temp = malloc(temp_elems > 0 ? temp_elems * esz : 1); /* mpi_ops.cc:1073-1077 */
+  if (!temp) return -2;
+  const int rc = oracle_ring_allreduce_rank(n, r, dtype, input, temp, output,
+                                            count, &tp, NULL);
+  free(temp);
   return rc;
 }
 

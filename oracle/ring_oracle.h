@@ -82,6 +82,16 @@ int oracle_ring_allreduce_rank(int n, int r, int dtype, const void* input,
                                void* temp, void* output, size_t count,
                                oracle_transport* tp, oracle_tap* tap);
 
+/* ring.h:136-228 for one rank alone: rs_segments[i] is what the rank receives
+ * at reduce-scatter step i, ag_segments[i] at allgather step i (n-1 of each,
+ * of the sizes the segment table gives those steps); what it sends is
+ * dropped. The per-rank data path on pre-staged peer segments. */
+int oracle_ring_allreduce_rank_prestaged(int n, int r, int dtype,
+                                         const void* input, void* output,
+                                         size_t count,
+                                         const void* const* rs_segments,
+                                         const void* const* ag_segments);
+
 /* ring.h:236-301 — RingAllgather for rank r of n. `rows[k]` is rank k's first
  * dimension, `input` holds rows[r]*elems_per_row elements, `output` the
  * concatenation. */

@@ -409,10 +409,12 @@ def test_prestaged_through_the_op_layer(oracle):
                 session.run(mpi.allreduce(cuda(ins[r]), average=False))
 
 
-def test_prestaged_1gib_float32_n64():
+def test_prestaged_1gib_float32_n64(oracle):
     """268,435,456 float32 (1 GiB), N=64: 63 + 63 steps on 16 MiB segments, one
-    launch per phase. Checked against numpy on the host: every reduce-scatter
-    step is input + received on its own segment, every allgather step a copy."""
+    launch per phase. The reduce-scatter alone is checked against numpy on the
+    host (every step is input + received on its own segment), the whole
+    per-rank allreduce against the oracle's rank 37 run alone on the same
+    incoming segments, and against what the schedule says of every segment."""
     n, r, count = 64, 37, 268_435_456
     seg = count // n
     gen = torch.Generator(device="cuda").manual_seed(r)
@@ -442,6 +444,8 @@ def test_prestaged_1gib_float32_n64():
     assert rc == 0, L.mpic_last_error()
     torch.cuda.synchronize()
     hout, hag = G.host(dout), G.host(ag)
+    G.assert_same_bits(hout, oracle.ring_allreduce_rank_prestaged(n, r, hin, list(hrs), list(hag)),
+                       "the oracle's rank %d alone on the same incoming segments" % r)
     owned = (r + 1) % n
     for i in range(n - 1):
         s = ring_abi.schedule(1, n, r, i)[1]
@@ -1093,6 +1097,9 @@ def test_allreduce_batch_is_one_node_per_tensor(oracle):
                                oracle.ring_allreduce([ins[q][0].reshape(-1) for q in range(n)])[r], "first of the batch")
             with pytest.raises(mpi.FailedPreconditionError):
                 handles[r][1].result()
+            # the one behind the bad node was enqueued in the same tick and completes like the first
+            G.assert_same_bits(G.host(handles[r][2].result()).reshape(-1),
+                               oracle.ring_allreduce([ins[q][4].reshape(-1) for q in range(n)])[r], "last of the batch")
 
 
 def test_prepared_batch_runs_the_same_nodes_every_step(oracle):
@@ -1182,6 +1189,8 @@ def test_prepared_batch_mixes_with_single_ops_and_reports_one_bad_node(oracle):
                                    "good node of a batch with a bad one")
                 with pytest.raises(mpi.FailedPreconditionError):
                     handles[r][1].result()
+                G.assert_same_bits(G.host(handles[r][2].result()), oracle.ring_allreduce([xs[q][2] for q in range(n)])[r],
+                                   "the node behind the bad one")
     with pytest.raises(mpi.FailedPreconditionError):
         batches[0].submit()                                 # its session is closed
 

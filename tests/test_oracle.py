@@ -147,6 +147,33 @@ def test_ring_order_matters_and_is_the_rotated_left_fold(oracle):
     assert not np.array_equal(naive, out)
 
 
+def test_one_rank_on_given_segments_by_hand_and_against_the_whole_ring(oracle):
+    """The per-rank data path (one rank, its incoming segments given): a case
+    worked out by hand from ring.h:183-225, then, for every rank of rings of
+    several sizes, what that rank received in the threaded ring replayed to it
+    alone must give its output of the threaded ring."""
+    # n=3, r=1, one element per segment. Reduce-scatter: step 0 receives segment (1-0-1)%3 = 0,
+    # step 1 segment (1-1-1)%3 = 2; allgather: step 0 receives segment 1, step 1 segment 0.
+    for dtype in DTYPES:
+        out = oracle.ring_allreduce_rank_prestaged(3, 1, np.array([1, 2, 4], dtype=dtype),
+                                                   [np.array([8], dtype=dtype), np.array([16], dtype=dtype)],
+                                                   [np.array([32], dtype=dtype), np.array([64], dtype=dtype)])
+        assert list(out) == [64, 32, 4 + 16]
+    # the same with the allgather of step 1 taken away would leave 1 + 8 in segment 0: the order of the
+    # steps is what the hand-made answer pins. A ragged rank: n=3, count=4 -> sizes [2, 1, 1], r=0:
+    # reduce-scatter receives segment 2 then 1, allgather segment 0 (2 elements) then 2.
+    out = oracle.ring_allreduce_rank_prestaged(3, 0, np.array([1, 2, 4, 8], dtype=np.int64),
+                                               [np.array([16]), np.array([32])],
+                                               [np.array([64, 128]), np.array([256])])
+    assert list(out) == [64, 128, 4 + 32, 256]
+    for dtype, n, count in itertools.product(DTYPES, (1, 2, 3, 5, 8), (0, 1, 7, 4913)):
+        ins = make_inputs(n, count, dtype, seed=100 * n + count)
+        outs, rs, ag = oracle.ring_allreduce(ins, tap=True)
+        for r in range(n):
+            alone = oracle.ring_allreduce_rank_prestaged(n, r, ins[r], list(rs[r]), list(ag[r]))
+            assert np.array_equal(bits(alone), bits(outs[r])), (np.dtype(dtype).name, n, count, r)
+
+
 def test_ring_known_answer_vectors(oracle):
     with open(os.path.join(GOLDEN, "ring_kats.json")) as f:
         kats = json.load(f)["cases"]
