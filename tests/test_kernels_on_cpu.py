@@ -10,6 +10,10 @@
    64-bit `min` ahead of a branch (v_cmp into vcc, branch on vcc, s_cselect on
    a stale SCC): every lane of a partial tile then ran, out of bounds on the
    GPU while the same source was correct on the CPU.
+3. The plugin's host code linked over the same CPU build of the kernels
+   (tests/cpp/plugin_emulation_test.cc): the coordinator's paths that end in a
+   launch, under the sanitizers, against the C oracle.
+4. ring_set_option against concurrent launches under ThreadSanitizer.
 """
 import os
 import re
@@ -32,20 +36,61 @@ def _clang():
     return None
 
 
+SANITIZE = ["-std=c++17", "-O0", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
+            "-fno-omit-frame-pointer", "-pthread"]
+SHIM = os.path.join(ROOT, "tests", "cpp", "hip_cpu_shim")
+
+
+def _run(cmd, **kw):
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, **kw)
+    assert res.returncode == 0, " ".join(cmd) + "\n" + res.stdout[-4000:]
+    return res.stdout
+
+
+def _kernel_library_for_the_cpu(clang):
+    """The kernel library as a sanitized CPU object, compiled once for the tests that link it."""
+    os.makedirs(BUILD, exist_ok=True)
+    obj = os.path.join(BUILD, "ring_kernels_cpu_asan.o")
+    sources = [SRC, os.path.join(ROOT, "include", "ring_abi.h"), os.path.join(SHIM, "hip", "hip_runtime.h"),
+               os.path.join(SHIM, "hip", "hip_ext.h"), os.path.abspath(__file__)]
+    if not os.path.exists(obj) or os.path.getmtime(obj) < max(os.path.getmtime(f) for f in sources):
+        _run([clang, "-x", "c++"] + SANITIZE + ["-I", SHIM, "-I", os.path.join(ROOT, "include"), "-c", "-o", obj, SRC])
+    return obj
+
+
 def test_kernels_under_sanitizers_on_the_cpu():
     clang = _clang()
     if clang is None:
         pytest.skip("no clang++ (the kernels use clang vector extensions)")
-    os.makedirs(BUILD, exist_ok=True)
+    obj = _kernel_library_for_the_cpu(clang)
     exe = os.path.join(BUILD, "kernel_emulation_test")
-    cmd = [clang, "-x", "c++", "-std=c++17", "-O0", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
-           "-fno-omit-frame-pointer", "-pthread",
-           "-I", os.path.join(ROOT, "tests", "cpp", "hip_cpu_shim"), "-I", os.path.join(ROOT, "include"),
-           "-o", exe, SRC, os.path.join(ROOT, "tests", "cpp", "kernel_emulation_test.cc")]
-    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    assert res.returncode == 0, res.stdout[-4000:]
-    res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=900)
-    assert res.returncode == 0 and "kernel emulation: ok" in res.stdout, res.stdout[-4000:]
+    _run([clang] + SANITIZE + ["-I", SHIM, "-I", os.path.join(ROOT, "include"), "-o", exe,
+                               os.path.join(ROOT, "tests", "cpp", "kernel_emulation_test.cc"), obj])
+    out = _run([exe], timeout=900)
+    assert "kernel emulation: ok" in out, out[-4000:]
+
+
+def test_plugin_over_the_emulated_kernels_under_sanitizers():
+    """The plugin's host code over the same CPU build of the kernel library:
+    the coordinator's paths that end in a launch (separate rings of a tick,
+    fused groups, prepared batches, allgather, a bad node among good ones),
+    bit for bit against the C oracle, under AddressSanitizer and UBSan."""
+    clang = _clang()
+    if clang is None:
+        pytest.skip("no clang++ (the kernels use clang vector extensions)")
+    obj = _kernel_library_for_the_cpu(clang)
+    host = os.path.join(ROOT, "tensorflow-allreduce_amd", "csrc", "host")
+    oracle_obj = os.path.join(BUILD, "ring_oracle_cpu.o")
+    _run(["gcc", "-O1", "-g", "-std=gnu11", "-fno-fast-math", "-c", os.path.join(ROOT, "oracle", "ring_oracle.c"),
+          "-o", oracle_obj])
+    exe = os.path.join(BUILD, "plugin_emulation_test")
+    _run([clang] + SANITIZE + ["-I", host, "-I", os.path.join(ROOT, "include"), "-I", os.path.join(ROOT, "oracle"),
+                               "-o", exe, os.path.join(ROOT, "tests", "cpp", "plugin_emulation_test.cc")] +
+         [os.path.join(host, f) for f in ("framework.cc", "wire.cc", "ring_driver.cc", "transport.cc", "collective_ops.cc")] +
+         [obj, oracle_obj])
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0")
+    out = _run([exe], timeout=900, env=env)
+    assert "plugin emulation: ok" in out, out[-4000:]
 
 
 SCC_WRITER = re.compile(r"^\s*(s_cmp|s_bitcmp|s_and_b|s_or_b|s_xor_b|s_andn2|s_orn2|s_add|s_sub|s_lshl|s_lshr|s_ashr|"
@@ -94,9 +139,10 @@ def test_no_scalar_select_on_a_stale_condition_code():
         pytest.skip("hipcc not found")
     os.makedirs(BUILD, exist_ok=True)
     asm = os.path.join(BUILD, "ring_kernels_gfx950.s")
-    cmd = [hipcc] + HIP_FLAGS + ["-I", os.path.join(ROOT, "include"), "-S", "--cuda-device-only", "-o", asm, SRC]
-    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    assert res.returncode == 0, res.stdout[-4000:]
+    # the assembly of this source and these flags is kept between runs (minutes of compiling otherwise)
+    sources = [SRC, os.path.join(ROOT, "include", "ring_abi.h"), os.path.abspath(__file__)]
+    if not os.path.exists(asm) or os.path.getmtime(asm) < max(os.path.getmtime(f) for f in sources):
+        _run([hipcc] + HIP_FLAGS + ["-I", os.path.join(ROOT, "include"), "-S", "--cuda-device-only", "-o", asm, SRC])
     text = open(asm).read()
     found = stale_selects(text)
     assert not found, "scalar selects on a stale condition code: %r" % (found[:5],)
