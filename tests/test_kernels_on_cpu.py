@@ -36,9 +36,15 @@ def _clang():
     return None
 
 
-SANITIZE = ["-std=c++17", "-O0", "-g", "-fsanitize=address,undefined", "-fno-sanitize-recover=all",
-            "-fno-omit-frame-pointer", "-pthread"]
+SANITIZERS = {
+    "asan": ["-fsanitize=address,undefined", "-fno-sanitize-recover=all"],
+    "tsan": ["-fsanitize=thread"],
+}
 SHIM = os.path.join(ROOT, "tests", "cpp", "hip_cpu_shim")
+
+
+def _flags(sanitizer):
+    return ["-std=c++17", "-O0", "-g"] + SANITIZERS[sanitizer] + ["-fno-omit-frame-pointer", "-pthread"]
 
 
 def _run(cmd, **kw):
@@ -47,14 +53,14 @@ def _run(cmd, **kw):
     return res.stdout
 
 
-def _kernel_library_for_the_cpu(clang):
+def _kernel_library_for_the_cpu(clang, sanitizer="asan"):
     """The kernel library as a sanitized CPU object, compiled once for the tests that link it."""
     os.makedirs(BUILD, exist_ok=True)
-    obj = os.path.join(BUILD, "ring_kernels_cpu_asan.o")
+    obj = os.path.join(BUILD, "ring_kernels_cpu_%s.o" % sanitizer)
     sources = [SRC, os.path.join(ROOT, "include", "ring_abi.h"), os.path.join(SHIM, "hip", "hip_runtime.h"),
                os.path.join(SHIM, "hip", "hip_ext.h"), os.path.abspath(__file__)]
     if not os.path.exists(obj) or os.path.getmtime(obj) < max(os.path.getmtime(f) for f in sources):
-        _run([clang, "-x", "c++"] + SANITIZE + ["-I", SHIM, "-I", os.path.join(ROOT, "include"), "-c", "-o", obj, SRC])
+        _run([clang, "-x", "c++"] + _flags(sanitizer) + ["-I", SHIM, "-I", os.path.join(ROOT, "include"), "-c", "-o", obj, SRC])
     return obj
 
 
@@ -64,31 +70,44 @@ def test_kernels_under_sanitizers_on_the_cpu():
         pytest.skip("no clang++ (the kernels use clang vector extensions)")
     obj = _kernel_library_for_the_cpu(clang)
     exe = os.path.join(BUILD, "kernel_emulation_test")
-    _run([clang] + SANITIZE + ["-I", SHIM, "-I", os.path.join(ROOT, "include"), "-o", exe,
-                               os.path.join(ROOT, "tests", "cpp", "kernel_emulation_test.cc"), obj])
-    out = _run([exe], timeout=900)
-    assert "kernel emulation: ok" in out, out[-4000:]
+    _run([clang] + _flags("asan") + ["-I", SHIM, "-I", os.path.join(ROOT, "include"), "-o", exe,
+                                     os.path.join(ROOT, "tests", "cpp", "kernel_emulation_test.cc"), obj])
+    # one process per element type, side by side: the stand-in runs a workgroup's lanes as OS threads
+    # and spends its time handing them work
+    procs = [(t, subprocess.Popen([exe, t], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True))
+             for t in ("float32", "int32", "int64")]
+    for t, proc in procs:
+        try:
+            out, _ = proc.communicate(timeout=900)
+        except subprocess.TimeoutExpired:
+            for _, other in procs:
+                other.kill()
+            raise
+        assert proc.returncode == 0 and "kernel emulation: ok" in out, t + "\n" + out[-4000:]
 
 
-def test_plugin_over_the_emulated_kernels_under_sanitizers():
+@pytest.mark.parametrize("sanitizer", ["asan", "tsan"])
+def test_plugin_over_the_emulated_kernels_under_sanitizers(sanitizer):
     """The plugin's host code over the same CPU build of the kernel library:
     the coordinator's paths that end in a launch (separate rings of a tick,
-    fused groups, prepared batches, allgather, a bad node among good ones),
-    bit for bit against the C oracle, under AddressSanitizer and UBSan."""
+    fused groups, prepared batches, allgather, a bad node among good ones,
+    ranks submitting from threads of their own), bit for bit against the C
+    oracle, once under AddressSanitizer and UBSan and once under
+    ThreadSanitizer."""
     clang = _clang()
     if clang is None:
         pytest.skip("no clang++ (the kernels use clang vector extensions)")
-    obj = _kernel_library_for_the_cpu(clang)
+    obj = _kernel_library_for_the_cpu(clang, sanitizer)
     host = os.path.join(ROOT, "tensorflow-allreduce_amd", "csrc", "host")
     oracle_obj = os.path.join(BUILD, "ring_oracle_cpu.o")
     _run(["gcc", "-O1", "-g", "-std=gnu11", "-fno-fast-math", "-c", os.path.join(ROOT, "oracle", "ring_oracle.c"),
           "-o", oracle_obj])
-    exe = os.path.join(BUILD, "plugin_emulation_test")
-    _run([clang] + SANITIZE + ["-I", host, "-I", os.path.join(ROOT, "include"), "-I", os.path.join(ROOT, "oracle"),
-                               "-o", exe, os.path.join(ROOT, "tests", "cpp", "plugin_emulation_test.cc")] +
+    exe = os.path.join(BUILD, "plugin_emulation_test_" + sanitizer)
+    _run([clang] + _flags(sanitizer) + ["-I", host, "-I", os.path.join(ROOT, "include"), "-I", os.path.join(ROOT, "oracle"),
+                                        "-o", exe, os.path.join(ROOT, "tests", "cpp", "plugin_emulation_test.cc")] +
          [os.path.join(host, f) for f in ("framework.cc", "wire.cc", "ring_driver.cc", "transport.cc", "collective_ops.cc")] +
          [obj, oracle_obj])
-    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0")
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0", TSAN_OPTIONS="halt_on_error=1:report_signal_unsafe=0")
     out = _run([exe], timeout=900, env=env)
     assert "plugin emulation: ok" in out, out[-4000:]
 
@@ -177,13 +196,10 @@ def test_options_set_while_another_thread_launches_under_thread_sanitizer():
     clang = _clang()
     if clang is None:
         pytest.skip("no clang++ (the kernels use clang vector extensions)")
-    os.makedirs(BUILD, exist_ok=True)
+    obj = _kernel_library_for_the_cpu(clang, "tsan")
     exe = os.path.join(BUILD, "options_race_test")
-    cmd = [clang, "-x", "c++", "-std=c++17", "-O0", "-g", "-fsanitize=thread", "-fno-omit-frame-pointer", "-pthread",
-           "-I", os.path.join(ROOT, "tests", "cpp", "hip_cpu_shim"), "-I", os.path.join(ROOT, "include"),
-           "-o", exe, SRC, os.path.join(ROOT, "tests", "cpp", "options_race_test.cc")]
-    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    assert res.returncode == 0, res.stdout[-4000:]
+    _run([clang] + _flags("tsan") + ["-I", SHIM, "-I", os.path.join(ROOT, "include"), "-o", exe,
+                                     os.path.join(ROOT, "tests", "cpp", "options_race_test.cc"), obj])
     env = dict(os.environ, TSAN_OPTIONS="halt_on_error=1:report_signal_unsafe=0")
-    res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600, env=env)
-    assert res.returncode == 0 and "options race test: ok" in res.stdout, res.stdout[-4000:]
+    out = _run([exe], timeout=600, env=env)
+    assert "options race test: ok" in out, out[-4000:]
