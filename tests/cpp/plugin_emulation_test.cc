@@ -387,6 +387,65 @@ int main() {
     CHECK(mpic_world_destroy(w) == MPIC_OK);
   }
 
+  // ---- fusion scheduling on random gradient sets: which tensors are reduced together follows from the
+  // submission order, the element types and the buffer size alone (consecutive ready allreduces of one
+  // type while they fit; a group of one is a ring of its own), in both forms of the fused reduction ----
+  for (int iteration = 0; iteration < 36; iteration++) {
+    const int n = 2 + static_cast<int>(next_random() % 4);
+    const size_t k = 1 + next_random() % 12;
+    const size_t per_rank = 16 * (1 + next_random() % 1024);  // 16 B .. 16 KiB
+    const int direct = static_cast<int>(next_random() % 2);
+    const int divisor = (next_random() % 3 == 0) ? 0 : n;
+    std::vector<Type> types;
+    std::vector<size_t> counts;
+    for (size_t j = 0; j < k; j++) {
+      const uint64_t x = next_random();
+      types.push_back(x % 8 < 5 ? kF32 : (x % 8 < 7 ? kI32 : kI64));  // runs of one type are common
+      counts.push_back((x >> 8) % 5 == 0 ? (x >> 16) % 3 : (x >> 16) % 1500);
+    }
+    mpic_world* w = nullptr;
+    CHECK(mpic_world_create(n, &w) == MPIC_OK);
+    init_world(w);
+    CHECK(mpic_world_set_option(w, "direct", direct) == MPIC_OK);
+    void* buffer = device_alloc(per_rank * static_cast<size_t>(n));
+    CHECK(mpic_world_set_fusion_buffer(w, buffer, per_rank) == MPIC_OK);
+    TensorSet s(n, types, counts, "random");
+    s.refill();
+    std::vector<std::vector<mpic_context*>> ctx;
+    submit_batches(w, s, n, divisor, &ctx, false);
+    CHECK(mpic_world_flush(w) == MPIC_OK);
+    wait_all_ok(&ctx);
+    char what[128];
+    std::snprintf(what, sizeof what, "random set %d (n=%d, k=%zu, buffer %zu, direct=%d, divisor=%d)", iteration, n, k,
+                  per_rank, direct, divisor);
+    size_t i = 0;
+    while (i < k) {
+      size_t j = i, bytes = 0;
+      while (j < k && types[j].mpic == types[i].mpic && bytes + counts[j] * types[j].size <= per_rank) {
+        bytes += counts[j] * types[j].size;
+        j++;
+      }
+      if (j - i >= 2) {
+        check_fused(s, n, i, j, divisor, what);
+        i = j;
+      } else {
+        std::vector<const void*> ins;
+        for (int r = 0; r < n; r++) ins.push_back(s.in[static_cast<size_t>(r)][i]);
+        auto want = oracle_allreduce(types[i], n, counts[i], ins);
+        for (int r = 0; r < n; r++) {
+          if (divisor) divide(types[i], want[static_cast<size_t>(r)].data(), counts[i], divisor);
+          if (!same_bytes(want[static_cast<size_t>(r)].data(), s.out[static_cast<size_t>(r)][i], counts[i] * types[i].size)) {
+            std::fprintf(stderr, "%s: tensor %zu (a ring of its own) of rank %d differs from the oracle\n", what, i, r);
+            std::exit(1);
+          }
+        }
+        i++;
+      }
+    }
+    CHECK(mpic_world_destroy(w) == MPIC_OK);
+    std::free(buffer);
+  }
+
   std::printf("plugin emulation: ok\n");
   return 0;
 }
