@@ -161,7 +161,9 @@ void check_separate(const TensorSet& s, int n, int divisor, const char* what) {
 }
 
 // tensors [first, last) fused: the oracle's ring on the concatenation, divided where asked
-void check_fused(const TensorSet& s, int n, size_t first, size_t last, int divisor, const char* what) {
+// divisors[j - first] divides tensor j of the group (0: the sum stays)
+void check_fused(const TensorSet& s, int n, size_t first, size_t last, const std::vector<int>& divisors,
+                 const char* what) {
   const Type& t = s.types[first];
   size_t total = 0;
   for (size_t j = first; j < last; j++) total += s.counts[j];
@@ -177,9 +179,9 @@ void check_fused(const TensorSet& s, int n, size_t first, size_t last, int divis
   }
   auto want = oracle_allreduce(t, n, total, ins);
   for (int r = 0; r < n; r++) {
-    if (divisor) divide(t, want[static_cast<size_t>(r)].data(), total, divisor);
     size_t at = 0;
     for (size_t j = first; j < last; j++) {
+      if (divisors[j - first]) divide(t, want[static_cast<size_t>(r)].data() + at, s.counts[j], divisors[j - first]);
       if (!same_bytes(want[static_cast<size_t>(r)].data() + at, s.out[static_cast<size_t>(r)][j], s.counts[j] * t.size)) {
         std::fprintf(stderr, "%s: fused tensor %zu of rank %d differs from the oracle on the packed buffer\n", what, j, r);
         std::exit(1);
@@ -187,6 +189,10 @@ void check_fused(const TensorSet& s, int n, size_t first, size_t last, int divis
       at += s.counts[j] * t.size;
     }
   }
+}
+
+void check_fused(const TensorSet& s, int n, size_t first, size_t last, int divisor, const char* what) {
+  check_fused(s, n, first, last, std::vector<int>(last - first, divisor), what);
 }
 
 void submit_batches(mpic_world* w, const TensorSet& s, int n, int divisor, std::vector<std::vector<mpic_context*>>* ctx,
@@ -324,6 +330,27 @@ int main() {
       }
       check_fused(s, n, 0, 6, n, direct ? "fusion, direct form" : "fusion through the buffer");
       check_fused(s, n, 6, 8, n, direct ? "fusion, direct form (int32)" : "fusion through the buffer (int32)");
+    }
+    // one group whose tensors ask for different divisions (an averaged gradient next to a summed one): it is
+    // still one ring on the packed buffer, and only the tensors that asked are divided
+    {
+      TensorSet mixed(n, {kF32, kF32, kF32, kF32, kF32}, {700, 3, 1025, 64, 333}, "mixed");
+      mixed.refill();
+      auto mnames = mixed.name_ptrs();
+      auto mdtypes = mixed.dtypes();
+      auto mdims = mixed.dims();
+      std::vector<int> mndims(mixed.k(), 1);
+      std::vector<std::vector<mpic_context*>> ctx(static_cast<size_t>(n), std::vector<mpic_context*>(mixed.k(), nullptr));
+      for (int r = 0; r < n; r++) {
+        const size_t rr = static_cast<size_t>(r);
+        CHECK(mpic_allreduce_batch(w, r, 2, mnames.data(), mdtypes.data(), mndims.data(), mdims.data(), mixed.in[rr].data(),
+                                   mixed.out[rr].data(), n, ctx[rr].data()) == MPIC_OK);
+        CHECK(mpic_allreduce_batch(w, r, 3, mnames.data() + 2, mdtypes.data() + 2, mndims.data() + 2, mdims.data() + 2,
+                                   mixed.in[rr].data() + 2, mixed.out[rr].data() + 2, 0, ctx[rr].data() + 2) == MPIC_OK);
+      }
+      CHECK(mpic_world_flush(w) == MPIC_OK);
+      wait_all_ok(&ctx);
+      check_fused(mixed, n, 0, 5, std::vector<int>{n, n, 0, 0, 0}, "a group of mixed divisors");
     }
     // a group that does not fit the buffer is cut where it is full: 3 x 5000 float32 against 64 KiB per rank
     {
