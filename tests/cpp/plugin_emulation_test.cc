@@ -98,9 +98,9 @@ std::vector<std::vector<char>> oracle_allreduce(const Type& t, int n, size_t cou
 
 bool same_bytes(const void* a, const void* b, size_t bytes) { return bytes == 0 || std::memcmp(a, b, bytes) == 0; }
 
-void init_world(mpic_world* w) {
+void init_world(mpic_world* w, int rank = 0) {
   mpic_context* c = nullptr;
-  CHECK(mpic_context_create(w, 0, "MPIInit", "MPIInit", "GPU", nullptr, nullptr, &c) == MPIC_OK);
+  CHECK(mpic_context_create(w, rank, "MPIInit", "MPIInit", "GPU", nullptr, nullptr, &c) == MPIC_OK);
   CHECK(mpic_context_compute(c) == MPIC_OK);
   CHECK(mpic_context_wait(c) == MPIC_OK);
   CHECK(mpic_context_destroy(c) == MPIC_OK);
@@ -412,6 +412,77 @@ int main() {
     }
     for (void* p : ins) std::free(p);
     CHECK(mpic_world_destroy(w) == MPIC_OK);
+  }
+
+  // ---- a world of ONE real rank whose peers' segments are pre-staged: what every rank received in the
+  // oracle's threaded ring is staged for it, and the op gives that rank's output; fuse_copy on and off,
+  // the average after the collective as the reference has it; nothing staged is an error, not a hang ----
+  for (const Type& t : {kF32, kI64}) {
+    const int n = 4;
+    const size_t count = 10007, slot = oracle_temp_elements(count, n);
+    std::vector<void*> ins;
+    std::vector<const void*> cins;
+    for (int r = 0; r < n; r++) {
+      ins.push_back(device_alloc(count * t.size));
+      fill(t, ins.back(), count);
+      cins.push_back(ins.back());
+    }
+    std::vector<std::vector<char>> outs(static_cast<size_t>(n), std::vector<char>(count * t.size));
+    std::vector<std::vector<char>> rs(static_cast<size_t>(n), std::vector<char>((n - 1) * slot * t.size));
+    std::vector<std::vector<char>> ag(static_cast<size_t>(n), std::vector<char>((n - 1) * slot * t.size));
+    std::vector<void*> out_ptrs;
+    std::vector<oracle_tap> taps(static_cast<size_t>(n));
+    for (int r = 0; r < n; r++) {
+      out_ptrs.push_back(outs[static_cast<size_t>(r)].data());
+      taps[static_cast<size_t>(r)] = oracle_tap{rs[static_cast<size_t>(r)].data(), ag[static_cast<size_t>(r)].data(), slot};
+    }
+    CHECK(oracle_ring_allreduce_threads(n, t.oracle, count, cins.data(), out_ptrs.data(), taps.data()) == 0);
+    for (int r = 0; r < n; r++) {
+      const size_t rr = static_cast<size_t>(r);
+      // the same from the oracle's rank run alone on these segments (its fourth way to run)
+      std::vector<const void*> rs_ptrs, ag_ptrs;
+      std::vector<void*> staged;  // "device" copies of the segments
+      for (int i = 0; i < n - 1; i++) {
+        for (auto* from : {&rs, &ag}) {
+          staged.push_back(device_alloc(slot * t.size));
+          std::memcpy(staged.back(), (*from)[rr].data() + static_cast<size_t>(i) * slot * t.size, slot * t.size);
+          (from == &rs ? rs_ptrs : ag_ptrs).push_back(staged.back());
+        }
+      }
+      std::vector<char> alone(count * t.size);
+      CHECK(oracle_ring_allreduce_rank_prestaged(n, r, t.oracle, ins[rr], alone.data(), count, rs_ptrs.data(),
+                                                 ag_ptrs.data()) == 0);
+      CHECK(same_bytes(alone.data(), outs[rr].data(), count * t.size));
+      for (int fuse_copy : {1, 0}) {
+        mpic_world* w = nullptr;
+        CHECK(mpic_world_create_prestaged(n, r, &w) == MPIC_OK);
+        init_world(w, r);
+        CHECK(mpic_world_set_option(w, "fuse_copy", fuse_copy) == MPIC_OK);
+        for (int staged_first : {1, 0}) {
+          if (staged_first) CHECK(mpic_stage_peers(w, "grad", rs_ptrs.data(), ag_ptrs.data()) == MPIC_OK);
+          mpic_context* c = nullptr;
+          CHECK(mpic_context_create(w, r, "MPIAllreduce", "grad", "GPU", malloc_output, nullptr, &c) == MPIC_OK);
+          const int64_t dims[1] = {static_cast<int64_t>(count)};
+          CHECK(mpic_context_add_input(c, t.mpic, 1, dims, ins[rr], 0) == MPIC_OK);
+          CHECK(mpic_context_compute(c) == MPIC_OK);
+          void* data = nullptr;
+          if (staged_first) {
+            CHECK(mpic_context_wait(c) == MPIC_OK);
+            CHECK(mpic_context_output(c, 0, nullptr, nullptr, nullptr, &data) == MPIC_OK);
+            CHECK(same_bytes(data, outs[rr].data(), count * t.size));
+          } else {
+            CHECK(mpic_context_wait(c) == MPIC_FAILED_PRECONDITION);  // the staged segments were consumed
+            CHECK(std::strstr(mpic_context_message(c), "No pre-staged peer segments") != nullptr);
+            CHECK(mpic_context_num_outputs(c) == 1 && mpic_context_output(c, 0, nullptr, nullptr, nullptr, &data) == MPIC_OK);
+          }
+          std::free(data);
+          CHECK(mpic_context_destroy(c) == MPIC_OK);
+        }
+        CHECK(mpic_world_destroy(w) == MPIC_OK);
+      }
+      for (void* p : staged) std::free(p);
+    }
+    for (void* p : ins) std::free(p);
   }
 
   // ---- fusion scheduling on random gradient sets: which tensors are reduced together follows from the

@@ -48,6 +48,7 @@ def _flags(sanitizer):
 
 
 def _run(cmd, **kw):
+    __tracebackhide__ = True  # a failure shows the command and its output, not this frame's arguments (the environment)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, **kw)
     assert res.returncode == 0, " ".join(cmd) + "\n" + res.stdout[-4000:]
     return res.stdout
