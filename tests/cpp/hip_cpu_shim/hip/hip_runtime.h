@@ -5,7 +5,8 @@
 // CPU before the same code runs on a GPU. The product never sees this header:
 // the package builds the library with hipcc against the real runtime.
 //
-// Model: a launch runs its workgroups one after the other; the threads of a
+// Model: launches run one at a time, whichever host thread makes them; a launch
+// runs its workgroups one after the other; the threads of a
 // workgroup are real OS threads (a pool of up to 1024) so that __syncthreads()
 // is a real barrier; __shared__ variables are function-local statics, shared by
 // the threads of the running workgroup. Streams and events do nothing: every
@@ -139,8 +140,13 @@ class Pool {
   bool stop_ = false;
 };
 
+// One device: launches from several host threads (one per rank of a ring over a
+// transport) run one after the other, each to its end.
+inline std::mutex g_device;
+
 template <typename Kernel, typename... Args>
 void launch(Kernel kernel, dim3 grid, dim3 block, Args... args) {
+  std::lock_guard<std::mutex> device(g_device);
   g_grid = {grid.x, grid.y, grid.z};
   g_block_dim = {block.x, block.y, block.z};
   const std::function<void()> body = [&]() { kernel(args...); };
@@ -174,8 +180,9 @@ inline hipError_t hipMalloc(void** p, size_t bytes) { *p = malloc(bytes ? bytes 
 template <typename T> inline hipError_t hipMalloc(T** p, size_t bytes) { return hipMalloc(reinterpret_cast<void**>(p), bytes); }
 inline hipError_t hipFree(void* p) { free(p); return hipSuccess; }
 inline hipError_t hipMemcpy(void* dst, const void* src, size_t bytes, int) { memcpy(dst, src, bytes); return hipSuccess; }
-inline hipError_t hipStreamCreateWithFlags(hipStream_t* s, unsigned) { *s = nullptr; return hipSuccess; }
-inline hipError_t hipStreamDestroy(hipStream_t) { return hipSuccess; }
+// a stream is an address of its own (code above the library tells "no stream yet" from a stream by it)
+inline hipError_t hipStreamCreateWithFlags(hipStream_t* s, unsigned) { *s = reinterpret_cast<hipStream_t>(malloc(1)); return hipSuccess; }
+inline hipError_t hipStreamDestroy(hipStream_t s) { free(s); return hipSuccess; }
 inline hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
 enum { hipEventDisableTiming = 2 };
 enum hipStreamCaptureStatus { hipStreamCaptureStatusNone = 0, hipStreamCaptureStatusActive = 1 };

@@ -485,6 +485,77 @@ int main() {
     for (void* p : ins) std::free(p);
   }
 
+  // ---- the ring over a transport, one thread per rank (the reference's loop with its MPI calls behind the
+  // loopback transport): whole segments, pieces, a temp of two segments, the average, allgather of unequal rows ----
+  for (const Type& t : {kF32, kI32}) {
+    const int n = 3;
+    const size_t count = 2003, seg = oracle_temp_elements(count, n);
+    struct { int chunks; size_t temp; int divisor; } forms[] = {{1, seg, 0}, {4, seg, 0}, {3, 2 * seg, n}, {16, 2 * seg, 0}};
+    for (auto& f : forms) {
+      std::vector<void*> ins, outs, temps;
+      std::vector<const void*> cins;
+      for (int r = 0; r < n; r++) {
+        ins.push_back(device_alloc(count * t.size));
+        fill(t, ins.back(), count);
+        cins.push_back(ins.back());
+        outs.push_back(device_alloc(count * t.size));
+        temps.push_back(device_alloc(f.temp * t.size));
+      }
+      auto want = oracle_allreduce(t, n, count, cins);
+      mpic_loopback* lb = nullptr;
+      CHECK(mpic_loopback_create(n, 60.0, &lb) == MPIC_OK);
+      std::vector<std::thread> ranks;
+      std::vector<int> rcs(static_cast<size_t>(n), -1);
+      for (int r = 0; r < n; r++) {
+        ranks.emplace_back([&, r] {
+          mpic_transport tp;
+          CHECK(mpic_loopback_endpoint(lb, r, &tp) == MPIC_OK);
+          const int flags = ((f.chunks - 1) << 4) | (f.divisor << 8);
+          rcs[static_cast<size_t>(r)] = mpic_ring_allreduce_transport(n, r, t.mpic, ins[static_cast<size_t>(r)],
+                                                                      outs[static_cast<size_t>(r)], temps[static_cast<size_t>(r)],
+                                                                      f.temp, count, &tp, nullptr, flags);
+          if (rcs[static_cast<size_t>(r)] != MPIC_OK) std::fprintf(stderr, "rank %d: %s\n", r, mpic_last_error());
+        });
+      }
+      for (auto& th : ranks) th.join();
+      for (int r = 0; r < n; r++) {
+        if (rcs[static_cast<size_t>(r)] != MPIC_OK) std::fprintf(stderr, "transport ring, rank %d: %d\n", r, rcs[static_cast<size_t>(r)]);
+        CHECK(rcs[static_cast<size_t>(r)] == MPIC_OK);
+        if (f.divisor) divide(t, want[static_cast<size_t>(r)].data(), count, f.divisor);
+        CHECK(same_bytes(want[static_cast<size_t>(r)].data(), outs[static_cast<size_t>(r)], count * t.size));
+      }
+      // allgather of unequal rows over the same transport
+      const size_t rows[3] = {5, 0, 2}, cols = 129;
+      std::vector<char> gathered_want;
+      std::vector<void*> gin, gout;
+      for (int r = 0; r < n; r++) {
+        gin.push_back(device_alloc(rows[r] * cols * t.size));
+        fill(t, gin.back(), rows[r] * cols);
+        gathered_want.insert(gathered_want.end(), static_cast<char*>(gin.back()),
+                             static_cast<char*>(gin.back()) + rows[r] * cols * t.size);
+        gout.push_back(device_alloc(7 * cols * t.size));
+      }
+      ranks.clear();
+      for (int r = 0; r < n; r++) {
+        ranks.emplace_back([&, r] {
+          mpic_transport tp;
+          CHECK(mpic_loopback_endpoint(lb, r, &tp) == MPIC_OK);
+          rcs[static_cast<size_t>(r)] = mpic_ring_allgather_transport(n, r, t.mpic, gin[static_cast<size_t>(r)], rows, cols,
+                                                                      gout[static_cast<size_t>(r)], &tp, nullptr,
+                                                                      (f.chunks - 1) << 4);
+        });
+      }
+      for (auto& th : ranks) th.join();
+      for (int r = 0; r < n; r++) {
+        CHECK(rcs[static_cast<size_t>(r)] == MPIC_OK);
+        CHECK(same_bytes(gathered_want.data(), gout[static_cast<size_t>(r)], gathered_want.size()));
+      }
+      CHECK(mpic_loopback_destroy(lb) == MPIC_OK);
+      for (auto* v : {&ins, &outs, &temps, &gin, &gout})
+        for (void* p : *v) std::free(p);
+    }
+  }
+
   // ---- fusion scheduling on random gradient sets: which tensors are reduced together follows from the
   // submission order, the element types and the buffer size alone (consecutive ready allreduces of one
   // type while they fit; a group of one is a ring of its own), in both forms of the fused reduction ----
