@@ -698,14 +698,14 @@ __device__ __forceinline__ void fold_tile(T* dst, const void* const* src, int m,
   }
 }
 
-// A row with one source and no divide is a plain copy (the finished segments a
-// rank takes in next to the fold of its own): touched once, so non-temporal
-// both ways whatever the fold rows use.
+// A row with one source, one destination and no divide is a plain copy (the
+// finished segments a rank takes in next to the fold of its own): touched once,
+// so non-temporal both ways whatever the fold rows use.
 template <typename T, bool DIV, int NT, int UNROLL, int GROUP>
 __device__ __forceinline__ void fold_row_tile(const FoldTable& tab, int row, uint32_t tile, uint32_t tiles_in_row) {
   const FoldRow r = tab.row[row];
   const bool divide = DIV && ((tab.div_mask >> row) & 1u);
-  if (r.m == 1 && !divide)
+  if (r.m == 1 && r.n_more == 0 && !divide)
     fold_tile<T, UNROLL, GROUP, false, 3>(static_cast<T*>(r.dst), tab.src + r.first_ptr, 1, r.count, tile, tiles_in_row,
                                           0, false);
   else

@@ -539,6 +539,7 @@ void run_all(const char* name) {
   test_fold_to_all<T>(8, 8, 10007, 8);
   test_fold_to_all<T>(3, 5, 4099, 0);
   test_fold_to_all<T>(1, 2, 700, 3);
+  test_fold_to_all<T>(1, 3, 700, 0);  // one source stored to several destinations as it is
   printf("%s: fusion\n", name); fflush(stdout);
   test_fusion<T>({5, 0, 4099, 1, 64, 0, 3}, 0, 3);
   test_fusion<T>({20000, 64, 64, 36864, 64, 64, 9001, 2, 12288}, 8, 8);

@@ -367,10 +367,10 @@ def test_fold_stored_to_every_rank(dtype):
     """ring_fold_to_all_rows: the numpy fold in the same order, stored to n_dst
     destinations of differing alignment; rows of unequal length, the divide, an
     allreduce in place (every destination is a source), more pointers than one
-    launch's table holds."""
+    launch's table holds, one source stored to several destinations."""
     rng = np.random.default_rng(7)
     code = G.NP2ABI[np.dtype(dtype)]
-    for m, n_dst, counts in ((1, 1, [33]), (2, 3, [4099, 0, 12]), (8, 8, [30_011] * 8), (5, 7, [9000, 5, 2049]),
+    for m, n_dst, counts in ((1, 1, [33]), (1, 4, [700, 3]), (2, 3, [4099, 0, 12]), (8, 8, [30_011] * 8), (5, 7, [9000, 5, 2049]),
                              (40, 40, [1500] * 6), (128, 129, [777])):
         for divisor in (0, 6):
             rows, checks, keep = [], [], []
