@@ -87,6 +87,30 @@ def test_kernels_under_sanitizers_on_the_cpu():
         assert proc.returncode == 0 and "kernel emulation: ok" in out, t + "\n" + out[-4000:]
 
 
+def test_random_shapes_through_the_emulated_kernels():
+    """A short, fixed sweep of tests/cpp/kernel_emulation_fuzz.cc (random shapes,
+    element types and launch options through the emulation test's cases); the
+    program takes a seed and a case count for longer ones. Two seeds side by
+    side."""
+    clang = _clang()
+    if clang is None:
+        pytest.skip("no clang++ (the kernels use clang vector extensions)")
+    obj = _kernel_library_for_the_cpu(clang)
+    exe = os.path.join(BUILD, "kernel_emulation_fuzz")
+    _run([clang] + _flags("asan") + ["-I", SHIM, "-I", os.path.join(ROOT, "include"), "-o", exe,
+                                     os.path.join(ROOT, "tests", "cpp", "kernel_emulation_fuzz.cc"), obj])
+    procs = [subprocess.Popen([exe, seed, "25"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+             for seed in ("1", "2")]
+    for proc in procs:
+        try:
+            out, _ = proc.communicate(timeout=900)
+        except subprocess.TimeoutExpired:
+            for other in procs:
+                other.kill()
+            raise
+        assert proc.returncode == 0 and "25 cases ok" in out, out[-3000:]
+
+
 @pytest.mark.parametrize("sanitizer", ["asan", "tsan"])
 def test_plugin_over_the_emulated_kernels_under_sanitizers(sanitizer):
     """The plugin's host code over the same CPU build of the kernel library:
