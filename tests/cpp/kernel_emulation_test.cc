@@ -112,6 +112,49 @@ void test_primitives() {
       }
 }
 
+// The one-direction launches of the measurement hook: a write probe fills exactly the whole
+// 16-byte vectors of every row (what lies behind them, and before the row, stays), a read probe
+// changes nothing; what it cannot take it refuses.
+template <typename T>
+void test_probe() {
+  constexpr size_t VEC = 16 / sizeof(T);
+  const size_t counts[] = {0, 1, VEC, 5 * VEC + 1, 1024 * VEC, 1024 * VEC + VEC - 1, 3000 * VEC + 2};
+  std::vector<Buf<T>> bufs;
+  bufs.reserve(8);
+  std::vector<ring_row> rows;
+  for (size_t c : counts) {
+    bufs.emplace_back(c, 4 * VEC);  // four vectors of poison ahead of an aligned row
+    CHECK(reinterpret_cast<uintptr_t>(bufs.back().p) % 16 == 0);
+    rows.push_back(ring_row{bufs.back().p, bufs.back().p, nullptr, c});
+  }
+  std::vector<std::vector<T>> before;
+  for (auto& b : bufs) before.emplace_back(b.p, b.p + b.count);
+  for (int mode : {0, 2}) {
+    OK(ring_probe_stream(rows.data(), static_cast<int>(rows.size()), code<T>(), mode, nullptr));
+    for (size_t k = 0; k < bufs.size(); k++) expect_equal(bufs[k].p, before[k], "a read probe leaves memory alone");
+  }
+  for (int mode : {1, 3}) {
+    for (size_t k = 0; k < bufs.size(); k++)
+      if (bufs[k].count) memcpy(bufs[k].p, before[k].data(), bufs[k].count * sizeof(T));
+    OK(ring_probe_stream(rows.data(), static_cast<int>(rows.size()), code<T>(), mode, nullptr));
+    for (size_t k = 0; k < bufs.size(); k++) {
+      const size_t whole = bufs[k].count / VEC;
+      const uint32_t* words = reinterpret_cast<const uint32_t*>(bufs[k].p);
+      for (size_t v = 0; v < whole; v++)
+        CHECK(words[4 * v] == 1u && words[4 * v + 1] == 2u && words[4 * v + 2] == 3u && words[4 * v + 3] == v % 256);
+      for (size_t e = whole * VEC; e < bufs[k].count; e++) CHECK(memcmp(&bufs[k].p[e], &before[k][e], sizeof(T)) == 0);
+      bufs[k].check_lead();
+    }
+  }
+  Buf<T> odd(64, 1);  // not 16-byte aligned
+  ring_row bad{odd.p, odd.p, nullptr, 64};
+  CHECK(ring_probe_stream(&bad, 1, code<T>(), 0, nullptr) == RING_ERR_ARGUMENT);
+  CHECK(ring_probe_stream(rows.data(), 1, code<T>(), 4, nullptr) == RING_ERR_ARGUMENT);
+  std::vector<ring_row> nine(9, rows[2]);
+  CHECK(ring_probe_stream(nine.data(), 9, code<T>(), 0, nullptr) == RING_ERR_ARGUMENT);
+  CHECK(ring_probe_stream(rows.data(), 1, 99, 0, nullptr) == RING_ERR_DTYPE);
+}
+
 // Rows of mixed kinds and lengths in one call: in-place adds, out-of-place adds,
 // copies; some divided. More rows than one table carries.
 template <typename T>
@@ -506,6 +549,7 @@ template <typename T>
 void run_all(const char* name) {
   printf("%s: primitives\n", name); fflush(stdout);
   test_primitives<T>();
+  test_probe<T>();
   printf("%s: mixed rows\n", name); fflush(stdout);
   test_mixed_rows<T>(1, 1, 20011);
   test_mixed_rows<T>(4, 8, 9000);

@@ -127,6 +127,37 @@ def _random_table(rng, n_rows, dtype, max_count):
     return [(offs[i], counts[i]) for i in order], at
 
 
+def test_one_direction_probes_touch_what_they_say():
+    """ring_probe_stream (the measurement hook behind bench.py's floors
+    workloads): a write probe fills exactly the whole 16-byte vectors of every
+    row with (1, 2, 3, lane) and nothing else, a read probe changes nothing,
+    and rows it cannot take are refused."""
+    counts = [1, 4, 21, 4096, 4099, 1_000_003, 3 * 1024 * 1024 + 2]      # float32 elements
+    for mode in (0, 2, 1, 3):
+        bufs = [torch.full((c + 8,), 7.0, dtype=torch.float32, device="cuda") for c in counts]
+        rows = [(b[4:].data_ptr(), b[4:].data_ptr(), None, c) for b, c in zip(bufs, counts)]    # 16 bytes in: aligned
+        ring_abi.probe_stream(rows, ring_abi.F32, mode, None)
+        G.sync()
+        for b, c in zip(bufs, counts):
+            h = G.host(b)
+            whole = c // 4
+            if mode & 1:
+                words = h[4:4 + 4 * whole].view(np.uint32).reshape(whole, 4)
+                assert (words[:, 0] == 1).all() and (words[:, 1] == 2).all() and (words[:, 2] == 3).all()
+                assert (words[:, 3] == np.arange(whole) % 256).all()
+                assert (h[:4] == 7.0).all() and (h[4 + 4 * whole:] == 7.0).all(), "a write probe stays inside its whole vectors"
+            else:
+                assert (h == 7.0).all(), "a read probe leaves memory alone"
+    x = torch.zeros(64, dtype=torch.float32, device="cuda")
+    with pytest.raises(ring_abi.RingError):
+        ring_abi.probe_stream([(x[1:].data_ptr(), x[1:].data_ptr(), None, 32)], ring_abi.F32, 0, None)   # misaligned
+    with pytest.raises(ring_abi.RingError):
+        ring_abi.probe_stream([(x.data_ptr(), x.data_ptr(), None, 32)] * 9, ring_abi.F32, 0, None)      # more than 8 rows
+    with pytest.raises(ring_abi.RingError):
+        ring_abi.probe_stream([(x.data_ptr(), x.data_ptr(), None, 32)], ring_abi.F32, 4, None)          # no such mode
+    G.sync()
+
+
 @pytest.mark.parametrize("dtype", G.DTYPES)
 @pytest.mark.parametrize("n_rows", [1, 7, 63, 64, 65, 150])
 def test_step_tables_match_oracle(oracle, dtype, n_rows):
