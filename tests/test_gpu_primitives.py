@@ -127,6 +127,48 @@ def _random_table(rng, n_rows, dtype, max_count):
     return [(offs[i], counts[i]) for i in order], at
 
 
+def test_launch_timing_hook_times_the_armed_launches_in_order():
+    """ring_time_next_launch / ring_event_elapsed_us (what bench.py's roofline
+    figures are measured with): each armed pair times one launch, in order; a
+    64 MiB copy takes longer than a 1 MiB one and both lie between what 8 TB/s
+    and 0.2 TB/s would give; pairs beyond 8 are refused; null events disarm;
+    the results of timed launches are the results of untimed ones."""
+    stream = ring_abi.stream_create()
+    try:
+        big_n, small_n = 16 << 20, 256 << 10                      # float32 elements: 64 MiB and 1 MiB
+        src = torch.arange(big_n, dtype=torch.float32, device="cuda")
+        dst = torch.zeros(big_n, dtype=torch.float32, device="cuda")
+        acc = torch.ones(small_n, dtype=torch.float32, device="cuda")
+        torch.cuda.synchronize()
+        events = [(ring_abi.event_create(), ring_abi.event_create()) for _ in range(9)]
+        for _ in range(2):                                          # the first round warms up
+            for pair in events[:3]:
+                ring_abi.time_next_launch(*pair)
+            ring_abi.copy_bytes(dst.data_ptr(), src.data_ptr(), big_n * 4, stream)
+            ring_abi.copy_bytes(dst.data_ptr(), src.data_ptr(), small_n * 4, stream)
+            ring_abi.accumulate(ring_abi.F32, acc.data_ptr(), src.data_ptr(), small_n, stream)
+            ring_abi.stream_synchronize(stream)
+        big, small, add = [ring_abi.event_elapsed_us(*pair) for pair in events[:3]]
+        assert 2 * (64 << 20) / 8e6 < big < 2 * (64 << 20) / 0.2e6, big           # 16.8 us at 8 TB/s
+        assert 0.5 < small < big / 4, (small, big)
+        assert 0.5 < add < big / 4, (add, big)
+        assert torch.equal(dst, src) and torch.equal(acc[:16], 1 + 2 * src[:16])
+        # nine pairs ahead: the ninth is refused, two nulls drop the eight that wait
+        for pair in events[:8]:
+            ring_abi.time_next_launch(*pair)
+        with pytest.raises(ring_abi.RingError):
+            ring_abi.time_next_launch(*events[8])
+        ring_abi.time_next_launch(None, None)
+        ring_abi.copy_bytes(dst.data_ptr(), src.data_ptr(), small_n * 4, stream)   # not timed any more
+        ring_abi.stream_synchronize(stream)
+        assert ring_abi.event_elapsed_us(*events[0]) == big         # still what the first round's launch took
+        for pair in events:
+            for e in pair:
+                ring_abi.event_destroy(e)
+    finally:
+        ring_abi.stream_destroy(stream)
+
+
 def test_one_direction_probes_touch_what_they_say():
     """ring_probe_stream (the measurement hook behind bench.py's floors
     workloads): a write probe fills exactly the whole 16-byte vectors of every
