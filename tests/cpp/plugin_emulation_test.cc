@@ -556,6 +556,56 @@ int main() {
     }
   }
 
+  // ---- the same on random rings: ranks, element type, count (fewer elements than ranks among them), pieces,
+  // size of the temp buffer between one and two segments, the average ----
+  for (int iteration = 0; iteration < 16; iteration++) {
+    const Type types[3] = {kF32, kI32, kI64};
+    const Type t = types[next_random() % 3];
+    const int n = 1 + static_cast<int>(next_random() % 6);
+    const size_t count = next_random() % 4 == 0 ? next_random() % 8 : next_random() % 6000;
+    const size_t seg = oracle_temp_elements(count, n);
+    const int chunks = 1 + static_cast<int>(next_random() % 16);
+    const size_t temp = next_random() % 3 == 0 ? 2 * seg : (next_random() % 2 ? seg : seg + next_random() % (seg + 1));
+    const int divisor = next_random() % 2 ? 0 : 1 + static_cast<int>(next_random() % 9);
+    std::vector<void*> ins, outs, temps;
+    std::vector<const void*> cins;
+    for (int r = 0; r < n; r++) {
+      ins.push_back(device_alloc(count * t.size));
+      fill(t, ins.back(), count);
+      cins.push_back(ins.back());
+      outs.push_back(device_alloc(count * t.size));
+      temps.push_back(device_alloc(temp * t.size));
+    }
+    auto want = oracle_allreduce(t, n, count, cins);
+    mpic_loopback* lb = nullptr;
+    CHECK(mpic_loopback_create(n, 60.0, &lb) == MPIC_OK);
+    std::vector<std::thread> ranks;
+    std::vector<int> rcs(static_cast<size_t>(n), -1);
+    for (int r = 0; r < n; r++) {
+      ranks.emplace_back([&, r] {
+        mpic_transport tp;
+        CHECK(mpic_loopback_endpoint(lb, r, &tp) == MPIC_OK);
+        const size_t rr = static_cast<size_t>(r);
+        rcs[rr] = mpic_ring_allreduce_transport(n, r, t.mpic, ins[rr], outs[rr], temps[rr], temp, count, &tp, nullptr,
+                                                ((chunks - 1) << 4) | (divisor << 8));
+        if (rcs[rr] != MPIC_OK) std::fprintf(stderr, "rank %d: %s\n", r, mpic_last_error());
+      });
+    }
+    for (auto& th : ranks) th.join();
+    for (int r = 0; r < n; r++) {
+      const size_t rr = static_cast<size_t>(r);
+      if (divisor) divide(t, want[rr].data(), count, divisor);
+      if (rcs[rr] != MPIC_OK || !same_bytes(want[rr].data(), outs[rr], count * t.size)) {
+        std::fprintf(stderr, "random ring %d: %zu-byte elements, n=%d, count=%zu, %d pieces, temp %zu of segment %zu, divisor %d, rank %d\n",
+                     iteration, t.size, n, count, chunks, temp, seg, divisor, r);
+        std::exit(1);
+      }
+    }
+    CHECK(mpic_loopback_destroy(lb) == MPIC_OK);
+    for (auto* v : {&ins, &outs, &temps})
+      for (void* p : *v) std::free(p);
+  }
+
   // ---- fusion scheduling on random gradient sets: which tensors are reduced together follows from the
   // submission order, the element types and the buffer size alone (consecutive ready allreduces of one
   // type while they fit; a group of one is a ring of its own), in both forms of the fused reduction ----
