@@ -22,9 +22,13 @@ void one_case(std::mt19937_64& r, int index) {
   CHECK(ring_set_option("phased_copy", phased) == RING_OK);
   CHECK(ring_set_option("unroll", unroll) == RING_OK);
   CHECK(ring_set_option("flat_grid", static_cast<int>(pick(2))) == RING_OK);
+  const int per_cu_choices[] = {0, 0, 1, 2, 8};  // 0: one workgroup per tile; else a grid of that many per CU that loops
+  const int per_cu = per_cu_choices[pick(5)];
+  CHECK(ring_set_option("blocks_per_cu", per_cu) == RING_OK);
   const int what = static_cast<int>(pick(6));
   const size_t big = pick(4) == 0 ? 1 + pick(600000) : 1 + pick(30000);
-  printf("[%d] %zu-byte elements, paced_copy=%d phased_copy=%d unroll=%d: ", index, sizeof(T), paced, phased, unroll);
+  printf("[%d] %zu-byte elements, paced_copy=%d phased_copy=%d unroll=%d blocks_per_cu=%d: ", index, sizeof(T), paced,
+         phased, unroll, per_cu);
   switch (what) {
     case 0: {
       const int rows = 1 + static_cast<int>(pick(80)), divisor = static_cast<int>(pick(9));
