@@ -558,7 +558,7 @@ int main() {
 
   // ---- the same on random rings: ranks, element type, count (fewer elements than ranks among them), pieces,
   // size of the temp buffer between one and two segments, the average ----
-  for (int iteration = 0; iteration < 16; iteration++) {
+  for (int iteration = 0; iteration < 10; iteration++) {
     const Type types[3] = {kF32, kI32, kI64};
     const Type t = types[next_random() % 3];
     const int n = 1 + static_cast<int>(next_random() % 6);
@@ -609,7 +609,7 @@ int main() {
   // ---- fusion scheduling on random gradient sets: which tensors are reduced together follows from the
   // submission order, the element types and the buffer size alone (consecutive ready allreduces of one
   // type while they fit; a group of one is a ring of its own), in both forms of the fused reduction ----
-  for (int iteration = 0; iteration < 36; iteration++) {
+  for (int iteration = 0; iteration < 24; iteration++) {
     const int n = 2 + static_cast<int>(next_random() % 4);
     const size_t k = 1 + next_random() % 12;
     const size_t per_rank = 16 * (1 + next_random() % 1024);  // 16 B .. 16 KiB
