@@ -76,7 +76,7 @@ struct Buf {
 template <typename T>
 void expect_equal(const T* got, const std::vector<T>& want, const char* what) {
   if (want.empty()) return;
-  if (memcmp(got, want.data(), want.size() * sizeof(T)) != 0) {
+  if (!want.empty() && memcmp(got, want.data(), want.size() * sizeof(T)) != 0) {
     for (size_t i = 0; i < want.size(); i++)
       if (memcmp(&got[i], &want[i], sizeof(T)) != 0) {
         fprintf(stderr, "%s: element %zu of %zu differs\n", what, i, want.size());
@@ -223,7 +223,7 @@ void test_step_tables(size_t count, int n) {
     Buf<T> out2(count, 0, false);
     OK(ring_reduce_scatter_steps_from(in.p, out2.p, rs.data(), n - 1, code<T>(), nullptr));
     for (int i = 0; i < n - 1; i++)
-      CHECK(memcmp(out2.p + rs[i].dst_offset, want.data() + rs[i].dst_offset, rs[i].count * sizeof(T)) == 0);
+      CHECK(rs[i].count == 0 || memcmp(out2.p + rs[i].dst_offset, want.data() + rs[i].dst_offset, rs[i].count * sizeof(T)) == 0);
     for (int i = 0; i < n - 1; i++) {
       int snd, rcv;
       OK(ring_schedule(RING_PHASE_ALLGATHER, n, r, i, &snd, &rcv));
@@ -348,7 +348,8 @@ void test_fused_allreduce_of_all_ranks(const std::vector<size_t>& counts, int di
     for (int r = 0; r < n; r++) {
       size_t at = 0;
       for (auto& t : got[r]) {
-        CHECK(memcmp(t.p, want.data() + at, t.count * sizeof(T)) == 0 || (fprintf(stderr, "%s, rank %d\n", what, r), false));
+        CHECK(t.count == 0 || memcmp(t.p, want.data() + at, t.count * sizeof(T)) == 0 ||
+              (fprintf(stderr, "%s, rank %d\n", what, r), false));
         t.check_lead();
         at += t.count;
       }
