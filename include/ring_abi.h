@@ -163,7 +163,8 @@ int ring_segment_table(size_t count, int n, size_t* sizes, size_t* starts);
 size_t ring_temp_elements(size_t count, int n);
 
 /* Allgather segment starts, in elements — ring.h:255-259. rows[k] is rank k's
- * first dimension; starts: host array of n. */
+ * first dimension; starts: host array of n. RING_ERR_ARGUMENT when the gathered
+ * tensor's element count does not fit size_t (the reference's table wraps). */
 int ring_allgather_table(const size_t* rows, int n, size_t elems_per_row,
                          size_t* starts);
 

@@ -2280,7 +2280,11 @@ int ring_allgather_table(const size_t* rows, int n, size_t elems_per_row, size_t
   size_t at = 0;
   for (int i = 0; i < n; i++) {
     starts[i] = at;
-    at += elems_per_row * rows[i];
+    // a gathered tensor that does not fit size_t is an error, not a table that wraps
+    if (rows[i] != 0 && elems_per_row > SIZE_MAX / rows[i]) return RING_ERR_ARGUMENT;
+    const size_t elems = elems_per_row * rows[i];
+    if (elems > SIZE_MAX - at) return RING_ERR_ARGUMENT;
+    at += elems;
   }
   return RING_OK;
 }
@@ -2593,6 +2597,8 @@ int ring_fusion_plan_create(const void* const* tensors, const size_t* counts, in
     if (!tensors[j] || (reinterpret_cast<uintptr_t>(tensors[j]) & (esz - 1))) return RING_ERR_ARGUMENT;
     offsets.push_back(total);
     ptrs.push_back(const_cast<void*>(tensors[j]));
+    // a set whose bytes do not fit 64 bits is an error, not a fused buffer that wraps
+    if (counts[j] > (UINT64_MAX / esz) - total) return RING_ERR_ARGUMENT;
     total += counts[j];
   }
   offsets.push_back(total);
@@ -2686,8 +2692,8 @@ int ring_fusion_run_static(int unpack, const void* const* tensors, const size_t*
     if (!tensors[j] || (reinterpret_cast<uintptr_t>(tensors[j]) & (esz - 1))) return RING_ERR_ARGUMENT;
     if (m == kStaticMaxTensors) return RING_ERR_LIMIT;
     m++;
+    if (counts[j] > static_cast<uint64_t>(kStaticMaxTiles) * tile_elems - total) return RING_ERR_LIMIT;  // (no sum that wraps)
     total += counts[j];
-    if (total > static_cast<uint64_t>(kStaticMaxTiles) * tile_elems) return RING_ERR_LIMIT;
   }
   if (total == 0) return RING_OK;
   if (!fused || (reinterpret_cast<uintptr_t>(fused) & 15u)) return RING_ERR_ARGUMENT;

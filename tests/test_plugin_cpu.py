@@ -83,6 +83,35 @@ def test_host_tables_agree_with_oracle(oracle):
     assert ring_abi.temp_elements(5, 0) == 0
 
 
+def test_sizes_that_do_not_fit_are_refused_not_wrapped():
+    """Element counts whose sum or product wraps 64 bits come back as an error
+    from the host-side tables and from the two fusion entry points that add
+    counts up, before anything is allocated or launched (no GPU needed)."""
+    L = ring_abi.lib()
+    top = 2 ** 64 - 1
+    with pytest.raises(ring_abi.RingError):
+        ring_abi.allgather_table([top // 2, top // 2], 8)            # rows x elements per row wraps
+    with pytest.raises(ring_abi.RingError):
+        ring_abi.allgather_table([top // 2, top // 2 + 2], 1)        # the sum of the rows wraps
+    assert ring_abi.allgather_table([top // 4, 1], 2) == [0, 2 * (top // 4)]
+    # a fusion plan over tensors whose counts add up past 64 bits (the pointers are never dereferenced:
+    # the call is refused while it looks at the sizes)
+    ptrs = (ctypes.c_void_p * 2)(4096, 8192)
+    plan = ctypes.c_void_p()
+    for counts in ((top, 2), (top // 4, top // 4 + 1), (top // 8 + 1, top // 8 + 1)):
+        c = (ctypes.c_size_t * 2)(*counts)
+        assert L.ring_fusion_plan_create(ptrs, c, 2, ring_abi.F32, ctypes.byref(plan)) == 2, counts
+        assert not plan.value
+    # the allocation-free entry point: beyond its stated size it says so, also when the sum wraps
+    for counts in ((2, top), (top, top), (2 ** 40, 1)):
+        c = (ctypes.c_size_t * 2)(*counts)
+        assert L.ring_fusion_run_static(0, ptrs, c, 2, ring_abi.F32, ctypes.c_void_p(4096), 0, None) == 5, counts
+    # the segment table and the temp size of a count at the top of the range
+    sizes, starts = ring_abi.segment_table(top, 4)
+    assert sum(sizes) == top and starts[3] + sizes[3] == top
+    assert ring_abi.temp_elements(top, 3) == top // 3
+
+
 def test_schedule_is_the_reference_index_algebra():
     # ring.h:184-185, 212-213, 280-281
     for n in (2, 3, 8):
