@@ -121,6 +121,9 @@ typedef void* (*mpic_alloc_fn)(void* user, int dtype, int ndims, const int64_t* 
  * matched by across ranks (mpi_ops.cc:1062, 1127-1131); `device`: "CPU"/"GPU". */
 int mpic_context_create(mpic_world* world, int rank, const char* op, const char* node_name,
                         const char* device, mpic_alloc_fn alloc, void* user, mpic_context** ctx);
+/* An input tensor: at most 8 dimensions, none negative, and a size in bytes that
+ * fits 63 bits (INVALID_ARGUMENT otherwise, here and for the tensors of
+ * mpic_allreduce_batch / mpic_batch_create). */
 int mpic_context_add_input(mpic_context* ctx, int dtype, int ndims, const int64_t* dims,
                            const void* data, int host_memory);
 /* Fuses the graph's tf.div(output, divisor) consumer into this node: the

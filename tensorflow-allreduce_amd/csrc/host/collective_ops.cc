@@ -970,6 +970,20 @@ int Fail(const Status& s) {
 // =============================================================================
 // C interface
 // =============================================================================
+// The dimensions an embedder hands over: none negative, and a byte size that
+// fits 63 bits (8-byte elements at most), so that no size computed from them
+// wraps.
+static bool DimsFit(const int64_t* dims, int ndims) {
+  uint64_t elements = 1;
+  for (int i = 0; i < ndims; i++) {
+    if (dims[i] < 0) return false;
+    const uint64_t d = static_cast<uint64_t>(dims[i]);
+    if (d != 0 && elements > (static_cast<uint64_t>(INT64_MAX) / 8) / d) return false;
+    elements *= d;
+  }
+  return true;
+}
+
 struct mpic_context {
   std::unique_ptr<mpic::OpKernelContext> ctx;
   std::unique_ptr<mpic::OpKernel> kernel;
@@ -1122,6 +1136,7 @@ int mpic_context_create(mpic_world* world, int rank, const char* op, const char*
 int mpic_context_add_input(mpic_context* c, int dtype, int ndims, const int64_t* dims, const void* data,
                            int host_memory) {
   if (!c || c->started || ndims < 0 || ndims > 8 || (ndims > 0 && !dims)) return MPIC_INVALID_ARGUMENT;
+  if (!DimsFit(dims, ndims)) return MPIC_INVALID_ARGUMENT;
   std::vector<int64_t> d(dims, dims + ndims);
   c->ctx->AddInput(mpic::Tensor(static_cast<mpic::DataType>(dtype), mpic::TensorShape(d), const_cast<void*>(data),
                                 host_memory != 0));
@@ -1207,7 +1222,8 @@ int mpic_allreduce_batch(mpic_world* world, int rank, int k, const char* const* 
   if (!kdef) return MPIC_NOT_FOUND;
   size_t at = 0;
   for (int j = 0; j < k; j++) {
-    if (ndims[j] < 0 || ndims[j] > 8 || (ndims[j] > 0 && !dims) || !node_names[j]) {
+    if (ndims[j] < 0 || ndims[j] > 8 || (ndims[j] > 0 && !dims) || !node_names[j] ||
+        !DimsFit(dims + at, ndims[j])) {
       for (int i = 0; i < j; i++) { delete contexts[i]; contexts[i] = nullptr; }
       return MPIC_INVALID_ARGUMENT;
     }
@@ -1283,7 +1299,8 @@ int mpic_batch_create(mpic_world* world, int rank, int k, const char* const* nod
   b->rank = rank;
   size_t at = 0;
   for (int j = 0; j < k; j++) {
-    if (ndims[j] < 0 || ndims[j] > 8 || (ndims[j] > 0 && !dims) || !node_names[j]) return MPIC_INVALID_ARGUMENT;
+    if (ndims[j] < 0 || ndims[j] > 8 || (ndims[j] > 0 && !dims) || !node_names[j] || !DimsFit(dims + at, ndims[j]))
+      return MPIC_INVALID_ARGUMENT;
     mpic::OpKernelConstruction construction(*node_names[j] ? node_names[j] : "MPIAllreduce");
     b->kernels.emplace_back(kdef->factory(&construction));
     void* out = outputs[j];

@@ -628,6 +628,38 @@ def test_a_batch_outlives_its_world_but_cannot_be_submitted():
     assert L.mpic_batch_destroy(batches[1]) == _plugin.OK      # after its world
 
 
+def test_dimensions_that_are_negative_or_do_not_fit_are_refused():
+    """mpic_context_add_input, mpic_allreduce_batch and mpic_batch_create take dimensions from the
+    embedder: a negative one, or a shape whose byte size wraps, is INVALID_ARGUMENT before anything is
+    filed (no GPU needed: nothing is computed)."""
+    L = _plugin.load_library()
+    w = ctypes.c_void_p()
+    assert L.mpic_world_create(2, ctypes.byref(w)) == 0
+    try:
+        c = ctypes.c_void_p()
+        assert L.mpic_context_create(w, 0, b"MPIAllreduce", b"x", b"GPU", _plugin.ALLOC_FN(0), None, ctypes.byref(c)) == 0
+        for dims in ((-1,), (4, -2), (2 ** 40, 2 ** 40), (2 ** 62, 2), (2 ** 60,)):
+            d = (ctypes.c_int64 * len(dims))(*dims)
+            assert L.mpic_context_add_input(c, _plugin.DT_FLOAT, len(dims), d, ctypes.c_void_p(4096), 0) == _plugin.INVALID_ARGUMENT, dims
+        d = (ctypes.c_int64 * 2)(2 ** 30, 2 ** 29)                  # 2^59 elements: the largest that still fits
+        assert L.mpic_context_add_input(c, _plugin.DT_FLOAT, 2, d, ctypes.c_void_p(4096), 0) == 0
+        assert L.mpic_context_destroy(c) == 0
+        names = (ctypes.c_char_p * 2)(b"a", b"b")
+        dtypes = (ctypes.c_int * 2)(_plugin.DT_FLOAT, _plugin.DT_FLOAT)
+        ndims = (ctypes.c_int * 2)(1, 2)
+        ptrs = (ctypes.c_void_p * 2)(4096, 8192)
+        for dims in ((4, 3, -1), (4, 2 ** 40, 2 ** 40)):
+            d = (ctypes.c_int64 * 3)(*dims)
+            contexts = (ctypes.c_void_p * 2)()
+            assert L.mpic_allreduce_batch(w, 0, 2, names, dtypes, ndims, d, ptrs, ptrs, 0, contexts) == _plugin.INVALID_ARGUMENT
+            assert not contexts[0] and not contexts[1]
+            batch = ctypes.c_void_p()
+            assert L.mpic_batch_create(w, 0, 2, names, dtypes, ndims, d, ptrs, ptrs, 0, ctypes.byref(batch)) == _plugin.INVALID_ARGUMENT
+            assert not batch.value
+    finally:
+        assert L.mpic_world_destroy(w) == 0
+
+
 def test_a_batch_that_fails_gives_its_node_names_back():
     """An entry the plugin cannot describe (more than 8 dimensions) fails the whole allreduce_batch
     call and files nothing; the auto-generated node names it took are given back, so the rank's
