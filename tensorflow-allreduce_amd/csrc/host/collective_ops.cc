@@ -710,6 +710,20 @@ void EnqueueTensorCollective(mpic_world* w, CollectiveOpRecord record, MPIReques
   if (wake) w->work_cv.notify_one();
 }
 
+// Dimensions that come from outside (an embedder's tensors, an allgather's
+// sizes): none negative, and a byte size that fits 63 bits (8-byte elements at
+// most), so that no size computed from them wraps.
+bool DimsFit(const int64_t* dims, int ndims) {
+  uint64_t elements = 1;
+  for (int i = 0; i < ndims; i++) {
+    if (dims[i] < 0) return false;
+    const uint64_t d = static_cast<uint64_t>(dims[i]);
+    if (d != 0 && elements > (static_cast<uint64_t>(INT64_MAX) / 8) / d) return false;
+    elements *= d;
+  }
+  return true;
+}
+
 mpic_world* WorldOf(OpKernelContext* context) { return static_cast<mpic_world*>(context->world()); }
 
 // ---- ops -------------------------------------------------------------------------
@@ -908,10 +922,19 @@ class MPIAllgatherOp : public AsyncOpKernel {
               : errors::InvalidArgument("sizes must be an int64 host tensor with one entry per rank."),
           done);
       const int64_t* sizing_array = static_cast<const int64_t*>(sizing_tensor->data());
+      bool sizes_fit = true;
       for (int i = 0; i < world->size; i++) {
+        sizes_fit = sizes_fit && sizing_array[i] >= 0 &&
+                    static_cast<uint64_t>(sizing_array[i]) <= static_cast<uint64_t>(INT64_MAX) / 8 - output_first_dim;
+        if (!sizes_fit) break;
         record.sizes_vec.push_back(static_cast<size_t>(sizing_array[i]));
         output_first_dim += static_cast<size_t>(sizing_array[i]);
       }
+      OP_REQUIRES_OK_ASYNC(
+          context,
+          sizes_fit ? Status::OK()
+                    : errors::InvalidArgument("sizes must be non-negative and add up to a tensor's first dimension."),
+          done);
     }
 
     record.dtype = TF_MPI_INVALID_TYPE;
@@ -920,6 +943,11 @@ class MPIAllgatherOp : public AsyncOpKernel {
     TensorShape output_shape;
     output_shape.AddDim(static_cast<int64_t>(output_first_dim));
     for (int i = 1; i < input_tensor->shape().dims(); i++) output_shape.AddDim(input_tensor->dim_size(i));
+    OP_REQUIRES_OK_ASYNC(context,
+                         DimsFit(output_shape.dim_sizes().data(), output_shape.dims())
+                             ? Status::OK()
+                             : errors::InvalidArgument("the gathered tensor is too large."),
+                         done);
     Tensor* output_tensor = nullptr;
     OP_REQUIRES_OK_ASYNC(context,
                          context->allocate_output(0, output_shape, input_tensor->dtype(), false, &output_tensor), done);
@@ -970,20 +998,6 @@ int Fail(const Status& s) {
 // =============================================================================
 // C interface
 // =============================================================================
-// The dimensions an embedder hands over: none negative, and a byte size that
-// fits 63 bits (8-byte elements at most), so that no size computed from them
-// wraps.
-static bool DimsFit(const int64_t* dims, int ndims) {
-  uint64_t elements = 1;
-  for (int i = 0; i < ndims; i++) {
-    if (dims[i] < 0) return false;
-    const uint64_t d = static_cast<uint64_t>(dims[i]);
-    if (d != 0 && elements > (static_cast<uint64_t>(INT64_MAX) / 8) / d) return false;
-    elements *= d;
-  }
-  return true;
-}
-
 struct mpic_context {
   std::unique_ptr<mpic::OpKernelContext> ctx;
   std::unique_ptr<mpic::OpKernel> kernel;
@@ -1136,7 +1150,7 @@ int mpic_context_create(mpic_world* world, int rank, const char* op, const char*
 int mpic_context_add_input(mpic_context* c, int dtype, int ndims, const int64_t* dims, const void* data,
                            int host_memory) {
   if (!c || c->started || ndims < 0 || ndims > 8 || (ndims > 0 && !dims)) return MPIC_INVALID_ARGUMENT;
-  if (!DimsFit(dims, ndims)) return MPIC_INVALID_ARGUMENT;
+  if (!mpic::DimsFit(dims, ndims)) return MPIC_INVALID_ARGUMENT;
   std::vector<int64_t> d(dims, dims + ndims);
   c->ctx->AddInput(mpic::Tensor(static_cast<mpic::DataType>(dtype), mpic::TensorShape(d), const_cast<void*>(data),
                                 host_memory != 0));
@@ -1223,7 +1237,7 @@ int mpic_allreduce_batch(mpic_world* world, int rank, int k, const char* const* 
   size_t at = 0;
   for (int j = 0; j < k; j++) {
     if (ndims[j] < 0 || ndims[j] > 8 || (ndims[j] > 0 && !dims) || !node_names[j] ||
-        !DimsFit(dims + at, ndims[j])) {
+        !mpic::DimsFit(dims + at, ndims[j])) {
       for (int i = 0; i < j; i++) { delete contexts[i]; contexts[i] = nullptr; }
       return MPIC_INVALID_ARGUMENT;
     }
@@ -1299,7 +1313,7 @@ int mpic_batch_create(mpic_world* world, int rank, int k, const char* const* nod
   b->rank = rank;
   size_t at = 0;
   for (int j = 0; j < k; j++) {
-    if (ndims[j] < 0 || ndims[j] > 8 || (ndims[j] > 0 && !dims) || !node_names[j] || !DimsFit(dims + at, ndims[j]))
+    if (ndims[j] < 0 || ndims[j] > 8 || (ndims[j] > 0 && !dims) || !node_names[j] || !mpic::DimsFit(dims + at, ndims[j]))
       return MPIC_INVALID_ARGUMENT;
     mpic::OpKernelConstruction construction(*node_names[j] ? node_names[j] : "MPIAllreduce");
     b->kernels.emplace_back(kdef->factory(&construction));

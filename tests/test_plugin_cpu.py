@@ -660,6 +660,34 @@ def test_dimensions_that_are_negative_or_do_not_fit_are_refused():
         assert L.mpic_world_destroy(w) == 0
 
 
+def test_allgather_sizes_that_are_negative_or_do_not_fit_are_refused():
+    """MPIAllgather's `sizes` input comes from the embedder (the reference takes it from the sizing
+    pre-pass, mpi_ops.py:152-160): a negative entry, or entries whose gathered tensor would not fit,
+    end the op with InvalidArgument before anything is filed."""
+    L = _plugin.load_library()
+    w = ctypes.c_void_p()
+    assert L.mpic_world_create(2, ctypes.byref(w)) == 0
+    try:
+        init = ctypes.c_void_p()
+        assert L.mpic_context_create(w, 0, b"MPIInit", b"MPIInit", b"CPU", _plugin.ALLOC_FN(0), None, ctypes.byref(init)) == 0
+        assert L.mpic_context_compute(init) == 0 and L.mpic_context_wait(init) == 0 and L.mpic_context_destroy(init) == 0
+        for sizes, message in (((3, -1), b"non-negative"), ((2 ** 62, 2 ** 62), b"non-negative"),
+                               ((2 ** 40, 2 ** 40), b"too large")):
+            c = ctypes.c_void_p()
+            assert L.mpic_context_create(w, 0, b"MPIAllgather", b"g", b"GPU", _plugin.ALLOC_FN(0), None, ctypes.byref(c)) == 0
+            dims = (ctypes.c_int64 * 2)(3, 2 ** 20)
+            assert L.mpic_context_add_input(c, _plugin.DT_FLOAT, 2, dims, ctypes.c_void_p(4096), 0) == 0
+            host_sizes = (ctypes.c_int64 * 2)(*sizes)
+            one = (ctypes.c_int64 * 1)(2)
+            assert L.mpic_context_add_input(c, _plugin.DT_INT64, 1, one, host_sizes, 1) == 0
+            assert L.mpic_context_compute(c) == 0
+            assert L.mpic_context_wait(c) == _plugin.INVALID_ARGUMENT, sizes
+            assert message in L.mpic_context_message(c), (sizes, L.mpic_context_message(c))
+            assert L.mpic_context_destroy(c) == 0
+    finally:
+        assert L.mpic_world_destroy(w) == 0
+
+
 def test_a_batch_that_fails_gives_its_node_names_back():
     """An entry the plugin cannot describe (more than 8 dimensions) fails the whole allreduce_batch
     call and files nothing; the auto-generated node names it took are given back, so the rank's
