@@ -132,7 +132,8 @@ def test_plugin_over_the_emulated_kernels_under_sanitizers(sanitizer):
                                         "-o", exe, os.path.join(ROOT, "tests", "cpp", "plugin_emulation_test.cc")] +
          [os.path.join(host, f) for f in ("framework.cc", "wire.cc", "ring_driver.cc", "transport.cc", "collective_ops.cc")] +
          [obj, oracle_obj])
-    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0", TSAN_OPTIONS="halt_on_error=1:report_signal_unsafe=0")
+    # (AddressSanitizer's leak check is on: what a world, a batch or a plan allocates goes when it is destroyed)
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1", TSAN_OPTIONS="halt_on_error=1:report_signal_unsafe=0")
     out = _run([exe], timeout=900, env=env)
     assert "plugin emulation: ok" in out, out[-4000:]
 
