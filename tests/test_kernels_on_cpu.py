@@ -73,10 +73,20 @@ def test_kernels_under_sanitizers_on_the_cpu():
     exe = os.path.join(BUILD, "kernel_emulation_test")
     _run([clang] + _flags("asan") + ["-I", SHIM, "-I", os.path.join(ROOT, "include"), "-o", exe,
                                      os.path.join(ROOT, "tests", "cpp", "kernel_emulation_test.cc"), obj])
+    # The same cases once more under ThreadSanitizer, for one element type: the lanes of a workgroup are
+    # threads and __syncthreads a real barrier, so a table in LDS that is read without a barrier behind its
+    # writes is a data race it reports.
+    tsan_exe = os.path.join(BUILD, "kernel_emulation_test_tsan")
+    _run([clang] + _flags("tsan") + ["-I", SHIM, "-I", os.path.join(ROOT, "include"), "-o", tsan_exe,
+                                     os.path.join(ROOT, "tests", "cpp", "kernel_emulation_test.cc"),
+                                     _kernel_library_for_the_cpu(clang, "tsan")])
+    env = dict(os.environ, TSAN_OPTIONS="halt_on_error=1:report_signal_unsafe=0")
     # one process per element type, side by side: the stand-in runs a workgroup's lanes as OS threads
     # and spends its time handing them work
     procs = [(t, subprocess.Popen([exe, t], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True))
              for t in ("float32", "int32", "int64")]
+    procs.append(("float32 under ThreadSanitizer",
+                  subprocess.Popen([tsan_exe, "float32"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env)))
     for t, proc in procs:
         try:
             out, _ = proc.communicate(timeout=900)
