@@ -54,7 +54,9 @@ struct CommunicationDoneCallback {
 // mpi_ops.cc:123-153
 struct CollectiveOpRecord {
   int rank = 0;                   // the (virtual) rank performing this piece of the op
-  std::string name;               // node name: the key collectives are matched by
+  // node name: the key collectives are matched by. The kernel's own string (the node outlives its
+  // execution, op_kernel.h:187-189), not a copy per execution.
+  const std::string* name = nullptr;
   OpKernelContext* context = nullptr;
   MPIDataType dtype = TF_MPI_INVALID_TYPE;
   const Tensor* in_t = nullptr;
@@ -456,7 +458,7 @@ void PerformFusedAllreduce(mpic_world* w, const std::vector<std::string>& names,
     for (auto& kv : rec) {
       if (kv.second.divisor != rec.begin()->second.divisor)
         status = errors::FailedPrecondition("Mismatched fused divisors: ranks asked for different divisions of " +
-                                            kv.second.name + ".");
+                                            *kv.second.name + ".");
     }
     uniform = uniform && rec.begin()->second.divisor == divisor;
   }
@@ -697,9 +699,9 @@ void EnqueueTensorCollective(mpic_world* w, CollectiveOpRecord record, MPIReques
   {
     std::lock_guard<std::mutex> guard(w->mu);
     // the MPIRequest of mpi_ops.cc:855-863, written straight into its wire form
-    AppendRequestFrame(&w->message_bytes, record.rank, rtype, record.dtype, record.name,
+    AppendRequestFrame(&w->message_bytes, record.rank, rtype, record.dtype, *record.name,
                        record.in_t->shape().dim_sizes());
-    RankRecords& by_rank = w->tensor_table[record.name];
+    RankRecords& by_rank = w->tensor_table[*record.name];
     if (by_rank.empty()) by_rank.reserve(static_cast<size_t>(w->expected_requests()));
     const int rank = record.rank;
     by_rank[rank] = std::move(record);
@@ -847,7 +849,7 @@ class MPIAllreduceOp : public AsyncOpKernel {
         done);
 
     record.rank = context->rank();
-    record.name = name();
+    record.name = &name();
     record.context = context;
     record.in_t = input_tensor;
     record.out_t = output_tensor;
@@ -901,7 +903,7 @@ class MPIAllgatherOp : public AsyncOpKernel {
 
     CollectiveOpRecord record;
     record.rank = context->rank();
-    record.name = name();
+    record.name = &name();
     record.context = context;
     record.in_t = input_tensor;
     record.on_gpu = IsGPUDevice<Device>() && !input_tensor->host_memory();
