@@ -540,10 +540,11 @@ void PerformReady(mpic_world* w, const std::vector<std::string>& ready) {
   // Each response goes through its wire form, as it would to ranks in other
   // processes (mpi_ops.cc:727-739).
   std::vector<MPIResponse> responses;
+  responses.reserve(ready.size());
   for (const std::string& name : ready) {
     MPIResponse received;
     if (received.ParseFromString(ConstructMPIResponse(&w->message_table, name).SerializeAsString()))
-      responses.push_back(received);
+      responses.push_back(std::move(received));
   }
   const WorldOptions opt = SnapshotOptions(w);
   const bool fusing = opt.fusion_bytes > 0 && opt.fusion_buffer && w->real_rank < 0 && w->size > 1;
